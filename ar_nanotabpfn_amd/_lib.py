@@ -1,0 +1,169 @@
+"""ctypes binding of ``libartab_attention.so`` (the C ABI in ``include/artab_attention.h``).
+
+There is no CPU fallback: if the shared library has not been built the first use
+raises ``RuntimeError`` naming the build command, and tensors that are not on a
+HIP device are rejected.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libartab_attention.so")
+
+ARTAB_BF16, ARTAB_F16, ARTAB_F32 = 0, 1, 2
+IMPL_AUTO, IMPL_PORTABLE, IMPL_MFMA = 0, 1, 2
+
+ARTAB_ERR_NULL_POINTER = -1
+ARTAB_ERR_BAD_SHAPE = -2
+ARTAB_ERR_BAD_STRIDE = -3
+ARTAB_ERR_UNSUPPORTED = -4
+ARTAB_ERR_WORKSPACE = -5
+ARTAB_ERR_CAPACITY = -6
+ARTAB_ERR_LAUNCH = -7
+
+_DTYPE_CODE = {torch.bfloat16: ARTAB_BF16, torch.float16: ARTAB_F16, torch.float32: ARTAB_F32}
+
+
+class ArtabView(ctypes.Structure):
+    _fields_ = [
+        ("data", ctypes.c_void_p),
+        ("stride_b", ctypes.c_int64),
+        ("stride_h", ctypes.c_int64),
+        ("stride_n", ctypes.c_int64),
+    ]
+
+
+_VP = ctypes.POINTER(ArtabView)
+_i, _f, _p, _sz, _i64 = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int64
+
+# name -> (restype, argtypes); every symbol declared in include/artab_attention.h
+SIGNATURES = {
+    "artab_version": (_i, []),
+    "artab_status_string": (ctypes.c_char_p, [_i]),
+    "artab_last_error": (ctypes.c_char_p, []),
+    "artab_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
+    "artab_context_attention": (_i, [_VP, _VP, _VP, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _p, _sz, _i, _p]),
+    "artab_decode_attention": (
+        _i,
+        [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p, _sz, _i, _p],
+    ),
+    "artab_teacher_forcing_attention": (_i, [_VP, _VP, _VP, _VP, _VP, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
+    "artab_prefill_attention": (_i, [_VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
+    "artab_buffer_attention": (_i, [_VP, _VP, _VP, _p, _i64, _i64, _i64, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _p]),
+    "artab_merge_attention_outputs": (_i, [_VP, _p, _VP, _p, _VP, _i, _i, _i, _i, _i, _p]),
+}
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def library_built() -> bool:
+    return os.path.exists(LIB_PATH)
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library once; raise loudly when it is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not library_built():
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: the HIP extension has not been built. "
+            "Build it with `python -m ar_nanotabpfn_amd.build_ext` (needs hipcc, targets gfx950). "
+            "There is no CPU fallback for the attention path."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    if lib.artab_version() != 1:
+        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.artab_version()} != 1; rebuild the extension")
+    _lib = lib
+    return lib
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise ValueError(f"unsupported dtype {dtype}; expected bfloat16, float16 or float32") from None
+
+
+def require_device(*tensors: Optional[torch.Tensor]) -> torch.device:
+    """All given tensors must live on one HIP device; returns it."""
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(
+                "ar_nanotabpfn_amd attention runs on a HIP device only (got a tensor on "
+                f"{t.device}); there is no CPU implementation in this package."
+            )
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise ValueError(f"tensors on different devices: {dev} and {t.device}")
+    if dev is None:
+        raise ValueError("no tensor given")
+    return dev
+
+
+def view4(t: Optional[torch.Tensor], shared_batch: bool = False) -> Optional[ArtabView]:
+    """Describe a ``[B,H,N,Dh]`` tensor (or ``[H,N,Dh]`` with ``shared_batch``) for the C ABI."""
+    if t is None:
+        return None
+    if shared_batch:
+        if t.dim() != 3:
+            raise ValueError(f"expected a [H,N,Dh] tensor, got {tuple(t.shape)}")
+        if t.shape[-1] > 1 and t.stride(-1) != 1:
+            raise ValueError("head_dim axis must be contiguous")
+        return ArtabView(t.data_ptr(), 0, t.stride(0), t.stride(1))
+    if t.dim() != 4:
+        raise ValueError(f"expected a [B,H,N,Dh] tensor, got {tuple(t.shape)}")
+    if t.shape[-1] > 1 and t.stride(-1) != 1:
+        raise ValueError("head_dim axis must be contiguous")
+    return ArtabView(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+
+
+def ref(v: Optional[ArtabView]):
+    return ctypes.byref(v) if v is not None else None
+
+
+def current_stream(device: torch.device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def check(status: int) -> None:
+    """Map a negative status to the exception the reference raises for that condition:
+    ``ValueError`` for shape/contract violations, ``RuntimeError`` for device-side
+    unavailability or launch failure."""
+    if status == 0:
+        return
+    lib = load()
+    msg = lib.artab_last_error().decode() or lib.artab_status_string(status).decode()
+    if status in (ARTAB_ERR_BAD_SHAPE, ARTAB_ERR_CAPACITY, ARTAB_ERR_BAD_STRIDE, ARTAB_ERR_NULL_POINTER):
+        raise ValueError(msg)
+    raise RuntimeError(msg)
+
+
+_workspaces = {}
+
+
+def workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
+    """A float32 scratch tensor of at least ``nbytes`` on ``device`` (grown on demand,
+    reused between calls: consecutive launches on one stream are ordered)."""
+    if nbytes <= 0:
+        return None
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() * 4 < nbytes:
+        ws = torch.empty((nbytes + 3) // 4, device=device, dtype=torch.float32)
+        _workspaces[key] = ws
+    return ws

@@ -1,0 +1,350 @@
+"""Attention entry points of the AR-TabPFN inference path, served by HIP kernels.
+
+Host-side mirror of the reference's ``ar_tabpfn/model/triton_kernels.py``: the
+same callables with the same argument meaning and error behaviour, each a thin
+wrapper that describes its tensors to the C ABI (``include/artab_attention.h``)
+and launches on the current stream.  All arithmetic happens on the device;
+tensors that are not on a HIP device raise ``RuntimeError``.
+
+The ``use_triton`` flag of the reference selects between its Triton kernel and
+its eager PyTorch path.  Here it selects between the MFMA kernels (True, the
+default; used whenever dtype/head_dim allow) and the portable float32-arithmetic
+kernel (False).
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from . import _lib
+
+__all__ = [
+    "hip_available",
+    "triton_available",
+    "context_attention",
+    "triton_context_attention",
+    "pytorch_context_attention",
+    "buffer_attention",
+    "pytorch_buffer_attention",
+    "teacher_forcing_buffer_attention",
+    "pytorch_teacher_forcing_buffer_attention",
+    "merge_attention_outputs",
+    "hybrid_attention",
+    "hybrid_teacher_forcing_attention",
+    "cross_attention",
+    "decode_attention",
+    "teacher_forcing_attention",
+    "prefill_attention",
+]
+
+
+def hip_available() -> bool:
+    """True when the HIP extension is built and a HIP device is visible."""
+    return _lib.library_built() and torch.cuda.is_available()
+
+
+def triton_available() -> bool:
+    """Availability probe under the reference's name (triton_kernels.py:527-529)."""
+    return hip_available()
+
+
+def _impl(use_triton: bool) -> int:
+    return _lib.IMPL_AUTO if use_triton else _lib.IMPL_PORTABLE
+
+
+def _alloc_out(q: Tensor) -> Tensor:
+    """Output ``[B,H,Lq,Dh]`` backed by ``[B,Lq,H,Dh]`` storage, so the caller's
+    ``out.transpose(1, 2).reshape(B, Lq, H*Dh)`` (inference.py:825) is a free view."""
+    B, H, Lq, Dh = q.shape
+    return torch.empty((B, Lq, H, Dh), device=q.device, dtype=q.dtype).transpose(1, 2)
+
+
+def _ctx_views(k_ctx: Tensor, v_ctx: Tensor):
+    if k_ctx.dim() == 3:
+        return _lib.view4(k_ctx, shared_batch=True), _lib.view4(v_ctx, shared_batch=True), k_ctx.shape[0], k_ctx.shape[1]
+    return _lib.view4(k_ctx), _lib.view4(v_ctx), k_ctx.shape[1], k_ctx.shape[2]
+
+
+def _workspace_for(q: Tensor, Nc: int):
+    B, H, Lq, Dh = q.shape
+    lib = _lib.load()
+    nbytes = lib.artab_workspace_bytes(B, H, Lq, Nc, Dh, _lib.dtype_code(q.dtype))
+    ws = _lib.workspace(q.device, nbytes)
+    if ws is None:
+        return None, 0
+    return ctypes.c_void_p(ws.data_ptr()), ws.numel() * 4
+
+
+def context_attention(
+    q: Tensor, k_ctx: Tensor, v_ctx: Tensor, scale: Optional[float] = None, use_triton: bool = True
+) -> Tuple[Tensor, Tensor]:
+    """Attention of ``q [B,H,Lq,D]`` over the context with log-sum-exp.
+
+    ``k_ctx``/``v_ctx``: ``[H,Nc,D]`` shared by the batch (triton_kernels.py:347-475,
+    :532-567) or ``[B,H,Nc,D]`` per dataset.  Returns ``out [B,H,Lq,D]`` (q's dtype)
+    and ``lse [B,H,Lq]`` float32.
+    """
+    dev = _lib.require_device(q, k_ctx, v_ctx)
+    lib = _lib.load()
+    B, H, Lq, Dh = q.shape
+    kv, vv, Hk, Nc = _ctx_views(k_ctx, v_ctx)
+    if Hk != H or k_ctx.shape[-1] != Dh or v_ctx.shape != k_ctx.shape:
+        raise ValueError(f"context K/V {tuple(k_ctx.shape)} do not match q {tuple(q.shape)}")
+    if k_ctx.dtype != q.dtype or v_ctx.dtype != q.dtype:
+        raise ValueError("q, k_ctx and v_ctx must share one dtype")
+    out = _alloc_out(q)
+    lse = torch.empty((B, H, Lq), device=dev, dtype=torch.float32)
+    ws_ptr, ws_bytes = _workspace_for(q, Nc)
+    qv, ov = _lib.view4(q), _lib.view4(out)
+    _lib.check(
+        lib.artab_context_attention(
+            _lib.ref(qv), _lib.ref(kv), _lib.ref(vv), _lib.ref(ov), ctypes.c_void_p(lse.data_ptr()),
+            B, H, Lq, Nc, Dh, float(scale) if scale is not None else 0.0, _lib.dtype_code(q.dtype),
+            ws_ptr, ws_bytes, _impl(use_triton), _lib.current_stream(dev),
+        )
+    )
+    return out, lse
+
+
+def triton_context_attention(q: Tensor, k_ctx: Tensor, v_ctx: Tensor, scale: Optional[float] = None):
+    """Name kept from triton_kernels.py:347-411; runs the MFMA kernel."""
+    return context_attention(q, k_ctx, v_ctx, scale=scale, use_triton=True)
+
+
+def pytorch_context_attention(q: Tensor, k_ctx: Tensor, v_ctx: Tensor, scale: Optional[float] = None):
+    """Name kept from triton_kernels.py:532-567; runs the portable float32 kernel."""
+    return context_attention(q, k_ctx, v_ctx, scale=scale, use_triton=False)
+
+
+def buffer_attention(
+    q: Tensor, k_buf: Tensor, v_buf: Tensor, mask: Optional[Tensor] = None, scale: Optional[float] = None
+) -> Tuple[Tensor, Tensor]:
+    """Per-trajectory attention over buffer K/V with an optional boolean mask
+    (True = attend, broadcastable to ``[B,H,Lq,Nb]``) and log-sum-exp
+    (triton_kernels.py:570-614).  Rows with no visible key: out 0, lse -inf."""
+    dev = _lib.require_device(q, k_buf, v_buf, mask)
+    lib = _lib.load()
+    B, H, Lq, Dh = q.shape
+    Nb = k_buf.shape[2]
+    if k_buf.shape != v_buf.shape or k_buf.shape[0] != B or k_buf.shape[1] != H or k_buf.shape[3] != Dh:
+        raise ValueError(f"buffer K/V {tuple(k_buf.shape)} do not match q {tuple(q.shape)}")
+    out = _alloc_out(q)
+    lse = torch.empty((B, H, Lq), device=dev, dtype=torch.float32)
+    mask_ptr, msb, msh, msq, keep = None, 0, 0, 0, None
+    if mask is not None and Nb > 0:
+        m = mask
+        if m.dtype != torch.uint8:
+            m = m.to(torch.uint8)  # before expanding: broadcast axes stay stride-0 views
+        while m.dim() < 4:
+            m = m.unsqueeze(0)
+        m = m.expand(B, H, Lq, Nb)
+        if m.stride(3) != 1:
+            m = m.contiguous()
+        keep = m
+        mask_ptr, msb, msh, msq = ctypes.c_void_p(m.data_ptr()), m.stride(0), m.stride(1), m.stride(2)
+    qv, ov = _lib.view4(q), _lib.view4(out)
+    kv = _lib.view4(k_buf) if Nb > 0 else None
+    vv = _lib.view4(v_buf) if Nb > 0 else None
+    _lib.check(
+        lib.artab_buffer_attention(
+            _lib.ref(qv), _lib.ref(kv), _lib.ref(vv), mask_ptr, msb, msh, msq, _lib.ref(ov),
+            ctypes.c_void_p(lse.data_ptr()), B, H, Lq, Nb, Dh,
+            float(scale) if scale is not None else 0.0, _lib.dtype_code(q.dtype), _lib.current_stream(dev),
+        )
+    )
+    del keep
+    return out, lse
+
+
+pytorch_buffer_attention = buffer_attention
+
+
+def _tf_mask(num_targets: int, device) -> Tensor:
+    """``[1,1,2Nt,Nt]`` teacher-forcing buffer mask (triton_kernels.py:620-637)."""
+    q_idx = torch.arange(2 * num_targets, device=device)
+    kv_idx = torch.arange(num_targets, device=device)
+    buffer_mask = kv_idx[None, :] <= q_idx[:, None]
+    target_mask = kv_idx[None, :] < (q_idx - num_targets)[:, None]
+    return torch.where((q_idx < num_targets)[:, None], buffer_mask, target_mask)[None, None]
+
+
+def teacher_forcing_buffer_attention(
+    q: Tensor, k_buf: Tensor, v_buf: Tensor, num_targets: int, scale: Optional[float] = None
+) -> Tuple[Tensor, Tensor]:
+    """Buffer part of teacher forcing with its LSE (triton_kernels.py:640-659)."""
+    if q.shape[2] != 2 * num_targets:
+        raise ValueError("Expected 2*num_targets queries for teacher forcing.")
+    if k_buf.shape[2] != num_targets:
+        raise ValueError("Expected buffer length to match num_targets.")
+    return buffer_attention(q, k_buf, v_buf, mask=_tf_mask(num_targets, q.device), scale=scale)
+
+
+pytorch_teacher_forcing_buffer_attention = teacher_forcing_buffer_attention
+
+
+def merge_attention_outputs(out_ctx: Tensor, lse_ctx: Tensor, out_buf: Tensor, lse_buf: Tensor) -> Tensor:
+    """Merge two partial attention outputs by their log-sum-exps (triton_kernels.py:478-524)."""
+    dev = _lib.require_device(out_ctx, lse_ctx, out_buf, lse_buf)
+    lib = _lib.load()
+    B, H, Lq, Dh = out_ctx.shape
+    if out_buf.shape != out_ctx.shape or lse_ctx.shape != (B, H, Lq) or lse_buf.shape != (B, H, Lq):
+        raise ValueError("merge_attention_outputs: shape mismatch")
+    if out_buf.dtype != out_ctx.dtype:
+        out_buf = out_buf.to(out_ctx.dtype)
+    la = lse_ctx.to(torch.float32).contiguous()
+    lb = lse_buf.to(torch.float32).contiguous()
+    out = _alloc_out(out_ctx)
+    av, bv, ov = _lib.view4(out_ctx), _lib.view4(out_buf), _lib.view4(out)
+    _lib.check(
+        lib.artab_merge_attention_outputs(
+            _lib.ref(av), ctypes.c_void_p(la.data_ptr()), _lib.ref(bv), ctypes.c_void_p(lb.data_ptr()),
+            _lib.ref(ov), B, H, Lq, Dh, _lib.dtype_code(out_ctx.dtype), _lib.current_stream(dev),
+        )
+    )
+    return out
+
+
+def decode_attention(
+    q: Tensor,
+    k_ctx: Tensor,
+    v_ctx: Tensor,
+    k_buf_cache: Optional[Tensor],
+    v_buf_cache: Optional[Tensor],
+    n_buf: int,
+    k_new: Optional[Tensor] = None,
+    v_new: Optional[Tensor] = None,
+    use_triton: bool = True,
+) -> Tensor:
+    """One decode step of row attention (inference.py:785-823) in one call.
+
+    ``q [B,H,Lq,D]`` with Lq in {1,2}; ``k_buf_cache``/``v_buf_cache`` are the
+    preallocated ``[B,H,cap,D]`` caches whose rows ``[0,n_buf)`` are valid.  With
+    ``k_new``/``v_new [B,H,1,D]`` the row is appended in place at slot ``n_buf`` and
+    all queries see it; the caller advances its cursor.  Raises ``ValueError`` for
+    Lq outside {1,2} (:765-768) and for a full cache (:247-250).
+    """
+    dev = _lib.require_device(q, k_ctx, v_ctx, k_buf_cache, v_buf_cache, k_new, v_new)
+    lib = _lib.load()
+    B, H, Lq, Dh = q.shape
+    if Lq not in (1, 2):
+        raise ValueError("Shared-context decode only supports N=1 (target) or N=2 (buffer, target).")
+    kv, vv, Hk, Nc = _ctx_views(k_ctx, v_ctx)
+    if Hk != H or k_ctx.shape[-1] != Dh:
+        raise ValueError(f"context K/V {tuple(k_ctx.shape)} do not match q {tuple(q.shape)}")
+    cap = k_buf_cache.shape[2] if k_buf_cache is not None else 0
+    out = _alloc_out(q)
+    ws_ptr, ws_bytes = _workspace_for(q, Nc)
+    qv, ov = _lib.view4(q), _lib.view4(out)
+    kbv, vbv = _lib.view4(k_buf_cache), _lib.view4(v_buf_cache)
+    knv, vnv = _lib.view4(k_new), _lib.view4(v_new)
+    _lib.check(
+        lib.artab_decode_attention(
+            _lib.ref(qv), _lib.ref(kv), _lib.ref(vv), _lib.ref(kbv), _lib.ref(vbv), _lib.ref(knv), _lib.ref(vnv),
+            _lib.ref(ov), B, H, Lq, Nc, int(n_buf), cap, Dh, 0.0, _lib.dtype_code(q.dtype),
+            ws_ptr, ws_bytes, _impl(use_triton), _lib.current_stream(dev),
+        )
+    )
+    return out
+
+
+def teacher_forcing_attention(
+    q: Tensor, k_ctx: Tensor, v_ctx: Tensor, k_buf: Tensor, v_buf: Tensor, num_targets: int,
+    use_triton: bool = True, return_lse: bool = False,
+):
+    """Teacher-forced attention with the mask as a tile schedule; context shared
+    ``[H,Nc,D]`` or per dataset ``[B,H,Nc,D]``."""
+    dev = _lib.require_device(q, k_ctx, v_ctx, k_buf, v_buf)
+    lib = _lib.load()
+    B, H, Lq, Dh = q.shape
+    if Lq != 2 * num_targets:
+        raise ValueError("Expected 2*num_targets queries for teacher forcing.")
+    if k_buf.shape[2] != num_targets:
+        raise ValueError("Expected buffer length to match num_targets.")
+    kv, vv, Hk, Nc = _ctx_views(k_ctx, v_ctx)
+    if Hk != H or k_ctx.shape[-1] != Dh:
+        raise ValueError(f"context K/V {tuple(k_ctx.shape)} do not match q {tuple(q.shape)}")
+    out = _alloc_out(q)
+    lse = torch.empty((B, H, Lq), device=dev, dtype=torch.float32) if return_lse else None
+    qv, ov, kbv, vbv = _lib.view4(q), _lib.view4(out), _lib.view4(k_buf), _lib.view4(v_buf)
+    _lib.check(
+        lib.artab_teacher_forcing_attention(
+            _lib.ref(qv), _lib.ref(kv), _lib.ref(vv), _lib.ref(kbv), _lib.ref(vbv), _lib.ref(ov),
+            ctypes.c_void_p(lse.data_ptr()) if lse is not None else None,
+            B, H, num_targets, Nc, Dh, 0.0, _lib.dtype_code(q.dtype), _impl(use_triton), _lib.current_stream(dev),
+        )
+    )
+    return (out, lse) if return_lse else out
+
+
+def prefill_attention(
+    q: Tensor, k: Tensor, v: Tensor, k_cache: Optional[Tensor] = None, v_cache: Optional[Tensor] = None,
+    use_triton: bool = True,
+) -> Tensor:
+    """Dense self-attention over the context rows plus the cache write
+    (inference.py:618-622, :672-676).  ``k_cache``/``v_cache``: ``[H,Nc',D]`` (shared:
+    batch entry 0 is stored) or ``[B,H,Nc',D]`` with Nc' >= Nc."""
+    dev = _lib.require_device(q, k, v, k_cache, v_cache)
+    lib = _lib.load()
+    B, H, Nc, Dh = q.shape
+    if k.shape != q.shape or v.shape != q.shape:
+        raise ValueError("prefill expects q, k, v of one shape [B,H,Nc,D]")
+    out = _alloc_out(q)
+    kcv = vcv = None
+    cache_batches = 0
+    if k_cache is not None:
+        shared = k_cache.dim() == 3
+        rows = k_cache.shape[1] if shared else k_cache.shape[2]
+        if rows < Nc:
+            raise ValueError(f"cache holds {rows} rows, context has {Nc}")
+        kcv, vcv = _lib.view4(k_cache, shared_batch=shared), _lib.view4(v_cache, shared_batch=shared)
+        cache_batches = 1 if shared else k_cache.shape[0]
+    qv, kv, vv, ov = _lib.view4(q), _lib.view4(k), _lib.view4(v), _lib.view4(out)
+    _lib.check(
+        lib.artab_prefill_attention(
+            _lib.ref(qv), _lib.ref(kv), _lib.ref(vv), _lib.ref(ov), _lib.ref(kcv), _lib.ref(vcv), cache_batches,
+            B, H, Nc, Dh, 0.0, _lib.dtype_code(q.dtype), _impl(use_triton), _lib.current_stream(dev),
+        )
+    )
+    return out
+
+
+def hybrid_attention(
+    q: Tensor, k_ctx: Tensor, v_ctx: Tensor, k_buf: Tensor, v_buf: Tensor,
+    buf_mask: Optional[Tensor] = None, use_triton: bool = True,
+) -> Tensor:
+    """Context attention + buffer attention + LSE merge (triton_kernels.py:705-755).
+
+    An empty buffer returns the context part alone (:735-741).  Without a mask and
+    with at most two queries this is one fused decode call; otherwise the three
+    device steps run one after another exactly as the reference composes them.
+    """
+    Lq = q.shape[2]
+    if k_buf.shape[2] == 0:
+        out, _ = context_attention(q, k_ctx, v_ctx, use_triton=use_triton)
+        return out
+    if buf_mask is None and Lq in (1, 2):
+        return decode_attention(q, k_ctx, v_ctx, k_buf, v_buf, k_buf.shape[2], use_triton=use_triton)
+    out_ctx, lse_ctx = context_attention(q, k_ctx, v_ctx, use_triton=use_triton)
+    out_buf, lse_buf = buffer_attention(q, k_buf, v_buf, mask=buf_mask)
+    return merge_attention_outputs(out_ctx, lse_ctx, out_buf, lse_buf)
+
+
+def hybrid_teacher_forcing_attention(
+    q: Tensor, k_ctx: Tensor, v_ctx: Tensor, k_buf: Tensor, v_buf: Tensor, num_targets: int,
+    use_triton: bool = True,
+) -> Tensor:
+    """Teacher-forcing attention (triton_kernels.py:662-702) as one kernel."""
+    if k_buf.shape[2] == 0:
+        out, _ = context_attention(q, k_ctx, v_ctx, use_triton=use_triton)
+        return out
+    return teacher_forcing_attention(q, k_ctx, v_ctx, k_buf, v_buf, num_targets, use_triton=use_triton)
+
+
+def cross_attention(q: Tensor, k_ctx: Tensor, v_ctx: Tensor, use_triton: bool = True) -> Tensor:
+    """Context attention without the LSE (triton_kernels.py:758-767)."""
+    out, _ = context_attention(q, k_ctx, v_ctx, use_triton=use_triton)
+    return out

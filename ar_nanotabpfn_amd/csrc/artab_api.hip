@@ -1,0 +1,578 @@
+// C ABI of the AR-TabPFN attention library for MI355X (gfx950): argument checks,
+// kernel selection and launches.  See include/artab_attention.h for the contract.
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/artab_attention.h"
+#include "common.h"
+#include "decode_buffer.h"
+#include "mfma_flash.h"
+#include "portable_kernels.h"
+
+namespace artab {
+
+static thread_local char g_err[512] = "";
+
+static int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+static inline int elem_size(int dtype) { return dtype == ARTAB_F32 ? 4 : 2; }
+
+static inline View dv(const artab_view *v) {
+    View r;
+    if (v) {
+        r.p = static_cast<char *>(v->data);
+        r.sb = v->stride_b;
+        r.sh = v->stride_h;
+        r.sn = v->stride_n;
+    } else {
+        r.p = nullptr;
+        r.sb = r.sh = r.sn = 0;
+    }
+    return r;
+}
+
+// Rows start on 16-byte boundaries and hold a whole number of 16-byte vectors.
+static inline bool vec_aligned(const artab_view *v, int dtype, int Dh) {
+    if (!v || !v->data) return true;
+    const int64_t per = 16 / elem_size(dtype);
+    return (reinterpret_cast<uintptr_t>(v->data) % 16 == 0) && (v->stride_b % per == 0) &&
+           (v->stride_h % per == 0) && (v->stride_n % per == 0) && (Dh % per == 0);
+}
+
+static inline bool elem_aligned(const artab_view *v, int dtype) {
+    return !v || !v->data || reinterpret_cast<uintptr_t>(v->data) % elem_size(dtype) == 0;
+}
+
+static int check_view(const artab_view *v, const char *name, int dtype, bool required) {
+    if (!v || !v->data) {
+        if (required) return fail(ARTAB_ERR_NULL_POINTER, "%s is NULL", name);
+        return ARTAB_OK;
+    }
+    if (!elem_aligned(v, dtype)) return fail(ARTAB_ERR_BAD_STRIDE, "%s is not aligned to its element size", name);
+    return ARTAB_OK;
+}
+
+static int check_common(int B, int H, int Lq, int Dh, int dtype) {
+    if (dtype != ARTAB_BF16 && dtype != ARTAB_F16 && dtype != ARTAB_F32)
+        return fail(ARTAB_ERR_UNSUPPORTED, "unknown dtype code %d", dtype);
+    if (B < 0 || H <= 0 || Lq < 0) return fail(ARTAB_ERR_BAD_SHAPE, "bad sizes B=%d H=%d Lq=%d", B, H, Lq);
+    if (Dh <= 0 || Dh > kPortableMaxDh)
+        return fail(ARTAB_ERR_UNSUPPORTED, "head_dim %d outside [1,%d]", Dh, kPortableMaxDh);
+    return ARTAB_OK;
+}
+
+static inline float resolve_scale(float scale, int Dh) {
+    return scale > 0.f ? scale : 1.0f / std::sqrt(static_cast<float>(Dh));
+}
+
+static inline bool mfma_shape_ok(int dtype, int Dh) {
+    return (dtype == ARTAB_BF16 || dtype == ARTAB_F16) && (Dh == 32 || Dh == 64 || Dh == 128);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Flash (MFMA) launch planning
+// ---------------------------------------------------------------------------------------------
+
+constexpr int kFlashBN = 64;
+constexpr int kTargetWorkgroups = 768;  // 3 per CU on a 256-CU part
+
+struct FlashPlan {
+    int BM;        // query rows per workgroup: 256, 128 or 64
+    int n_split;   // context slices
+    int kv_per_split;
+    int tiles_per_group;
+    int n_groups;
+    int G;
+};
+
+static FlashPlan plan_flash(int B, int H, int Lq, int Nc, int Dh, bool stacked, bool allow_split) {
+    FlashPlan pl;
+    pl.n_groups = stacked ? 1 : B;
+    pl.G = stacked ? B * Lq : Lq;
+    const int cands[3] = {256, 128, 64};
+    int pick = 64;
+    for (int ci = 0; ci < 3; ++ci) {
+        int bm = cands[ci];
+        if (Dh == 128 && bm == 256) continue;  // register budget: one 32-row block per wavefront
+        long wgs = static_cast<long>((pl.G + bm - 1) / bm) * pl.n_groups * H;
+        if (wgs >= kTargetWorkgroups) {
+            pick = bm;
+            break;
+        }
+    }
+    pl.BM = pick;
+    pl.tiles_per_group = (pl.G + pick - 1) / pick;
+    long base = static_cast<long>(pl.tiles_per_group) * pl.n_groups * H;
+    int n_split = 1;
+    if (allow_split && base < kTargetWorkgroups) {
+        int max_split = Nc / 256 > 0 ? Nc / 256 : 1;
+        int want = static_cast<int>((kTargetWorkgroups + base - 1) / base);
+        n_split = want < max_split ? want : max_split;
+        if (n_split > 64) n_split = 64;
+    }
+    int per = (Nc + n_split - 1) / n_split;
+    per = (per + kFlashBN - 1) / kFlashBN * kFlashBN;
+    if (per <= 0) per = kFlashBN;
+    pl.kv_per_split = per;
+    pl.n_split = (Nc + per - 1) / per;
+    if (pl.n_split < 1) pl.n_split = 1;
+    return pl;
+}
+
+template <typename T, int DH>
+static hipError_t launch_flash_bm(const FlashParams &P, int BM, hipStream_t stream) {
+    const int W = P.tiles_per_group * P.n_split;
+    const int n_kvg = P.H * P.n_groups;
+    const unsigned grid = static_cast<unsigned>(((n_kvg + 7) / 8) * W * 8);
+    if (grid == 0) return hipSuccess;
+    if constexpr (DH <= 64) {
+        if (BM == 256) {
+            hipLaunchKernelGGL((flash_kernel<T, DH, 2, 4, kFlashBN>), dim3(grid), dim3(256), 0, stream, P);
+            return hipGetLastError();
+        }
+    }
+    if (BM == 128) {
+        hipLaunchKernelGGL((flash_kernel<T, DH, 1, 4, kFlashBN>), dim3(grid), dim3(256), 0, stream, P);
+    } else {
+        hipLaunchKernelGGL((flash_kernel<T, DH, 1, 2, kFlashBN>), dim3(grid), dim3(128), 0, stream, P);
+    }
+    return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_flash(const FlashParams &P, int Dh, int BM, hipStream_t stream) {
+    switch (Dh) {
+        case 32: return launch_flash_bm<T, 32>(P, BM, stream);
+        case 64: return launch_flash_bm<T, 64>(P, BM, stream);
+        default: return launch_flash_bm<T, 128>(P, BM, stream);
+    }
+}
+
+static hipError_t launch_flash_dtype(const FlashParams &P, int dtype, int Dh, int BM, hipStream_t stream) {
+    return dtype == ARTAB_BF16 ? launch_flash<bf16_t>(P, Dh, BM, stream) : launch_flash<f16_t>(P, Dh, BM, stream);
+}
+
+template <typename T, int LQ>
+static hipError_t launch_decode_lq(const DecodeParams &P, int Dh, hipStream_t stream) {
+    const long pairs = static_cast<long>(P.B) * P.H;
+    if (pairs == 0) return hipSuccess;
+    dim3 grid(static_cast<unsigned>((pairs + kDecodeWaves - 1) / kDecodeWaves)), block(kDecodeWaves * 64);
+    switch (Dh) {
+        case 32: hipLaunchKernelGGL((decode_buffer_kernel<T, 32, LQ>), grid, block, 0, stream, P); break;
+        case 64: hipLaunchKernelGGL((decode_buffer_kernel<T, 64, LQ>), grid, block, 0, stream, P); break;
+        default: hipLaunchKernelGGL((decode_buffer_kernel<T, 128, LQ>), grid, block, 0, stream, P); break;
+    }
+    return hipGetLastError();
+}
+
+static hipError_t launch_decode(const DecodeParams &P, int dtype, int Dh, int Lq, hipStream_t stream) {
+    if (dtype == ARTAB_BF16)
+        return Lq == 1 ? launch_decode_lq<bf16_t, 1>(P, Dh, stream) : launch_decode_lq<bf16_t, 2>(P, Dh, stream);
+    return Lq == 1 ? launch_decode_lq<f16_t, 1>(P, Dh, stream) : launch_decode_lq<f16_t, 2>(P, Dh, stream);
+}
+
+static hipError_t launch_portable_dtype(const PortableParams &P, int dtype, hipStream_t stream) {
+    switch (dtype) {
+        case ARTAB_BF16: return launch_portable<bf16_t>(P, stream);
+        case ARTAB_F16: return launch_portable<f16_t>(P, stream);
+        default: return launch_portable<float>(P, stream);
+    }
+}
+
+// Combine split-context partials of arbitrary Lq into the final output: one thread
+// per (row, 4 output elements).
+struct CombineParams {
+    View out;
+    const float *part_o, *part_lse;
+    float *lse;
+    long rows;
+    int H, Lq, Dh, n_split;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void combine_kernel(CombineParams P) {
+    const int per_row = P.Dh / 4;
+    long idx = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= P.rows * per_row) return;
+    long row = idx / per_row;
+    int d0 = static_cast<int>(idx % per_row) * 4;
+    float mx = -INFINITY;
+    for (int s = 0; s < P.n_split; ++s) mx = fmaxf(mx, P.part_lse[s * P.rows + row]);
+    float wsum = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < P.n_split; ++s) {
+        float w = expf(P.part_lse[s * P.rows + row] - mx);
+        f32x4 o = *reinterpret_cast<const f32x4 *>(P.part_o + (s * P.rows + row) * P.Dh + d0);
+        wsum += w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] = fmaf(w, o[e], acc[e]);
+    }
+    int i = static_cast<int>(row % P.Lq);
+    int h = static_cast<int>((row / P.Lq) % P.H);
+    long b = row / (static_cast<long>(P.Lq) * P.H);
+    T *orow = view_row<T>(P.out, b, h, i) + d0;
+    float inv = 1.f / wsum;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) orow[e] = from_f32<T>(acc[e] * inv);
+    if (P.lse && d0 == 0) P.lse[row] = mx + logf(wsum);
+}
+
+static size_t split_workspace_bytes(long rows, int Dh, int n_split) {
+    return static_cast<size_t>(n_split) * static_cast<size_t>(rows) * (Dh + 1) * sizeof(float);
+}
+
+}  // namespace artab
+
+using namespace artab;
+
+#define ARTAB_TRY(expr)                 \
+    do {                                \
+        int rc__ = (expr);              \
+        if (rc__ != ARTAB_OK) return rc__; \
+    } while (0)
+
+static int launch_status(hipError_t e, const char *what) {
+    if (e == hipSuccess) return ARTAB_OK;
+    return fail(ARTAB_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+extern "C" {
+
+int artab_version(void) { return ARTAB_VERSION; }
+
+const char *artab_status_string(int status) {
+    switch (status) {
+        case ARTAB_OK: return "ok";
+        case ARTAB_ERR_NULL_POINTER: return "null pointer";
+        case ARTAB_ERR_BAD_SHAPE: return "bad shape";
+        case ARTAB_ERR_BAD_STRIDE: return "bad stride or alignment";
+        case ARTAB_ERR_UNSUPPORTED: return "unsupported dtype/head_dim/implementation";
+        case ARTAB_ERR_WORKSPACE: return "workspace missing or too small";
+        case ARTAB_ERR_CAPACITY: return "buffer cache capacity exceeded";
+        case ARTAB_ERR_LAUNCH: return "kernel launch failed";
+        default: return "unknown status";
+    }
+}
+
+const char *artab_last_error(void) { return g_err; }
+
+size_t artab_workspace_bytes(int B, int H, int Lq, int Nc, int Dh, int dtype) {
+    if (B <= 0 || H <= 0 || Lq <= 0 || Nc <= 0 || !mfma_shape_ok(dtype, Dh)) return 0;
+    // Upper bound over the two schedules (queries stacked over a shared context, or
+    // grouped per batch entry over per-dataset contexts).
+    FlashPlan a = plan_flash(B, H, Lq, Nc, Dh, /*stacked=*/true, /*allow_split=*/true);
+    FlashPlan b = plan_flash(B, H, Lq, Nc, Dh, /*stacked=*/false, /*allow_split=*/true);
+    const int n_split = a.n_split > b.n_split ? a.n_split : b.n_split;
+    return split_workspace_bytes(static_cast<long>(B) * H * Lq, Dh, n_split);
+}
+
+int artab_context_attention(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                            const artab_view *out, float *lse, int B, int H, int Lq, int Nc, int Dh,
+                            float scale, int dtype, void *workspace, size_t workspace_bytes, int impl,
+                            void *stream) {
+    ARTAB_TRY(check_common(B, H, Lq, Dh, dtype));
+    if (Nc < 1) return fail(ARTAB_ERR_BAD_SHAPE, "context attention needs Nc >= 1 (got %d)", Nc);
+    if (B == 0 || Lq == 0) return ARTAB_OK;
+    ARTAB_TRY(check_view(q, "q", dtype, true));
+    ARTAB_TRY(check_view(k_ctx, "k_ctx", dtype, true));
+    ARTAB_TRY(check_view(v_ctx, "v_ctx", dtype, true));
+    ARTAB_TRY(check_view(out, "out", dtype, true));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    scale = resolve_scale(scale, Dh);
+    const bool aligned = vec_aligned(q, dtype, Dh) && vec_aligned(k_ctx, dtype, Dh) &&
+                         vec_aligned(v_ctx, dtype, Dh) && vec_aligned(out, dtype, Dh);
+    bool use_mfma = impl != ARTAB_IMPL_PORTABLE && mfma_shape_ok(dtype, Dh) && aligned;
+    if (impl == ARTAB_IMPL_MFMA && !use_mfma)
+        return fail(ARTAB_ERR_UNSUPPORTED, "MFMA path needs bf16/f16, head_dim in {32,64,128}, 16-byte aligned rows");
+
+    if (!use_mfma) {
+        PortableParams P;
+        memset(&P, 0, sizeof(P));
+        P.q = dv(q); P.kc = dv(k_ctx); P.vc = dv(v_ctx); P.out = dv(out);
+        P.lse = lse;
+        P.B = B; P.H = H; P.Lq = Lq; P.Nc = Nc; P.Nb = 0;
+        P.new_row = -1; P.mode = kModePlain; P.Dh = Dh; P.scale = scale;
+        P.vec_ok = aligned ? 1 : 0;
+        return launch_status(launch_portable_dtype(P, dtype, st), "context attention (portable)");
+    }
+
+    const bool stacked = (k_ctx->stride_b == 0 && v_ctx->stride_b == 0) || B == 1;
+    const long rows = static_cast<long>(B) * H * Lq;
+    FlashPlan pl = plan_flash(B, H, Lq, Nc, Dh, stacked, /*allow_split=*/true);
+    if (pl.n_split > 1) {
+        size_t need = split_workspace_bytes(rows, Dh, pl.n_split);
+        if (!workspace || workspace_bytes < need) {
+            // Without a workspace the unsplit schedule is still correct, only less parallel.
+            pl.n_split = 1;
+            pl.kv_per_split = (Nc + kFlashBN - 1) / kFlashBN * kFlashBN;
+        }
+    }
+    FlashParams F;
+    memset(&F, 0, sizeof(F));
+    F.q = dv(q); F.kc = dv(k_ctx); F.vc = dv(v_ctx); F.out = dv(out);
+    F.lse = lse;
+    F.B = B; F.H = H; F.Lq = Lq; F.Nc = Nc;
+    F.G = pl.G; F.tiles_per_group = pl.tiles_per_group; F.n_groups = pl.n_groups;
+    F.n_split = pl.n_split; F.kv_per_split = pl.kv_per_split;
+    F.qscale = scale * kLog2e;
+    F.mode = kFlashContext;
+    if (pl.n_split > 1) {
+        F.part_o = static_cast<float *>(workspace);
+        F.part_lse = F.part_o + static_cast<size_t>(pl.n_split) * rows * Dh;
+    }
+    ARTAB_TRY(launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "context attention (mfma)"));
+    if (pl.n_split > 1) {
+        CombineParams C;
+        C.out = dv(out); C.part_o = F.part_o; C.part_lse = F.part_lse; C.lse = lse;
+        C.rows = rows; C.H = H; C.Lq = Lq; C.Dh = Dh; C.n_split = pl.n_split;
+        unsigned grid = static_cast<unsigned>((rows * (Dh / 4) + 255) / 256);
+        if (dtype == ARTAB_BF16)
+            hipLaunchKernelGGL((combine_kernel<bf16_t>), dim3(grid), dim3(256), 0, st, C);
+        else
+            hipLaunchKernelGGL((combine_kernel<f16_t>), dim3(grid), dim3(256), 0, st, C);
+        return launch_status(hipGetLastError(), "split combine");
+    }
+    return ARTAB_OK;
+}
+
+int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                           const artab_view *k_buf, const artab_view *v_buf, const artab_view *k_new,
+                           const artab_view *v_new, const artab_view *out, int B, int H, int Lq, int Nc,
+                           int n_buf, int buf_capacity, int Dh, float scale, int dtype, void *workspace,
+                           size_t workspace_bytes, int impl, void *stream) {
+    ARTAB_TRY(check_common(B, H, Lq, Dh, dtype));
+    if (Lq != 1 && Lq != 2)
+        return fail(ARTAB_ERR_BAD_SHAPE, "decode supports Lq=1 (target) or Lq=2 (buffer, target); got %d", Lq);
+    if (Nc < 1) return fail(ARTAB_ERR_BAD_SHAPE, "decode needs a prefilled context (Nc=%d)", Nc);
+    if (n_buf < 0 || buf_capacity < 0) return fail(ARTAB_ERR_BAD_SHAPE, "negative buffer length");
+    const bool k_new_given = k_new && k_new->data, v_new_given = v_new && v_new->data;
+    if (k_new_given != v_new_given) return fail(ARTAB_ERR_NULL_POINTER, "k_new and v_new must be given together");
+    const int has_new = k_new_given ? 1 : 0;
+    if (n_buf + has_new > buf_capacity)
+        return fail(ARTAB_ERR_CAPACITY, "buffer cache exceeded: %d rows + %d new > capacity %d", n_buf, has_new,
+                    buf_capacity);
+    if (B == 0) return ARTAB_OK;
+    ARTAB_TRY(check_view(q, "q", dtype, true));
+    ARTAB_TRY(check_view(k_ctx, "k_ctx", dtype, true));
+    ARTAB_TRY(check_view(v_ctx, "v_ctx", dtype, true));
+    ARTAB_TRY(check_view(out, "out", dtype, true));
+    const bool need_buf = n_buf + has_new > 0;
+    ARTAB_TRY(check_view(k_buf, "k_buf", dtype, need_buf));
+    ARTAB_TRY(check_view(v_buf, "v_buf", dtype, need_buf));
+    ARTAB_TRY(check_view(k_new, "k_new", dtype, false));
+    ARTAB_TRY(check_view(v_new, "v_new", dtype, false));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    scale = resolve_scale(scale, Dh);
+
+    const bool aligned = vec_aligned(q, dtype, Dh) && vec_aligned(k_ctx, dtype, Dh) &&
+                         vec_aligned(v_ctx, dtype, Dh) && vec_aligned(out, dtype, Dh) &&
+                         vec_aligned(k_buf, dtype, Dh) && vec_aligned(v_buf, dtype, Dh) &&
+                         vec_aligned(k_new, dtype, Dh) && vec_aligned(v_new, dtype, Dh);
+    const bool shared_ctx = (k_ctx->stride_b == 0 && v_ctx->stride_b == 0) || B == 1;
+    bool use_mfma = impl != ARTAB_IMPL_PORTABLE && mfma_shape_ok(dtype, Dh) && aligned && shared_ctx;
+    const long rows = static_cast<long>(B) * H * Lq;
+    FlashPlan pl;
+    size_t need_ws = 0;
+    if (use_mfma) {
+        pl = plan_flash(B, H, Lq, Nc, Dh, /*stacked=*/true, /*allow_split=*/true);
+        const bool direct = !need_buf && pl.n_split == 1;  // context pass writes the final output
+        need_ws = direct ? 0 : split_workspace_bytes(rows, Dh, pl.n_split);
+        if (need_ws && (!workspace || workspace_bytes < need_ws)) {
+            if (impl == ARTAB_IMPL_MFMA)
+                return fail(ARTAB_ERR_WORKSPACE, "decode needs %zu workspace bytes, got %zu", need_ws,
+                            workspace_bytes);
+            use_mfma = false;
+        }
+    } else if (impl == ARTAB_IMPL_MFMA) {
+        return fail(ARTAB_ERR_UNSUPPORTED,
+                    "MFMA decode needs bf16/f16, head_dim in {32,64,128}, aligned rows and a shared context");
+    }
+
+    if (!use_mfma) {
+        PortableParams P;
+        memset(&P, 0, sizeof(P));
+        P.q = dv(q); P.kc = dv(k_ctx); P.vc = dv(v_ctx); P.kb = dv(k_buf); P.vb = dv(v_buf);
+        P.knew = dv(k_new); P.vnew = dv(v_new); P.out = dv(out);
+        P.B = B; P.H = H; P.Lq = Lq; P.Nc = Nc; P.Nb = n_buf + has_new;
+        P.new_row = has_new ? n_buf : -1;
+        P.append = has_new;
+        P.mode = kModePlain; P.Dh = Dh; P.scale = scale;
+        P.vec_ok = aligned ? 1 : 0;
+        return launch_status(launch_portable_dtype(P, dtype, st), "decode attention (portable)");
+    }
+
+    FlashParams F;
+    memset(&F, 0, sizeof(F));
+    F.q = dv(q); F.kc = dv(k_ctx); F.vc = dv(v_ctx); F.out = dv(out);
+    F.B = B; F.H = H; F.Lq = Lq; F.Nc = Nc;
+    F.G = pl.G; F.tiles_per_group = pl.tiles_per_group; F.n_groups = pl.n_groups;
+    F.n_split = pl.n_split; F.kv_per_split = pl.kv_per_split;
+    F.qscale = scale * kLog2e;
+    F.mode = kFlashContext;
+    if (need_ws) {
+        F.part_o = static_cast<float *>(workspace);
+        F.part_lse = F.part_o + static_cast<size_t>(pl.n_split) * rows * Dh;
+    }
+    ARTAB_TRY(launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "decode context pass"));
+    if (!need_ws) return ARTAB_OK;
+
+    DecodeParams D;
+    memset(&D, 0, sizeof(D));
+    D.q = dv(q); D.kb = dv(k_buf); D.vb = dv(v_buf); D.knew = dv(k_new); D.vnew = dv(v_new); D.out = dv(out);
+    D.part_o = F.part_o; D.part_lse = F.part_lse; D.lse = nullptr;
+    D.B = B; D.H = H; D.n_split = pl.n_split; D.n_buf = n_buf; D.has_new = has_new;
+    D.qscale = scale * kLog2e;
+    return launch_status(launch_decode(D, dtype, Dh, Lq, st), "decode buffer pass");
+}
+
+int artab_teacher_forcing_attention(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                                    const artab_view *k_buf, const artab_view *v_buf, const artab_view *out,
+                                    float *lse, int B, int H, int Nt, int Nc, int Dh, float scale, int dtype,
+                                    int impl, void *stream) {
+    ARTAB_TRY(check_common(B, H, 2 * Nt, Dh, dtype));
+    if (Nt < 0) return fail(ARTAB_ERR_BAD_SHAPE, "negative num_targets");
+    if (Nc < 1) return fail(ARTAB_ERR_BAD_SHAPE, "teacher forcing needs a context (Nc=%d)", Nc);
+    if (B == 0 || Nt == 0) return ARTAB_OK;
+    ARTAB_TRY(check_view(q, "q", dtype, true));
+    ARTAB_TRY(check_view(k_ctx, "k_ctx", dtype, true));
+    ARTAB_TRY(check_view(v_ctx, "v_ctx", dtype, true));
+    ARTAB_TRY(check_view(k_buf, "k_buf", dtype, true));
+    ARTAB_TRY(check_view(v_buf, "v_buf", dtype, true));
+    ARTAB_TRY(check_view(out, "out", dtype, true));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    scale = resolve_scale(scale, Dh);
+    const bool aligned = vec_aligned(q, dtype, Dh) && vec_aligned(k_ctx, dtype, Dh) &&
+                         vec_aligned(v_ctx, dtype, Dh) && vec_aligned(out, dtype, Dh) &&
+                         vec_aligned(k_buf, dtype, Dh) && vec_aligned(v_buf, dtype, Dh);
+    const bool use_mfma = impl != ARTAB_IMPL_PORTABLE && mfma_shape_ok(dtype, Dh) && aligned;
+    if (impl == ARTAB_IMPL_MFMA && !use_mfma)
+        return fail(ARTAB_ERR_UNSUPPORTED, "MFMA path needs bf16/f16, head_dim in {32,64,128}, 16-byte aligned rows");
+    const int Lq = 2 * Nt;
+    if (!use_mfma) {
+        PortableParams P;
+        memset(&P, 0, sizeof(P));
+        P.q = dv(q); P.kc = dv(k_ctx); P.vc = dv(v_ctx); P.kb = dv(k_buf); P.vb = dv(v_buf); P.out = dv(out);
+        P.lse = lse;
+        P.B = B; P.H = H; P.Lq = Lq; P.Nc = Nc; P.Nb = Nt; P.Nt = Nt;
+        P.new_row = -1; P.mode = kModeTeacher; P.Dh = Dh; P.scale = scale;
+        P.vec_ok = aligned ? 1 : 0;
+        return launch_status(launch_portable_dtype(P, dtype, st), "teacher forcing (portable)");
+    }
+    FlashPlan pl = plan_flash(B, H, Lq, Nc, Dh, /*stacked=*/false, /*allow_split=*/false);
+    FlashParams F;
+    memset(&F, 0, sizeof(F));
+    F.q = dv(q); F.kc = dv(k_ctx); F.vc = dv(v_ctx); F.kb = dv(k_buf); F.vb = dv(v_buf); F.out = dv(out);
+    F.lse = lse;
+    F.B = B; F.H = H; F.Lq = Lq; F.Nc = Nc; F.Nb = Nt; F.Nt = Nt;
+    F.G = pl.G; F.tiles_per_group = pl.tiles_per_group; F.n_groups = pl.n_groups;
+    F.n_split = 1; F.kv_per_split = pl.kv_per_split;
+    F.qscale = scale * kLog2e;
+    F.mode = kFlashTeacher;
+    return launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "teacher forcing (mfma)");
+}
+
+int artab_prefill_attention(const artab_view *q, const artab_view *k, const artab_view *v, const artab_view *out,
+                            const artab_view *k_cache, const artab_view *v_cache, int cache_batches, int B, int H,
+                            int Nc, int Dh, float scale, int dtype, int impl, void *stream) {
+    ARTAB_TRY(check_common(B, H, Nc, Dh, dtype));
+    if (B == 0 || Nc == 0) return ARTAB_OK;
+    ARTAB_TRY(check_view(q, "q", dtype, true));
+    ARTAB_TRY(check_view(k, "k", dtype, true));
+    ARTAB_TRY(check_view(v, "v", dtype, true));
+    ARTAB_TRY(check_view(out, "out", dtype, true));
+    const bool kc_given = k_cache && k_cache->data, vc_given = v_cache && v_cache->data;
+    if (kc_given != vc_given) return fail(ARTAB_ERR_NULL_POINTER, "k_cache and v_cache must be given together");
+    if (kc_given && (cache_batches < 1 || cache_batches > B))
+        return fail(ARTAB_ERR_BAD_SHAPE, "cache_batches=%d outside [1,%d]", cache_batches, B);
+    ARTAB_TRY(check_view(k_cache, "k_cache", dtype, false));
+    ARTAB_TRY(check_view(v_cache, "v_cache", dtype, false));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    scale = resolve_scale(scale, Dh);
+    const bool aligned = vec_aligned(q, dtype, Dh) && vec_aligned(k, dtype, Dh) && vec_aligned(v, dtype, Dh) &&
+                         vec_aligned(out, dtype, Dh) && vec_aligned(k_cache, dtype, Dh) &&
+                         vec_aligned(v_cache, dtype, Dh);
+    const bool use_mfma = impl != ARTAB_IMPL_PORTABLE && mfma_shape_ok(dtype, Dh) && aligned;
+    if (impl == ARTAB_IMPL_MFMA && !use_mfma)
+        return fail(ARTAB_ERR_UNSUPPORTED, "MFMA path needs bf16/f16, head_dim in {32,64,128}, 16-byte aligned rows");
+    if (!use_mfma) {
+        PortableParams P;
+        memset(&P, 0, sizeof(P));
+        P.q = dv(q); P.kc = dv(k); P.vc = dv(v); P.out = dv(out);
+        P.kcache = dv(kc_given ? k_cache : nullptr); P.vcache = dv(kc_given ? v_cache : nullptr);
+        P.cache_batches = kc_given ? cache_batches : 0;
+        P.B = B; P.H = H; P.Lq = Nc; P.Nc = Nc; P.Nb = 0;
+        P.new_row = -1; P.mode = kModePlain; P.Dh = Dh; P.scale = scale;
+        P.vec_ok = aligned ? 1 : 0;
+        return launch_status(launch_portable_dtype(P, dtype, st), "prefill (portable)");
+    }
+    FlashPlan pl = plan_flash(B, H, Nc, Nc, Dh, /*stacked=*/false, /*allow_split=*/false);
+    FlashParams F;
+    memset(&F, 0, sizeof(F));
+    F.q = dv(q); F.kc = dv(k); F.vc = dv(v); F.out = dv(out);
+    F.kcache = dv(kc_given ? k_cache : nullptr); F.vcache = dv(kc_given ? v_cache : nullptr);
+    F.cache_batches = kc_given ? cache_batches : 0;
+    F.B = B; F.H = H; F.Lq = Nc; F.Nc = Nc;
+    F.G = pl.G; F.tiles_per_group = pl.tiles_per_group; F.n_groups = pl.n_groups;
+    F.n_split = 1; F.kv_per_split = pl.kv_per_split;
+    F.qscale = scale * kLog2e;
+    F.mode = kFlashPrefill;
+    return launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "prefill (mfma)");
+}
+
+int artab_buffer_attention(const artab_view *q, const artab_view *k_buf, const artab_view *v_buf,
+                           const uint8_t *mask, int64_t mask_sb, int64_t mask_sh, int64_t mask_sq,
+                           const artab_view *out, float *lse, int B, int H, int Lq, int Nb, int Dh, float scale,
+                           int dtype, void *stream) {
+    ARTAB_TRY(check_common(B, H, Lq, Dh, dtype));
+    if (Nb < 0) return fail(ARTAB_ERR_BAD_SHAPE, "negative buffer length");
+    if (B == 0 || Lq == 0) return ARTAB_OK;
+    ARTAB_TRY(check_view(q, "q", dtype, true));
+    ARTAB_TRY(check_view(out, "out", dtype, true));
+    ARTAB_TRY(check_view(k_buf, "k_buf", dtype, Nb > 0));
+    ARTAB_TRY(check_view(v_buf, "v_buf", dtype, Nb > 0));
+    PortableParams P;
+    memset(&P, 0, sizeof(P));
+    P.q = dv(q); P.kb = dv(k_buf); P.vb = dv(v_buf); P.out = dv(out);
+    P.lse = lse;
+    P.mask = mask; P.m_sb = mask_sb; P.m_sh = mask_sh; P.m_sq = mask_sq;
+    P.B = B; P.H = H; P.Lq = Lq; P.Nc = 0; P.Nb = Nb;
+    P.new_row = -1; P.mode = mask ? kModeMasked : kModePlain; P.Dh = Dh;
+    P.scale = resolve_scale(scale, Dh);
+    P.vec_ok = (vec_aligned(q, dtype, Dh) && vec_aligned(k_buf, dtype, Dh) && vec_aligned(v_buf, dtype, Dh)) ? 1 : 0;
+    return launch_status(launch_portable_dtype(P, dtype, static_cast<hipStream_t>(stream)), "buffer attention");
+}
+
+int artab_merge_attention_outputs(const artab_view *out_a, const float *lse_a, const artab_view *out_b,
+                                  const float *lse_b, const artab_view *out, int B, int H, int Lq, int Dh,
+                                  int dtype, void *stream) {
+    ARTAB_TRY(check_common(B, H, Lq, Dh, dtype));
+    if (B == 0 || Lq == 0) return ARTAB_OK;
+    ARTAB_TRY(check_view(out_a, "out_a", dtype, true));
+    ARTAB_TRY(check_view(out_b, "out_b", dtype, true));
+    ARTAB_TRY(check_view(out, "out", dtype, true));
+    if (!lse_a || !lse_b) return fail(ARTAB_ERR_NULL_POINTER, "lse_a / lse_b is NULL");
+    MergeParams P;
+    P.a = dv(out_a); P.b = dv(out_b); P.out = dv(out);
+    P.lse_a = lse_a; P.lse_b = lse_b;
+    P.rows = static_cast<long>(B) * H * Lq; P.H = H; P.Lq = Lq; P.Dh = Dh;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipError_t e;
+    switch (dtype) {
+        case ARTAB_BF16: e = launch_merge<bf16_t>(P, st); break;
+        case ARTAB_F16: e = launch_merge<f16_t>(P, st); break;
+        default: e = launch_merge<float>(P, st); break;
+    }
+    return launch_status(e, "merge");
+}
+
+}  // extern "C"

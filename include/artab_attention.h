@@ -1,0 +1,186 @@
+/*
+ * artab_attention.h — C ABI of the MI355X (gfx950) attention library for the
+ * AR-TabPFN inference hot path.
+ *
+ * The reference implementation (conorhassan/AR-nanoTabPFN) has no FFI layer: its
+ * boundary is a set of Python callables in ar_tabpfn/model/triton_kernels.py and
+ * the cache attributes handled by ar_tabpfn/model/inference.py.  Each entry point
+ * below names the reference callable(s) it replaces.  A maintainer binds them
+ * with ctypes (no torch types cross the boundary): device pointers, sizes,
+ * element strides and a hipStream_t.
+ *
+ * Conventions
+ *  - All tensors live in device memory of the current HIP device.  The library
+ *    never allocates, frees or retains a pointer past the call, never
+ *    synchronises, and launches only on `stream` (0 = the null stream).
+ *  - A tensor is described by an artab_view: pointer to element [0,0,0,:] plus
+ *    element strides for batch, head and row.  The head_dim axis is contiguous.
+ *    A batch stride of 0 means "one copy shared by every batch entry"; that is
+ *    how the shared context K/V `[H, Nc, Dh]` is passed.
+ *  - dtype selects the element type of q/k/v/out (and caches); log-sum-exp
+ *    outputs and workspaces are always float32.  Softmax statistics and
+ *    accumulation are float32 for every dtype.
+ *  - `scale` <= 0 selects the default head_dim^-0.5.
+ *  - Every function returns ARTAB_OK (0) or a negative artab_status; on error
+ *    nothing has been launched.  artab_last_error() gives a thread-local text.
+ */
+#ifndef ARTAB_ATTENTION_H
+#define ARTAB_ATTENTION_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ARTAB_VERSION 1
+
+typedef enum artab_dtype {
+    ARTAB_BF16 = 0,
+    ARTAB_F16 = 1,
+    ARTAB_F32 = 2
+} artab_dtype;
+
+typedef enum artab_status {
+    ARTAB_OK = 0,
+    ARTAB_ERR_NULL_POINTER = -1,   /* a required pointer is NULL                       */
+    ARTAB_ERR_BAD_SHAPE = -2,      /* a size is negative/zero where that is not allowed */
+    ARTAB_ERR_BAD_STRIDE = -3,     /* misaligned pointer or stride for the chosen dtype */
+    ARTAB_ERR_UNSUPPORTED = -4,    /* dtype / head_dim / flag combination not built     */
+    ARTAB_ERR_WORKSPACE = -5,      /* workspace missing or too small                    */
+    ARTAB_ERR_CAPACITY = -6,       /* buffer cache slot beyond its capacity             */
+    ARTAB_ERR_LAUNCH = -7          /* hipLaunch reported an error                       */
+} artab_status;
+
+/* Selects the kernel family.  AUTO picks the MFMA kernels for 16-bit dtypes with
+ * head_dim in {32, 64, 128} and the portable wave-per-row kernel otherwise. */
+typedef enum artab_impl {
+    ARTAB_IMPL_AUTO = 0,
+    ARTAB_IMPL_PORTABLE = 1,
+    ARTAB_IMPL_MFMA = 2
+} artab_impl;
+
+typedef struct artab_view {
+    void *data;       /* device pointer to element [0,0,0,0]                  */
+    int64_t stride_b; /* elements between batch entries (0 = shared)          */
+    int64_t stride_h; /* elements between heads                                */
+    int64_t stride_n; /* elements between rows; head_dim elements contiguous   */
+} artab_view;
+
+int artab_version(void);
+const char *artab_status_string(int status);
+const char *artab_last_error(void);
+
+/* Bytes of float32 workspace the split-context paths need for the given problem
+ * (artab_context_attention, artab_decode_attention).  0 means no workspace is
+ * needed.  Pure host arithmetic, no device access. */
+size_t artab_workspace_bytes(int B, int H, int Lq, int Nc, int Dh, int dtype);
+
+/*
+ * Context attention with log-sum-exp.
+ * Replaces triton_context_attention / triton_context_attention_multiq /
+ * pytorch_context_attention (ar_tabpfn/model/triton_kernels.py:347-475, :532-567).
+ *   q    [B,H,Lq,Dh]           out [B,H,Lq,Dh]
+ *   k_ctx, v_ctx [*,H,Nc,Dh]   (stride_b 0 = shared context, else one per batch entry)
+ *   lse  float32, contiguous [B,H,Lq]; may be NULL
+ * Nc >= 1.
+ */
+int artab_context_attention(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                            const artab_view *out, float *lse,
+                            int B, int H, int Lq, int Nc, int Dh, float scale, int dtype,
+                            void *workspace, size_t workspace_bytes, int impl, void *stream);
+
+/*
+ * One decode step of row attention for Lq in {1,2} queries per trajectory.
+ * Replaces the body of ARTabPFNPredictor._layer_decode_with_cache_shared between
+ * the projections and out_proj (ar_tabpfn/model/inference.py:785-823): the two
+ * hybrid_attention calls (triton_kernels.py:705-755: context pass, buffer pass,
+ * merge_attention_outputs :478-524), the per-step torch.cat (:806-807) and the
+ * slice-assign cache append (:816-821).
+ *   q            [B,H,Lq,Dh]
+ *   k_ctx,v_ctx  [*,H,Nc,Dh]   context K/V (stride_b 0 = shared)
+ *   k_buf,v_buf  [B,H,cap,Dh]  preallocated buffer cache; rows [0,n_buf) are valid
+ *   k_new,v_new  [B,H,1,Dh]    may be NULL (both).  When given, the row is written
+ *                              in place to slot n_buf of the cache and every query
+ *                              attends to rows [0,n_buf] (the new one included);
+ *                              otherwise queries attend to rows [0,n_buf).
+ *   out          [B,H,Lq,Dh]
+ * An empty buffer (n_buf == 0 and no new row) gives context attention alone
+ * (triton_kernels.py:735-741).  The caller advances n_buf (inference.py:256).
+ */
+int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                           const artab_view *k_buf, const artab_view *v_buf,
+                           const artab_view *k_new, const artab_view *v_new,
+                           const artab_view *out,
+                           int B, int H, int Lq, int Nc, int n_buf, int buf_capacity, int Dh,
+                           float scale, int dtype,
+                           void *workspace, size_t workspace_bytes, int impl, void *stream);
+
+/*
+ * Teacher-forced attention over [Buffer_0..Nt-1, Target_0..Nt-1] queries.
+ * Replaces hybrid_teacher_forcing_attention (triton_kernels.py:662-702: context
+ * pass + masked buffer pass :620-659 + merge) and, with a per-batch context, the
+ * flex_attention call under _create_teacher_forcing_mask
+ * (inference.py:525-577, :735).  The mask is a tile schedule: buffer query i
+ * sees buffer keys j <= i, target query i sees j < i, everyone sees the context,
+ * target keys are never visited.
+ *   q            [B,H,2*Nt,Dh]   out [B,H,2*Nt,Dh]
+ *   k_ctx,v_ctx  [*,H,Nc,Dh]     (stride_b 0 = shared, else per dataset)
+ *   k_buf,v_buf  [B,H,Nt,Dh]     K/V of the Nt buffer rows
+ *   lse          float32 [B,H,2*Nt] contiguous, may be NULL (lse over context+buffer)
+ */
+int artab_teacher_forcing_attention(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                                    const artab_view *k_buf, const artab_view *v_buf,
+                                    const artab_view *out, float *lse,
+                                    int B, int H, int Nt, int Nc, int Dh, float scale, int dtype,
+                                    int impl, void *stream);
+
+/*
+ * Context prefill: dense bidirectional self-attention plus the K/V cache write.
+ * Replaces, in _layer_forward_with_cache(_shared), the cache slice-assign and the
+ * flex_attention call under the dense mask (inference.py:618-622, :672-676;
+ * mask from attention.py:72-83).
+ *   q,k,v    [B,H,Nc,Dh]   (strided views of the [B,Nc,H*Dh] projections)
+ *   out      [B,H,Nc,Dh]
+ *   k_cache, v_cache  may be NULL (both).  When given, rows [0,Nc) of k and v are
+ *            copied to k_cache[b,h,row,:] for b in [0, cache_batches) — use
+ *            cache_batches = 1 with any stride_b for the shared `[H,Nc,Dh]` cache
+ *            (only batch entry 0 is cached, inference.py:672-673) and
+ *            cache_batches = B for the per-dataset cache (:618-619).
+ */
+int artab_prefill_attention(const artab_view *q, const artab_view *k, const artab_view *v,
+                            const artab_view *out,
+                            const artab_view *k_cache, const artab_view *v_cache, int cache_batches,
+                            int B, int H, int Nc, int Dh, float scale, int dtype,
+                            int impl, void *stream);
+
+/*
+ * Buffer attention with log-sum-exp and an optional boolean mask.
+ * Replaces pytorch_buffer_attention (triton_kernels.py:570-614).
+ *   q [B,H,Lq,Dh], k_buf,v_buf [B,H,Nb,Dh], out [B,H,Lq,Dh], lse float32 [B,H,Lq] or NULL
+ *   mask: uint8 (non-zero = attend), element strides (mask_sb, mask_sh, mask_sq) and
+ *         contiguous along keys; NULL = no mask.  Strides of 0 broadcast.
+ * Rows with no visible key give out = 0 and lse = -inf (:598-611).  Nb may be 0.
+ */
+int artab_buffer_attention(const artab_view *q, const artab_view *k_buf, const artab_view *v_buf,
+                           const uint8_t *mask, int64_t mask_sb, int64_t mask_sh, int64_t mask_sq,
+                           const artab_view *out, float *lse,
+                           int B, int H, int Lq, int Nb, int Dh, float scale, int dtype, void *stream);
+
+/*
+ * Merge two partial attention results through their log-sum-exps.
+ * Replaces merge_attention_outputs (triton_kernels.py:478-524).
+ *   out_a, out_b, out [B,H,Lq,Dh]; lse_a, lse_b float32 contiguous [B,H,Lq].
+ * A side whose lse is -inf contributes nothing; both -inf gives NaN, as the
+ * reference formula does.
+ */
+int artab_merge_attention_outputs(const artab_view *out_a, const float *lse_a,
+                                  const artab_view *out_b, const float *lse_b,
+                                  const artab_view *out,
+                                  int B, int H, int Lq, int Dh, int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ARTAB_ATTENTION_H */

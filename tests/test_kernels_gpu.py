@@ -1,0 +1,398 @@
+"""Parity of every C-ABI entry point (through the Python mirror) against the numpy
+oracle on identical seeded inputs.  Tolerances: 2e-2 max-abs on 16-bit outputs,
+1e-3 on float32 LSE; 1e-5 for float32 inputs (the reference's own kernel-vs-PyTorch
+tolerance, tests/test_triton_kernel.py:51-66)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention_oracle as ao
+from tests.helpers import lse_tol, max_abs, out_tol, randn, to_np
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.bfloat16, torch.float16, torch.float32]
+
+
+def _ak():
+    import ar_nanotabpfn_amd.attention_kernels as ak
+
+    return ak
+
+
+def _ctx_inputs(B, H, Lq, Nc, D, dtype, seed=42, scale=1.0, per_batch=False):
+    q = randn((B, H, Lq, D), seed, dtype, scale)
+    kshape = (B, H, Nc, D) if per_batch else (H, Nc, D)
+    k = randn(kshape, seed + 1, dtype, scale)
+    v = randn(kshape, seed + 2, dtype, scale)
+    return q, k, v
+
+
+# ----- context attention (reference grid: tests/test_triton_kernel.py:28-129) -----------------
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("use_mfma", [True, False])
+@pytest.mark.parametrize(
+    "B,H,Lq,Nc,D",
+    [
+        (1, 4, 1, 32, 32),
+        (16, 8, 1, 64, 64),
+        (64, 4, 1, 128, 32),
+        (128, 8, 1, 256, 64),
+        (37, 4, 1, 64, 32),  # batch not divisible by any tile
+        (32, 4, 1, 100, 32),  # context not divisible by any tile
+        (8, 2, 5, 64, 32),  # multi-query
+        (1, 2, 2, 32, 32),
+        (3, 2, 7, 333, 128),
+        (5, 3, 3, 70, 16),  # head_dim only the portable kernel covers
+    ],
+)
+def test_context_attention_matches_oracle(device, dtype, use_mfma, B, H, Lq, Nc, D):
+    ak = _ak()
+    q, k, v = _ctx_inputs(B, H, Lq, Nc, D, dtype)
+    out, lse = ak.context_attention(q.to(device), k.to(device), v.to(device), use_triton=use_mfma)
+    ref_out, ref_lse = ao.context_attention(to_np(q), to_np(k), to_np(v))
+    assert out.shape == (B, H, Lq, D) and out.dtype == dtype
+    assert lse.shape == (B, H, Lq) and lse.dtype == torch.float32
+    tol_o, tol_l = out_tol(dtype), lse_tol(dtype)
+    if dtype == torch.float32:
+        tol_o = tol_l = 2e-5  # randn-scale scores up to ~20: float32 rounding of the scores themselves
+    else:
+        # unit-variance q,k give peaked softmaxes (a handful of keys carry the mass).  The
+        # MFMA kernel sums the 16-bit-rounded probabilities it feeds to the PV product, so
+        # the LSE carries their rounding: <= 2^-9 relative for a one-key softmax, shrinking
+        # as 1/sqrt(#effective keys).  At the 1/sqrt(64)-scaled inputs the 1e-3 target is
+        # stated for (test_decode_attention_config1_shape etc.) the error is ~1e-5.
+        tol_l = 2.5e-3
+    assert max_abs(to_np(out), ref_out) <= tol_o
+    assert max_abs(to_np(lse), ref_lse) <= tol_l
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_context_attention_per_dataset_context(device, dtype):
+    ak = _ak()
+    B, H, Lq, Nc, D = 6, 4, 9, 150, 32
+    q, k, v = _ctx_inputs(B, H, Lq, Nc, D, dtype, per_batch=True, scale=0.5)
+    out, lse = ak.context_attention(q.to(device), k.to(device), v.to(device))
+    ref_out, ref_lse = ao.context_attention(to_np(q), to_np(k), to_np(v))
+    assert max_abs(to_np(out), ref_out) <= out_tol(dtype)
+    assert max_abs(to_np(lse), ref_lse) <= lse_tol(dtype)
+
+
+def test_context_attention_split_context_large(device):
+    """Long context, few query rows: the split-context schedule with the LSE combine."""
+    ak = _ak()
+    B, H, Lq, Nc, D = 64, 8, 2, 4096, 32
+    q, k, v = _ctx_inputs(B, H, Lq, Nc, D, torch.bfloat16, scale=0.6)
+    out, lse = ak.context_attention(q.to(device), k.to(device), v.to(device))
+    ref_out, ref_lse = ao.context_attention(to_np(q), to_np(k), to_np(v))
+    assert max_abs(to_np(out), ref_out) <= 2e-2
+    assert max_abs(to_np(lse), ref_lse) <= 1e-3
+
+
+def test_context_attention_strided_q_view(device):
+    """q arrives as the transposed view of a [B,N,H*Dh] projection (inference.py:781)."""
+    ak = _ak()
+    B, H, Lq, Nc, D = 9, 4, 2, 96, 32
+    proj = randn((B, Lq, H * D), 7, torch.bfloat16)
+    q = proj.view(B, Lq, H, D).transpose(1, 2)
+    _, k, v = _ctx_inputs(B, H, Lq, Nc, D, torch.bfloat16)
+    qd = proj.to(device).view(B, Lq, H, D).transpose(1, 2)
+    assert not qd.is_contiguous()
+    out, lse = ak.context_attention(qd, k.to(device), v.to(device))
+    ref_out, ref_lse = ao.context_attention(to_np(q), to_np(k), to_np(v))
+    assert max_abs(to_np(out), ref_out) <= 2e-2
+    assert max_abs(to_np(lse), ref_lse) <= 1e-3
+    # the output's transposed reshape must be a view (free for out_proj)
+    flat = out.transpose(1, 2).reshape(B, Lq, H * D)
+    assert flat.data_ptr() == out.data_ptr()
+
+
+# ----- decode step ------------------------------------------------------------------------------
+
+
+def _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, use_mfma, scale=1.0, seed=3):
+    ak = _ak()
+    q, k_ctx, v_ctx = _ctx_inputs(B, H, Lq, Nc, D, dtype, seed=seed, scale=scale)
+    k_cache = randn((B, H, cap, D), seed + 10, dtype, scale)
+    v_cache = randn((B, H, cap, D), seed + 11, dtype, scale)
+    k_new = randn((B, H, 1, D), seed + 12, dtype, scale) if with_new else None
+    v_new = randn((B, H, 1, D), seed + 13, dtype, scale) if with_new else None
+    kc_d, vc_d = k_cache.to(device), v_cache.to(device)
+    out = ak.decode_attention(
+        q.to(device), k_ctx.to(device), v_ctx.to(device), kc_d, vc_d, n_buf,
+        k_new.to(device) if with_new else None, v_new.to(device) if with_new else None, use_triton=use_mfma,
+    )
+    ref, k_all, v_all = ao.decode_step_attention(
+        to_np(q), to_np(k_ctx), to_np(v_ctx), to_np(k_cache[:, :, :n_buf]), to_np(v_cache[:, :, :n_buf]),
+        to_np(k_new) if with_new else None, to_np(v_new) if with_new else None,
+    )
+    tol = out_tol(dtype) if dtype != torch.float32 else 2e-5
+    assert max_abs(to_np(out), ref) <= tol
+    # cache after the call: appended row in place, everything else untouched (bit-exact)
+    exp_k, exp_v = k_cache.clone(), v_cache.clone()
+    if with_new:
+        exp_k[:, :, n_buf] = k_new[:, :, 0]
+        exp_v[:, :, n_buf] = v_new[:, :, 0]
+    assert torch.equal(kc_d.cpu(), exp_k) and torch.equal(vc_d.cpu(), exp_v)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("use_mfma", [True, False])
+@pytest.mark.parametrize(
+    "B,H,Lq,Nc,D,n_buf,cap,with_new",
+    [
+        (8, 4, 1, 64, 32, 0, 16, False),  # first target: context only
+        (8, 4, 2, 64, 32, 0, 16, True),  # second step: buffer is just the new row
+        (8, 4, 2, 64, 32, 5, 16, True),
+        (8, 4, 2, 64, 32, 15, 16, True),  # last slot
+        (8, 4, 1, 64, 32, 7, 16, False),  # target only over committed buffers
+        (33, 8, 2, 100, 64, 19, 64, True),
+        (5, 2, 2, 300, 128, 70, 80, True),
+        (4, 3, 2, 50, 16, 9, 12, True),  # portable-only head_dim
+    ],
+)
+def test_decode_attention_matches_oracle(device, dtype, use_mfma, B, H, Lq, Nc, D, n_buf, cap, with_new):
+    _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, use_mfma)
+
+
+@pytest.mark.parametrize("n_buf", [1, 2, 17, 33, 64])
+def test_decode_attention_config1_shape(device, n_buf):
+    """BASELINE configs[1]: H=8, Dh=64, Nc=1024, B=256, entries ~N(0,1)/8, N_buf swept."""
+    _decode_case(device, torch.bfloat16, 256, 8, 1, 1024, 64, n_buf, 64, False, True, scale=0.125, seed=0)
+
+
+def test_decode_attention_long_context_split(device):
+    """Many context slices + buffer pass + merge (the configs[3] schedule, smaller)."""
+    _decode_case(device, torch.bfloat16, 128, 8, 2, 8192, 32, 100, 128, True, True, scale=0.6)
+
+
+def test_hybrid_attention_empty_buffer_is_context_only(device):
+    """tests/test_triton_kernel.py:319-339."""
+    ak = _ak()
+    B, H, Lq, Nc, D = 32, 4, 1, 64, 32
+    q, k, v = _ctx_inputs(B, H, Lq, Nc, D, torch.float32)
+    kb = torch.empty(B, H, 0, D)
+    out = ak.hybrid_attention(q.to(device), k.to(device), v.to(device), kb.to(device), kb.to(device), use_triton=False)
+    ref, _ = ao.context_attention(to_np(q), to_np(k), to_np(v))
+    assert max_abs(to_np(out), ref) <= 2e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_hybrid_attention_matches_full_attention(device, dtype):
+    """tests/test_triton_kernel.py:288-317: hybrid == one softmax over cat(ctx, buffer)."""
+    ak = _ak()
+    B, H, Lq, D, Nc, Nb = 64, 4, 1, 32, 128, 32
+    q, k, v = _ctx_inputs(B, H, Lq, Nc, D, dtype)
+    kb, vb = randn((B, H, Nb, D), 50, dtype), randn((B, H, Nb, D), 51, dtype)
+    out = ak.hybrid_attention(q.to(device), k.to(device), v.to(device), kb.to(device), vb.to(device))
+    k_full = np.concatenate([np.broadcast_to(to_np(k)[None], (B, H, Nc, D)), to_np(kb)], axis=2)
+    v_full = np.concatenate([np.broadcast_to(to_np(v)[None], (B, H, Nc, D)), to_np(vb)], axis=2)
+    ref, _ = ao.masked_full_attention(to_np(q), k_full, v_full)
+    assert max_abs(to_np(out), ref) <= (2e-5 if dtype == torch.float32 else 2e-2)
+
+
+def test_hybrid_attention_with_buffer_mask(device):
+    """tests/test_triton_kernel.py:242-282: masked buffer + merge == masked full attention."""
+    ak = _ak()
+    B, H, Lq, D, Nc, Nb = 8, 4, 1, 32, 32, 8
+    q, k, v = _ctx_inputs(B, H, Lq, Nc, D, torch.float32)
+    kb, vb = randn((B, H, Nb, D), 50, torch.float32), randn((B, H, Nb, D), 51, torch.float32)
+    mask = torch.zeros(B, H, Lq, Nb, dtype=torch.bool)
+    mask[..., :4] = True
+    out = ak.hybrid_attention(
+        q.to(device), k.to(device), v.to(device), kb.to(device), vb.to(device), buf_mask=mask.to(device)
+    )
+    k_full = np.concatenate([np.broadcast_to(to_np(k)[None], (B, H, Nc, D)), to_np(kb)], axis=2)
+    v_full = np.concatenate([np.broadcast_to(to_np(v)[None], (B, H, Nc, D)), to_np(vb)], axis=2)
+    full_mask = np.ones((B, H, Lq, Nc + Nb), dtype=bool)
+    full_mask[..., Nc:] = mask.numpy()
+    ref, _ = ao.masked_full_attention(to_np(q), k_full, v_full, mask=full_mask)
+    assert max_abs(to_np(out), ref) <= 2e-5
+
+
+# ----- buffer attention / merge -------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_buffer_attention_masked_rows(device, dtype):
+    """Target 0 sees no buffer: out 0, lse -inf (tests/test_triton_kernel.py:135-151)."""
+    ak = _ak()
+    B, H, Nt, D = 4, 2, 3, 16
+    q = randn((B, H, 2 * Nt, D), 1, dtype)
+    kb, vb = randn((B, H, Nt, D), 2, dtype), randn((B, H, Nt, D), 3, dtype)
+    out, lse = ak.pytorch_teacher_forcing_buffer_attention(q.to(device), kb.to(device), vb.to(device), Nt)
+    ref_out, ref_lse = ao.teacher_forcing_buffer_attention(to_np(q), to_np(kb), to_np(vb), Nt)
+    assert torch.all(out[:, :, Nt] == 0)
+    assert torch.isneginf(lse[:, :, Nt]).all()
+    assert max_abs(to_np(out), ref_out) <= (2e-5 if dtype == torch.float32 else 2e-2)
+    assert max_abs(to_np(lse), ref_lse) <= (2e-5 if dtype == torch.float32 else 1e-3)
+
+
+def test_buffer_attention_shape_errors(device):
+    ak = _ak()
+    q = torch.zeros(2, 2, 6, 16, device=device)
+    kb = torch.zeros(2, 2, 3, 16, device=device)
+    with pytest.raises(ValueError):
+        ak.pytorch_teacher_forcing_buffer_attention(q, kb, kb, 4)
+    with pytest.raises(ValueError):
+        ak.pytorch_teacher_forcing_buffer_attention(q[:, :, :4], kb, kb, 2)
+
+
+def test_merge_closed_forms(device):
+    """tests/test_triton_kernel.py:345-382."""
+    ak = _ak()
+    B, H, Lq, D = 8, 4, 1, 32
+    a, b = randn((B, H, Lq, D), 1, torch.float32), randn((B, H, Lq, D), 2, torch.float32)
+    hi = torch.full((B, H, Lq), 10.0)
+    lo = torch.full((B, H, Lq), -10.0)
+    out = ak.merge_attention_outputs(a.to(device), hi.to(device), b.to(device), lo.to(device))
+    assert max_abs(to_np(out), to_np(a)) <= 1e-4
+    eq = torch.full((B, H, Lq), 5.0)
+    out = ak.merge_attention_outputs(a.to(device), eq.to(device), b.to(device), eq.to(device))
+    assert max_abs(to_np(out), (to_np(a) + to_np(b)) / 2) <= 1e-5
+    ninf = torch.full((B, H, Lq), float("-inf"))
+    out = ak.merge_attention_outputs(a.to(device), eq.to(device), b.to(device), ninf.to(device))
+    assert torch.equal(out.cpu(), a)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_merge_matches_oracle(device, dtype):
+    ak = _ak()
+    B, H, Lq, D = 5, 3, 4, 32
+    a, b = randn((B, H, Lq, D), 1, dtype), randn((B, H, Lq, D), 2, dtype)
+    la, lb = randn((B, H, Lq), 3, torch.float32, 3.0), randn((B, H, Lq), 4, torch.float32, 3.0)
+    out = ak.merge_attention_outputs(a.to(device), la.to(device), b.to(device), lb.to(device))
+    ref = ao.merge_attention_outputs(to_np(a), to_np(la), to_np(b), to_np(lb))
+    assert max_abs(to_np(out), ref) <= (1e-5 if dtype == torch.float32 else 2e-2)
+
+
+# ----- teacher forcing ------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("use_mfma", [True, False])
+@pytest.mark.parametrize("per_batch", [False, True])
+@pytest.mark.parametrize(
+    "B,H,Nt,Nc,D",
+    [
+        (2, 3, 4, 5, 16),  # tests/test_triton_kernel.py:157-198
+        (2, 2, 1, 40, 32),  # Nt = 1 (tests/test_triton_joint_density.py:255-260)
+        (4, 4, 16, 64, 32),
+        (3, 2, 50, 130, 32),  # nothing divides a tile
+        (2, 8, 128, 512, 32),  # configs[2] per (b,h) shape
+        (2, 2, 150, 96, 64),  # Nt > 128: several q tiles, tiles straddling the buffer/target border
+        (1, 2, 37, 70, 128),
+    ],
+)
+def test_teacher_forcing_matches_oracle(device, dtype, use_mfma, per_batch, B, H, Nt, Nc, D):
+    ak = _ak()
+    q, k, v = _ctx_inputs(B, H, 2 * Nt, Nc, D, dtype, per_batch=per_batch, scale=0.7)
+    kb, vb = randn((B, H, Nt, D), 60, dtype, 0.7), randn((B, H, Nt, D), 61, dtype, 0.7)
+    out, lse = ak.teacher_forcing_attention(
+        q.to(device), k.to(device), v.to(device), kb.to(device), vb.to(device), Nt,
+        use_triton=use_mfma, return_lse=True,
+    )
+    # ground truth: one masked softmax over cat(context, buffer, [never-visible targets])
+    kc = to_np(k) if per_batch else np.broadcast_to(to_np(k)[None], (B, H, Nc, D))
+    vc = to_np(v) if per_batch else np.broadcast_to(to_np(v)[None], (B, H, Nc, D))
+    pad = np.zeros((B, H, Nt, D))
+    k_full = np.concatenate([kc, to_np(kb), pad], axis=2)
+    v_full = np.concatenate([vc, to_np(vb), pad], axis=2)
+    mask = ao.teacher_forcing_mask(Nc, Nt)[None, None]
+    ref_out, ref_lse = ao.masked_full_attention(to_np(q), k_full, v_full, mask=mask)
+    tol_o = 2e-5 if dtype == torch.float32 else 2e-2
+    tol_l = 2e-5 if dtype == torch.float32 else 1e-3
+    assert max_abs(to_np(out), ref_out) <= tol_o
+    assert max_abs(to_np(lse), ref_lse) <= tol_l
+    # and the reference's own composition (context + masked buffer + merge)
+    ref2 = ao.hybrid_teacher_forcing_attention(to_np(q), to_np(k), to_np(v), to_np(kb), to_np(vb), Nt)
+    assert max_abs(to_np(out), ref2) <= tol_o
+
+
+def test_teacher_forcing_strided_views(device):
+    """q/k_buf/v_buf as views of the fresh [B,2Nt,H*Dh] projections (inference.py:869-876)."""
+    ak = _ak()
+    B, H, Nt, Nc, D = 3, 4, 20, 64, 32
+    pq, pk, pv = (randn((B, 2 * Nt, H * D), s, torch.bfloat16, 0.7) for s in (1, 2, 3))
+    k_ctx, v_ctx = randn((H, Nc, D), 4, torch.bfloat16, 0.7), randn((H, Nc, D), 5, torch.bfloat16, 0.7)
+
+    def heads(t):
+        return t.view(B, 2 * Nt, H, D).transpose(1, 2)
+
+    qd, kd, vd = heads(pq.to(device)), heads(pk.to(device)), heads(pv.to(device))
+    out = ak.hybrid_teacher_forcing_attention(
+        qd, k_ctx.to(device), v_ctx.to(device), kd[:, :, :Nt], vd[:, :, :Nt], Nt
+    )
+    ref = ao.hybrid_teacher_forcing_attention(
+        to_np(heads(pq)), to_np(k_ctx), to_np(v_ctx), to_np(heads(pk)[:, :, :Nt]), to_np(heads(pv)[:, :, :Nt]), Nt
+    )
+    assert max_abs(to_np(out), ref) <= 2e-2
+
+
+# ----- prefill -----------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("use_mfma", [True, False])
+@pytest.mark.parametrize("shared_cache", [True, False])
+@pytest.mark.parametrize("B,H,Nc,D", [(1, 4, 64, 32), (3, 2, 100, 32), (2, 8, 512, 32), (2, 2, 300, 64), (1, 2, 130, 128)])
+def test_prefill_matches_oracle_and_writes_cache(device, dtype, use_mfma, shared_cache, B, H, Nc, D):
+    ak = _ak()
+    # strided views of [B,Nc,H*D] projections, as the predictor produces them
+    pq, pk, pv = (randn((B, Nc, H * D), s, dtype, 0.7) for s in (11, 12, 13))
+
+    def heads(t):
+        return t.view(B, Nc, H, D).transpose(1, 2)
+
+    cap = Nc + 3
+    if shared_cache:
+        kc = torch.full((H, cap, D), 7.0, dtype=dtype, device=device)
+    else:
+        kc = torch.full((B, H, cap, D), 7.0, dtype=dtype, device=device)
+    vc = kc.clone()
+    out = ak.prefill_attention(
+        heads(pq.to(device)), heads(pk.to(device)), heads(pv.to(device)), kc, vc, use_triton=use_mfma
+    )
+    ref, _ = ao.dense_self_attention(to_np(heads(pq)), to_np(heads(pk)), to_np(heads(pv)))
+    assert max_abs(to_np(out), ref) <= (2e-5 if dtype == torch.float32 else 2e-2)
+    k_exp = heads(pk)[0] if shared_cache else heads(pk)
+    v_exp = heads(pv)[0] if shared_cache else heads(pv)
+    assert torch.equal(kc[..., :Nc, :].cpu(), k_exp) and torch.equal(vc[..., :Nc, :].cpu(), v_exp)
+    assert torch.all(kc[..., Nc:, :] == 7.0) and torch.all(vc[..., Nc:, :] == 7.0)
+
+
+def test_prefill_permutation_invariance(device):
+    """Context is bidirectional with no positions: permuting rows permutes outputs."""
+    ak = _ak()
+    B, H, Nc, D = 2, 4, 200, 32
+    q, k, v = (randn((B, H, Nc, D), s, torch.bfloat16, 0.7).to(device) for s in (1, 2, 3))
+    perm = torch.randperm(Nc, generator=torch.Generator().manual_seed(0)).to(device)
+    out = ak.prefill_attention(q, k, v)
+    out_p = ak.prefill_attention(q[:, :, perm], k[:, :, perm], v[:, :, perm])
+    assert max_abs(to_np(out[:, :, perm]), to_np(out_p)) <= 1e-2
+
+
+# ----- error behaviour through the ABI ---------------------------------------------------------------
+
+
+def test_decode_errors(device):
+    ak = _ak()
+    q = torch.zeros(2, 2, 3, 32, device=device, dtype=torch.bfloat16)
+    kc = torch.zeros(2, 8, 32, device=device, dtype=torch.bfloat16)
+    cache = torch.zeros(2, 2, 4, 32, device=device, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):  # N not in {1,2} (inference.py:765-768)
+        ak.decode_attention(q, kc, kc, cache, cache, 0)
+    new = torch.zeros(2, 2, 1, 32, device=device, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):  # cache full (inference.py:247-250)
+        ak.decode_attention(q[:, :, :2], kc, kc, cache, cache, 4, new, new)
+
+
+def test_cpu_tensors_are_rejected():
+    ak = _ak()
+    q = torch.zeros(1, 1, 1, 32)
+    k = torch.zeros(1, 4, 32)
+    with pytest.raises(RuntimeError):
+        ak.context_attention(q, k, k)
