@@ -22,6 +22,8 @@ HIPCC_FLAGS = [
     "-fPIC",
     # packed-FP32 VALU forms are switched off for device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA accumulators live in VGPRs (no AGPR<->VGPR copies around every product)
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
 ]
 
 

@@ -6,6 +6,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "../../include/artab_attention.h"
@@ -85,7 +86,7 @@ static inline bool mfma_shape_ok(int dtype, int Dh) {
 // ---------------------------------------------------------------------------------------------
 
 constexpr int kFlashBN = 64;
-constexpr int kTargetWorkgroups = 768;  // 3 per CU on a 256-CU part
+constexpr int kTargetWorkgroups = 512;  // 2 per CU on a 256-CU part
 
 struct FlashPlan {
     int BM;        // query rows per workgroup: 256, 128 or 64
@@ -96,30 +97,39 @@ struct FlashPlan {
     int G;
 };
 
+static int env_int(const char *name, int fallback) {
+    const char *v = getenv(name);
+    return (v && *v) ? atoi(v) : fallback;
+}
+
+// Tile planning.  Query tiles of 256 rows (two 32-row blocks per wavefront) give the
+// best MFMA-per-LDS-byte ratio; smaller tiles are used only when a group has fewer
+// rows (no wavefronts of pure padding) or, for the unsplittable phases, when the
+// grid would not cover the chip.  Missing parallelism on long contexts comes from
+// slicing the context (each slice returns a normalised partial + log-sum-exp).
+// ARTAB_BM / ARTAB_SPLIT override the choice (tuning aid).
 static FlashPlan plan_flash(int B, int H, int Lq, int Nc, int Dh, bool stacked, bool allow_split) {
     FlashPlan pl;
     pl.n_groups = stacked ? 1 : B;
     pl.G = stacked ? B * Lq : Lq;
-    const int cands[3] = {256, 128, 64};
-    int pick = 64;
-    for (int ci = 0; ci < 3; ++ci) {
-        int bm = cands[ci];
-        if (Dh == 128 && bm == 256) continue;  // register budget: one 32-row block per wavefront
-        long wgs = static_cast<long>((pl.G + bm - 1) / bm) * pl.n_groups * H;
-        if (wgs >= kTargetWorkgroups) {
-            pick = bm;
-            break;
-        }
-    }
-    pl.BM = pick;
-    pl.tiles_per_group = (pl.G + pick - 1) / pick;
-    long base = static_cast<long>(pl.tiles_per_group) * pl.n_groups * H;
+    auto wgs = [&](int bm) { return static_cast<long>((pl.G + bm - 1) / bm) * pl.n_groups * H; };
+    int bm = Dh == 128 ? 128 : 256;  // head_dim 128: one 32-row block per wavefront (register budget)
+    while (bm > 64 && pl.G <= bm / 2) bm /= 2;
+    if (!allow_split)
+        while (bm > 64 && wgs(bm) < 512) bm /= 2;
+    const int bm_env = env_int("ARTAB_BM", 0);
+    if ((bm_env == 64 || bm_env == 128 || (bm_env == 256 && Dh != 128))) bm = bm_env;
+    pl.BM = bm;
+    pl.tiles_per_group = (pl.G + bm - 1) / bm;
+    const long base = wgs(bm);
     int n_split = 1;
     if (allow_split && base < kTargetWorkgroups) {
-        int max_split = Nc / 256 > 0 ? Nc / 256 : 1;
-        int want = static_cast<int>((kTargetWorkgroups + base - 1) / base);
+        const int max_split = Nc / 512 > 0 ? Nc / 512 : 1;  // at least 512 keys per slice
+        const int want = static_cast<int>((kTargetWorkgroups + base - 1) / base);
         n_split = want < max_split ? want : max_split;
-        if (n_split > 64) n_split = 64;
+        if (n_split > 32) n_split = 32;
+        const int sp_env = env_int("ARTAB_SPLIT", 0);
+        if (sp_env > 0) n_split = sp_env < max_split ? sp_env : max_split;
     }
     int per = (Nc + n_split - 1) / n_split;
     per = (per + kFlashBN - 1) / kFlashBN * kFlashBN;

@@ -11,19 +11,31 @@
 // Layout.  Everything is computed transposed so that softmax statistics are
 // per-lane scalars and P never leaves registers:
 //     S^T[kv, q] = K[kv, :] . Q[q, :]        (A = K tile from LDS, B = Q in registers)
-//     O^T[d,  q] = V^T[d, kv] . P^T[kv, q]   (A = V^T tile from LDS, B = P in registers)
+//     O^T[d,  q] = V^T[d, kv] . P^T[kv, q]   (A = V^T from LDS,    B = P in registers)
 // With v_mfma_f32_32x32x16 a lane (c = lane % 32, hb = lane / 32) owns query
 // column c and, in accumulator register v = 4g + r, row 8g + 4hb + r.  The 16
 // scores a lane holds for one 32-key block are therefore keys {8g + 4hb + r};
 // used directly as the B operand of the second product this enumerates the
-// contraction index as e = 4(g mod 2) + r per 16-wide step t = g / 2.  V is
-// staged into LDS transposed and with its key columns permuted to exactly that
-// order, so one 16-byte LDS read yields the matching A operand.
+// contraction index as e = 4(g mod 2) + r per 16-wide step t = g / 2.  V stays
+// row-major in LDS; ds_read_b64_tr_b16 (the CDNA4 transposing LDS read) hands
+// each lane the four keys {base + r} of one output dimension, so two such reads
+// give the matching A operand for step t without any shuffling.
+//
+// Softmax.  Q is pre-multiplied by scale*log2(e) and rounded to the input type
+// (the rounding model of the reference kernel, triton_kernels.py:120-121), so
+// p = 2^s needs no multiply.  The fast path subtracts no running maximum at all:
+// float32 holds 2^s for |s| < 126, bf16 keeps that exponent range, and the
+// accumulators are float32.  A row whose probability mass leaves [2^-100, 2^100]
+// (or any NaN/inf) makes the whole workgroup redo its tile range with the
+// classical online-softmax (running maximum, rescaled accumulators); fp16, whose
+// exponent range is too small for the fast path, always takes that robust path.
 #pragma once
 
 #include "common.h"
 
 namespace artab {
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
 
 template <typename T>
 struct MfmaOps;
@@ -31,6 +43,7 @@ struct MfmaOps;
 template <>
 struct MfmaOps<bf16_t> {
     typedef bf16x8 vec;
+    static constexpr bool kWideExponent = true;
     static __device__ __forceinline__ f32x16 mma(vec a, vec b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
@@ -44,6 +57,7 @@ struct MfmaOps<bf16_t> {
 template <>
 struct MfmaOps<f16_t> {
     typedef f16x8 vec;
+    static constexpr bool kWideExponent = false;
     static __device__ __forceinline__ f32x16 mma(vec a, vec b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
@@ -71,11 +85,14 @@ struct FlashParams {
     int n_split, kv_per_split;
     float qscale;  // softmax scale * log2(e), folded into Q
     int mode;
+    int force_robust;  // 1: skip the fast path (testing the online-softmax path)
 };
 
-constexpr float kRescaleSum = 4096.0f;  // block probability sum (16 keys) that forces a refresh of the offset
+// Probability mass (sum of 2^s over a row) the fast path accepts.
+constexpr float kFastMassMax = 1.2676506e30f;  // 2^100
+constexpr float kFastMassMin = 7.8886091e-31f; // 2^-100
 
-// Largest teacher-forcing key limit over query rows [a, b] (inclusive).
+// Largest / smallest teacher-forcing key limit over query rows [a, b] (inclusive).
 __host__ __device__ inline int tf_range_max(int a, int b, int Nt) {
     int best = 0;
     if (a < Nt) best = tf_limit(b < Nt ? b : Nt - 1, Nt);
@@ -92,6 +109,11 @@ __host__ __device__ inline int tf_range_min(int a, int b, int Nt) {
     return best;
 }
 
+template <bool V>
+struct BoolTag {
+    static constexpr bool value = V;
+};
+
 template <typename T, int DH, int QB, int NW, int BN>
 __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
     typedef MfmaOps<T> Ops;
@@ -99,18 +121,18 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
     constexpr int KS = DH / 16;
     constexpr int DB = DH / 32;
     constexpr int SB = BN / 32;
-    constexpr int KPAD = DH + 8;
-    constexpr int VPAD = BN + 8;
+    constexpr int KPAD = DH + 8;   // K rows: 16-byte reads by 8 consecutive lanes hit 8 distinct bank groups
+    constexpr int VPAD = DH + 16;  // V rows: row stride = 32 or 96 bytes mod 128 for the transposing reads
     constexpr int NT = NW * 64;
     constexpr int ROWS_W = 32 * QB;
     constexpr int BM = NW * ROWS_W;
-    constexpr int K_CHUNKS = BN * DH / 8;         // 16-byte pieces of a K tile
-    constexpr int V_TASKS = (BN / 4) * (DH / 4);  // 4 keys x 4 dims transposes of a V tile
-    constexpr int KCH = (K_CHUNKS + NT - 1) / NT;
-    constexpr int VTK = (V_TASKS + NT - 1) / NT;
+    constexpr int CHUNKS = BN * DH / 8;  // 16-byte pieces of a K (or V) tile
+    constexpr int NCH = (CHUNKS + NT - 1) / NT;
+    constexpr int CPR = DH / 8;  // chunks per row
 
-    __shared__ __attribute__((aligned(16))) T k_lds[2][BN * KPAD];
-    __shared__ __attribute__((aligned(16))) T v_lds[2][DH * VPAD];
+    __shared__ __attribute__((aligned(16))) T k_lds[3][BN * KPAD];
+    __shared__ __attribute__((aligned(16))) T v_lds[3][BN * VPAD];
+    __shared__ int redo_flag;
 
     // ---- workgroup -> (kv-sharing group, q tile, context split); XCD-aware: the
     // hardware deals consecutive workgroup ids round-robin over the 8 XCDs, so all
@@ -134,11 +156,8 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
     const int row0_wg = tile * BM;
     const int row0_w = row0_wg + wave * ROWS_W;
 
-    // ---- Q fragments (B operand of S^T), pre-scaled by scale*log2e in float32 and
-    // split into two 16-bit terms (hi + lo) so the scaling adds no rounding of its
-    // own: scores carry ~16 mantissa bits of q, which keeps the log-sum-exp within
-    // 1e-3 at unit-variance scores.  The extra MFMAs ride on a pipe that has slack.
-    vec qhi[QB][KS], qlo[QB][KS];
+    // ---- Q fragments (B operand of S^T), pre-scaled by scale*log2e.
+    vec qreg[QB][KS];
     long orow_idx[QB];  // (b*H + h)*Lq + i of this lane's query per block, or -1
     int qi[QB];         // query index i within its batch entry
     long qb[QB];
@@ -157,23 +176,19 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
         for (int ks = 0; ks < KS; ++ks) {
             u32x4 raw = {0u, 0u, 0u, 0u};
             if (valid) raw = *reinterpret_cast<const u32x4 *>(qrow + 16 * ks + 8 * hb);
-            u32x4 hi, lo;
+            u32x4 sc;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float a = unpack_lo<T>(raw[e]) * P.qscale, bq = unpack_hi<T>(raw[e]) * P.qscale;
-                hi[e] = pack2<T>(a, bq);
-                lo[e] = pack2<T>(a - unpack_lo<T>(hi[e]), bq - unpack_hi<T>(hi[e]));
-            }
-            qhi[j][ks] = __builtin_bit_cast(vec, hi);
-            qlo[j][ks] = __builtin_bit_cast(vec, lo);
+            for (int e = 0; e < 4; ++e)
+                sc[e] = pack2<T>(unpack_lo<T>(raw[e]) * P.qscale, unpack_hi<T>(raw[e]) * P.qscale);
+            qreg[j][ks] = __builtin_bit_cast(vec, sc);
         }
     }
 
     // ---- prefill: this tile's own K/V rows go to the cache.
     if (P.mode == kFlashPrefill && P.kcache.p && g < P.cache_batches) {
         int nrows = min(BM, P.G - row0_wg);
-        for (int idx = tid; idx < nrows * (DH / 8); idx += NT) {
-            int rr = row0_wg + idx / (DH / 8), ch = idx % (DH / 8);
+        for (int idx = tid; idx < nrows * CPR; idx += NT) {
+            int rr = row0_wg + idx / CPR, ch = idx % CPR;
             *reinterpret_cast<u32x4 *>(view_row<T>(P.kcache, g, h, rr) + 8 * ch) =
                 *reinterpret_cast<const u32x4 *>(view_row<T>(P.kc, kvb, h, rr) + 8 * ch);
             *reinterpret_cast<u32x4 *>(view_row<T>(P.vcache, g, h, rr) + 8 * ch) =
@@ -186,8 +201,10 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
     const int ctx_end = min(P.Nc, ctx_begin + P.kv_per_split);
     const int ctx_tiles = (ctx_end - ctx_begin + BN - 1) / BN;
     int buf_tiles = 0;
-    int lim[QB];         // per-lane visible buffer keys
+    int lim[QB];  // per-lane visible buffer keys
     int wave_lim_min = 0, wave_lim_max = 0;
+#pragma unroll
+    for (int j = 0; j < QB; ++j) lim[j] = 0;
     if (P.mode == kFlashTeacher) {
         int last = min(row0_wg + BM, P.G) - 1;
         int wg_max = min(P.Nb, tf_range_max(row0_wg, last, P.Nt));
@@ -200,15 +217,19 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
         }
 #pragma unroll
         for (int j = 0; j < QB; ++j) lim[j] = qi[j] >= 0 ? min(P.Nb, tf_limit(qi[j], P.Nt)) : 0;
-    } else {
-#pragma unroll
-        for (int j = 0; j < QB; ++j) lim[j] = 0;
     }
     const int n_tiles = ctx_tiles + buf_tiles;
 
-    // ---- staging registers (global -> registers -> LDS, one tile ahead).
-    u32x4 kst[KCH];
-    u32x2 vst[VTK][4];
+    // ---- staging: global -> registers -> LDS, one tile ahead.  Each thread owns
+    // NCH 16-byte chunks (row kvl, chunk ch) of the K tile and the same of V.
+    int st_row[NCH], st_col[NCH];
+#pragma unroll
+    for (int x = 0; x < NCH; ++x) {
+        int idx = tid + x * NT;
+        st_row[x] = idx / CPR;
+        st_col[x] = (idx % CPR) * 8;
+    }
+    u32x4 kst[NCH], vst[NCH];
 
     auto fetch = [&](int it) {
         const bool is_ctx = it < ctx_tiles;
@@ -216,193 +237,341 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
         const View &vs_ = is_ctx ? P.vc : P.vb;
         const long bb = is_ctx ? kvb : g;
         const int kv0 = is_ctx ? ctx_begin + it * BN : (it - ctx_tiles) * BN;
-        const int seg_end = is_ctx ? ctx_end : P.Nb;
+        const int rows_left = (is_ctx ? ctx_end : P.Nb) - kv0;
+        const T *kbase = view_row<T>(ks_, bb, h, kv0);
+        const T *vbase = view_row<T>(vs_, bb, h, kv0);
+        if (rows_left >= BN) {
 #pragma unroll
-        for (int x = 0; x < KCH; ++x) {
-            int idx = tid + x * NT;
-            int kvl = idx / (DH / 8), ch = idx % (DH / 8);
-            u32x4 val = {0u, 0u, 0u, 0u};
-            if (idx < K_CHUNKS && kv0 + kvl < seg_end)
-                val = *reinterpret_cast<const u32x4 *>(view_row<T>(ks_, bb, h, kv0 + kvl) + 8 * ch);
-            kst[x] = val;
-        }
+            for (int x = 0; x < NCH; ++x) {
+                if (NCH * NT == CHUNKS || tid + x * NT < CHUNKS) {
+                    kst[x] = *reinterpret_cast<const u32x4 *>(kbase + st_row[x] * ks_.sn + st_col[x]);
+                    vst[x] = *reinterpret_cast<const u32x4 *>(vbase + st_row[x] * vs_.sn + st_col[x]);
+                }
+            }
+        } else {
 #pragma unroll
-        for (int x = 0; x < VTK; ++x) {
-            int idx = tid + x * NT;
-            int kg4 = idx / (DH / 4), dq = idx % (DH / 4);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                u32x2 val = {0u, 0u};
-                int kv = kv0 + 4 * kg4 + r;
-                if (idx < V_TASKS && kv < seg_end)
-                    val = *reinterpret_cast<const u32x2 *>(view_row<T>(vs_, bb, h, kv) + 4 * dq);
-                vst[x][r] = val;
+            for (int x = 0; x < NCH; ++x) {
+                kst[x] = u32x4{0u, 0u, 0u, 0u};
+                vst[x] = u32x4{0u, 0u, 0u, 0u};
+                if ((NCH * NT == CHUNKS || tid + x * NT < CHUNKS) && st_row[x] < rows_left) {
+                    kst[x] = *reinterpret_cast<const u32x4 *>(kbase + st_row[x] * ks_.sn + st_col[x]);
+                    vst[x] = *reinterpret_cast<const u32x4 *>(vbase + st_row[x] * vs_.sn + st_col[x]);
+                }
             }
         }
     };
 
     auto stash = [&](int buf) {
 #pragma unroll
-        for (int x = 0; x < KCH; ++x) {
-            int idx = tid + x * NT;
-            int kvl = idx / (DH / 8), ch = idx % (DH / 8);
-            if (idx < K_CHUNKS) *reinterpret_cast<u32x4 *>(&k_lds[buf][kvl * KPAD + 8 * ch]) = kst[x];
-        }
-#pragma unroll
-        for (int x = 0; x < VTK; ++x) {
-            int idx = tid + x * NT;
-            if (idx < V_TASKS) {
-                int kg4 = idx / (DH / 4), dq = idx % (DH / 4);
-                int kvl = 4 * kg4;
-                int sbk = kvl >> 5, kl = kvl & 31;
-                int pcol = sbk * 32 + ((kl >> 2) & 1) * 16 + (kl >> 3) * 4;
-                // 4x4 transpose of 16-bit elements: rows = keys r, columns = dims dd.
-                unsigned a0 = vst[x][0][0], a1 = vst[x][1][0], a2 = vst[x][2][0], a3 = vst[x][3][0];
-                unsigned b0 = vst[x][0][1], b1 = vst[x][1][1], b2 = vst[x][2][1], b3 = vst[x][3][1];
-                u32x2 d0 = {(a0 & 0xffffu) | (a1 << 16), (a2 & 0xffffu) | (a3 << 16)};
-                u32x2 d1 = {(a0 >> 16) | (a1 & 0xffff0000u), (a2 >> 16) | (a3 & 0xffff0000u)};
-                u32x2 d2 = {(b0 & 0xffffu) | (b1 << 16), (b2 & 0xffffu) | (b3 << 16)};
-                u32x2 d3 = {(b0 >> 16) | (b1 & 0xffff0000u), (b2 >> 16) | (b3 & 0xffff0000u)};
-                T *base = &v_lds[buf][(4 * dq) * VPAD + pcol];
-                *reinterpret_cast<u32x2 *>(base) = d0;
-                *reinterpret_cast<u32x2 *>(base + VPAD) = d1;
-                *reinterpret_cast<u32x2 *>(base + 2 * VPAD) = d2;
-                *reinterpret_cast<u32x2 *>(base + 3 * VPAD) = d3;
+        for (int x = 0; x < NCH; ++x) {
+            if (NCH * NT == CHUNKS || tid + x * NT < CHUNKS) {
+                *reinterpret_cast<u32x4 *>(&k_lds[buf][st_row[x] * KPAD + st_col[x]]) = kst[x];
+                *reinterpret_cast<u32x4 *>(&v_lds[buf][st_row[x] * VPAD + st_col[x]]) = vst[x];
             }
         }
     };
 
-    // ---- running softmax state.  m is the offset already subtracted from the
-    // scores (log2 domain); it starts at 0, is set exactly on the first block and
-    // afterwards only moves when a block's maximum exceeds it by the threshold.
+    // ---- per-lane LDS read offsets (elements).
+    const int k_rd = c * KPAD + 8 * hb;                                       // + 32*sb*KPAD + 16*ks
+    const int v_rd = (4 * hb + ((lane & 15) >> 2)) * VPAD + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    //                                            + (32*sb + 16*t + 8*u)*VPAD + 32*db
+
     float m_run[QB], l_run[QB];
-    f32x16 negm[QB];
     f32x16 o_acc[QB][DB];
-#pragma unroll
-    for (int j = 0; j < QB; ++j) {
-        m_run[j] = 0.f;
-        l_run[j] = 0.f;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) negm[j][v] = 0.f;
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) o_acc[j][db][v] = 0.f;
-    }
-    bool first = true;
 
-    if (n_tiles > 0) {
-        fetch(0);
-        stash(0);
-    }
-    __syncthreads();
-
-    for (int it = 0; it < n_tiles; ++it) {
-        const int cur = it & 1;
-        if (it + 1 < n_tiles) fetch(it + 1);
-
-        const bool is_ctx = it < ctx_tiles;
-        const int kv0 = is_ctx ? ctx_begin + it * BN : (it - ctx_tiles) * BN;
-        const int seg_end = is_ctx ? ctx_end : P.Nb;
-        const int w_min = is_ctx ? seg_end : wave_lim_min;
-        const int w_max = is_ctx ? seg_end : wave_lim_max;
-
+    // One pass over this workgroup's key tiles.  ROBUST selects the online softmax
+    // with a running maximum; otherwise p = 2^s is accumulated as is.
+    auto run_pass = [&](auto robust_tag) {
+        constexpr bool ROBUST = decltype(robust_tag)::value;
 #pragma unroll
-        for (int sb = 0; sb < SB; ++sb) {
-            const int blk0 = kv0 + 32 * sb;
-            if (blk0 >= w_max) continue;  // wave-uniform: nothing visible to this wavefront
-            const bool need_mask = blk0 + 32 > w_min;
-
-            vec ak[KS];
+        for (int j = 0; j < QB; ++j) {
+            m_run[j] = ROBUST ? -INFINITY : 0.f;
+            l_run[j] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks)
-                ak[ks] = *reinterpret_cast<const vec *>(&k_lds[cur][(32 * sb + c) * KPAD + 16 * ks + 8 * hb]);
-
-            f32x16 s[QB];
+            for (int db = 0; db < DB; ++db)
 #pragma unroll
-            for (int j = 0; j < QB; ++j) {
-                s[j] = negm[j];
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    s[j] = Ops::mma(ak[ks], qhi[j][ks], s[j]);
-                    s[j] = Ops::mma(ak[ks], qlo[j][ks], s[j]);
-                }
-            }
+                for (int v = 0; v < 16; ++v) o_acc[j][db][v] = 0.f;
+        }
 
-            if (need_mask) {
+        if (n_tiles > 0) {
+            fetch(0);
+            stash(0);
+        }
+        __syncthreads();
+
+        for (int it = 0; it < n_tiles; ++it) {
+            const int cur = it & 1;
+            if (it + 1 < n_tiles) fetch(it + 1);
+
+            const bool is_ctx = it < ctx_tiles;
+            const int kv0 = is_ctx ? ctx_begin + it * BN : (it - ctx_tiles) * BN;
+            const int seg_end = is_ctx ? ctx_end : P.Nb;
+            const int w_min = is_ctx ? seg_end : wave_lim_min;
+            const int w_max = is_ctx ? seg_end : wave_lim_max;
+            const T *kt = &k_lds[cur][k_rd];
+            const T *vt = &v_lds[cur][v_rd];
+
+            auto block = [&](int sb, auto mask_tag) {
+                constexpr bool MASK = decltype(mask_tag)::value;
+                const int blk0 = kv0 + 32 * sb;
+                vec ak[KS];
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    ak[ks] = *reinterpret_cast<const vec *>(kt + 32 * sb * KPAD + 16 * ks);
+
+                f32x16 s[QB];
 #pragma unroll
                 for (int j = 0; j < QB; ++j) {
-                    const int lj = is_ctx ? seg_end : lim[j];
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        int kv = blk0 + 8 * (v >> 2) + 4 * hb + (v & 3);
-                        if (kv >= lj) s[j][v] = -INFINITY;
+                    for (int v = 0; v < 16; ++v) s[j][v] = 0.f;
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) s[j] = Ops::mma(ak[ks], qreg[j][ks], s[j]);
+                }
+
+                if constexpr (MASK) {
+#pragma unroll
+                    for (int j = 0; j < QB; ++j) {
+                        const int lj = is_ctx ? seg_end : lim[j];
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            int kv = blk0 + 8 * (v >> 2) + 4 * hb + (v & 3);
+                            if (kv >= lj) s[j][v] = -INFINITY;
+                        }
                     }
                 }
-            }
 
-            unsigned pk[QB][8];
+                unsigned pk[QB][8];
 #pragma unroll
-            for (int j = 0; j < QB; ++j) {
-                // Common path: the scores already carry -m (accumulator init), so
-                // p = 2^s directly.  The running offset m is stale by design; it is
-                // refreshed only when this block's probabilities sum past
-                // 16 * 2^threshold (or overflow), which also covers any single
-                // score more than `threshold` above m.
-                float lsum = 0.f;
-                if (!first) {
+                for (int j = 0; j < QB; ++j) {
+                    if constexpr (ROBUST) {
+                        float tmax = s[j][0];
+#pragma unroll
+                        for (int v = 1; v < 16; ++v) tmax = fmaxf(tmax, s[j][v]);
+                        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+                        const float m_new = fmaxf(m_run[j], tmax);
+                        // m_new = -inf only while every key so far was masked: keep state at zero
+                        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+                        const float alpha = fast_exp2(m_run[j] - m_use);  // 2^(-inf) = 0 on the first block
+                        if (__any(alpha != 1.f)) {
+                            l_run[j] *= alpha;
+#pragma unroll
+                            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                                for (int v = 0; v < 16; ++v) o_acc[j][db][v] *= alpha;
+                        }
+                        m_run[j] = m_new;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) s[j][v] -= m_use;
+                    }
+                    float lsum = l_run[j];
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
                         pk[j][e] = pack2<T>(fast_exp2(s[j][2 * e]), fast_exp2(s[j][2 * e + 1]));
                         lsum = Ops::dot2(pk[j][e], lsum);
                     }
+                    l_run[j] = lsum;
                 }
-                const bool need = first || !(lsum <= kRescaleSum);
-                if (__any(need)) {
-                    float tmax = s[j][0];
+
 #pragma unroll
-                    for (int v = 1; v < 16; ++v) tmax = fmaxf(tmax, s[j][v]);
-                    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-                    float delta = first ? tmax : fmaxf(tmax, 0.f);
-                    if (delta == -INFINITY) delta = 0.f;
-                    const float alpha = fast_exp2(-delta);
-                    m_run[j] += delta;
-                    l_run[j] *= alpha;
+                for (int db = 0; db < DB; ++db) {
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        const T *vp = vt + (32 * sb + 16 * t) * VPAD + 32 * db;
+                        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (__attribute__((address_space(3))) s16x4 *)(vp));
+                        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (__attribute__((address_space(3))) s16x4 *)(vp + 8 * VPAD));
+                        typedef short s16x8 __attribute__((ext_vector_type(8)));
+                        s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                        vec av = __builtin_bit_cast(vec, both);
+#pragma unroll
+                        for (int j = 0; j < QB; ++j) {
+                            u32x4 pb = {pk[j][4 * t], pk[j][4 * t + 1], pk[j][4 * t + 2], pk[j][4 * t + 3]};
+                            o_acc[j][db] = Ops::mma(av, __builtin_bit_cast(vec, pb), o_acc[j][db]);
+                        }
+                    }
+                }
+            };
+
+#pragma unroll
+            for (int sb = 0; sb < SB; ++sb) {
+                const int blk0 = kv0 + 32 * sb;
+                if (blk0 >= w_max) continue;  // wave-uniform: nothing visible to this wavefront
+                if (blk0 + 32 > w_min)
+                    block(sb, BoolTag<true>{});
+                else
+                    block(sb, BoolTag<false>{});
+            }
+
+            if (it + 1 < n_tiles) stash(cur ^ 1);
+            __syncthreads();
+        }
+    };
+
+    // Fast pass: p = 2^s without a running maximum, software-pipelined so that the
+    // MFMAs of the next block's scores and of the previous block's PV product are
+    // issued between the exp/convert/sum VALU work of the current block.  Three LDS
+    // stages with one barrier per tile: tile it+2 is stored while tile it is
+    // computed and block 0 of tile it+1 is already being multiplied.
+    auto fast_pass = [&]() {
+#pragma unroll
+        for (int j = 0; j < QB; ++j) {
+            m_run[j] = 0.f;
+            l_run[j] = 0.f;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) o_acc[j][db][v] = 0.f;
+        }
+        if (n_tiles > 0) {
+            fetch(0);
+            stash(0);
+        }
+        if (n_tiles > 1) {
+            fetch(1);
+            stash(1);
+        }
+        __syncthreads();
+        if (n_tiles == 0) return;
+
+        auto scores = [&](f32x16(&dst)[QB], const T *kblk) {
+            vec ak[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) ak[ks] = *reinterpret_cast<const vec *>(kblk + 16 * ks);
+#pragma unroll
+            for (int j = 0; j < QB; ++j) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) dst[j][v] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) dst[j] = Ops::mma(ak[ks], qreg[j][ks], dst[j]);
+            }
+        };
+
+        f32x16 s_cur[QB];
+        scores(s_cur, &k_lds[0][k_rd]);
+
+        int stage = 0;
+        for (int it = 0; it < n_tiles; ++it) {
+            if (it > 0) __syncthreads();
+            if (it + 2 < n_tiles) fetch(it + 2);
+            const int stage_next = stage == 2 ? 0 : stage + 1;
+            const bool is_ctx = it < ctx_tiles;
+            const int kv0 = is_ctx ? ctx_begin + it * BN : (it - ctx_tiles) * BN;
+            const int seg_end = is_ctx ? ctx_end : P.Nb;
+            const int w_min = is_ctx ? seg_end : wave_lim_min;
+            const T *kt = &k_lds[stage][k_rd];
+            const T *vt = &v_lds[stage][v_rd];
+            // block after the last one of this tile: block 0 of the next tile (or, on the
+            // very last tile, any valid block — its scores are never used)
+            const T *kt_next = (it + 1 < n_tiles) ? &k_lds[stage_next][k_rd] : kt;
+
+            auto tile_body = [&](auto mask_tag) {
+                constexpr bool MASK = decltype(mask_tag)::value;
+#pragma unroll
+                for (int sb = 0; sb < SB; ++sb) {
+                    if constexpr (MASK) {
+                        const int blk0 = kv0 + 32 * sb;
+#pragma unroll
+                        for (int j = 0; j < QB; ++j) {
+                            const int lj = is_ctx ? seg_end : lim[j];
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) {
+                                int kv = blk0 + 8 * (v >> 2) + 4 * hb + (v & 3);
+                                if (kv >= lj) s_cur[j][v] = -INFINITY;
+                            }
+                        }
+                    }
+                    // LDS operands: V of this block, K of the next one
+                    vec av[DB][2];
 #pragma unroll
                     for (int db = 0; db < DB; ++db)
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) o_acc[j][db][v] *= alpha;
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) negm[j][v] = -m_run[j];
-                    lsum = 0.f;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        pk[j][e] = pack2<T>(fast_exp2(s[j][2 * e] - delta), fast_exp2(s[j][2 * e + 1] - delta));
-                        lsum = Ops::dot2(pk[j][e], lsum);
-                    }
-                }
-                l_run[j] += lsum;
-            }
-            first = false;
+                        for (int t = 0; t < 2; ++t) {
+                            const T *vp = vt + (32 * sb + 16 * t) * VPAD + 32 * db;
+                            s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                (__attribute__((address_space(3))) s16x4 *)(vp));
+                            s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                (__attribute__((address_space(3))) s16x4 *)(vp + 8 * VPAD));
+                            typedef short s16x8 __attribute__((ext_vector_type(8)));
+                            s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                            av[db][t] = __builtin_bit_cast(vec, both);
+                        }
+                    f32x16 s_next[QB];
+                    scores(s_next, sb + 1 < SB ? kt + 32 * (sb + 1) * KPAD : kt_next);
 
-#pragma unroll
-            for (int db = 0; db < DB; ++db) {
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    vec av = *reinterpret_cast<const vec *>(
-                        &v_lds[cur][(32 * db + c) * VPAD + 32 * sb + 16 * hb + 8 * t]);
+                    unsigned pk[QB][8];
 #pragma unroll
                     for (int j = 0; j < QB; ++j) {
-                        u32x4 pb = {pk[j][4 * t], pk[j][4 * t + 1], pk[j][4 * t + 2], pk[j][4 * t + 3]};
-                        o_acc[j][db] = Ops::mma(av, __builtin_bit_cast(vec, pb), o_acc[j][db]);
+                        float lsum = l_run[j];
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            pk[j][e] = pack2<T>(fast_exp2(s_cur[j][2 * e]), fast_exp2(s_cur[j][2 * e + 1]));
+                            lsum = Ops::dot2(pk[j][e], lsum);
+                        }
+                        l_run[j] = lsum;
+                    }
+#pragma unroll
+                    for (int j = 0; j < QB; ++j)
+#pragma unroll
+                        for (int db = 0; db < DB; ++db)
+#pragma unroll
+                            for (int t = 0; t < 2; ++t) {
+                                u32x4 pb = {pk[j][4 * t], pk[j][4 * t + 1], pk[j][4 * t + 2], pk[j][4 * t + 3]};
+                                o_acc[j][db] = Ops::mma(av[db][t], __builtin_bit_cast(vec, pb), o_acc[j][db]);
+                            }
+#pragma unroll
+                    for (int j = 0; j < QB; ++j) s_cur[j] = s_next[j];
+
+                    if constexpr (!MASK) {
+                        // Issue order for this block: the score MFMAs of the next block ride
+                        // under the first query block's exps, the PV MFMAs of query block j
+                        // under the exps of block j+1.
+                        __builtin_amdgcn_sched_group_barrier(0x100, KS + 4 * DB, 0);  // DS reads
+#pragma unroll
+                        for (int i = 0; i < QB * KS; ++i) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x400, 16 / (QB * KS) > 0 ? 16 / (QB * KS) : 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x002, 16 / (QB * KS) > 0 ? 16 / (QB * KS) : 1, 0);
+                        }
+#pragma unroll
+                        for (int j = 1; j < QB; ++j)
+#pragma unroll
+                            for (int i = 0; i < 2 * DB; ++i) {
+                                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x400, 16 / (2 * DB), 0);
+                                __builtin_amdgcn_sched_group_barrier(0x002, 16 / (2 * DB), 0);
+                            }
                     }
                 }
-            }
-        }
+            };
 
-        if (it + 1 < n_tiles) stash(cur ^ 1);
+            if (kv0 + BN > w_min)
+                tile_body(BoolTag<true>{});
+            else
+                tile_body(BoolTag<false>{});
+
+            if (it + 2 < n_tiles) stash(stage == 0 ? 2 : stage - 1);
+            stage = stage_next;
+        }
         __syncthreads();
+    };
+
+    bool robust = !Ops::kWideExponent || P.force_robust;
+    if (!robust) {
+        fast_pass();
+        bool bad = false;
+#pragma unroll
+        for (int j = 0; j < QB; ++j) {
+            const float l_tot = l_run[j] + __shfl_xor(l_run[j], 32, 64);
+            bad = bad || !(l_tot > kFastMassMin && l_tot < kFastMassMax);
+        }
+        if (tid == 0) redo_flag = 0;
+        __syncthreads();
+        if (bad) redo_flag = 1;
+        __syncthreads();
+        robust = redo_flag != 0;
     }
+    if (robust) run_pass(BoolTag<true>{});
 
     // ---- epilogue: normalise, write output (final or split partial) and log-sum-exp.
     const long total_rows = static_cast<long>(P.B) * P.H * P.Lq;
@@ -411,7 +580,8 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
         float l_tot = l_run[j] + __shfl_xor(l_run[j], 32, 64);
         if (orow_idx[j] < 0) continue;
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-        const float lse = l_tot > 0.f ? (m_run[j] + fast_log2(l_tot)) * kLn2 : -INFINITY;
+        const float m_fin = m_run[j] == -INFINITY ? 0.f : m_run[j];
+        const float lse = l_tot > 0.f ? (m_fin + fast_log2(l_tot)) * kLn2 : -INFINITY;
         if (P.part_o) {
             float *po = P.part_o + (static_cast<long>(split) * total_rows + orow_idx[j]) * DH;
 #pragma unroll
