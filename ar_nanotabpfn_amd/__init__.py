@@ -23,4 +23,23 @@ from .attention_kernels import (  # noqa: F401
     triton_context_attention,
 )
 
+from .attention import (  # noqa: F401,E402
+    DecodeMask,
+    DenseMask,
+    MultiheadAttention,
+    TeacherForcingMask,
+    clear_mask_cache,
+    create_context_self_attention_mask,
+    create_dense_mask,
+    create_row_mask,
+)
+from .inference import ARTabPFNPredictor  # noqa: F401,E402
+from .model import (  # noqa: F401,E402
+    ARTabPFN,
+    Embedder,
+    MixtureGaussianHead,
+    TwoStageTransformer,
+    TwoStageTransformerLayer,
+)
+
 __version__ = "0.1.0"

@@ -47,6 +47,8 @@ SIGNATURES = {
     "artab_version": (_i, []),
     "artab_status_string": (ctypes.c_char_p, [_i]),
     "artab_last_error": (ctypes.c_char_p, []),
+    "artab_profile_begin": (_i, [_i]),
+    "artab_profile_end": (_i, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_i)]),
     "artab_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
     "artab_context_attention": (_i, [_VP, _VP, _VP, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _p, _sz, _i, _p]),
     "artab_decode_attention": (

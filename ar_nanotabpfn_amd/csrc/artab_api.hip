@@ -19,6 +19,29 @@ namespace artab {
 
 static thread_local char g_err[512] = "";
 
+// Optional timing of the MFMA context-pass launches (benchmark aid; off by default).
+// While enabled, each such launch is bracketed by a pair of HIP events on its stream.
+struct ProfileState {
+    bool enabled = false;
+    int capacity = 0, used = 0;
+    hipEvent_t *start = nullptr, *stop = nullptr;
+};
+static ProfileState g_prof;
+
+struct ProfileScope {
+    hipStream_t stream;
+    int slot;
+    explicit ProfileScope(hipStream_t st) : stream(st), slot(-1) {
+        if (g_prof.enabled && g_prof.used < g_prof.capacity) {
+            slot = g_prof.used++;
+            (void)hipEventRecord(g_prof.start[slot], stream);
+        }
+    }
+    ~ProfileScope() {
+        if (slot >= 0) (void)hipEventRecord(g_prof.stop[slot], stream);
+    }
+};
+
 static int fail(int code, const char *fmt, ...) {
     va_list ap;
     va_start(ap, fmt);
@@ -276,6 +299,47 @@ const char *artab_status_string(int status) {
 
 const char *artab_last_error(void) { return g_err; }
 
+int artab_profile_begin(int max_records) {
+    if (max_records <= 0) return fail(ARTAB_ERR_BAD_SHAPE, "max_records must be positive");
+    if (g_prof.capacity < max_records) {
+        for (int i = 0; i < g_prof.capacity; ++i) {
+            (void)hipEventDestroy(g_prof.start[i]);
+            (void)hipEventDestroy(g_prof.stop[i]);
+        }
+        delete[] g_prof.start;
+        delete[] g_prof.stop;
+        g_prof.start = new hipEvent_t[max_records];
+        g_prof.stop = new hipEvent_t[max_records];
+        g_prof.capacity = 0;
+        for (int i = 0; i < max_records; ++i) {
+            if (hipEventCreate(&g_prof.start[i]) != hipSuccess || hipEventCreate(&g_prof.stop[i]) != hipSuccess)
+                return fail(ARTAB_ERR_LAUNCH, "hipEventCreate failed");
+            g_prof.capacity = i + 1;
+        }
+    }
+    g_prof.used = 0;
+    g_prof.enabled = true;
+    return ARTAB_OK;
+}
+
+int artab_profile_end(double *total_ms, int *records) {
+    g_prof.enabled = false;
+    double sum = 0.0;
+    int n = 0;
+    for (int i = 0; i < g_prof.used; ++i) {
+        if (hipEventSynchronize(g_prof.stop[i]) != hipSuccess) continue;
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, g_prof.start[i], g_prof.stop[i]) == hipSuccess) {
+            sum += ms;
+            ++n;
+        }
+    }
+    if (total_ms) *total_ms = sum;
+    if (records) *records = n;
+    g_prof.used = 0;
+    return ARTAB_OK;
+}
+
 size_t artab_workspace_bytes(int B, int H, int Lq, int Nc, int Dh, int dtype) {
     if (B <= 0 || H <= 0 || Lq <= 0 || Nc <= 0 || !mfma_shape_ok(dtype, Dh)) return 0;
     // Upper bound over the two schedules (queries stacked over a shared context, or
@@ -340,7 +404,10 @@ int artab_context_attention(const artab_view *q, const artab_view *k_ctx, const 
         F.part_o = static_cast<float *>(workspace);
         F.part_lse = F.part_o + static_cast<size_t>(pl.n_split) * rows * Dh;
     }
-    ARTAB_TRY(launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "context attention (mfma)"));
+    {
+        ProfileScope prof(st);
+        ARTAB_TRY(launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "context attention (mfma)"));
+    }
     if (pl.n_split > 1) {
         CombineParams C;
         C.out = dv(out); C.part_o = F.part_o; C.part_lse = F.part_lse; C.lse = lse;
@@ -433,7 +500,10 @@ int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const a
         F.part_o = static_cast<float *>(workspace);
         F.part_lse = F.part_o + static_cast<size_t>(pl.n_split) * rows * Dh;
     }
-    ARTAB_TRY(launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "decode context pass"));
+    {
+        ProfileScope prof(st);
+        ARTAB_TRY(launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "decode context pass"));
+    }
     if (!need_ws) return ARTAB_OK;
 
     DecodeParams D;
@@ -488,6 +558,7 @@ int artab_teacher_forcing_attention(const artab_view *q, const artab_view *k_ctx
     F.n_split = 1; F.kv_per_split = pl.kv_per_split;
     F.qscale = scale * kLog2e;
     F.mode = kFlashTeacher;
+    ProfileScope prof(st);
     return launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "teacher forcing (mfma)");
 }
 
@@ -536,6 +607,7 @@ int artab_prefill_attention(const artab_view *q, const artab_view *k, const arta
     F.n_split = 1; F.kv_per_split = pl.kv_per_split;
     F.qscale = scale * kLog2e;
     F.mode = kFlashPrefill;
+    ProfileScope prof(st);
     return launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "prefill (mfma)");
 }
 

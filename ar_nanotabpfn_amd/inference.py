@@ -1,0 +1,317 @@
+"""Autoregressive predictor with KV caching (host-side mirror of the reference's
+``ar_tabpfn/model/inference.py``), driving the HIP attention kernels.
+
+Same constructor, method names, cache attributes and state as the reference's
+``ARTabPFNPredictor``.  Two cache layouts, selected by ``backend`` under the
+reference's names:
+
+* ``"triton_shared_context"`` — one context K/V ``[H,Nc,Dh]`` for every trajectory
+  (``layer.k_ctx_cache`` / ``v_ctx_cache``) plus a preallocated per-trajectory buffer
+  cache ``[B,H,max_buf,Dh]`` (``layer.k_buf_cache`` / ``v_buf_cache``) that decode
+  steps append to in place (inference.py:107-122, :746-833).
+* ``"flex_attention"`` — one full cache ``[B,H,max_seq,Dh]`` per batch entry
+  (``layer.k_cache`` / ``v_cache``) for per-dataset contexts (inference.py:124-135,
+  :687-744).
+
+Both run on the same kernels; the names only choose the layout.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch import Tensor
+
+from . import attention_kernels as ak
+from .attention import DecodeMask, TeacherForcingMask
+
+__all__ = ["ARTabPFNPredictor"]
+
+_SHARED = "triton_shared_context"
+_PER_DATASET = "flex_attention"
+_ALIASES = {"shared_context": _SHARED, "per_dataset": _PER_DATASET}
+
+
+class ARTabPFNPredictor:
+    """Joint sampling and log-density evaluation (inference.py:32-453)."""
+
+    def __init__(self, embedder, backbone, head, ar_tokens, backend: str = "flex_attention"):
+        self.embedder = embedder
+        self.backbone = backbone
+        self.head = head
+        self.ar_tokens = ar_tokens
+        backend = _ALIASES.get(backend, backend)
+        if backend not in (_PER_DATASET, _SHARED):
+            raise ValueError(f"Unsupported backend: {backend}")
+        self.backend = backend
+        self.seq_len = 0          # committed keys in the full cache (per-dataset layout)
+        self.context_len = 0      # context rows (shared layout)
+        self.buffer_len = 0       # committed buffer rows (shared layout)
+        self.max_buffer_len = 0   # capacity of the buffer cache (shared layout)
+        self._device = None
+        self._dtype = None
+
+    @classmethod
+    def from_trained_model(cls, model, backend: str = "flex_attention") -> "ARTabPFNPredictor":
+        return cls(model.embedder, model.backbone, model.head, model.ar_tokens, backend=backend)
+
+    # ------------------------------------------------------------------ cache state
+
+    def init_kv_cache(self, batch_size: int, max_seq_len: int, device=None, dtype=None) -> None:
+        """Allocate the caches.  ``max_seq_len`` is the buffer capacity for the shared
+        layout and context + buffers (+ targets for teacher forcing) for the full cache,
+        as in the reference (inference.py:94-95)."""
+        if device is None or dtype is None:
+            param = next(self.backbone.parameters())
+            device = device or param.device
+            dtype = dtype or param.dtype
+        self._device, self._dtype = device, dtype
+        self.seq_len = self.context_len = self.buffer_len = 0
+        if self.backend == _SHARED:
+            self.max_buffer_len = max_seq_len
+            for layer in self.backbone.layers:
+                H, Dh = layer.attn_rows.n_heads, layer.attn_rows.head_dim
+                layer.k_ctx_cache = torch.empty((H, 0, Dh), device=device, dtype=dtype)
+                layer.v_ctx_cache = torch.empty_like(layer.k_ctx_cache)
+                layer.k_buf_cache = torch.zeros(batch_size, H, max_seq_len, Dh, device=device, dtype=dtype)
+                layer.v_buf_cache = torch.zeros_like(layer.k_buf_cache)
+            return
+        self.max_buffer_len = 0
+        for layer in self.backbone.layers:
+            H, Dh = layer.attn_rows.n_heads, layer.attn_rows.head_dim
+            layer.k_cache = torch.zeros(batch_size, H, max_seq_len, Dh, device=device, dtype=dtype)
+            layer.v_cache = torch.zeros_like(layer.k_cache)
+
+    def clear_cache(self) -> None:
+        """Reset the cursors, keep the memory (inference.py:137-141)."""
+        self.seq_len = self.context_len = self.buffer_len = 0
+
+    # ------------------------------------------------------------------ per-layer pieces
+
+    @staticmethod
+    def _qkv(layer, x_row: Tensor):
+        a = layer.attn_rows
+        return a.split_heads(a.q_proj(x_row)), a.split_heads(a.k_proj(x_row)), a.split_heads(a.v_proj(x_row))
+
+    # ------------------------------------------------------------------ prefill
+
+    @torch.no_grad()
+    def prefill_context(self, x_context: Tensor, y_context: Tensor) -> None:
+        """Encode the context and fill the caches; rows ``[0,Nc)`` hold context K/V
+        afterwards (inference.py:143-178)."""
+        if self.backend == _SHARED:
+            self.prefill_context_shared(x_context, y_context)
+            return
+        x_row = self.embedder.embed_context(x_context, y_context)
+        Nc = x_row.shape[1]
+        for layer in self.backbone.layers:
+            if layer.k_cache.shape[2] < Nc:
+                raise ValueError("KV cache too small for the context; call init_kv_cache with a larger max_seq_len.")
+            x_row = layer.feature_stage(x_row)
+            q, k, v = self._qkv(layer, x_row)
+            attn = ak.prefill_attention(q, k, v, layer.k_cache, layer.v_cache)
+            x_row = layer.finish(x_row, attn)
+        self.seq_len = Nc
+
+    @torch.no_grad()
+    def prefill_context_shared(self, x_context: Tensor, y_context: Tensor) -> None:
+        """Shared layout: only batch entry 0 is encoded — the context is taken to be the
+        same for every trajectory (inference.py:180-223)."""
+        Nc = x_context.shape[1]
+        x_row = self.embedder.embed_context(x_context[0:1], y_context[0:1])
+        for layer in self.backbone.layers:
+            H, Dh = layer.attn_rows.n_heads, layer.attn_rows.head_dim
+            if layer.k_ctx_cache.shape[1] != Nc or layer.k_ctx_cache.shape[0] != H:
+                layer.k_ctx_cache = torch.zeros(H, Nc, Dh, device=x_row.device, dtype=x_row.dtype)
+                layer.v_ctx_cache = torch.zeros_like(layer.k_ctx_cache)
+            x_row = layer.feature_stage(x_row)
+            q, k, v = self._qkv(layer, x_row)
+            attn = ak.prefill_attention(q, k, v, layer.k_ctx_cache, layer.v_ctx_cache)
+            x_row = layer.finish(x_row, attn)
+        self.context_len = Nc
+        self.buffer_len = 0
+        self.seq_len = Nc
+        self._prefill_batch_size = x_context.shape[0]
+
+    # ------------------------------------------------------------------ decode
+
+    @torch.no_grad()
+    def transformer_decode(self, embedding: Tensor, commit: int) -> Tensor:
+        """Run ``[B,N,D]`` new rows through the stack against the caches and commit the
+        first ``commit`` of them (N-1 for ``[buffer, target]``, 0 for ``[target]``);
+        returns the normed ``[B,N,D]`` (inference.py:225-276)."""
+        B, N, D = embedding.shape
+        x_row = embedding
+        if self.backend == _SHARED:
+            if self.buffer_len + commit > self.max_buffer_len:
+                raise ValueError("Shared-context buffer cache exceeded; increase max buffer length.")
+            for layer in self.backbone.layers:
+                x_row = self._layer_decode_with_cache_shared(layer, x_row, commit)
+            self.buffer_len += commit
+            self.seq_len = self.context_len + self.buffer_len
+            return self.backbone.norm(x_row)
+
+        mask = DecodeMask(num_cached=self.seq_len, num_new=N)
+        for layer in self.backbone.layers:
+            x_row = self._layer_decode_with_cache(layer, x_row, mask, cache_start=self.seq_len)
+        self.seq_len += commit
+        return self.backbone.norm(x_row)
+
+    def _layer_decode_with_cache_shared(self, layer, x_row: Tensor, commit: int = 1) -> Tensor:
+        """One layer of a decode step on the shared layout (inference.py:746-833): both
+        queries of a ``[buffer, target]`` pair see context + committed buffers + the new
+        buffer row, which is appended in place by the same kernel call."""
+        B, N, D = x_row.shape
+        if N not in (1, 2):
+            raise ValueError("Shared-context decode only supports N=1 (target) or N=2 (buffer, target).")
+        x_row = layer.feature_stage(x_row)
+        q, k_new, v_new = self._qkv(layer, x_row)
+        k_ctx = layer.k_ctx_cache[:, : self.context_len]
+        v_ctx = layer.v_ctx_cache[:, : self.context_len]
+        if N == 1:
+            attn = ak.decode_attention(q, k_ctx, v_ctx, layer.k_buf_cache, layer.v_buf_cache, self.buffer_len)
+        else:
+            attn = ak.decode_attention(
+                q, k_ctx, v_ctx, layer.k_buf_cache, layer.v_buf_cache, self.buffer_len,
+                k_new[:, :, 0:1], v_new[:, :, 0:1],
+            )
+        return layer.finish(x_row, attn)
+
+    def _layer_decode_with_cache(self, layer, x_row: Tensor, mask, cache_start: int) -> Tensor:
+        """One layer on the full per-dataset cache (inference.py:687-744): the new K/V are
+        written at ``[cache_start, cache_start+N)`` and the queries attend under ``mask``."""
+        B, N, D = x_row.shape
+        x_row = layer.feature_stage(x_row)
+        q, k_new, v_new = self._qkv(layer, x_row)
+        if layer.k_cache.shape[2] < cache_start + N:
+            raise ValueError("KV cache exceeded; increase max_seq_len.")
+        if isinstance(mask, TeacherForcingMask):
+            Nt = mask.num_targets
+            layer.k_cache[:, :, cache_start : cache_start + N] = k_new
+            layer.v_cache[:, :, cache_start : cache_start + N] = v_new
+            attn = ak.teacher_forcing_attention(
+                q, layer.k_cache[:, :, :cache_start], layer.v_cache[:, :, :cache_start],
+                k_new[:, :, :Nt], v_new[:, :, :Nt], Nt,
+            )
+        elif N in (1, 2):
+            # context = cached keys of this batch entry; the new buffer row lands in slot
+            # cache_start of the same cache (the "buffer" view starts there)
+            k_tail, v_tail = layer.k_cache[:, :, cache_start:], layer.v_cache[:, :, cache_start:]
+            attn = ak.decode_attention(
+                q, layer.k_cache[:, :, :cache_start], layer.v_cache[:, :, :cache_start], k_tail, v_tail, 0,
+                k_new[:, :, 0:1] if N == 2 else None, v_new[:, :, 0:1] if N == 2 else None,
+            )
+            if N == 2:  # the reference also parks the target's K/V behind it until the next step
+                layer.k_cache[:, :, cache_start + 1 : cache_start + 2] = k_new[:, :, 1:2]
+                layer.v_cache[:, :, cache_start + 1 : cache_start + 2] = v_new[:, :, 1:2]
+            else:
+                layer.k_cache[:, :, cache_start : cache_start + 1] = k_new
+                layer.v_cache[:, :, cache_start : cache_start + 1] = v_new
+        else:
+            # general N: cached keys + causal part among the new rows (inference.py:512-519)
+            layer.k_cache[:, :, cache_start : cache_start + N] = k_new
+            layer.v_cache[:, :, cache_start : cache_start + N] = v_new
+            out_c, lse_c = ak.context_attention(q, layer.k_cache[:, :, :cache_start], layer.v_cache[:, :, :cache_start])
+            qi = torch.arange(N, device=q.device)[:, None]
+            kj = torch.arange(N, device=q.device)[None, :]
+            new_mask = torch.where(qi == N - 1, kj < qi, kj <= qi)[None, None]
+            out_n, lse_n = ak.buffer_attention(q, k_new, v_new, mask=new_mask)
+            attn = ak.merge_attention_outputs(out_c, lse_c, out_n, lse_n)
+        return layer.finish(x_row, attn)
+
+    @torch.no_grad()
+    def autoregressive_decode(self, x_target: Tensor, prev_x: Optional[Tensor] = None,
+                              prev_y: Optional[Tensor] = None, ar_idx: int = 0) -> Tensor:
+        """Decode one target, feeding the previous prediction back as a buffer row;
+        returns the sampled ``[B,1]`` (inference.py:278-320)."""
+        target_emb = self.embedder.embed_target(x_target)
+        if prev_x is not None and prev_y is not None:
+            buffer_emb = self.embedder.embed_buffer(prev_x, prev_y) + self.ar_tokens[ar_idx]
+            embedding, commit = torch.cat([buffer_emb, target_emb], dim=1), 1
+        else:
+            embedding, commit = target_emb, 0
+        z = self.transformer_decode(embedding, commit=commit)
+        return self.head.sample(z[:, -1:, :])[:, :, 0, 0]
+
+    @torch.no_grad()
+    def sample_sequence(self, x_context: Tensor, y_context: Tensor, x_target: Tensor) -> Tensor:
+        """Sample all targets autoregressively -> ``[B,Nt]`` (inference.py:322-366)."""
+        B, Nc, _ = x_context.shape
+        Nt = x_target.shape[1]
+        device, dtype = x_context.device, x_context.dtype
+        self.init_kv_cache(B, Nt if self.backend == _SHARED else Nc + Nt, device, dtype)
+        self.prefill_context(x_context, y_context)
+        preds = []
+        prev_x = prev_y = None
+        for t in range(Nt):
+            x_t = x_target[:, t : t + 1, :]
+            y_t = self.autoregressive_decode(x_t, prev_x, prev_y, t % self.ar_tokens.shape[0])
+            preds.append(y_t)
+            prev_x, prev_y = x_t, y_t
+        return torch.cat(preds, dim=1)
+
+    # ------------------------------------------------------------------ teacher forcing
+
+    @torch.no_grad()
+    def evaluate_joint_density(self, x_context: Tensor, y_context: Tensor, x_target: Tensor,
+                               y_target: Tensor) -> Tensor:
+        """Log-density ``[B,Nt]`` of the targets in one teacher-forced pass
+        (inference.py:368-453)."""
+        if self.backend == _SHARED:
+            return self._evaluate_joint_density_shared(x_context, y_context, x_target, y_target)
+        return self._evaluate_joint_density_flex(x_context, y_context, x_target, y_target)
+
+    def _teacher_forcing_embedding(self, x_target: Tensor, y_target: Tensor) -> Tensor:
+        Nt = x_target.shape[1]
+        pos = torch.arange(Nt, device=x_target.device) % self.ar_tokens.shape[0]
+        buffer_emb = self.embedder.embed_buffer(x_target, y_target) + self.ar_tokens[pos]
+        return torch.cat([buffer_emb, self.embedder.embed_target(x_target)], dim=1)
+
+    def _evaluate_joint_density_shared(self, x_context, y_context, x_target, y_target) -> Tensor:
+        B, Nt = x_context.shape[0], x_target.shape[1]
+        self.init_kv_cache(B, Nt, x_context.device, x_context.dtype)
+        self.prefill_context(x_context, y_context)
+        z = self._teacher_forcing_decode_shared(self._teacher_forcing_embedding(x_target, y_target), Nt)
+        return self.head.log_likelihood(z[:, Nt:, :], y_target.unsqueeze(-1))
+
+    def _evaluate_joint_density_flex(self, x_context, y_context, x_target, y_target) -> Tensor:
+        B, Nc = x_context.shape[0], x_context.shape[1]
+        Nt = x_target.shape[1]
+        self.init_kv_cache(B, Nc + 2 * Nt, x_context.device, x_context.dtype)
+        self.prefill_context(x_context, y_context)
+        z = self._teacher_forcing_decode(self._teacher_forcing_embedding(x_target, y_target), Nt)
+        return self.head.log_likelihood(z[:, Nt:, :], y_target.unsqueeze(-1))
+
+    @torch.no_grad()
+    def _teacher_forcing_decode(self, embedding: Tensor, num_targets: int) -> Tensor:
+        """``[buffers, targets]`` under the teacher-forcing mask on the full cache
+        (inference.py:455-471)."""
+        if embedding.shape[1] != 2 * num_targets:
+            raise ValueError("Expected N == 2*num_targets for teacher forcing.")
+        mask = TeacherForcingMask(num_cached=self.seq_len, num_targets=num_targets)
+        x_row = embedding
+        for layer in self.backbone.layers:
+            x_row = self._layer_decode_with_cache(layer, x_row, mask, cache_start=self.seq_len)
+        return self.backbone.norm(x_row)
+
+    @torch.no_grad()
+    def _teacher_forcing_decode_shared(self, embedding: Tensor, num_targets: int) -> Tensor:
+        x_row = embedding
+        for layer in self.backbone.layers:
+            x_row = self._layer_teacher_forcing_shared(layer, x_row, num_targets)
+        return self.backbone.norm(x_row)
+
+    def _layer_teacher_forcing_shared(self, layer, x_row: Tensor, num_targets: int) -> Tensor:
+        """inference.py:835-890: buffer K/V are the fresh projections of the first Nt
+        rows; the buffer cache is neither read nor written."""
+        B, N, D = x_row.shape
+        if N != 2 * num_targets:
+            raise ValueError("Expected N == 2*num_targets for teacher forcing.")
+        x_row = layer.feature_stage(x_row)
+        q, k, v = self._qkv(layer, x_row)
+        attn = ak.hybrid_teacher_forcing_attention(
+            q, layer.k_ctx_cache[:, : self.context_len], layer.v_ctx_cache[:, : self.context_len],
+            k[:, :, :num_targets], v[:, :, :num_targets], num_targets,
+        )
+        return layer.finish(x_row, attn)

@@ -1,0 +1,198 @@
+"""AR-TabPFN modules (host-side mirror of the reference's ``ar_tabpfn/model/model.py``).
+
+Plain PyTorch-ROCm around the HIP attention kernels.  Module names, parameter
+shapes, construction order (hence seeded initialisation) and ``state_dict`` keys
+follow the reference so checkpoints interchange: ``embedder.{x_embed,y_embed}``,
+``embedder.marker_embed``, ``backbone.layers.{i}.{attn_features,attn_rows}.*_proj``,
+``backbone.layers.{i}.ff.{0,2}``, ``backbone.layers.{i}.norm{1,2,3}``,
+``backbone.norm``, ``head.head.{0,2}``, ``head.{mean_bias,std_bias,weight_bias}``,
+``ar_tokens`` (model.py:33-37, :89-98, :138, :172-184, :315).
+
+The training forward (flex_attention with the context/buffer/target row mask,
+model.py:317-369) is not part of this package; inference goes through
+``ARTabPFNPredictor``.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+
+from .attention import DenseMask, MultiheadAttention
+
+__all__ = ["Embedder", "TwoStageTransformerLayer", "TwoStageTransformer", "MixtureGaussianHead", "ARTabPFN"]
+
+_MARKERS = {"target": 0, "context": 1, "buffer": 2}  # model.py:36-38
+
+
+class Embedder(nn.Module):
+    """Scalar-wise feature embedding averaged over features, plus the y embedding and a
+    learned marker per row kind (model.py:23-76)."""
+
+    def __init__(self, d_model: int):
+        super().__init__()
+        self.x_embed = nn.Linear(1, d_model)
+        self.y_embed = nn.Linear(1, d_model)
+        self.marker_embed = nn.Embedding(3, d_model)
+
+    def _x(self, x: Tensor) -> Tensor:
+        # mean_c(x_c * w + b) == mean_c(x_c) * w + b: one [B,N,D] result instead of [B,N,C,D]
+        return self.x_embed(x.mean(dim=-1, keepdim=True))
+
+    def _y(self, y: Tensor) -> Tensor:
+        return self.y_embed(y.unsqueeze(-1) if y.dim() == 2 else y)
+
+    def _marker(self, kind: str) -> Tensor:
+        return self.marker_embed.weight[_MARKERS[kind]]
+
+    def embed_context(self, x: Tensor, y: Tensor) -> Tensor:
+        """x ``[B,N,C]``, y ``[B,N]`` or ``[B,N,1]`` -> ``[B,N,D]``."""
+        return self._x(x) + self._y(y) + self._marker("context")
+
+    def embed_buffer(self, x: Tensor, y: Tensor) -> Tensor:
+        """Buffer rows; the AR position token is added by the caller."""
+        return self._x(x) + self._y(y) + self._marker("buffer")
+
+    def embed_target(self, x: Tensor) -> Tensor:
+        return self._x(x) + self._marker("target")
+
+
+class TwoStageTransformerLayer(nn.Module):
+    """Feature attention over columns, row attention, feed-forward; post-norm
+    (model.py:79-126)."""
+
+    def __init__(self, d_model: int, n_heads: int, d_ff: int):
+        super().__init__()
+        self.attn_features = MultiheadAttention(d_model, n_heads)
+        self.attn_rows = MultiheadAttention(d_model, n_heads)
+        self.ff = nn.Sequential(nn.Linear(d_model, d_ff), nn.GELU(), nn.Linear(d_ff, d_model))
+        self.norm1 = nn.LayerNorm(d_model)
+        self.norm2 = nn.LayerNorm(d_model)
+        self.norm3 = nn.LayerNorm(d_model)
+
+    def feature_stage(self, x_row: Tensor) -> Tensor:
+        """Feature attention for the single-column case (C = 1) followed by norm1.
+
+        One key per query: the softmax weight is exactly 1, so the attention output is
+        ``out_proj(v_proj(x))`` and the q/k projections do not enter
+        (attention.py:52-61 with S = 1; inference.py:771-773)."""
+        a = self.attn_features
+        return self.norm1(a.out_proj(a.v_proj(x_row)) + x_row)
+
+    def finish(self, x_row: Tensor, attn_heads: Tensor) -> Tensor:
+        """``out_proj`` on ``[B,H,N,Dh]`` attention output, then norm2 / FFN / norm3
+        (inference.py:825-831)."""
+        B, H, N, Dh = attn_heads.shape
+        attn = self.attn_rows.out_proj(attn_heads.transpose(1, 2).reshape(B, N, H * Dh))
+        x_row = self.norm2(x_row + attn)
+        return self.norm3(x_row + self.ff(x_row))
+
+    def forward(self, x: Tensor, mask_features: DenseMask, mask_rows: DenseMask) -> Tuple[Tensor, Tuple[Tensor, Tensor]]:
+        """``[B,R,C,D]`` with dense masks only (the bidirectional context pass)."""
+        B, R, C, D = x.shape
+        if C != 1:
+            raise NotImplementedError("only the single-column layout (C = 1) is used by this model")
+        x_row = self.feature_stage(x.squeeze(2))
+        attn, kv = self.attn_rows(x_row, x_row, x_row, mask_rows)
+        x_row = self.norm2(x_row + attn)
+        return self.norm3(x_row + self.ff(x_row)).unsqueeze(2), kv
+
+
+class TwoStageTransformer(nn.Module):
+    def __init__(self, d_model: int, n_heads: int, n_layers: int, d_ff: int):
+        super().__init__()
+        self.d_model = d_model
+        self.layers = nn.ModuleList([TwoStageTransformerLayer(d_model, n_heads, d_ff) for _ in range(n_layers)])
+        self.norm = nn.LayerNorm(d_model)
+
+    def forward(self, x: Tensor, mask_features: DenseMask, mask_rows: DenseMask) -> Tuple[Tensor, List[Tuple[Tensor, Tensor]]]:
+        kvs = []
+        for layer in self.layers:
+            x, kv = layer(x, mask_features, mask_rows)
+            kvs.append(kv)
+        return self.norm(x), kvs
+
+
+class MixtureGaussianHead(nn.Module):
+    """Mixture-of-Gaussians regression head (model.py:150-272)."""
+
+    def __init__(self, d_model: int, d_ff: int, dim_y: int = 1, num_components: int = 5, std_min: float = 1e-3):
+        super().__init__()
+        self.dim_y = dim_y
+        self.num_components = num_components
+        self.std_min = std_min
+        self.head = nn.Sequential(nn.Linear(d_model, d_ff), nn.GELU(), nn.Linear(d_ff, num_components * dim_y * 3))
+        self.mean_bias = nn.Parameter(torch.linspace(-1.0, 1.0, num_components))
+        delta = 1.0 / (num_components - 1)
+        self.std_bias = nn.Parameter(torch.full((num_components,), math.log(math.expm1(delta))))
+        self.weight_bias = nn.Parameter(torch.zeros(num_components))
+
+    def _parameterize(self, z: Tensor) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+        """``[B,T,D] -> mean, std, weight, log_weight`` each ``[B,T,K,dim_y]``; the raw
+        output is laid out ``(K, dim_y, 3)`` (model.py:195-196)."""
+        B, T, _ = z.shape
+        raw = self.head(z).view(B, T, self.num_components, self.dim_y, 3)
+        bias = lambda p: p.view(1, 1, -1, 1)  # noqa: E731
+        mean = raw[..., 0] + bias(self.mean_bias)
+        std = F.softplus(raw[..., 1] + bias(self.std_bias)).clamp(max=2.0) + self.std_min
+        log_weight = F.log_softmax(raw[..., 2] + bias(self.weight_bias), dim=2)
+        return mean, std, log_weight.exp(), log_weight
+
+    @staticmethod
+    def _log_likelihood(y: Tensor, mean: Tensor, std: Tensor, log_weight: Tensor) -> Tensor:
+        z = (y.unsqueeze(2) - mean) / std
+        comp = -0.5 * (math.log(2 * math.pi) + z * z) - std.log() + log_weight
+        return torch.logsumexp(comp, dim=2)
+
+    def forward(self, z: Tensor, y: Optional[Tensor] = None, loss_mask: Optional[Tensor] = None):
+        mean, std, weight, log_weight = self._parameterize(z)
+        loss = None
+        if y is not None:
+            ll = self._log_likelihood(y, mean, std, log_weight)
+            if loss_mask is not None:
+                ll = ll.mean(-1) * loss_mask
+                denom = loss_mask.sum().clamp(min=1)
+            else:
+                denom = ll.numel()
+            loss = -ll.sum() / denom
+        return loss, mean, std, weight
+
+    def sample(self, z: Tensor, num_samples: int = 1) -> Tensor:
+        """``[B,T,D] -> [B,T,num_samples,dim_y]``: pick a component per draw, then a normal."""
+        mean, std, weight, _ = self._parameterize(z)
+        B, T, K, Dy = mean.shape
+        flat = lambda t: t.permute(0, 1, 3, 2).reshape(B * T * Dy, K)  # noqa: E731
+        idx = torch.multinomial(flat(weight), num_samples, replacement=True)
+        mu = torch.gather(flat(mean), 1, idx).view(B, T, Dy, num_samples)
+        sd = torch.gather(flat(std), 1, idx).view(B, T, Dy, num_samples)
+        return (mu + sd * torch.randn_like(mu)).permute(0, 1, 3, 2)
+
+    def log_likelihood(self, z: Tensor, y: Tensor) -> Tensor:
+        """``z [B,T,D]``, ``y [B,T,dim_y]`` -> ``[B,T]``."""
+        mean, std, _, log_weight = self._parameterize(z)
+        return self._log_likelihood(y, mean, std, log_weight).sum(dim=-1)
+
+
+class ARTabPFN(nn.Module):
+    """Container with the reference's constructor and attribute names (model.py:275-315)."""
+
+    def __init__(self, d_model: int = 128, n_heads: int = 4, n_layers: int = 6, d_ff: int = 256,
+                 num_features: int = 10, buffer_size: int = 8, num_components: int = 5):
+        super().__init__()
+        self.d_model = d_model
+        self.num_features = num_features
+        self.buffer_size = buffer_size
+        self.embedder = Embedder(d_model)
+        self.backbone = TwoStageTransformer(d_model, n_heads, n_layers, d_ff)
+        self.head = MixtureGaussianHead(d_model, d_ff, dim_y=1, num_components=num_components)
+        self.ar_tokens = nn.Parameter(torch.randn(buffer_size, d_model) * 0.02)
+
+    def forward(self, *args, **kwargs):
+        raise NotImplementedError(
+            "the training forward (context/buffer/target row mask with a backward pass) is not part of this "
+            "inference package; use ARTabPFNPredictor.from_trained_model(model)"
+        )

@@ -1,0 +1,292 @@
+#!/usr/bin/env python3
+"""Benchmark of the AR-TabPFN attention hot path on one MI355X.
+
+Workload (BASELINE.json configs[3], the configuration the headline metric is quoted
+on): long-context autoregressive sampling with the 12-layer d_model=256 / 8-head
+(head_dim 32) bf16 model, one shared context of N_ctx=16384 rows, B=1024
+trajectories.  One *step* is one decode step: every trajectory advances by one
+target through all 12 layers (projections, shared-context decode attention with the
+in-place buffer append and LSE merge, FFN, mixture head, sampling).  Steps are timed
+from the first target on, so step t attends to t-1 buffer rows; the default K=256
+is the whole configuration.  The context prefill runs before the timed region and is
+reported separately.
+
+Prints one JSON line:
+  metric/value   target-steps per second over the K timed steps (inputs resident in HBM)
+  roofline       the dominant kernel (MFMA context pass of the decode attention):
+                 algorithmic flops 4*B*H*Lq*N_ctx*Dh per launch over its average
+                 launch duration, measured with HIP events around every launch in a
+                 second, instrumented run of the same K steps; peak 2.5 PFLOP/s bf16
+  cpu_baseline   the numpy oracle (a port of the reference's arithmetic, float32) timed
+                 on this box's host cores on a bounded sample of the same workload
+  log_density    configs[2] (B=64 datasets, 512 context + 128 target rows): one
+                 teacher-forced evaluation on the GPU vs the same on the host CPU
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+
+CFG3 = dict(d_model=256, n_heads=8, n_layers=12, d_ff=256, num_features=10, buffer_size=256, num_components=5)
+B3, NC3, NT3 = 1024, 16384, 256
+B2, NC2, NT2 = 64, 512, 128
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def build_model(device, dtype):
+    from ar_nanotabpfn_amd.model import ARTabPFN
+
+    torch.manual_seed(0)
+    return ARTabPFN(**CFG3).eval().to(device=device, dtype=dtype)
+
+
+def gp_context(n, feats, seed, lengthscale=1.0, noise=0.05, n_rff=2048):
+    """GP draw with an RBF kernel via random Fourier features (exact Cholesky at
+    n=16384 would be a 2 GB float64 matrix); values do not affect throughput."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(n, feats, generator=g)
+    w = torch.randn(feats, n_rff, generator=g) / lengthscale
+    b = torch.rand(n_rff, generator=g) * 2 * math.pi
+    a = torch.randn(n_rff, generator=g)
+    y = math.sqrt(2.0 / n_rff) * torch.cos(x @ w + b) @ a + noise * torch.randn(n, generator=g)
+    return x, y
+
+
+def decode_inputs(device, dtype):
+    x_ctx, y_ctx = gp_context(NC3, CFG3["num_features"], seed=3)
+    g = torch.Generator().manual_seed(4)
+    x_tgt = torch.randn(NT3, CFG3["num_features"], generator=g)
+    x_context = x_ctx.to(device, dtype).unsqueeze(0).expand(B3, -1, -1)
+    y_context = y_ctx.to(device, dtype).unsqueeze(0).expand(B3, -1)
+    x_target = x_tgt.to(device, dtype).unsqueeze(0).expand(B3, -1, -1)
+    return x_context, y_context, x_target
+
+
+def run_decode(pred, x_context, y_context, x_target, steps, device, dtype):
+    """Prefill (untimed) + `steps` decode steps; returns (prefill_ms, decode_ms)."""
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+    pred.init_kv_cache(B3, NT3, device, dtype)
+    torch.cuda.synchronize()
+    ev[0].record()
+    pred.prefill_context(x_context, y_context)
+    ev[1].record()
+    torch.cuda.synchronize()
+    prev_x = prev_y = None
+    t0 = time.perf_counter()
+    ev[2].record()
+    for t in range(steps):
+        x_t = x_target[:, t : t + 1, :]
+        y_t = pred.autoregressive_decode(x_t, prev_x, prev_y, t % pred.ar_tokens.shape[0])
+        prev_x, prev_y = x_t, y_t
+    ev[3].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return ev[0].elapsed_time(ev[1]), ev[2].elapsed_time(ev[3]), wall_ms
+
+
+def cpu_decode_baseline(model, x_context, y_context, x_target, sample_steps=(1, 128)):
+    """The numpy oracle on the host: prefill is skipped (random K/V of the right shape
+    stand in for the context cache: attention cost does not depend on values), then one
+    decode step at each buffer length in `sample_steps` with B=1024."""
+    from oracle import model_oracle as mo
+
+    sd = {k: v.detach().float().cpu().numpy() for k, v in model.state_dict().items()}
+    om = mo.OracleModel(sd, CFG3["n_heads"], compute=np.float32)
+    op = mo.OraclePredictor(om, "shared")
+    H, Dh, L = CFG3["n_heads"], CFG3["d_model"] // CFG3["n_heads"], CFG3["n_layers"]
+    rng = np.random.default_rng(0)
+    xt = x_target[:, :2].float().cpu().numpy()
+    times = []
+    for n in sample_steps:
+        op.init_kv_cache(B3, NT3)
+        op.context_len = NC3
+        op.k_ctx = [rng.standard_normal((H, NC3, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
+        op.v_ctx = [rng.standard_normal((H, NC3, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
+        op.k_buf = [rng.standard_normal((B3, H, n - 1, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
+        op.v_buf = [rng.standard_normal((B3, H, n - 1, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
+        op.buffer_len = n - 1
+        emb = np.concatenate(
+            [om.embed_buffer(xt[:, 0:1], np.zeros((B3, 1), np.float32)) + om.ar_tokens[n % om.ar_tokens.shape[0]],
+             om.embed_target(xt[:, 1:2])], axis=1)
+        t0 = time.perf_counter()
+        z = op.transformer_decode(emb, commit=1)
+        om.head_parameterize(z[:, -1:])
+        times.append(time.perf_counter() - t0)
+        log(f"[cpu] decode step at n_buf={n}: {times[-1]:.2f} s")
+    return float(np.mean(times)), list(sample_steps)
+
+
+def log_density_bench(device, dtype, model, with_cpu):
+    from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
+
+    g = torch.Generator().manual_seed(2)
+    F = CFG3["num_features"]
+    x = torch.randn(B2, NC2 + NT2, F, generator=g)
+    w1 = torch.randn(B2, F, 64, generator=g) / F**0.5
+    w2 = torch.randn(B2, 64, 64, generator=g) / 8.0
+    w3 = torch.randn(B2, 64, 1, generator=g) / 8.0
+    y = (torch.tanh(torch.tanh(x @ w1) @ w2) @ w3).squeeze(-1) + 0.1 * torch.randn(B2, NC2 + NT2, generator=g)
+    y = (y - y[:, :NC2].mean(1, keepdim=True)) / y[:, :NC2].std(1, keepdim=True)
+    xd, yd = x.to(device, dtype), y.to(device, dtype)
+    args = (xd[:, :NC2], yd[:, :NC2], xd[:, NC2:], yd[:, NC2:])
+    pred = ARTabPFNPredictor.from_trained_model(model, backend="flex_attention")
+    for _ in range(3):
+        ll = pred.evaluate_joint_density(*args)
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(10):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        ll = pred.evaluate_joint_density(*args)
+        b.record()
+        torch.cuda.synchronize()
+        ts.append(a.elapsed_time(b))
+    gpu_ms = float(np.median(ts))
+    res = {"workload": "configs[2]: B=64 datasets x (512 context + 128 target rows), 12-layer d_model=256 bf16, "
+                       "per-dataset contexts", "gpu_ms": round(gpu_ms, 3), "finite": bool(torch.isfinite(ll).all())}
+    if with_cpu:
+        from oracle import model_oracle as mo
+
+        sd = {k: v.detach().float().cpu().numpy() for k, v in model.state_dict().items()}
+        om = mo.OracleModel(sd, CFG3["n_heads"], compute=np.float32)
+        a32 = [t.float().cpu().numpy() for t in args]
+        t0 = time.perf_counter()
+        ll_cpu = mo.OraclePredictor(om, "per_dataset").evaluate_joint_density(*a32)
+        cpu_s = time.perf_counter() - t0
+        d = np.abs(ll.float().cpu().numpy() - ll_cpu)
+        res.update(cpu_s=round(cpu_s, 3), speedup=round(cpu_s * 1e3 / gpu_ms, 1),
+                   mean_abs_dlogp_vs_cpu_f32=float(d.mean()))
+        log(f"[cpu] configs[2] log-density: {cpu_s:.2f} s  (GPU {gpu_ms:.2f} ms)")
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=NT3)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: trajectories are independent given the context, so more GPUs "
+                 "shard B with no per-step exchange; run with --gpus 1.")
+    if not 1 <= args.steps <= NT3:
+        sys.exit(f"--steps must be in [1, {NT3}] (one step per target of the configuration)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a HIP device")
+
+    from ar_nanotabpfn_amd import _lib
+    from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
+
+    lib = _lib.load()  # fails loudly when the extension is not built
+    device, dtype = torch.device("cuda:0"), torch.bfloat16
+    model = build_model(device, dtype)
+    x_context, y_context, x_target = decode_inputs(device, dtype)
+    pred = ARTabPFNPredictor.from_trained_model(model, backend="triton_shared_context")
+
+    torch.manual_seed(0)
+    if args.warmup:
+        run_decode(pred, x_context, y_context, x_target, min(args.warmup, NT3), device, dtype)
+    prefill_ms, decode_ms, wall_ms = run_decode(pred, x_context, y_context, x_target, args.steps, device, dtype)
+    ms_per_step = decode_ms / args.steps
+    value = 1e3 / ms_per_step
+    log(f"[gpu] prefill {prefill_ms:.2f} ms; {args.steps} decode steps in {decode_ms:.2f} ms "
+        f"({ms_per_step:.3f} ms/step, host wall {wall_ms:.1f} ms)")
+
+    # instrumented re-run of the same steps: HIP events around every context-pass launch
+    import ctypes
+
+    lib.artab_profile_begin(CFG3["n_layers"] * (args.steps + 1) + 64)
+    run_decode(pred, x_context, y_context, x_target, args.steps, device, dtype)
+    tot, cnt = ctypes.c_double(0.0), ctypes.c_int(0)
+    lib.artab_profile_end(ctypes.byref(tot), ctypes.byref(cnt))
+    # the first L launches are the prefill's dense passes, the first decode step has Lq=1
+    H, Dh, L = CFG3["n_heads"], CFG3["d_model"] // CFG3["n_heads"], CFG3["n_layers"]
+    n_dec = cnt.value - L
+    # per-launch algorithmic flops: 4*B*H*Lq*Nc*Dh with Lq=1 for step 0 and 2 afterwards
+    flops_total = 4.0 * B3 * H * NC3 * Dh * L * (1 + 2 * (args.steps - 1))
+    # time of the decode launches = total - prefill launches; measure prefill launches separately
+    lib.artab_profile_begin(L + 8)
+    pred.init_kv_cache(B3, NT3, device, dtype)
+    pred.prefill_context(x_context, y_context)
+    ptot, pcnt = ctypes.c_double(0.0), ctypes.c_int(0)
+    lib.artab_profile_end(ctypes.byref(ptot), ctypes.byref(pcnt))
+    dec_kernel_ms = tot.value - ptot.value
+    avg_launch_us = dec_kernel_ms * 1e3 / max(n_dec, 1)
+    achieved = flops_total / (dec_kernel_ms * 1e-3) / 1e12 if dec_kernel_ms > 0 else 0.0
+    prefill_flops = 4.0 * H * NC3 * NC3 * Dh * L
+    roofline = {
+        "kernel": "flash_kernel<bf16,32> context pass of artab_decode_attention",
+        "bound": "mfma",
+        "achieved": round(achieved, 2),
+        "peak": MFMA_BF16_PEAK_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
+        "traffic": None,
+        "launches": n_dec,
+        "avg_launch_us": round(avg_launch_us, 2),
+        "flops_per_launch_lq2": 4.0 * B3 * H * 2 * NC3 * Dh,
+        "prefill_tflops": round(prefill_flops / (ptot.value * 1e-3) / 1e12, 2) if ptot.value > 0 else None,
+    }
+    log(f"[gpu] context-pass kernel: {n_dec} launches, avg {avg_launch_us:.1f} us, {achieved:.1f} TFLOP/s")
+
+    out = {
+        "metric": "ar_decode_target_steps_per_sec",
+        "value": round(value, 2),
+        "unit": "target-steps/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[3] long-context AR sampling: shared context N_ctx=16384 (x in R^10, GP prior via "
+                        "random Fourier features), B=1024 trajectories, 12-layer d_model=256 8-head bf16 model, "
+                        "decode steps 0..K-1 with the in-place buffer K/V (N_buf = step-1) and LSE merge",
+            "B": B3, "N_ctx": NC3, "N_targets": NT3, "layers": L, "heads": H, "head_dim": Dh,
+        },
+        "trajectory_steps_per_sec": round(value * B3, 1),
+        "prefill_ms": round(prefill_ms, 3),
+        "roofline": roofline,
+    }
+
+    if not args.no_cpu:
+        cpu_s, sample = cpu_decode_baseline(model, x_context, y_context, x_target)
+        out["cpu_baseline"] = {
+            "value": round(1.0 / cpu_s, 4),
+            "unit": "target-steps/s",
+            "cores": os.cpu_count() if not os.environ.get("OMP_NUM_THREADS") else int(os.environ["OMP_NUM_THREADS"]),
+            "kind": "port",
+            "sample": f"numpy float32 oracle, one full 12-layer decode step (B=1024, N_ctx=16384) at each of "
+                      f"N_buf={sample}, mean; context K/V random (prefill skipped)",
+        }
+    else:
+        out["cpu_baseline"] = None
+    out["log_density"] = log_density_bench(device, dtype, model, with_cpu=not args.no_cpu)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -72,6 +72,18 @@ int artab_version(void);
 const char *artab_status_string(int status);
 const char *artab_last_error(void);
 
+/*
+ * Benchmark aid without a counterpart in the reference (which times whole calls with
+ * perf_counter + synchronize, tests/test_triton_gpu.py:255-293).  Between
+ * artab_profile_begin and artab_profile_end every launch of the MFMA attention kernel
+ * (context pass of artab_context_attention / artab_decode_attention, teacher forcing,
+ * prefill) is bracketed by a pair of HIP events on its stream; _end waits for them and
+ * returns the summed kernel time and the number of launches.  These two calls create
+ * events and synchronise, unlike every other entry point; not thread-safe.
+ */
+int artab_profile_begin(int max_records);
+int artab_profile_end(double *total_ms, int *records);
+
 /* Bytes of float32 workspace the split-context paths need for the given problem
  * (artab_context_attention, artab_decode_attention).  0 means no workspace is
  * needed.  Pure host arithmetic, no device access. */

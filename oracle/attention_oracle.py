@@ -103,10 +103,19 @@ def context_attention(
     D = q.shape[-1]
     if scale is None:
         scale = D ** -0.5
-    scores = np.einsum("bhqd,bhkd->bhqk", q, np.broadcast_to(k, (q.shape[0],) + k.shape[1:])) * scale
+    B, H, Lq, _ = q.shape
+    if k.shape[0] == 1 and B > 1:
+        # one context for the whole batch: fold (b, lq) into the row axis so the products are
+        # plain per-head matrix multiplications (same arithmetic, BLAS speed)
+        q2 = q.transpose(1, 0, 2, 3).reshape(H, B * Lq, D)
+        scores = np.matmul(q2, k[0].transpose(0, 2, 1)) * scale  # [H, B*Lq, Nc]
+        lse = _logsumexp(scores)
+        out = np.matmul(_softmax(scores), v[0])
+        out = out.reshape(H, B, Lq, D).transpose(1, 0, 2, 3)
+        return out, lse.reshape(H, B, Lq).transpose(1, 0, 2)
+    scores = np.matmul(q, k.transpose(0, 1, 3, 2)) * scale
     lse = _logsumexp(scores)
-    attn = _softmax(scores)
-    out = np.einsum("bhqk,bhkd->bhqd", attn, np.broadcast_to(v, (q.shape[0],) + v.shape[1:]))
+    out = np.matmul(_softmax(scores), v)
     return out, lse
 
 
@@ -125,7 +134,7 @@ def buffer_attention(
     D = q.shape[-1]
     if scale is None:
         scale = D ** -0.5
-    scores = np.einsum("bhqd,bhkd->bhqk", q, k) * scale
+    scores = np.matmul(q, k.transpose(0, 1, 3, 2)) * scale
     no_kv = None
     if mask is not None:
         mask = np.broadcast_to(np.asarray(mask, dtype=bool), scores.shape)
@@ -135,7 +144,7 @@ def buffer_attention(
     attn = _softmax(scores)
     if no_kv is not None:
         attn = np.where(no_kv[..., None], 0.0, attn)
-    out = np.einsum("bhqk,bhkd->bhqd", attn, v)
+    out = np.matmul(attn, v)
     return out, lse
 
 
