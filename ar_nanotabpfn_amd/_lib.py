@@ -53,12 +53,14 @@ SIGNATURES = {
     "artab_context_attention": (_i, [_VP, _VP, _VP, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _p, _sz, _i, _p]),
     "artab_decode_attention": (
         _i,
-        [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p, _sz, _i, _p],
+        [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _p, _i, _i, _f, _i, _p, _sz, _i, _p],
     ),
     "artab_teacher_forcing_attention": (_i, [_VP, _VP, _VP, _VP, _VP, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "artab_prefill_attention": (_i, [_VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "artab_buffer_attention": (_i, [_VP, _VP, _VP, _p, _i64, _i64, _i64, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _p]),
     "artab_merge_attention_outputs": (_i, [_VP, _p, _VP, _p, _VP, _i, _i, _i, _i, _i, _p]),
+    "artab_add_layernorm": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _i, _f, _i, _p]),
+    "artab_bias_gelu": (_i, [_p, _i64, _p, _p, _i64, _i, _i, _p]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

@@ -218,6 +218,7 @@ def decode_attention(
     k_new: Optional[Tensor] = None,
     v_new: Optional[Tensor] = None,
     use_triton: bool = True,
+    n_buf_device: Optional[Tensor] = None,
 ) -> Tensor:
     """One decode step of row attention (inference.py:785-823) in one call.
 
@@ -226,6 +227,10 @@ def decode_attention(
     ``k_new``/``v_new [B,H,1,D]`` the row is appended in place at slot ``n_buf`` and
     all queries see it; the caller advances its cursor.  Raises ``ValueError`` for
     Lq outside {1,2} (:765-768) and for a full cache (:247-250).
+
+    ``n_buf_device`` (one int32 on the device) makes the kernels read the committed
+    length at run time, for launches recorded in a HIP graph; ``n_buf`` is then the
+    upper bound that is validated against the cache capacity.
     """
     dev = _lib.require_device(q, k_ctx, v_ctx, k_buf_cache, v_buf_cache, k_new, v_new)
     lib = _lib.load()
@@ -236,6 +241,8 @@ def decode_attention(
     if Hk != H or k_ctx.shape[-1] != Dh:
         raise ValueError(f"context K/V {tuple(k_ctx.shape)} do not match q {tuple(q.shape)}")
     cap = k_buf_cache.shape[2] if k_buf_cache is not None else 0
+    if n_buf_device is not None and (n_buf_device.dtype != torch.int32 or not n_buf_device.is_cuda):
+        raise ValueError("n_buf_device must be an int32 tensor on the device")
     out = _alloc_out(q)
     ws_ptr, ws_bytes = _workspace_for(q, Nc)
     qv, ov = _lib.view4(q), _lib.view4(out)
@@ -244,7 +251,9 @@ def decode_attention(
     _lib.check(
         lib.artab_decode_attention(
             _lib.ref(qv), _lib.ref(kv), _lib.ref(vv), _lib.ref(kbv), _lib.ref(vbv), _lib.ref(knv), _lib.ref(vnv),
-            _lib.ref(ov), B, H, Lq, Nc, int(n_buf), cap, Dh, 0.0, _lib.dtype_code(q.dtype),
+            _lib.ref(ov), B, H, Lq, Nc, int(n_buf),
+            ctypes.c_void_p(n_buf_device.data_ptr()) if n_buf_device is not None else None,
+            cap, Dh, 0.0, _lib.dtype_code(q.dtype),
             ws_ptr, ws_bytes, _impl(use_triton), _lib.current_stream(dev),
         )
     )

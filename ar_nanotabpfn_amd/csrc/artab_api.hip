@@ -12,6 +12,7 @@
 #include "../../include/artab_attention.h"
 #include "common.h"
 #include "decode_buffer.h"
+#include "glue_kernels.h"
 #include "mfma_flash.h"
 #include "portable_kernels.h"
 
@@ -155,13 +156,16 @@ static FlashPlan plan_flash(int B, int H, int Lq, int Nc, int Dh, bool stacked, 
         if (sp_env > 0) n_split = sp_env < max_split ? sp_env : max_split;
     }
     int per = (Nc + n_split - 1) / n_split;
-    per = (per + kFlashBN - 1) / kFlashBN * kFlashBN;
-    if (per <= 0) per = kFlashBN;
+    per = (per + 127) / 128 * 128;  // whole LDS tiles for either tile length
+    if (per <= 0) per = 128;
     pl.kv_per_split = per;
     pl.n_split = (Nc + per - 1) / per;
     if (pl.n_split < 1) pl.n_split = 1;
     return pl;
 }
+
+// Keys per LDS tile: 64, or 128 for head_dim 32 when ARTAB_BN=128 (tuning aid).
+static int flash_bn(int Dh) { return (Dh == 32 && env_int("ARTAB_BN", 64) == 128) ? 128 : 64; }
 
 template <typename T, int DH>
 static hipError_t launch_flash_bm(const FlashParams &P, int BM, hipStream_t stream) {
@@ -169,6 +173,17 @@ static hipError_t launch_flash_bm(const FlashParams &P, int BM, hipStream_t stre
     const int n_kvg = P.H * P.n_groups;
     const unsigned grid = static_cast<unsigned>(((n_kvg + 7) / 8) * W * 8);
     if (grid == 0) return hipSuccess;
+    if constexpr (DH == 32) {
+        if (flash_bn(DH) == 128) {
+            if (BM == 256)
+                hipLaunchKernelGGL((flash_kernel<T, DH, 2, 4, 128>), dim3(grid), dim3(256), 0, stream, P);
+            else if (BM == 128)
+                hipLaunchKernelGGL((flash_kernel<T, DH, 1, 4, 128>), dim3(grid), dim3(256), 0, stream, P);
+            else
+                hipLaunchKernelGGL((flash_kernel<T, DH, 1, 2, 128>), dim3(grid), dim3(128), 0, stream, P);
+            return hipGetLastError();
+        }
+    }
     if constexpr (DH <= 64) {
         if (BM == 256) {
             hipLaunchKernelGGL((flash_kernel<T, DH, 2, 4, kFlashBN>), dim3(grid), dim3(256), 0, stream, P);
@@ -388,7 +403,7 @@ int artab_context_attention(const artab_view *q, const artab_view *k_ctx, const 
         if (!workspace || workspace_bytes < need) {
             // Without a workspace the unsplit schedule is still correct, only less parallel.
             pl.n_split = 1;
-            pl.kv_per_split = (Nc + kFlashBN - 1) / kFlashBN * kFlashBN;
+            pl.kv_per_split = (Nc + 127) / 128 * 128;
         }
     }
     FlashParams F;
@@ -425,8 +440,8 @@ int artab_context_attention(const artab_view *q, const artab_view *k_ctx, const 
 int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
                            const artab_view *k_buf, const artab_view *v_buf, const artab_view *k_new,
                            const artab_view *v_new, const artab_view *out, int B, int H, int Lq, int Nc,
-                           int n_buf, int buf_capacity, int Dh, float scale, int dtype, void *workspace,
-                           size_t workspace_bytes, int impl, void *stream) {
+                           int n_buf, const int32_t *n_buf_device, int buf_capacity, int Dh, float scale,
+                           int dtype, void *workspace, size_t workspace_bytes, int impl, void *stream) {
     ARTAB_TRY(check_common(B, H, Lq, Dh, dtype));
     if (Lq != 1 && Lq != 2)
         return fail(ARTAB_ERR_BAD_SHAPE, "decode supports Lq=1 (target) or Lq=2 (buffer, target); got %d", Lq);
@@ -443,7 +458,7 @@ int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const a
     ARTAB_TRY(check_view(k_ctx, "k_ctx", dtype, true));
     ARTAB_TRY(check_view(v_ctx, "v_ctx", dtype, true));
     ARTAB_TRY(check_view(out, "out", dtype, true));
-    const bool need_buf = n_buf + has_new > 0;
+    const bool need_buf = n_buf + has_new > 0 || n_buf_device != nullptr;
     ARTAB_TRY(check_view(k_buf, "k_buf", dtype, need_buf));
     ARTAB_TRY(check_view(v_buf, "v_buf", dtype, need_buf));
     ARTAB_TRY(check_view(k_new, "k_new", dtype, false));
@@ -483,6 +498,7 @@ int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const a
         P.B = B; P.H = H; P.Lq = Lq; P.Nc = Nc; P.Nb = n_buf + has_new;
         P.new_row = has_new ? n_buf : -1;
         P.append = has_new;
+        P.nbuf_dev = n_buf_device;
         P.mode = kModePlain; P.Dh = Dh; P.scale = scale;
         P.vec_ok = aligned ? 1 : 0;
         return launch_status(launch_portable_dtype(P, dtype, st), "decode attention (portable)");
@@ -510,7 +526,7 @@ int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const a
     memset(&D, 0, sizeof(D));
     D.q = dv(q); D.kb = dv(k_buf); D.vb = dv(v_buf); D.knew = dv(k_new); D.vnew = dv(v_new); D.out = dv(out);
     D.part_o = F.part_o; D.part_lse = F.part_lse; D.lse = nullptr;
-    D.B = B; D.H = H; D.n_split = pl.n_split; D.n_buf = n_buf; D.has_new = has_new;
+    D.B = B; D.H = H; D.n_split = pl.n_split; D.n_buf = n_buf; D.n_buf_dev = n_buf_device; D.has_new = has_new;
     D.qscale = scale * kLog2e;
     return launch_status(launch_decode(D, dtype, Dh, Lq, st), "decode buffer pass");
 }
@@ -655,6 +671,59 @@ int artab_merge_attention_outputs(const artab_view *out_a, const float *lse_a, c
         default: e = launch_merge<float>(P, st); break;
     }
     return launch_status(e, "merge");
+}
+
+int artab_add_layernorm(const void *x, int64_t ldx, const void *y, int64_t ldy, const void *bias, const void *gamma,
+                        const void *beta, void *out, int64_t rows, int D, float eps, int dtype, void *stream) {
+    if (dtype != ARTAB_BF16 && dtype != ARTAB_F16 && dtype != ARTAB_F32)
+        return fail(ARTAB_ERR_UNSUPPORTED, "unknown dtype code %d", dtype);
+    if (rows < 0 || D <= 0) return fail(ARTAB_ERR_BAD_SHAPE, "bad sizes rows=%lld D=%d", (long long)rows, D);
+    if (D % 4 || D > 256 * kGlueMaxPerLane)
+        return fail(ARTAB_ERR_UNSUPPORTED, "add_layernorm needs D %% 4 == 0 and D <= %d (got %d)", 256 * kGlueMaxPerLane, D);
+    if (rows == 0) return ARTAB_OK;
+    if (!x || !gamma || !beta || !out) return fail(ARTAB_ERR_NULL_POINTER, "x, gamma, beta and out are required");
+    const int64_t per = 16 / elem_size(dtype) / 2;  // 4-element vectors: 8 bytes (16-bit) or 16 bytes (float32)
+    const uintptr_t align = dtype == ARTAB_F32 ? 16 : 8;
+    auto bad = [&](const void *p) { return p && reinterpret_cast<uintptr_t>(p) % align != 0; };
+    if (bad(x) || bad(y) || bad(bias) || bad(gamma) || bad(beta) || bad(out) || ldx % 4 || (y && ldy % 4))
+        return fail(ARTAB_ERR_BAD_STRIDE, "add_layernorm operands must be aligned to 4 elements");
+    (void)per;
+    AddLayerNormParams P;
+    P.x = x; P.y = y; P.bias = bias; P.gamma = gamma; P.beta = beta; P.out = out;
+    P.rows = rows; P.ldx = ldx; P.ldy = ldy; P.D = D; P.eps = eps;
+    dim3 grid(static_cast<unsigned>((rows + kGlueWaves - 1) / kGlueWaves)), block(kGlueWaves * 64);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case ARTAB_BF16: hipLaunchKernelGGL((add_layernorm_kernel<bf16_t>), grid, block, 0, st, P); break;
+        case ARTAB_F16: hipLaunchKernelGGL((add_layernorm_kernel<f16_t>), grid, block, 0, st, P); break;
+        default: hipLaunchKernelGGL((add_layernorm_kernel<float>), grid, block, 0, st, P); break;
+    }
+    return launch_status(hipGetLastError(), "add_layernorm");
+}
+
+int artab_bias_gelu(const void *x, int64_t ldx, const void *bias, void *out, int64_t rows, int D, int dtype,
+                    void *stream) {
+    if (dtype != ARTAB_BF16 && dtype != ARTAB_F16 && dtype != ARTAB_F32)
+        return fail(ARTAB_ERR_UNSUPPORTED, "unknown dtype code %d", dtype);
+    if (rows < 0 || D <= 0) return fail(ARTAB_ERR_BAD_SHAPE, "bad sizes rows=%lld D=%d", (long long)rows, D);
+    if (D % 4) return fail(ARTAB_ERR_UNSUPPORTED, "bias_gelu needs D %% 4 == 0 (got %d)", D);
+    if (rows == 0) return ARTAB_OK;
+    if (!x || !out) return fail(ARTAB_ERR_NULL_POINTER, "x and out are required");
+    const uintptr_t align = dtype == ARTAB_F32 ? 16 : 8;
+    auto bad = [&](const void *p) { return p && reinterpret_cast<uintptr_t>(p) % align != 0; };
+    if (bad(x) || bad(bias) || bad(out) || ldx % 4)
+        return fail(ARTAB_ERR_BAD_STRIDE, "bias_gelu operands must be aligned to 4 elements");
+    BiasGeluParams P;
+    P.x = x; P.bias = bias; P.out = out; P.rows = rows; P.ldx = ldx; P.D = D;
+    const long total = rows * (D / 4);
+    dim3 grid(static_cast<unsigned>((total + 255) / 256));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case ARTAB_BF16: hipLaunchKernelGGL((bias_gelu_kernel<bf16_t>), grid, dim3(256), 0, st, P); break;
+        case ARTAB_F16: hipLaunchKernelGGL((bias_gelu_kernel<f16_t>), grid, dim3(256), 0, st, P); break;
+        default: hipLaunchKernelGGL((bias_gelu_kernel<float>), grid, dim3(256), 0, st, P); break;
+    }
+    return launch_status(hipGetLastError(), "bias_gelu");
 }
 
 }  // extern "C"

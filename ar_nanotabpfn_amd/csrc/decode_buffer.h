@@ -23,6 +23,7 @@ struct DecodeParams {
     int B, H;
     int n_split;
     int n_buf;    // committed buffer rows
+    const int *n_buf_dev;  // when set, the committed length is read from here at run time
     int has_new;  // 1: row n_buf comes from knew/vnew, is attended and appended
     float qscale; // scale * log2(e)
 };
@@ -70,7 +71,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
         for (int e = 0; e < 8; ++e) acc[i][e] = 0.f;
     }
 
-    const int n_total = P.n_buf + (P.has_new ? 1 : 0);
+    const int n_buf = P.n_buf_dev ? *P.n_buf_dev : P.n_buf;
+    const int n_total = n_buf + (P.has_new ? 1 : 0);
     const T *knew_row = P.has_new ? view_row<T>(P.knew, b, h, 0) : nullptr;
     const T *vnew_row = P.has_new ? view_row<T>(P.vnew, b, h, 0) : nullptr;
 
@@ -84,7 +86,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
             kraw[u] = u32x4{0u, 0u, 0u, 0u};
             vraw[u] = u32x4{0u, 0u, 0u, 0u};
             if (ok[u]) {
-                const bool is_new = P.has_new && kv == P.n_buf;
+                const bool is_new = P.has_new && kv == n_buf;
                 const T *kr = is_new ? knew_row : view_row<T>(P.kb, b, h, kv);
                 const T *vr = is_new ? vnew_row : view_row<T>(P.vb, b, h, kv);
                 kraw[u] = *reinterpret_cast<const u32x4 *>(kr + 8 * sub);
@@ -190,9 +192,9 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
         }
     } else if (grp == 1 && P.has_new) {
         // In-place append: slot n_buf of the cache receives the new row.
-        *reinterpret_cast<u32x4 *>(view_row<T>(P.kb, b, h, P.n_buf) + 8 * sub) =
+        *reinterpret_cast<u32x4 *>(view_row<T>(P.kb, b, h, n_buf) + 8 * sub) =
             *reinterpret_cast<const u32x4 *>(knew_row + 8 * sub);
-        *reinterpret_cast<u32x4 *>(view_row<T>(P.vb, b, h, P.n_buf) + 8 * sub) =
+        *reinterpret_cast<u32x4 *>(view_row<T>(P.vb, b, h, n_buf) + 8 * sub) =
             *reinterpret_cast<const u32x4 *>(vnew_row + 8 * sub);
     }
 }

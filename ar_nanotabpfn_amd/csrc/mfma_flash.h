@@ -220,8 +220,9 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
     }
     const int n_tiles = ctx_tiles + buf_tiles;
 
-    // ---- staging: global -> registers -> LDS, one tile ahead.  Each thread owns
-    // NCH 16-byte chunks (row kvl, chunk ch) of the K tile and the same of V.
+    // ---- staging: global -> registers -> LDS.  Each thread owns NCH 16-byte chunks
+    // (row st_row, column st_col) of the K tile and the same of V; their global
+    // addresses are kept as running pointers that advance by one tile per fetch.
     int st_row[NCH], st_col[NCH];
 #pragma unroll
     for (int x = 0; x < NCH; ++x) {
@@ -230,22 +231,39 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
         st_col[x] = (idx % CPR) * 8;
     }
     u32x4 kst[NCH], vst[NCH];
+    const T *kp[NCH], *vp[NCH];
+    long k_step = 0, v_step = 0;  // elements per tile
+    int fetch_rows_left = 0;      // rows of the current segment from the next tile to fetch
 
-    auto fetch = [&](int it) {
+    // Point the running pointers at tile `it` (first tile of the context slice or of
+    // the buffer segment).
+    auto seek = [&](int it) {
         const bool is_ctx = it < ctx_tiles;
         const View &ks_ = is_ctx ? P.kc : P.kb;
         const View &vs_ = is_ctx ? P.vc : P.vb;
         const long bb = is_ctx ? kvb : g;
         const int kv0 = is_ctx ? ctx_begin + it * BN : (it - ctx_tiles) * BN;
-        const int rows_left = (is_ctx ? ctx_end : P.Nb) - kv0;
+        fetch_rows_left = (is_ctx ? ctx_end : P.Nb) - kv0;
         const T *kbase = view_row<T>(ks_, bb, h, kv0);
         const T *vbase = view_row<T>(vs_, bb, h, kv0);
-        if (rows_left >= BN) {
+        k_step = static_cast<long>(BN) * ks_.sn;
+        v_step = static_cast<long>(BN) * vs_.sn;
+#pragma unroll
+        for (int x = 0; x < NCH; ++x) {
+            kp[x] = kbase + st_row[x] * ks_.sn + st_col[x];
+            vp[x] = vbase + st_row[x] * vs_.sn + st_col[x];
+        }
+    };
+
+    // Load tile `it` (the one the running pointers are at) and advance them.
+    auto fetch = [&](int it) {
+        if (it == 0 || it == ctx_tiles) seek(it);
+        if (fetch_rows_left >= BN) {
 #pragma unroll
             for (int x = 0; x < NCH; ++x) {
                 if (NCH * NT == CHUNKS || tid + x * NT < CHUNKS) {
-                    kst[x] = *reinterpret_cast<const u32x4 *>(kbase + st_row[x] * ks_.sn + st_col[x]);
-                    vst[x] = *reinterpret_cast<const u32x4 *>(vbase + st_row[x] * vs_.sn + st_col[x]);
+                    kst[x] = *reinterpret_cast<const u32x4 *>(kp[x]);
+                    vst[x] = *reinterpret_cast<const u32x4 *>(vp[x]);
                 }
             }
         } else {
@@ -253,11 +271,17 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
             for (int x = 0; x < NCH; ++x) {
                 kst[x] = u32x4{0u, 0u, 0u, 0u};
                 vst[x] = u32x4{0u, 0u, 0u, 0u};
-                if ((NCH * NT == CHUNKS || tid + x * NT < CHUNKS) && st_row[x] < rows_left) {
-                    kst[x] = *reinterpret_cast<const u32x4 *>(kbase + st_row[x] * ks_.sn + st_col[x]);
-                    vst[x] = *reinterpret_cast<const u32x4 *>(vbase + st_row[x] * vs_.sn + st_col[x]);
+                if ((NCH * NT == CHUNKS || tid + x * NT < CHUNKS) && st_row[x] < fetch_rows_left) {
+                    kst[x] = *reinterpret_cast<const u32x4 *>(kp[x]);
+                    vst[x] = *reinterpret_cast<const u32x4 *>(vp[x]);
                 }
             }
+        }
+        fetch_rows_left -= BN;
+#pragma unroll
+        for (int x = 0; x < NCH; ++x) {
+            kp[x] += k_step;
+            vp[x] += v_step;
         }
     };
 
@@ -434,10 +458,27 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
         __syncthreads();
         if (n_tiles == 0) return;
 
-        auto scores = [&](f32x16(&dst)[QB], const T *kblk) {
-            vec ak[KS];
+        // LDS operand fetches: K fragments of one 32-key block (A operand of S^T) and
+        // the transposed V fragments of one block (A operand of O^T).
+        auto load_k = [&](vec(&ak)[KS], const T *kblk) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) ak[ks] = *reinterpret_cast<const vec *>(kblk + 16 * ks);
+        };
+        auto load_v = [&](vec(&av)[DB][2], const T *vblk) {
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const T *vp_ = vblk + 16 * t * VPAD + 32 * db;
+                    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp_));
+                    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) s16x4 *)(vp_ + 8 * VPAD));
+                    typedef short s16x8 __attribute__((ext_vector_type(8)));
+                    s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    av[db][t] = __builtin_bit_cast(vec, both);
+                }
+        };
+        auto scores = [&](f32x16(&dst)[QB], const vec(&ak)[KS]) {
 #pragma unroll
             for (int j = 0; j < QB; ++j) {
 #pragma unroll
@@ -448,7 +489,11 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
         };
 
         f32x16 s_cur[QB];
-        scores(s_cur, &k_lds[0][k_rd]);
+        {
+            vec ak0[KS];
+            load_k(ak0, &k_lds[0][k_rd]);
+            scores(s_cur, ak0);
+        }
 
         int stage = 0;
         for (int it = 0; it < n_tiles; ++it) {
@@ -461,8 +506,8 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
             const int w_min = is_ctx ? seg_end : wave_lim_min;
             const T *kt = &k_lds[stage][k_rd];
             const T *vt = &v_lds[stage][v_rd];
-            // block after the last one of this tile: block 0 of the next tile (or, on the
-            // very last tile, any valid block — its scores are never used)
+            // the block after this tile's last one is block 0 of the next tile (on the very
+            // last tile any valid address will do: those scores are never used)
             const T *kt_next = (it + 1 < n_tiles) ? &k_lds[stage_next][k_rd] : kt;
 
             auto tile_body = [&](auto mask_tag) {
@@ -481,23 +526,12 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
                             }
                         }
                     }
-                    // LDS operands: V of this block, K of the next one
-                    vec av[DB][2];
-#pragma unroll
-                    for (int db = 0; db < DB; ++db)
-#pragma unroll
-                        for (int t = 0; t < 2; ++t) {
-                            const T *vp = vt + (32 * sb + 16 * t) * VPAD + 32 * db;
-                            s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                                (__attribute__((address_space(3))) s16x4 *)(vp));
-                            s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                                (__attribute__((address_space(3))) s16x4 *)(vp + 8 * VPAD));
-                            typedef short s16x8 __attribute__((ext_vector_type(8)));
-                            s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                            av[db][t] = __builtin_bit_cast(vec, both);
-                        }
+                    vec ak_nx[KS], av_cu[DB][2];
+                    load_v(av_cu, vt + 32 * sb * VPAD);
+                    load_k(ak_nx, sb + 1 < SB ? kt + 32 * (sb + 1) * KPAD : kt_next);
+
                     f32x16 s_next[QB];
-                    scores(s_next, sb + 1 < SB ? kt + 32 * (sb + 1) * KPAD : kt_next);
+                    scores(s_next, ak_nx);
 
                     unsigned pk[QB][8];
 #pragma unroll
@@ -517,7 +551,7 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
 #pragma unroll
                             for (int t = 0; t < 2; ++t) {
                                 u32x4 pb = {pk[j][4 * t], pk[j][4 * t + 1], pk[j][4 * t + 2], pk[j][4 * t + 3]};
-                                o_acc[j][db] = Ops::mma(av[db][t], __builtin_bit_cast(vec, pb), o_acc[j][db]);
+                                o_acc[j][db] = Ops::mma(av_cu[db][t], __builtin_bit_cast(vec, pb), o_acc[j][db]);
                             }
 #pragma unroll
                     for (int j = 0; j < QB; ++j) s_cur[j] = s_next[j];

@@ -23,6 +23,7 @@ struct PortableParams {
     long m_sb, m_sh, m_sq;
     int B, H, Lq, Nc, Nb;
     int new_row;  // buffer row index served from knew/vnew, or -1
+    const int *nbuf_dev;  // decode: committed buffer length read at run time (overrides Nb / new_row)
     int append;   // copy knew/vnew to kb/vb[new_row]
     int mode;
     int Nt;
@@ -136,6 +137,11 @@ __global__ __launch_bounds__(kPortableWaves * 64) void portable_attention_kernel
     }
 
     // Buffer segment: keys [0, limit) with the mode's visibility rule.
+    if (P.nbuf_dev) {
+        const int n = *P.nbuf_dev;
+        P.Nb = n + (P.new_row >= 0 ? 1 : 0);
+        if (P.new_row >= 0) P.new_row = n;
+    }
     int limit = P.Nb;
     if (P.mode == kModeTeacher) limit = min(P.Nb, tf_limit(i, P.Nt));
     const T *knew_row = P.new_row >= 0 ? view_row<T>(P.knew, b, h, 0) : nullptr;

@@ -25,8 +25,14 @@ from torch import Tensor
 
 from . import attention_kernels as ak
 from .attention import DecodeMask, TeacherForcingMask
+from .glue import add_layer_norm
 
 __all__ = ["ARTabPFNPredictor"]
+
+
+class _GraphState:
+    """Static tensors and the recorded graph of the sampling loop."""
+
 
 _SHARED = "triton_shared_context"
 _PER_DATASET = "flex_attention"
@@ -51,6 +57,10 @@ class ARTabPFNPredictor:
         self.max_buffer_len = 0   # capacity of the buffer cache (shared layout)
         self._device = None
         self._dtype = None
+        # Replay the decode step of sample_sequence from a recorded HIP graph (shared
+        # layout on a HIP device only).  Set to False to launch every kernel from Python.
+        self.use_hip_graph = True
+        self._graph_state = None
 
     @classmethod
     def from_trained_model(cls, model, backend: str = "flex_attention") -> "ARTabPFNPredictor":
@@ -68,20 +78,33 @@ class ARTabPFNPredictor:
             dtype = dtype or param.dtype
         self._device, self._dtype = device, dtype
         self.seq_len = self.context_len = self.buffer_len = 0
+        def zeros(layer, name, shape):
+            # same contents as a fresh torch.zeros; memory (and its address, which recorded
+            # HIP graphs refer to) is kept when the shape, dtype and device are unchanged
+            old = getattr(layer, name, None)
+            if (isinstance(old, torch.Tensor) and tuple(old.shape) == tuple(shape) and old.dtype == dtype
+                    and old.device == torch.device(device) and old.is_contiguous()):
+                old.zero_()
+            else:
+                setattr(layer, name, torch.zeros(shape, device=device, dtype=dtype))
+
         if self.backend == _SHARED:
             self.max_buffer_len = max_seq_len
             for layer in self.backbone.layers:
                 H, Dh = layer.attn_rows.n_heads, layer.attn_rows.head_dim
-                layer.k_ctx_cache = torch.empty((H, 0, Dh), device=device, dtype=dtype)
-                layer.v_ctx_cache = torch.empty_like(layer.k_ctx_cache)
-                layer.k_buf_cache = torch.zeros(batch_size, H, max_seq_len, Dh, device=device, dtype=dtype)
-                layer.v_buf_cache = torch.zeros_like(layer.k_buf_cache)
+                old = getattr(layer, "k_ctx_cache", None)
+                if not (isinstance(old, torch.Tensor) and old.dim() == 3 and old.shape[0] == H and old.shape[2] == Dh
+                        and old.dtype == dtype and old.device == torch.device(device)):
+                    layer.k_ctx_cache = torch.empty((H, 0, Dh), device=device, dtype=dtype)
+                    layer.v_ctx_cache = torch.empty_like(layer.k_ctx_cache)
+                zeros(layer, "k_buf_cache", (batch_size, H, max_seq_len, Dh))
+                zeros(layer, "v_buf_cache", (batch_size, H, max_seq_len, Dh))
             return
         self.max_buffer_len = 0
         for layer in self.backbone.layers:
             H, Dh = layer.attn_rows.n_heads, layer.attn_rows.head_dim
-            layer.k_cache = torch.zeros(batch_size, H, max_seq_len, Dh, device=device, dtype=dtype)
-            layer.v_cache = torch.zeros_like(layer.k_cache)
+            zeros(layer, "k_cache", (batch_size, H, max_seq_len, Dh))
+            zeros(layer, "v_cache", (batch_size, H, max_seq_len, Dh))
 
     def clear_cache(self) -> None:
         """Reset the cursors, keep the memory (inference.py:137-141)."""
@@ -91,8 +114,7 @@ class ARTabPFNPredictor:
 
     @staticmethod
     def _qkv(layer, x_row: Tensor):
-        a = layer.attn_rows
-        return a.split_heads(a.q_proj(x_row)), a.split_heads(a.k_proj(x_row)), a.split_heads(a.v_proj(x_row))
+        return layer.qkv_heads(x_row)
 
     # ------------------------------------------------------------------ prefill
 
@@ -150,15 +172,16 @@ class ARTabPFNPredictor:
                 x_row = self._layer_decode_with_cache_shared(layer, x_row, commit)
             self.buffer_len += commit
             self.seq_len = self.context_len + self.buffer_len
-            return self.backbone.norm(x_row)
+            return add_layer_norm(x_row, None, None, self.backbone.norm)
 
         mask = DecodeMask(num_cached=self.seq_len, num_new=N)
         for layer in self.backbone.layers:
             x_row = self._layer_decode_with_cache(layer, x_row, mask, cache_start=self.seq_len)
         self.seq_len += commit
-        return self.backbone.norm(x_row)
+        return add_layer_norm(x_row, None, None, self.backbone.norm)
 
-    def _layer_decode_with_cache_shared(self, layer, x_row: Tensor, commit: int = 1) -> Tensor:
+    def _layer_decode_with_cache_shared(self, layer, x_row: Tensor, commit: int = 1,
+                                        n_buf_device: Optional[Tensor] = None) -> Tensor:
         """One layer of a decode step on the shared layout (inference.py:746-833): both
         queries of a ``[buffer, target]`` pair see context + committed buffers + the new
         buffer row, which is appended in place by the same kernel call."""
@@ -169,12 +192,15 @@ class ARTabPFNPredictor:
         q, k_new, v_new = self._qkv(layer, x_row)
         k_ctx = layer.k_ctx_cache[:, : self.context_len]
         v_ctx = layer.v_ctx_cache[:, : self.context_len]
+        # with a device-side length the host value is only the bound that is validated
+        n_buf = self.buffer_len if n_buf_device is None else self.max_buffer_len - (N - 1)
         if N == 1:
-            attn = ak.decode_attention(q, k_ctx, v_ctx, layer.k_buf_cache, layer.v_buf_cache, self.buffer_len)
+            attn = ak.decode_attention(q, k_ctx, v_ctx, layer.k_buf_cache, layer.v_buf_cache, n_buf,
+                                       n_buf_device=n_buf_device)
         else:
             attn = ak.decode_attention(
-                q, k_ctx, v_ctx, layer.k_buf_cache, layer.v_buf_cache, self.buffer_len,
-                k_new[:, :, 0:1], v_new[:, :, 0:1],
+                q, k_ctx, v_ctx, layer.k_buf_cache, layer.v_buf_cache, n_buf,
+                k_new[:, :, 0:1], v_new[:, :, 0:1], n_buf_device=n_buf_device,
             )
         return layer.finish(x_row, attn)
 
@@ -236,12 +262,27 @@ class ARTabPFNPredictor:
 
     @torch.no_grad()
     def sample_sequence(self, x_context: Tensor, y_context: Tensor, x_target: Tensor) -> Tensor:
-        """Sample all targets autoregressively -> ``[B,Nt]`` (inference.py:322-366)."""
+        """Sample all targets autoregressively -> ``[B,Nt]`` (inference.py:322-366).
+
+        On a HIP device with the shared layout the steps after the first are replayed
+        from one recorded HIP graph (same kernels, same order; the step index and the
+        buffer length live in device memory), which removes the per-kernel launch cost
+        of the Python loop."""
         B, Nc, _ = x_context.shape
         Nt = x_target.shape[1]
         device, dtype = x_context.device, x_context.dtype
         self.init_kv_cache(B, Nt if self.backend == _SHARED else Nc + Nt, device, dtype)
         self.prefill_context(x_context, y_context)
+        return self.decode_targets(x_target)
+
+    @torch.no_grad()
+    def decode_targets(self, x_target: Tensor) -> Tensor:
+        """The decode loop of ``sample_sequence`` (inference.py:353-366) on caches that
+        are already initialised and prefilled: samples ``x_target [B,Nt,F]`` in order."""
+        Nt = x_target.shape[1]
+        if (self.use_hip_graph and self.backend == _SHARED and x_target.is_cuda and Nt >= 3
+                and self.buffer_len == 0 and Nt <= self.max_buffer_len):
+            return self._sample_sequence_graph(x_target)
         preds = []
         prev_x = prev_y = None
         for t in range(Nt):
@@ -250,6 +291,74 @@ class ARTabPFNPredictor:
             preds.append(y_t)
             prev_x, prev_y = x_t, y_t
         return torch.cat(preds, dim=1)
+
+    def _graph_step(self, st) -> None:
+        """One ``[buffer, target]`` decode step driven entirely by device-side state
+        (the body that is recorded): step index ``st.t``, buffer length ``st.nbuf``."""
+        bs = self.ar_tokens.shape[0]
+        x_t = st.x_target.index_select(1, st.t)
+        x_p = st.x_target.index_select(1, st.t - 1)
+        tok = self.ar_tokens.index_select(0, torch.remainder(st.t, bs))  # ar_tokens[t % bs], inference.py:359
+        buffer_emb = self.embedder.embed_buffer(x_p, st.y_prev) + tok
+        x_row = torch.cat([buffer_emb, self.embedder.embed_target(x_t)], dim=1)
+        for layer in self.backbone.layers:
+            x_row = self._layer_decode_with_cache_shared(layer, x_row, 1, n_buf_device=st.nbuf)
+        z = add_layer_norm(x_row, None, None, self.backbone.norm)
+        y = self.head.sample(z[:, -1:, :])[:, :, 0, 0]
+        st.preds.index_copy_(1, st.t, y)
+        st.y_prev.copy_(y)
+        st.t.add_(1)
+        st.nbuf.add_(1)
+
+    def _sample_sequence_graph(self, x_target: Tensor) -> Tensor:
+        B, Nt, F_ = x_target.shape
+        device, dtype = x_target.device, x_target.dtype
+        layer0 = self.backbone.layers[0]
+        key = (B, Nt, F_, self.context_len, dtype, str(device), layer0.k_ctx_cache.data_ptr(),
+               layer0.k_buf_cache.data_ptr(), tuple(p._version for p in self.backbone.parameters()))
+        st = self._graph_state
+        if st is None or st.key != key:
+            st = _GraphState()
+            st.key = key
+            st.x_target = torch.empty((B, Nt, F_), device=device, dtype=dtype)
+            st.y_prev = torch.zeros((B, 1), device=device, dtype=dtype)
+            st.preds = torch.zeros((B, Nt), device=device, dtype=dtype)
+            st.t = torch.ones(1, device=device, dtype=torch.long)
+            st.nbuf = torch.zeros(1, device=device, dtype=torch.int32)
+            st.graph = None
+            self._graph_state = st
+        st.x_target.copy_(x_target)
+
+        # first target: no buffer row yet (N = 1), launched directly
+        y0 = self.autoregressive_decode(st.x_target[:, 0:1, :], None, None, 0)
+
+        def reset():
+            st.y_prev.copy_(y0)
+            st.preds[:, 0:1] = y0
+            st.t.fill_(1)
+            st.nbuf.zero_()
+
+        if st.graph is None:
+            # warm-up on a side stream (workspace allocation, GEMM heuristics), then record;
+            # the rows the warm-up steps append are overwritten by the real steps
+            side = torch.cuda.Stream(device=device)
+            side.wait_stream(torch.cuda.current_stream(device))
+            with torch.cuda.stream(side):
+                reset()
+                for _ in range(2):
+                    self._graph_step(st)
+            torch.cuda.current_stream(device).wait_stream(side)
+            reset()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                self._graph_step(st)
+            st.graph = graph
+        reset()
+        for _ in range(Nt - 1):
+            st.graph.replay()
+        self.buffer_len = Nt - 1
+        self.seq_len = self.context_len + self.buffer_len
+        return st.preds.clone()
 
     # ------------------------------------------------------------------ teacher forcing
 
@@ -293,14 +402,14 @@ class ARTabPFNPredictor:
         x_row = embedding
         for layer in self.backbone.layers:
             x_row = self._layer_decode_with_cache(layer, x_row, mask, cache_start=self.seq_len)
-        return self.backbone.norm(x_row)
+        return add_layer_norm(x_row, None, None, self.backbone.norm)
 
     @torch.no_grad()
     def _teacher_forcing_decode_shared(self, embedding: Tensor, num_targets: int) -> Tensor:
         x_row = embedding
         for layer in self.backbone.layers:
             x_row = self._layer_teacher_forcing_shared(layer, x_row, num_targets)
-        return self.backbone.norm(x_row)
+        return add_layer_norm(x_row, None, None, self.backbone.norm)
 
     def _layer_teacher_forcing_shared(self, layer, x_row: Tensor, num_targets: int) -> Tensor:
         """inference.py:835-890: buffer K/V are the fresh projections of the first Nt

@@ -23,6 +23,7 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from .attention import DenseMask, MultiheadAttention
+from .glue import add_layer_norm, bias_gelu
 
 __all__ = ["Embedder", "TwoStageTransformerLayer", "TwoStageTransformer", "MixtureGaussianHead", "ARTabPFN"]
 
@@ -74,22 +75,61 @@ class TwoStageTransformerLayer(nn.Module):
         self.norm2 = nn.LayerNorm(d_model)
         self.norm3 = nn.LayerNorm(d_model)
 
+    def fused_weights(self):
+        """Weights of the fused inference GEMMs, rebuilt when a source weight changes.
+
+        * ``w_fo = out_proj.weight @ v_proj.weight`` of the feature attention: with a
+          single column the block is ``out_proj(v_proj(x))`` — one matrix (product taken
+          in float32, stored in the model dtype);
+        * ``w_qkv``: the three row-attention projections stacked, so q, k, v come out of
+          one GEMM as strided views of one ``[..., 3D]`` tensor.
+        """
+        af, ar = self.attn_features, self.attn_rows
+        srcs = (af.v_proj.weight, af.out_proj.weight, ar.q_proj.weight, ar.k_proj.weight, ar.v_proj.weight)
+        key = tuple((p.data_ptr(), p._version, p.dtype, p.device) for p in srcs)
+        cached = getattr(self, "_fused_cache", None)
+        if cached is None or cached[0] != key:
+            with torch.no_grad():
+                w_fo = (af.out_proj.weight.float() @ af.v_proj.weight.float()).to(af.v_proj.weight.dtype)
+                w_qkv = torch.cat([ar.q_proj.weight, ar.k_proj.weight, ar.v_proj.weight], dim=0).contiguous()
+            cached = (key, w_fo, w_qkv)
+            self._fused_cache = cached
+        return cached[1], cached[2]
+
     def feature_stage(self, x_row: Tensor) -> Tensor:
         """Feature attention for the single-column case (C = 1) followed by norm1.
 
         One key per query: the softmax weight is exactly 1, so the attention output is
         ``out_proj(v_proj(x))`` and the q/k projections do not enter
-        (attention.py:52-61 with S = 1; inference.py:771-773)."""
-        a = self.attn_features
-        return self.norm1(a.out_proj(a.v_proj(x_row)) + x_row)
+        (attention.py:52-61 with S = 1; inference.py:771-773).  One GEMM, then residual and
+        norm1 in one fused pass."""
+        w_fo, _ = self.fused_weights()
+        x2d = x_row.reshape(-1, x_row.shape[-1])
+        return add_layer_norm(x_row, torch.mm(x2d, w_fo.t()).view_as(x_row), None, self.norm1)
+
+    def qkv_heads(self, x_row: Tensor):
+        """q, k, v of the row attention as ``[B,H,N,Dh]`` strided views of one GEMM output."""
+        _, w_qkv = self.fused_weights()
+        B, N, D = x_row.shape
+        a = self.attn_rows
+        qkv = F.linear(x_row, w_qkv).view(B, N, 3, a.n_heads, a.head_dim)
+        return qkv[:, :, 0].transpose(1, 2), qkv[:, :, 1].transpose(1, 2), qkv[:, :, 2].transpose(1, 2)
 
     def finish(self, x_row: Tensor, attn_heads: Tensor) -> Tensor:
         """``out_proj`` on ``[B,H,N,Dh]`` attention output, then norm2 / FFN / norm3
         (inference.py:825-831)."""
         B, H, N, Dh = attn_heads.shape
-        attn = self.attn_rows.out_proj(attn_heads.transpose(1, 2).reshape(B, N, H * Dh))
-        x_row = self.norm2(x_row + attn)
-        return self.norm3(x_row + self.ff(x_row))
+        D = H * Dh
+        attn2d = attn_heads.transpose(1, 2).reshape(B * N, D)
+        x_row = add_layer_norm(x_row, torch.mm(attn2d, self.attn_rows.out_proj.weight.t()).view(B, N, D), None, self.norm2)
+        return self.feed_forward(x_row)
+
+    def feed_forward(self, x_row: Tensor) -> Tensor:
+        """``norm3(x + ff(x))`` with bias+GELU and bias+residual+norm fused around the two GEMMs."""
+        lin1, lin2 = self.ff[0], self.ff[2]
+        x2d = x_row.reshape(-1, x_row.shape[-1])
+        h = bias_gelu(torch.mm(x2d, lin1.weight.t()), lin1.bias)
+        return add_layer_norm(x_row, torch.mm(h, lin2.weight.t()).view_as(x_row), lin2.bias, self.norm3)
 
     def forward(self, x: Tensor, mask_features: DenseMask, mask_rows: DenseMask) -> Tuple[Tensor, Tuple[Tensor, Tensor]]:
         """``[B,R,C,D]`` with dense masks only (the bidirectional context pass)."""
@@ -98,8 +138,8 @@ class TwoStageTransformerLayer(nn.Module):
             raise NotImplementedError("only the single-column layout (C = 1) is used by this model")
         x_row = self.feature_stage(x.squeeze(2))
         attn, kv = self.attn_rows(x_row, x_row, x_row, mask_rows)
-        x_row = self.norm2(x_row + attn)
-        return self.norm3(x_row + self.ff(x_row)).unsqueeze(2), kv
+        x_row = add_layer_norm(x_row, attn, None, self.norm2)
+        return self.feed_forward(x_row).unsqueeze(2), kv
 
 
 class TwoStageTransformer(nn.Module):
@@ -114,7 +154,7 @@ class TwoStageTransformer(nn.Module):
         for layer in self.layers:
             x, kv = layer(x, mask_features, mask_rows)
             kvs.append(kv)
-        return self.norm(x), kvs
+        return add_layer_norm(x, None, None, self.norm), kvs
 
 
 class MixtureGaussianHead(nn.Module):

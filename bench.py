@@ -89,13 +89,9 @@ def run_decode(pred, x_context, y_context, x_target, steps, device, dtype):
     pred.prefill_context(x_context, y_context)
     ev[1].record()
     torch.cuda.synchronize()
-    prev_x = prev_y = None
     t0 = time.perf_counter()
     ev[2].record()
-    for t in range(steps):
-        x_t = x_target[:, t : t + 1, :]
-        y_t = pred.autoregressive_decode(x_t, prev_x, prev_y, t % pred.ar_tokens.shape[0])
-        prev_x, prev_y = x_t, y_t
+    pred.decode_targets(x_target[:, :steps])
     ev[3].record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
@@ -214,10 +210,13 @@ def main():
     # instrumented re-run of the same steps: HIP events around every context-pass launch
     import ctypes
 
+    # (launched kernel by kernel from Python: events cannot be recorded into a replayed graph)
+    pred.use_hip_graph = False
     lib.artab_profile_begin(CFG3["n_layers"] * (args.steps + 1) + 64)
     run_decode(pred, x_context, y_context, x_target, args.steps, device, dtype)
     tot, cnt = ctypes.c_double(0.0), ctypes.c_int(0)
     lib.artab_profile_end(ctypes.byref(tot), ctypes.byref(cnt))
+    pred.use_hip_graph = True
     # the first L launches are the prefill's dense passes, the first decode step has Lq=1
     H, Dh, L = CFG3["n_heads"], CFG3["d_model"] // CFG3["n_heads"], CFG3["n_layers"]
     n_dec = cnt.value - L

@@ -120,13 +120,19 @@ int artab_context_attention(const artab_view *q, const artab_view *k_ctx, const 
  *   out          [B,H,Lq,Dh]
  * An empty buffer (n_buf == 0 and no new row) gives context attention alone
  * (triton_kernels.py:735-741).  The caller advances n_buf (inference.py:256).
+ *   n_buf_device may be NULL.  When given it points to one int32 in device memory
+ *                that holds the committed length; the kernels read it when they run
+ *                instead of using `n_buf`, so a launch recorded in a HIP graph can be
+ *                replayed while the length advances.  `n_buf` must then be an upper
+ *                bound of every value the cell will hold (it is what is validated
+ *                against buf_capacity).
  */
 int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
                            const artab_view *k_buf, const artab_view *v_buf,
                            const artab_view *k_new, const artab_view *v_new,
                            const artab_view *out,
-                           int B, int H, int Lq, int Nc, int n_buf, int buf_capacity, int Dh,
-                           float scale, int dtype,
+                           int B, int H, int Lq, int Nc, int n_buf, const int32_t *n_buf_device,
+                           int buf_capacity, int Dh, float scale, int dtype,
                            void *workspace, size_t workspace_bytes, int impl, void *stream);
 
 /*
@@ -191,6 +197,23 @@ int artab_merge_attention_outputs(const artab_view *out_a, const float *lse_a,
                                   const artab_view *out_b, const float *lse_b,
                                   const artab_view *out,
                                   int B, int H, int Lq, int Dh, int dtype, void *stream);
+
+/*
+ * Row-wise glue of the transformer layer around the attention call (the norm2 / feed-forward /
+ * norm3 sequence of ar_tabpfn/model/inference.py:825-831 and the norm1 of :771-773), fused so a
+ * decode step is not dominated by small launches.  Matrices are row-major with a row stride in
+ * elements (ld*); `out` is contiguous [rows, D]; vectors are [D]; all of one dtype.
+ *
+ *   artab_add_layernorm:  out = LayerNorm(x + y + bias; gamma, beta, eps)   (y, bias may be NULL)
+ *                         float32 statistics, biased variance — torch.nn.LayerNorm semantics.
+ *                         D % 4 == 0, D <= 1024.
+ *   artab_bias_gelu:      out = gelu(x + bias), erf form (torch.nn.GELU default); bias may be NULL.
+ */
+int artab_add_layernorm(const void *x, int64_t ldx, const void *y, int64_t ldy, const void *bias,
+                        const void *gamma, const void *beta, void *out,
+                        int64_t rows, int D, float eps, int dtype, void *stream);
+int artab_bias_gelu(const void *x, int64_t ldx, const void *bias, void *out,
+                    int64_t rows, int D, int dtype, void *stream);
 
 #ifdef __cplusplus
 }

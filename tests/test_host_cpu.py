@@ -46,11 +46,11 @@ def test_argument_validation_returns_before_launch():
     v = L.ArtabView(0x1000, 64, 32, 32)  # never dereferenced: every call below fails validation
     r = ctypes.byref
     # decode: Lq outside {1,2}
-    rc = lib.artab_decode_attention(r(v), r(v), r(v), r(v), r(v), None, None, r(v), 2, 2, 3, 8, 0, 4, 32, 0.0, 0,
+    rc = lib.artab_decode_attention(r(v), r(v), r(v), r(v), r(v), None, None, r(v), 2, 2, 3, 8, 0, None, 4, 32, 0.0, 0,
                                     None, 0, 0, None)
     assert rc == L.ARTAB_ERR_BAD_SHAPE and b"Lq" in lib.artab_last_error()
     # decode: cache full
-    rc = lib.artab_decode_attention(r(v), r(v), r(v), r(v), r(v), r(v), r(v), r(v), 2, 2, 2, 8, 4, 4, 32, 0.0, 0,
+    rc = lib.artab_decode_attention(r(v), r(v), r(v), r(v), r(v), r(v), r(v), r(v), 2, 2, 2, 8, 4, None, 4, 32, 0.0, 0,
                                     None, 0, 0, None)
     assert rc == L.ARTAB_ERR_CAPACITY
     # context attention: empty context, unknown dtype, NULL q, oversized head_dim

@@ -427,3 +427,59 @@ def test_context_attention_extreme_scores(device, shift, gain):
     assert np.isfinite(to_np(out)).all() and np.isfinite(to_np(lse)).all()
     assert max_abs(to_np(out), ref_out) <= 2e-2
     assert max_abs(to_np(lse), ref_lse) <= 2.5e-3
+
+
+# ----- layer glue kernels -----------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,D", [(1, 4), (37, 128), (2048, 256), (5, 512), (3, 1024), (9, 36)])
+@pytest.mark.parametrize("with_y,with_bias", [(True, True), (True, False), (False, False)])
+def test_add_layernorm_matches_torch(device, dtype, rows, D, with_y, with_bias):
+    """LayerNorm(x + y + bias) against torch.nn.LayerNorm evaluated in float64 on the same bits."""
+    from ar_nanotabpfn_amd.glue import add_layer_norm
+
+    x = randn((rows, D), 1, dtype, 2.0)
+    y = randn((rows, D), 2, dtype) if with_y else None
+    b = randn((D,), 3, dtype, 0.3) if with_bias else None
+    norm = torch.nn.LayerNorm(D)
+    with torch.no_grad():
+        norm.weight.copy_(randn((D,), 4, torch.float32) * 0.2 + 1)
+        norm.bias.copy_(randn((D,), 5, torch.float32) * 0.2)
+    norm = norm.to(dtype)
+    out = add_layer_norm(x.to(device), y.to(device) if with_y else None, b.to(device) if with_bias else None,
+                         norm.to(device))
+    t = x.double() + (y.double() if with_y else 0) + (b.double() if with_bias else 0)
+    ref = torch.nn.functional.layer_norm(t, (D,), norm.weight.detach().cpu().double(), norm.bias.detach().cpu().double(), norm.eps)
+    tol = 2e-5 if dtype == torch.float32 else 2.0 ** -8 * max(1.0, float(ref.abs().max()))  # half an output ulp
+    assert out.shape == x.shape and out.dtype == dtype
+    assert max_abs(to_np(out), ref.numpy()) <= tol
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_add_layernorm_strided_input(device, dtype):
+    """x and y as column slices of a wider matrix (row stride != D)."""
+    from ar_nanotabpfn_amd.glue import add_layer_norm
+
+    wide = randn((64, 3 * 128), 1, dtype).to(device)
+    x, y = wide[:, 128:256], wide[:, 256:]
+    norm = torch.nn.LayerNorm(128).to(device=device, dtype=dtype)
+    out = add_layer_norm(x, y, None, norm)
+    ref = torch.nn.functional.layer_norm((x.double() + y.double()).cpu(), (128,), norm.weight.detach().cpu().double(),
+                                         norm.bias.detach().cpu().double(), norm.eps)
+    assert max_abs(to_np(out), ref.numpy()) <= (2e-5 if dtype == torch.float32 else 3e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,D", [(1, 4), (2048, 256), (7, 36)])
+def test_bias_gelu_matches_torch(device, dtype, rows, D):
+    from ar_nanotabpfn_amd.glue import bias_gelu
+
+    x, b = randn((rows, D), 1, dtype, 2.0), randn((D,), 2, dtype, 0.5)
+    out = bias_gelu(x.to(device), b.to(device))
+    ref = torch.nn.functional.gelu(x.double() + b.double())
+    # 16-bit outputs: half an output ulp (2^-8 relative for bf16) at the value's magnitude
+    tol = 2e-6 if dtype == torch.float32 else 2.0 ** -8 * max(1.0, float(ref.abs().max()))
+    assert max_abs(to_np(out), ref.numpy()) <= tol
+    out2 = bias_gelu(x.to(device), None)
+    assert max_abs(to_np(out2), torch.nn.functional.gelu(x.double()).numpy()) <= tol
