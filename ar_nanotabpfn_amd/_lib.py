@@ -61,6 +61,9 @@ SIGNATURES = {
     "artab_merge_attention_outputs": (_i, [_VP, _p, _VP, _p, _VP, _i, _i, _i, _i, _i, _p]),
     "artab_add_layernorm": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _i, _f, _i, _p]),
     "artab_bias_gelu": (_i, [_p, _i64, _p, _p, _i64, _i, _i, _p]),
+    "artab_pack_linear_weight": (_i, [_p, _p, _i, _i, _i, _p]),
+    "artab_layer_pre": (_i, [_p, _i64, _p, _p, _p, _f, _p, _p, _p, _i64, _i, _i, _p]),
+    "artab_layer_post": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _f, _p, _i64, _i, _i, _i, _p]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

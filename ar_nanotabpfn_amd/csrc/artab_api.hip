@@ -12,6 +12,7 @@
 #include "../../include/artab_attention.h"
 #include "common.h"
 #include "decode_buffer.h"
+#include "fused_layer.h"
 #include "glue_kernels.h"
 #include "mfma_flash.h"
 #include "portable_kernels.h"
@@ -189,6 +190,10 @@ static hipError_t launch_flash_bm(const FlashParams &P, int BM, hipStream_t stre
             hipLaunchKernelGGL((flash_kernel<T, DH, 2, 4, kFlashBN>), dim3(grid), dim3(256), 0, stream, P);
             return hipGetLastError();
         }
+        if (BM == 128 && env_int("ARTAB_NW", 4) == 2) {  // two wavefronts of two query blocks each
+            hipLaunchKernelGGL((flash_kernel<T, DH, 2, 2, kFlashBN>), dim3(grid), dim3(128), 0, stream, P);
+            return hipGetLastError();
+        }
     }
     if (BM == 128) {
         hipLaunchKernelGGL((flash_kernel<T, DH, 1, 4, kFlashBN>), dim3(grid), dim3(256), 0, stream, P);
@@ -293,6 +298,44 @@ static int launch_status(hipError_t e, const char *what) {
     if (e == hipSuccess) return ARTAB_OK;
     return fail(ARTAB_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
 }
+
+namespace {
+
+template <typename T>
+hipError_t launch_pre(const FusedPreParams &P, int D, hipStream_t st) {
+    dim3 grid(static_cast<unsigned>((P.rows + kFusedRows - 1) / kFusedRows)), block(fused_waves(D) * 64);
+    switch (D) {
+        case 128: hipLaunchKernelGGL((fused_pre_kernel<T, 128>), grid, block, 0, st, P); break;
+        case 256: hipLaunchKernelGGL((fused_pre_kernel<T, 256>), grid, block, 0, st, P); break;
+        default: hipLaunchKernelGGL((fused_pre_kernel<T, 512>), grid, block, 0, st, P); break;
+    }
+    return hipGetLastError();
+}
+
+template <typename T, int D>
+hipError_t launch_post_d(const FusedPostParams &P, int F, hipStream_t st) {
+    dim3 grid(static_cast<unsigned>((P.rows + kFusedRows - 1) / kFusedRows)), block(fused_waves(D) * 64);
+    switch (F) {
+        case 128: hipLaunchKernelGGL((fused_post_kernel<T, D, 128>), grid, block, 0, st, P); break;
+        case 256: hipLaunchKernelGGL((fused_post_kernel<T, D, 256>), grid, block, 0, st, P); break;
+        default: hipLaunchKernelGGL((fused_post_kernel<T, D, 512>), grid, block, 0, st, P); break;
+    }
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_post(const FusedPostParams &P, int D, int F, hipStream_t st) {
+    switch (D) {
+        case 128: return launch_post_d<T, 128>(P, F, st);
+        case 256: return launch_post_d<T, 256>(P, F, st);
+        default: return launch_post_d<T, 512>(P, F, st);
+    }
+}
+
+bool fused_width_ok(int n) { return n == 128 || n == 256 || n == 512; }
+bool misaligned16(const void *p) { return p && reinterpret_cast<uintptr_t>(p) % 16 != 0; }
+
+}  // namespace
 
 extern "C" {
 
@@ -724,6 +767,76 @@ int artab_bias_gelu(const void *x, int64_t ldx, const void *bias, void *out, int
         default: hipLaunchKernelGGL((bias_gelu_kernel<float>), grid, dim3(256), 0, st, P); break;
     }
     return launch_status(hipGetLastError(), "bias_gelu");
+}
+
+int artab_pack_linear_weight(const void *w, void *packed, int N, int K, int dtype, void *stream) {
+    if (dtype != ARTAB_BF16 && dtype != ARTAB_F16)
+        return fail(ARTAB_ERR_UNSUPPORTED, "pack_linear_weight supports bf16 and fp16 only (dtype code %d)", dtype);
+    if (N <= 0 || K <= 0 || N % 32 || K % 16)
+        return fail(ARTAB_ERR_BAD_SHAPE, "pack_linear_weight needs N %% 32 == 0 and K %% 16 == 0 (got %d, %d)", N, K);
+    if (!w || !packed) return fail(ARTAB_ERR_NULL_POINTER, "w and packed are required");
+    if (misaligned16(w) || misaligned16(packed)) return fail(ARTAB_ERR_BAD_STRIDE, "w and packed must be 16-byte aligned");
+    const char *a = static_cast<const char *>(w), *b = static_cast<const char *>(packed);
+    const size_t bytes = static_cast<size_t>(N) * K * 2;
+    if (a < b + bytes && b < a + bytes) return fail(ARTAB_ERR_BAD_STRIDE, "packed must not overlap w");
+    const long chunks = static_cast<long>(N) * K / 8;
+    dim3 grid(static_cast<unsigned>((chunks + 255) / 256));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == ARTAB_BF16)
+        hipLaunchKernelGGL((pack_weight_kernel<bf16_t>), grid, dim3(256), 0, st, static_cast<const bf16_t *>(w),
+                           static_cast<bf16_t *>(packed), N, K);
+    else
+        hipLaunchKernelGGL((pack_weight_kernel<f16_t>), grid, dim3(256), 0, st, static_cast<const f16_t *>(w),
+                           static_cast<f16_t *>(packed), N, K);
+    return launch_status(hipGetLastError(), "pack_linear_weight");
+}
+
+int artab_layer_pre(const void *x, int64_t ldx, const void *w_fo, const void *ln1_gamma, const void *ln1_beta,
+                    float eps1, const void *w_qkv, void *y, void *qkv, int64_t rows, int D, int dtype,
+                    void *stream) {
+    if (dtype != ARTAB_BF16 && dtype != ARTAB_F16)
+        return fail(ARTAB_ERR_UNSUPPORTED, "layer_pre supports bf16 and fp16 only (dtype code %d)", dtype);
+    if (rows < 0 || D <= 0) return fail(ARTAB_ERR_BAD_SHAPE, "bad sizes rows=%lld D=%d", (long long)rows, D);
+    if (!fused_width_ok(D)) return fail(ARTAB_ERR_UNSUPPORTED, "layer_pre needs D in {128, 256, 512} (got %d)", D);
+    if (rows == 0) return ARTAB_OK;
+    if (!x || !w_fo || !ln1_gamma || !ln1_beta || !w_qkv || !y || !qkv)
+        return fail(ARTAB_ERR_NULL_POINTER, "layer_pre: every pointer is required");
+    if (misaligned16(x) || misaligned16(w_fo) || misaligned16(w_qkv) || misaligned16(y) || misaligned16(qkv) ||
+        misaligned16(ln1_gamma) || misaligned16(ln1_beta) || ldx % 8 || ldx < D)
+        return fail(ARTAB_ERR_BAD_STRIDE, "layer_pre operands must be 16-byte aligned with ldx %% 8 == 0, ldx >= D");
+    FusedPreParams P;
+    P.x = x; P.ldx = ldx; P.w_fo = w_fo; P.g1 = ln1_gamma; P.b1 = ln1_beta; P.w_qkv = w_qkv;
+    P.y = y; P.qkv = qkv; P.rows = rows; P.eps = eps1;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipError_t e = dtype == ARTAB_BF16 ? launch_pre<bf16_t>(P, D, st) : launch_pre<f16_t>(P, D, st);
+    return launch_status(e, "layer_pre");
+}
+
+int artab_layer_post(const void *attn, int64_t lda, const void *y, int64_t ldy, const void *w_o,
+                     const void *ln2_gamma, const void *ln2_beta, float eps2, const void *w_1, const void *b_1,
+                     const void *w_2, const void *b_2, const void *ln3_gamma, const void *ln3_beta, float eps3,
+                     void *out, int64_t rows, int D, int F, int dtype, void *stream) {
+    if (dtype != ARTAB_BF16 && dtype != ARTAB_F16)
+        return fail(ARTAB_ERR_UNSUPPORTED, "layer_post supports bf16 and fp16 only (dtype code %d)", dtype);
+    if (rows < 0 || D <= 0 || F <= 0)
+        return fail(ARTAB_ERR_BAD_SHAPE, "bad sizes rows=%lld D=%d F=%d", (long long)rows, D, F);
+    if (!fused_width_ok(D) || !fused_width_ok(F))
+        return fail(ARTAB_ERR_UNSUPPORTED, "layer_post needs D and F in {128, 256, 512} (got %d, %d)", D, F);
+    if (rows == 0) return ARTAB_OK;
+    if (!attn || !y || !w_o || !ln2_gamma || !ln2_beta || !w_1 || !w_2 || !ln3_gamma || !ln3_beta || !out)
+        return fail(ARTAB_ERR_NULL_POINTER, "layer_post: only b_1 and b_2 may be NULL");
+    if (misaligned16(attn) || misaligned16(y) || misaligned16(w_o) || misaligned16(w_1) || misaligned16(w_2) ||
+        misaligned16(b_1) || misaligned16(b_2) || misaligned16(ln2_gamma) || misaligned16(ln2_beta) ||
+        misaligned16(ln3_gamma) || misaligned16(ln3_beta) || misaligned16(out) || lda % 8 || ldy % 8 || lda < D ||
+        ldy < D)
+        return fail(ARTAB_ERR_BAD_STRIDE, "layer_post operands must be 16-byte aligned with row strides %% 8 == 0");
+    FusedPostParams P;
+    P.attn = attn; P.lda = lda; P.y = y; P.ldy = ldy; P.w_o = w_o; P.g2 = ln2_gamma; P.b2 = ln2_beta;
+    P.w_1 = w_1; P.bias_1 = b_1; P.w_2 = w_2; P.bias_2 = b_2; P.g3 = ln3_gamma; P.b3 = ln3_beta;
+    P.out = out; P.rows = rows; P.eps2 = eps2; P.eps3 = eps3;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipError_t e = dtype == ARTAB_BF16 ? launch_post<bf16_t>(P, D, F, st) : launch_post<f16_t>(P, D, F, st);
+    return launch_status(e, "layer_post");
 }
 
 }  // extern "C"

@@ -1,0 +1,401 @@
+// Fused transformer-layer glue around the attention call (gfx950, bf16/f16).
+//
+// A decode step touches only B*N token rows (2048 at B=1024), so the GEMMs of a layer
+// are tiny and the step is dominated by the number of launches.  Two kernels replace
+// the nine launches of a layer's non-attention part:
+//
+//   fused_pre_kernel :  y = LN1(x + x W_fo^T);  qkv = y W_qkv^T
+//   fused_post_kernel:  x1 = LN2(y + attn W_o^T);  h = gelu(x1 W_1^T + b_1);
+//                       out = LN3(x1 + h W_2^T + b_2)
+//
+// One workgroup owns 32 token rows and all columns.  Products are computed transposed
+// with v_mfma_f32_32x32x16 (C^T[n, m] = sum_k W[n, k] A[m, k]): the weight rows are the
+// A operand, read straight from global memory in a pre-packed operand order (weights are
+// constants, packed once), so every wavefront load is one contiguous KiB; the
+// activation rows are the B operand, staged once in LDS and re-read per 16 contraction
+// elements; a lane then owns one token column, so LayerNorm statistics are per-lane sums
+// plus one exchange between the four wavefronts.  Activations stay in LDS between the
+// chained products.
+#pragma once
+
+#include "common.h"
+#include "mfma_flash.h"
+
+namespace artab {
+
+constexpr int kFusedRows = 32;  // token rows per workgroup
+
+// Stands in for an absent bias vector (1024 16-bit zeros; widths go up to 512).
+static __device__ const unsigned int kZeroVector[512] = {0u};
+
+// Wavefronts per workgroup: one 32-column output block each where the width allows, so that
+// a wavefront has every weight fragment of a product in flight at once (the kernels are
+// latency-bound at decode sizes: 64 workgroups for 2048 rows).
+constexpr int fused_waves(int D) { return D >= 256 ? 8 : 4; }
+
+struct FusedPreParams {
+    const void *x;   long ldx;   // [rows, D]
+    const void *w_fo;            // [D, D] packed
+    const void *g1, *b1;         // LayerNorm 1
+    const void *w_qkv;           // [3D, D] packed
+    void *y;                     // [rows, D] contiguous
+    void *qkv;                   // [rows, 3D] contiguous
+    long rows;
+    float eps;
+};
+
+struct FusedPostParams {
+    const void *attn; long lda;  // [rows, D]
+    const void *y;    long ldy;  // [rows, D] residual stream (output of the pre kernel)
+    const void *w_o;             // [D, D] packed
+    const void *g2, *b2;         // LayerNorm 2
+    const void *w_1, *bias_1;    // [F, D] packed, [F]
+    const void *w_2, *bias_2;    // [D, F] packed, [D]
+    const void *g3, *b3;         // LayerNorm 3
+    void *out;                   // [rows, D] contiguous
+    long rows;
+    float eps2, eps3;
+};
+
+// Packed weight layout.  A torch.nn.Linear weight W [N, K] (row-major) is stored as
+// [N/32][K/16][64 lanes][8]: element (blk, ks, lane, e) = W[32*blk + lane%32][16*ks + 8*(lane/32) + e],
+// i.e. exactly the A operand of v_mfma_f32_32x32x16 for output block blk and contraction step ks,
+// so that one wavefront load reads 1 KiB of consecutive memory.
+template <typename T>
+__global__ void pack_weight_kernel(const T *w, T *packed, int N, int K) {
+    const long chunk = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;  // one 16-byte chunk each
+    const long total = static_cast<long>(N) * K / 8;
+    if (chunk >= total) return;
+    const int lane = static_cast<int>(chunk % 64);
+    const long t = chunk / 64;
+    const int ks = static_cast<int>(t % (K / 16));
+    const int blk = static_cast<int>(t / (K / 16));
+    const T *src = w + static_cast<long>(32 * blk + (lane & 31)) * K + 16 * ks + 8 * (lane >> 5);
+    *reinterpret_cast<u32x4 *>(packed + chunk * 8) = *reinterpret_cast<const u32x4 *>(src);
+}
+
+// One transposed product: acc[b][v] = sum_k W[32*nblk[b] + row(v)][k] * A[c][k] for NB blocks of
+// 32 output columns; A is the [32, K] activation tile in LDS (row stride ld), W the packed weight.
+// The weight fragments are fetched explicitly ahead of their use — start() issues the first PF
+// contraction steps and can be called long before run(), e.g. ahead of the previous product's
+// epilogue, so that the memory round trips of chained products overlap.  (Left to itself the
+// compiler issues each load right before the MFMA that needs it: one round trip per step.)
+template <typename T, int K, int NB>
+struct WeightStream {
+    typedef MfmaOps<T> Ops;
+    typedef typename Ops::vec vec;
+    static constexpr int KS = K / 16;
+    static constexpr int PFW = NB >= 4 ? 4 : (NB == 2 ? 8 : 16);
+    static constexpr int PF = PFW < KS ? PFW : KS;
+    const T *wl[NB];
+    vec wf[PF][NB];
+
+    __device__ __forceinline__ void start(const T *wp, const int (&nblk)[NB], int lane) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) wl[b] = wp + static_cast<long>(nblk[b]) * KS * 512 + lane * 8;
+#pragma unroll
+        for (int p = 0; p < PF; ++p)
+#pragma unroll
+            for (int b = 0; b < NB; ++b) wf[p][b] = *reinterpret_cast<const vec *>(wl[b] + p * 512);
+        __builtin_amdgcn_sched_barrier(0);  // the prefetch stays where it was written
+    }
+
+    __device__ __forceinline__ void run(f32x16 (&acc)[NB], const T *a_lds, int ld, int c, int hb) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[b][v] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const vec af = *reinterpret_cast<const vec *>(a_lds + c * ld + 16 * ks + 8 * hb);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) acc[b] = Ops::mma(wf[ks % PF][b], af, acc[b]);
+            if (ks + PF < KS) {
+#pragma unroll
+                for (int b = 0; b < NB; ++b) wf[ks % PF][b] = *reinterpret_cast<const vec *>(wl[b] + (ks + PF) * 512);
+            }
+        }
+    }
+};
+
+// Column index of accumulator element (block nb, register v) for this lane.
+__device__ __forceinline__ int col_of(int nb, int v, int hb) { return 32 * nb + 8 * (v >> 2) + 4 * hb + (v & 3); }
+
+template <typename T>
+__device__ __forceinline__ void load4f(const T *p, float *f) {
+    u32x2 r = *reinterpret_cast<const u32x2 *>(p);
+    f[0] = unpack_lo<T>(r[0]);
+    f[1] = unpack_hi<T>(r[0]);
+    f[2] = unpack_lo<T>(r[1]);
+    f[3] = unpack_hi<T>(r[1]);
+}
+template <typename T>
+__device__ __forceinline__ void store4f(T *p, float a, float b, float c, float d) {
+    u32x2 r = {pack2<T>(a, b), pack2<T>(c, d)};
+    *reinterpret_cast<u32x2 *>(p) = r;
+}
+
+// The entries of a length-N vector (bias, gamma, beta) at this lane's accumulator columns;
+// a missing bias is read from a zero vector the caller substitutes.
+template <typename T, int NB>
+__device__ __forceinline__ void load_cols(const T *vec, const int (&nblk)[NB], int hb, float (&out)[NB][16]) {
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) load4f<T>(vec + col_of(nblk[b], 4 * g, hb), &out[b][4 * g]);
+}
+
+// Row statistics over all N columns of the tile: each lane holds, for its token column, the
+// values of NB blocks; sums are completed across the lane pair (hb) and the wavefronts.
+// red_a / red_b are two [NW*32] exchange arrays (two, so that back-to-back calls need no
+// trailing barrier).
+template <int NB, int NW>
+__device__ __forceinline__ void row_mean_rstd(const float (&v)[NB][16], float *red_a, float *red_b, int wave, int c,
+                                              int hb, int N, float eps, float &mean, float &rstd) {
+    float s = 0.f;
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s += v[b][e];
+    s += __shfl_xor(s, 32, 64);
+    if (hb == 0) red_a[wave * 32 + c] = s;
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) tot += red_a[w * 32 + c];
+    mean = tot / N;
+    float q = 0.f;
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const float d = v[b][e] - mean;
+            q += d * d;
+        }
+    q += __shfl_xor(q, 32, 64);
+    if (hb == 0) red_b[wave * 32 + c] = q;
+    __syncthreads();
+    float var = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) var += red_b[w * 32 + c];
+    rstd = rsqrtf(var / N + eps);
+}
+
+// Cooperative copy of a [32, W] tile between global memory (row stride ld) and LDS (row stride
+// lds_ld) with 16-byte accesses along rows.  Loading zero-fills rows beyond `valid`.
+template <typename T, int W, int NT>
+__device__ __forceinline__ void stage_tile(T *dst, int lds_ld, const T *src, long ld, int valid, int tid) {
+    constexpr int CPR = W / 8;
+#pragma unroll
+    for (int idx = tid; idx < kFusedRows * CPR; idx += NT) {
+        const int r = idx / CPR, ch = idx % CPR;
+        u32x4 val = {0u, 0u, 0u, 0u};
+        if (r < valid) val = *reinterpret_cast<const u32x4 *>(src + r * ld + 8 * ch);
+        *reinterpret_cast<u32x4 *>(dst + r * lds_ld + 8 * ch) = val;
+    }
+}
+template <typename T, int W, int NT>
+__device__ __forceinline__ void unstage_tile(T *dst, long ld, const T *src, int lds_ld, int valid, int tid) {
+    constexpr int CPR = W / 8;
+#pragma unroll
+    for (int idx = tid; idx < kFusedRows * CPR; idx += NT) {
+        const int r = idx / CPR, ch = idx % CPR;
+        if (r < valid)
+            *reinterpret_cast<u32x4 *>(dst + r * ld + 8 * ch) = *reinterpret_cast<const u32x4 *>(src + r * lds_ld + 8 * ch);
+    }
+}
+
+// LayerNorm over the tile rows of v (statistics across all wavefronts), result written as T
+// into the LDS tile `dst` at this lane's (row c, accumulator columns).
+template <typename T, int NB, int NW>
+__device__ __forceinline__ void layer_norm_to_lds(const float (&v)[NB][16], const float (&gam)[NB][16],
+                                                  const float (&bet)[NB][16], const int (&nblk)[NB], T *dst, int ld,
+                                                  float *red_a, float *red_b, int wave, int c, int hb, int N,
+                                                  float eps) {
+    float mean, rstd;
+    row_mean_rstd<NB, NW>(v, red_a, red_b, wave, c, hb, N, eps, mean, rstd);
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = (v[b][4 * g + e] - mean) * rstd * gam[b][4 * g + e] + bet[b][4 * g + e];
+            store4f<T>(dst + c * ld + col_of(nblk[b], 4 * g, hb), o[0], o[1], o[2], o[3]);
+        }
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(fused_waves(D) * 64) void fused_pre_kernel(FusedPreParams P) {
+    constexpr int NW = fused_waves(D), NT = NW * 64;
+    constexpr int LD = D + 8;
+    constexpr int NB = D / 32 / NW;  // 32-column blocks per wavefront per D columns
+    static_assert(D % (32 * NW) == 0, "D must be a multiple of 32 * wavefronts");
+    __shared__ __attribute__((aligned(16))) T a0[kFusedRows * LD];  // x tile, later qkv staging
+    __shared__ __attribute__((aligned(16))) T a1[kFusedRows * LD];  // y tile
+    __shared__ float red_a[NW * 32], red_b[NW * 32];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hb = lane >> 5;
+    const long row0 = static_cast<long>(blockIdx.x) * kFusedRows;
+    const int valid = static_cast<int>(min(static_cast<long>(kFusedRows), P.rows - row0));
+
+    int nblk[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) nblk[b] = wave + NW * b;
+
+    WeightStream<T, D, NB> w_a, w_b;
+    w_a.start(static_cast<const T *>(P.w_fo), nblk, lane);
+    stage_tile<T, D, NT>(a0, LD, static_cast<const T *>(P.x) + row0 * P.ldx, P.ldx, valid, tid);
+    float gam[NB][16], bet[NB][16];
+    load_cols<T, NB>(static_cast<const T *>(P.g1), nblk, hb, gam);
+    load_cols<T, NB>(static_cast<const T *>(P.b1), nblk, hb, bet);
+    w_b.start(static_cast<const T *>(P.w_qkv), nblk, lane);  // q columns
+    __syncthreads();
+
+    // ---- y = LN1(x + x W_fo^T)
+    {
+        f32x16 acc[NB];
+        w_a.run(acc, a0, LD, c, hb);
+        float v[NB][16];
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float r[4];
+                load4f<T>(a0 + c * LD + col_of(nblk[b], 4 * g, hb), r);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[b][4 * g + e] = acc[b][4 * g + e] + r[e];
+            }
+        layer_norm_to_lds<T, NB, NW>(v, gam, bet, nblk, a1, LD, red_a, red_b, wave, c, hb, D, P.eps);
+    }
+    __syncthreads();  // y complete in a1; a0 no longer read
+    unstage_tile<T, D, NT>(static_cast<T *>(P.y) + row0 * D, D, a1, LD, valid, tid);
+
+    // ---- qkv = y W_qkv^T, three passes of D columns, each staged through a0 for row-contiguous
+    // stores; the weights of the next pass are requested before the current one is computed
+#pragma unroll
+    for (int part = 0; part < 3; ++part) {
+        WeightStream<T, D, NB> &cur = (part & 1) ? w_a : w_b, &nxt = (part & 1) ? w_b : w_a;
+        if (part < 2) {
+            int nb2[NB];
+#pragma unroll
+            for (int b = 0; b < NB; ++b) nb2[b] = (part + 1) * (D / 32) + nblk[b];
+            nxt.start(static_cast<const T *>(P.w_qkv), nb2, lane);
+        }
+        f32x16 acc[NB];
+        cur.run(acc, a1, LD, c, hb);
+        if (part) __syncthreads();  // the previous pass has been copied out of a0
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                store4f<T>(a0 + c * LD + col_of(nblk[b], 4 * g, hb), acc[b][4 * g], acc[b][4 * g + 1],
+                           acc[b][4 * g + 2], acc[b][4 * g + 3]);
+        __syncthreads();
+        unstage_tile<T, D, NT>(static_cast<T *>(P.qkv) + row0 * (3 * D) + part * D, 3 * D, a0, LD, valid, tid);
+    }
+}
+
+template <typename T, int D, int F>
+__global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_kernel(FusedPostParams P) {
+    constexpr int NW = fused_waves(D), NT = NW * 64;
+    constexpr int LDD = D + 8, LDF = F + 8;
+    constexpr int LDM = LDD > LDF ? LDD : LDF;
+    constexpr int NBD = D / 32 / NW;
+    constexpr int NBF = (F / 32 + NW - 1) / NW;  // with F/32 < NW the upper wavefronts sit the product out
+    static_assert(D % (32 * NW) == 0 && F % 32 == 0, "unsupported widths");
+    static_assert(F / 32 >= NW ? (F / 32) % NW == 0 : true, "unsupported widths");
+    __shared__ __attribute__((aligned(16))) T a0[kFusedRows * LDM];  // attn tile, gelu output, out staging
+    __shared__ __attribute__((aligned(16))) T a1[kFusedRows * LDD];  // y tile, then x1 = LN2(...)
+    __shared__ float red_a[NW * 32], red_b[NW * 32];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hb = lane >> 5;
+    const long row0 = static_cast<long>(blockIdx.x) * kFusedRows;
+    const int valid = static_cast<int>(min(static_cast<long>(kFusedRows), P.rows - row0));
+
+    int nbd[NBD], nbf[NBF];
+#pragma unroll
+    for (int b = 0; b < NBD; ++b) nbd[b] = wave + NW * b;
+#pragma unroll
+    for (int b = 0; b < NBF; ++b) nbf[b] = wave + NW * b;
+    const bool ff_active = wave < F / 32;  // wavefront-uniform
+
+    WeightStream<T, D, NBD> w_o;
+    WeightStream<T, D, NBF> w_1;
+    WeightStream<T, F, NBD> w_2;
+    w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
+    stage_tile<T, D, NT>(a0, LDD, static_cast<const T *>(P.attn) + row0 * P.lda, P.lda, valid, tid);
+    stage_tile<T, D, NT>(a1, LDD, static_cast<const T *>(P.y) + row0 * P.ldy, P.ldy, valid, tid);
+    if (ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane);
+    __syncthreads();
+
+    // ---- x1 = LN2(y + attn W_o^T); each lane replaces exactly the y entries it read
+    {
+        float gam[NBD][16], bet[NBD][16];
+        load_cols<T, NBD>(static_cast<const T *>(P.g2), nbd, hb, gam);
+        load_cols<T, NBD>(static_cast<const T *>(P.b2), nbd, hb, bet);
+        f32x16 acc[NBD];
+        w_o.run(acc, a0, LDD, c, hb);
+        w_2.start(static_cast<const T *>(P.w_2), nbd, lane);
+        float v[NBD][16];
+#pragma unroll
+        for (int b = 0; b < NBD; ++b)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float r[4];
+                load4f<T>(a1 + c * LDD + col_of(nbd[b], 4 * g, hb), r);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[b][4 * g + e] = acc[b][4 * g + e] + r[e];
+            }
+        layer_norm_to_lds<T, NBD, NW>(v, gam, bet, nbd, a1, LDD, red_a, red_b, wave, c, hb, D, P.eps2);
+    }
+    __syncthreads();  // x1 complete in a1; every wavefront is done reading a0
+
+    // ---- h = gelu(x1 W_1^T + b_1)  -> a0
+    if (ff_active) {
+        float bias[NBF][16];
+        load_cols<T, NBF>(P.bias_1 ? static_cast<const T *>(P.bias_1) : reinterpret_cast<const T *>(kZeroVector), nbf,
+                          hb, bias);
+        f32x16 acc[NBF];
+        w_1.run(acc, a1, LDD, c, hb);
+#pragma unroll
+        for (int b = 0; b < NBF; ++b)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float t = acc[b][4 * g + e] + bias[b][4 * g + e];
+                    o[e] = 0.5f * t * (1.f + erff(t * 0.70710678118654752f));
+                }
+                store4f<T>(a0 + c * LDF + col_of(nbf[b], 4 * g, hb), o[0], o[1], o[2], o[3]);
+            }
+    }
+    float gam[NBD][16], bet[NBD][16], bias[NBD][16];
+    load_cols<T, NBD>(static_cast<const T *>(P.g3), nbd, hb, gam);
+    load_cols<T, NBD>(static_cast<const T *>(P.b3), nbd, hb, bet);
+    load_cols<T, NBD>(P.bias_2 ? static_cast<const T *>(P.bias_2) : reinterpret_cast<const T *>(kZeroVector), nbd, hb,
+                      bias);
+    __syncthreads();
+
+    // ---- out = LN3(x1 + h W_2^T + b_2), staged through a0 for row-contiguous stores
+    {
+        f32x16 acc[NBD];
+        w_2.run(acc, a0, LDF, c, hb);
+        float v[NBD][16];
+#pragma unroll
+        for (int b = 0; b < NBD; ++b)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float r[4];
+                load4f<T>(a1 + c * LDD + col_of(nbd[b], 4 * g, hb), r);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[b][4 * g + e] = acc[b][4 * g + e] + r[e] + bias[b][4 * g + e];
+            }
+        // the barriers inside the statistics also order every wavefront's last read of a0
+        // (the product above) before the first write of the result into it
+        layer_norm_to_lds<T, NBD, NW>(v, gam, bet, nbd, a0, LDD, red_a, red_b, wave, c, hb, D, P.eps3);
+    }
+    __syncthreads();
+    unstage_tile<T, D, NT>(static_cast<T *>(P.out) + row0 * D, D, a0, LDD, valid, tid);
+}
+
+}  // namespace artab

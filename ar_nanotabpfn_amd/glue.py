@@ -1,7 +1,9 @@
-"""Row-wise glue ops of the transformer layer (residual + bias + LayerNorm, bias + GELU).
+"""Row-wise glue ops of the transformer layer (residual + bias + LayerNorm, bias + GELU)
+and the two whole-layer fusions around the attention call.
 
 On a HIP device they are single fused kernels of ``libartab_attention.so``
-(``artab_add_layernorm``, ``artab_bias_gelu``); on CPU tensors — the model itself is
+(``artab_add_layernorm``, ``artab_bias_gelu``, ``artab_layer_pre``, ``artab_layer_post``);
+on CPU tensors — the model itself is
 plain PyTorch and can be built and inspected anywhere — the same arithmetic is spelled
 with torch ops.  The attention path has no such CPU spelling.
 """
@@ -17,7 +19,7 @@ from torch import Tensor, nn
 
 from . import _lib
 
-__all__ = ["add_layer_norm", "bias_gelu"]
+__all__ = ["add_layer_norm", "bias_gelu", "layer_fusable", "pack_weight", "layer_pre", "layer_post"]
 
 
 def _rows2d(t: Tensor) -> Tensor:
@@ -67,3 +69,72 @@ def bias_gelu(x: Tensor, bias: Optional[Tensor]) -> Tensor:
                             _lib.dtype_code(x.dtype), _lib.current_stream(x.device))
     )
     return out.view(x.shape)
+
+
+_FUSED_WIDTHS = (128, 256, 512)
+
+
+def layer_fusable(x: Tensor, d_model: int, d_ff: int) -> bool:
+    """True when ``layer_pre`` / ``layer_post`` cover this layer (16-bit dtype on a HIP device,
+    widths the kernels are built for)."""
+    return (x.is_cuda and x.dtype in (torch.bfloat16, torch.float16)
+            and d_model in _FUSED_WIDTHS and d_ff in _FUSED_WIDTHS)
+
+
+def _rows16(t: Tensor) -> Tensor:
+    """[rows, D] view with unit column stride, 16-byte aligned rows."""
+    t2 = t.reshape(-1, t.shape[-1])
+    if t2.stride(1) != 1 or t2.stride(0) % 8 or t2.data_ptr() % 16:
+        t2 = t2.contiguous()
+    return t2
+
+
+def pack_weight(w: Tensor) -> Tensor:
+    """A ``torch.nn.Linear`` weight ``[N, K]`` in the operand order of the fused layer kernels
+    (``[N/32, K/16, 64, 8]``, see ``artab_pack_linear_weight``); done once per weight."""
+    w = w.detach().contiguous()
+    N, K = w.shape
+    packed = torch.empty((N // 32, K // 16, 64, 8), device=w.device, dtype=w.dtype)
+    _lib.check(_lib.load().artab_pack_linear_weight(_ptr(w), _ptr(packed), N, K, _lib.dtype_code(w.dtype),
+                                                    _lib.current_stream(w.device)))
+    return packed
+
+
+def layer_pre(x: Tensor, w_fo: Tensor, norm1: nn.LayerNorm, w_qkv: Tensor):
+    """``y = norm1(x + x @ W_fo.T)``, ``qkv = y @ W_qkv.T`` in one launch; ``w_fo`` and
+    ``w_qkv`` are the packed forms (``pack_weight``) of ``W_fo [D, D]`` and ``W_qkv [3D, D]``.
+
+    Returns ``(y [rows, D], qkv [rows, 3D])``."""
+    D = x.shape[-1]
+    x2 = _rows16(x)
+    rows = x2.shape[0]
+    y = torch.empty((rows, D), device=x.device, dtype=x.dtype)
+    qkv = torch.empty((rows, 3 * D), device=x.device, dtype=x.dtype)
+    _lib.check(
+        _lib.load().artab_layer_pre(
+            _ptr(x2), x2.stride(0), _ptr(w_fo), _ptr(norm1.weight), _ptr(norm1.bias), float(norm1.eps),
+            _ptr(w_qkv), _ptr(y), _ptr(qkv), rows, D, _lib.dtype_code(x.dtype), _lib.current_stream(x.device),
+        )
+    )
+    return y, qkv
+
+
+def layer_post(attn: Tensor, y: Tensor, w_o: Tensor, norm2: nn.LayerNorm, w_1: Tensor, b_1: Optional[Tensor],
+               w_2: Tensor, b_2: Optional[Tensor], norm3: nn.LayerNorm) -> Tensor:
+    """``x1 = norm2(y + attn @ W_o.T)``; ``norm3(x1 + gelu(x1 @ W_1.T + b_1) @ W_2.T + b_2)`` in
+    one launch; ``w_o``, ``w_1``, ``w_2`` are packed (``pack_weight``).
+
+    ``attn`` and ``y`` are ``[rows, D]``-shaped (any leading dims); returns ``[rows, D]``."""
+    D = y.shape[-1]
+    a2, y2 = _rows16(attn), _rows16(y)
+    rows = y2.shape[0]
+    out = torch.empty((rows, D), device=y.device, dtype=y.dtype)
+    _lib.check(
+        _lib.load().artab_layer_post(
+            _ptr(a2), a2.stride(0), _ptr(y2), y2.stride(0), _ptr(w_o), _ptr(norm2.weight), _ptr(norm2.bias),
+            float(norm2.eps), _ptr(w_1), _ptr(b_1), _ptr(w_2), _ptr(b_2),
+            _ptr(norm3.weight), _ptr(norm3.bias), float(norm3.eps), _ptr(out), rows, D, w_1.shape[0] * 32,
+            _lib.dtype_code(y.dtype), _lib.current_stream(y.device),
+        )
+    )
+    return out

@@ -110,12 +110,6 @@ class ARTabPFNPredictor:
         """Reset the cursors, keep the memory (inference.py:137-141)."""
         self.seq_len = self.context_len = self.buffer_len = 0
 
-    # ------------------------------------------------------------------ per-layer pieces
-
-    @staticmethod
-    def _qkv(layer, x_row: Tensor):
-        return layer.qkv_heads(x_row)
-
     # ------------------------------------------------------------------ prefill
 
     @torch.no_grad()
@@ -130,8 +124,7 @@ class ARTabPFNPredictor:
         for layer in self.backbone.layers:
             if layer.k_cache.shape[2] < Nc:
                 raise ValueError("KV cache too small for the context; call init_kv_cache with a larger max_seq_len.")
-            x_row = layer.feature_stage(x_row)
-            q, k, v = self._qkv(layer, x_row)
+            x_row, q, k, v = layer.pre_attention(x_row)
             attn = ak.prefill_attention(q, k, v, layer.k_cache, layer.v_cache)
             x_row = layer.finish(x_row, attn)
         self.seq_len = Nc
@@ -147,8 +140,7 @@ class ARTabPFNPredictor:
             if layer.k_ctx_cache.shape[1] != Nc or layer.k_ctx_cache.shape[0] != H:
                 layer.k_ctx_cache = torch.zeros(H, Nc, Dh, device=x_row.device, dtype=x_row.dtype)
                 layer.v_ctx_cache = torch.zeros_like(layer.k_ctx_cache)
-            x_row = layer.feature_stage(x_row)
-            q, k, v = self._qkv(layer, x_row)
+            x_row, q, k, v = layer.pre_attention(x_row)
             attn = ak.prefill_attention(q, k, v, layer.k_ctx_cache, layer.v_ctx_cache)
             x_row = layer.finish(x_row, attn)
         self.context_len = Nc
@@ -188,8 +180,7 @@ class ARTabPFNPredictor:
         B, N, D = x_row.shape
         if N not in (1, 2):
             raise ValueError("Shared-context decode only supports N=1 (target) or N=2 (buffer, target).")
-        x_row = layer.feature_stage(x_row)
-        q, k_new, v_new = self._qkv(layer, x_row)
+        x_row, q, k_new, v_new = layer.pre_attention(x_row)
         k_ctx = layer.k_ctx_cache[:, : self.context_len]
         v_ctx = layer.v_ctx_cache[:, : self.context_len]
         # with a device-side length the host value is only the bound that is validated
@@ -208,8 +199,7 @@ class ARTabPFNPredictor:
         """One layer on the full per-dataset cache (inference.py:687-744): the new K/V are
         written at ``[cache_start, cache_start+N)`` and the queries attend under ``mask``."""
         B, N, D = x_row.shape
-        x_row = layer.feature_stage(x_row)
-        q, k_new, v_new = self._qkv(layer, x_row)
+        x_row, q, k_new, v_new = layer.pre_attention(x_row)
         if layer.k_cache.shape[2] < cache_start + N:
             raise ValueError("KV cache exceeded; increase max_seq_len.")
         if isinstance(mask, TeacherForcingMask):
@@ -417,8 +407,7 @@ class ARTabPFNPredictor:
         B, N, D = x_row.shape
         if N != 2 * num_targets:
             raise ValueError("Expected N == 2*num_targets for teacher forcing.")
-        x_row = layer.feature_stage(x_row)
-        q, k, v = self._qkv(layer, x_row)
+        x_row, q, k, v = layer.pre_attention(x_row)
         attn = ak.hybrid_teacher_forcing_attention(
             q, layer.k_ctx_cache[:, : self.context_len], layer.v_ctx_cache[:, : self.context_len],
             k[:, :, :num_targets], v[:, :, :num_targets], num_targets,

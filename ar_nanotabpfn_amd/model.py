@@ -23,7 +23,7 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from .attention import DenseMask, MultiheadAttention
-from .glue import add_layer_norm, bias_gelu
+from .glue import add_layer_norm, bias_gelu, layer_fusable, layer_post, layer_pre, pack_weight
 
 __all__ = ["Embedder", "TwoStageTransformerLayer", "TwoStageTransformer", "MixtureGaussianHead", "ARTabPFN"]
 
@@ -115,12 +115,47 @@ class TwoStageTransformerLayer(nn.Module):
         qkv = F.linear(x_row, w_qkv).view(B, N, 3, a.n_heads, a.head_dim)
         return qkv[:, :, 0].transpose(1, 2), qkv[:, :, 1].transpose(1, 2), qkv[:, :, 2].transpose(1, 2)
 
+    def packed_weights(self):
+        """The five matrices of the layer in the operand order of the fused kernels
+        (``pack_weight``), rebuilt when a source weight changes:
+        ``(w_fo, w_qkv, out_proj, ff[0], ff[2])``."""
+        w_fo, w_qkv = self.fused_weights()
+        srcs = (w_fo, w_qkv, self.attn_rows.out_proj.weight, self.ff[0].weight, self.ff[2].weight)
+        key = tuple((p.data_ptr(), p._version, p.dtype, p.device) for p in srcs)
+        cached = getattr(self, "_packed_cache", None)
+        if cached is None or cached[0] != key:
+            cached = (key, tuple(pack_weight(p) for p in srcs))
+            self._packed_cache = cached
+        return cached[1]
+
+    def _fusable(self, x_row: Tensor) -> bool:
+        return layer_fusable(x_row, x_row.shape[-1], self.ff[0].out_features)
+
+    def pre_attention(self, x_row: Tensor):
+        """Everything before the row-attention call: ``(y, q, k, v)`` with ``y`` the normed
+        feature stage ``[B,N,D]`` and q, k, v ``[B,H,N,Dh]`` views of one ``[B,N,3D]`` tensor.
+        One launch where the fused kernel covers the layer, otherwise two GEMMs and norm1."""
+        if not self._fusable(x_row):
+            y = self.feature_stage(x_row)
+            return (y,) + tuple(self.qkv_heads(y))
+        p_fo, p_qkv = self.packed_weights()[:2]
+        B, N, D = x_row.shape
+        a = self.attn_rows
+        y, qkv = layer_pre(x_row, p_fo, self.norm1, p_qkv)
+        qkv = qkv.view(B, N, 3, a.n_heads, a.head_dim)
+        return (y.view(B, N, D), qkv[:, :, 0].transpose(1, 2), qkv[:, :, 1].transpose(1, 2),
+                qkv[:, :, 2].transpose(1, 2))
+
     def finish(self, x_row: Tensor, attn_heads: Tensor) -> Tensor:
         """``out_proj`` on ``[B,H,N,Dh]`` attention output, then norm2 / FFN / norm3
-        (inference.py:825-831)."""
+        (inference.py:825-831); one launch where the fused kernel covers the layer."""
         B, H, N, Dh = attn_heads.shape
         D = H * Dh
         attn2d = attn_heads.transpose(1, 2).reshape(B * N, D)
+        if self._fusable(x_row):
+            p_o, p_1, p_2 = self.packed_weights()[2:]
+            return layer_post(attn2d, x_row, p_o, self.norm2, p_1, self.ff[0].bias, p_2, self.ff[2].bias,
+                              self.norm3).view(B, N, D)
         x_row = add_layer_norm(x_row, torch.mm(attn2d, self.attn_rows.out_proj.weight.t()).view(B, N, D), None, self.norm2)
         return self.feed_forward(x_row)
 

@@ -215,6 +215,40 @@ int artab_add_layernorm(const void *x, int64_t ldx, const void *y, int64_t ldy, 
 int artab_bias_gelu(const void *x, int64_t ldx, const void *bias, void *out,
                     int64_t rows, int D, int dtype, void *stream);
 
+/*
+ * The whole non-attention part of one layer of the cached decode / teacher-forcing pass
+ * (ar_tabpfn/model/inference.py:771-789 before the attention call, :825-831 after it) in two
+ * launches.  bf16 / fp16 only; D and F (feed-forward width) in {128, 256, 512}; anything else
+ * returns ARTAB_ERR_UNSUPPORTED and the caller composes the layer from GEMMs and the two
+ * kernels above.  Projections carry no bias, as in ar_tabpfn/model/attention.py:23-26.
+ *
+ * Weights are constants of the model, so they are handed over pre-packed in the order the
+ * matrix cores consume them: artab_pack_linear_weight turns a torch.nn.Linear weight W [N, K]
+ * (row-major, contiguous, N % 32 == 0, K % 16 == 0) into [N/32][K/16][64][8] with
+ *   packed[blk][ks][lane][e] = W[32*blk + lane%32][16*ks + 8*(lane/32) + e]
+ * (same dtype, same number of elements; `packed` must not alias `w`).  Pack once per weight.
+ *
+ *   artab_layer_pre:   y   = LayerNorm1(x + x w_fo^T)        w_fo = pack(out_proj.weight @ v_proj.weight)
+ *                      qkv = y w_qkv^T                       of the single-column feature attention,
+ *                                                            w_qkv = pack([q_proj; k_proj; v_proj].weight)
+ *                      x [rows, D] (row stride ldx), y [rows, D] and qkv [rows, 3D] contiguous.
+ *   artab_layer_post:  x1  = LayerNorm2(y + attn w_o^T)
+ *                      out = LayerNorm3(x1 + gelu(x1 w_1^T + b_1) w_2^T + b_2)
+ *                      attn [rows, D] (row stride lda), y [rows, D] (row stride ldy),
+ *                      out [rows, D] contiguous; w_o, w_1, w_2 packed; b_1, b_2 may be NULL.
+ * Accumulation, residual sums and LayerNorm statistics are float32; the intermediates x1 and
+ * gelu(...) are rounded to the storage dtype once, as operands of the next product.
+ */
+int artab_pack_linear_weight(const void *w, void *packed, int N, int K, int dtype, void *stream);
+int artab_layer_pre(const void *x, int64_t ldx, const void *w_fo, const void *ln1_gamma, const void *ln1_beta,
+                    float eps1, const void *w_qkv, void *y, void *qkv,
+                    int64_t rows, int D, int dtype, void *stream);
+int artab_layer_post(const void *attn, int64_t lda, const void *y, int64_t ldy, const void *w_o,
+                     const void *ln2_gamma, const void *ln2_beta, float eps2,
+                     const void *w_1, const void *b_1, const void *w_2, const void *b_2,
+                     const void *ln3_gamma, const void *ln3_beta, float eps3, void *out,
+                     int64_t rows, int D, int F, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

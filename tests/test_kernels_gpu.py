@@ -483,3 +483,132 @@ def test_bias_gelu_matches_torch(device, dtype, rows, D):
     assert max_abs(to_np(out), ref.numpy()) <= tol
     out2 = bias_gelu(x.to(device), None)
     assert max_abs(to_np(out2), torch.nn.functional.gelu(x.double()).numpy()) <= tol
+
+
+# ----- whole-layer fusions ------------------------------------------------------------------------------
+
+
+def _ln64(t, norm):
+    return torch.nn.functional.layer_norm(t, (t.shape[-1],), norm.weight.detach().cpu().double(),
+                                          norm.bias.detach().cpu().double(), norm.eps)
+
+
+def _mk_norm(D, seed, dtype):
+    norm = torch.nn.LayerNorm(D)
+    with torch.no_grad():
+        norm.weight.copy_(randn((D,), seed, torch.float32) * 0.2 + 1)
+        norm.bias.copy_(randn((D,), seed + 1, torch.float32) * 0.2)
+    return norm.to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,D", [(1, 128), (33, 128), (2048, 256), (70, 512)])
+def test_layer_pre_matches_float64(device, dtype, rows, D):
+    """y = LN1(x + x Wfo^T), qkv = y Wqkv^T against float64 on the same bits; the reference
+    chain rounds y to the storage dtype before the second product, as the kernel does."""
+    from ar_nanotabpfn_amd.glue import layer_pre, pack_weight
+
+    x = randn((rows, D), 1, dtype, 1.5)
+    w_fo = randn((D, D), 2, dtype, D ** -0.5)
+    w_qkv = randn((3 * D, D), 3, dtype, D ** -0.5)
+    norm = _mk_norm(D, 4, dtype)
+    y, qkv = layer_pre(x.to(device), pack_weight(w_fo.to(device)), norm.to(device), pack_weight(w_qkv.to(device)))
+    y_ref = _ln64(x.double() + x.double() @ w_fo.double().t(), norm)
+    qkv_ref = y_ref.to(dtype).double() @ w_qkv.double().t()
+    assert y.shape == (rows, D) and qkv.shape == (rows, 3 * D) and y.dtype == dtype
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    assert max_abs(to_np(y), y_ref.numpy()) <= 1.02 * ulp * max(1.0, float(y_ref.abs().max()))
+    # a flipped rounding of one y element moves a qkv entry by at most ulp*|y|*|w|; allow a few
+    assert max_abs(to_np(qkv), qkv_ref.numpy()) <= 2 * ulp * max(1.0, float(qkv_ref.abs().max()))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,D,F,with_bias", [(1, 128, 256, True), (33, 128, 128, False), (2048, 256, 256, True),
+                                               (70, 512, 256, True), (40, 256, 512, True), (5, 512, 512, False)])
+def test_layer_post_matches_float64(device, dtype, rows, D, F, with_bias):
+    """x1 = LN2(y + attn Wo^T); out = LN3(x1 + gelu(x1 W1^T + b1) W2^T + b2) against float64
+    with the kernel's two intermediate roundings."""
+    from ar_nanotabpfn_amd.glue import layer_post, pack_weight
+
+    attn = randn((rows, D), 1, dtype)
+    y = randn((rows, D), 2, dtype, 1.5)
+    w_o = randn((D, D), 3, dtype, D ** -0.5)
+    lin1, lin2 = torch.nn.Linear(D, F, bias=with_bias), torch.nn.Linear(F, D, bias=with_bias)
+    with torch.no_grad():
+        lin1.weight.copy_(randn((F, D), 4, torch.float32, D ** -0.5))
+        lin2.weight.copy_(randn((D, F), 5, torch.float32, F ** -0.5))
+        if with_bias:
+            lin1.bias.copy_(randn((F,), 6, torch.float32, 0.3))
+            lin2.bias.copy_(randn((D,), 7, torch.float32, 0.3))
+    lin1, lin2 = lin1.to(dtype), lin2.to(dtype)
+    n2, n3 = _mk_norm(D, 8, dtype), _mk_norm(D, 10, dtype)
+    lin1, lin2 = lin1.to(device), lin2.to(device)
+    out = layer_post(attn.to(device), y.to(device), pack_weight(w_o.to(device)), n2.to(device),
+                     pack_weight(lin1.weight), lin1.bias, pack_weight(lin2.weight), lin2.bias, n3.to(device))
+    d = lambda t: t.detach().cpu().double()  # noqa: E731
+    x1 = _ln64(y.double() + attn.double() @ w_o.double().t(), n2)
+    x1r = x1.to(dtype).double()
+    h = x1r @ d(lin1.weight).t() + (d(lin1.bias) if with_bias else 0)
+    hr = torch.nn.functional.gelu(h).to(dtype).double()
+    # the residual entering LN3 is the rounded copy of x1 staged for the product
+    ref = _ln64(x1r + hr @ d(lin2.weight).t() + (d(lin2.bias) if with_bias else 0), n3)
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    assert out.shape == (rows, D) and out.dtype == dtype
+    assert max_abs(to_np(out), ref.numpy()) <= 3 * ulp * max(1.0, float(ref.abs().max()))
+
+
+def test_layer_fusion_strided_inputs_and_errors(device):
+    """attn given as the [B,N,H,Dh]-backed view the attention kernels return, x as a column
+    slice; unsupported widths and dtypes raise."""
+    from ar_nanotabpfn_amd.glue import layer_fusable, layer_pre, pack_weight
+
+    dtype, D = torch.bfloat16, 256
+    wide = randn((96, 2 * D), 1, dtype).to(device)
+    x = wide[:, D:]
+    w_fo = pack_weight(randn((D, D), 2, dtype, D ** -0.5).to(device))
+    w_qkv = pack_weight(randn((3 * D, D), 3, dtype, D ** -0.5).to(device))
+    norm = _mk_norm(D, 4, dtype).to(device)
+    y, qkv = layer_pre(x, w_fo, norm, w_qkv)
+    y2, qkv2 = layer_pre(x.contiguous(), w_fo, norm, w_qkv)
+    assert torch.equal(y, y2) and torch.equal(qkv, qkv2)
+    assert not layer_fusable(x, 96, 256) and not layer_fusable(x.float(), 256, 256) and layer_fusable(x, 256, 512)
+    assert not layer_fusable(x.cpu(), 256, 256)
+    with pytest.raises((ValueError, RuntimeError)):
+        layer_pre(randn((4, 96), 1, dtype).to(device), randn((96, 96), 2, dtype).to(device),
+                  torch.nn.LayerNorm(96).to(device=device, dtype=dtype), randn((288, 96), 3, dtype).to(device))
+    with pytest.raises((ValueError, RuntimeError)):
+        layer_pre(x.float(), w_fo.float(), norm.float(), w_qkv.float())
+    with pytest.raises((ValueError, RuntimeError)):
+        pack_weight(randn((40, 64), 1, dtype).to(device))  # N % 32 != 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("N,K", [(32, 16), (768, 256), (256, 512)])
+def test_pack_weight_layout(device, dtype, N, K):
+    """packed[blk][ks][lane][e] = W[32*blk + lane%32][16*ks + 8*(lane/32) + e], bit-exact."""
+    from ar_nanotabpfn_amd.glue import pack_weight
+
+    w = randn((N, K), 1, dtype)
+    packed = pack_weight(w.to(device)).cpu()
+    ref = w.view(N // 32, 32, K // 16, 2, 8).permute(0, 2, 3, 1, 4).reshape(N // 32, K // 16, 64, 8)
+    assert packed.shape == ref.shape and torch.equal(packed, ref)
+
+
+@pytest.mark.parametrize("D,F,H", [(128, 256, 4), (256, 256, 8), (512, 256, 16)])
+def test_layer_fused_equals_unfused_composition(device, monkeypatch, D, F, H):
+    """TwoStageTransformerLayer.pre_attention / finish: the two-launch path against the path
+    composed from GEMMs and the row-wise kernels, same weights, bf16 tolerance."""
+    from ar_nanotabpfn_amd import model as m
+
+    torch.manual_seed(0)
+    layer = m.TwoStageTransformerLayer(D, H, F).to(device=device, dtype=torch.bfloat16)
+    x = randn((64, 2, D), 1, torch.bfloat16, 1.0).to(device)
+    attn = randn((64, 2, H, D // H), 2, torch.bfloat16).to(device).transpose(1, 2)
+    y_f, q_f, k_f, v_f = layer.pre_attention(x)
+    out_f = layer.finish(y_f, attn)
+    monkeypatch.setattr(m, "layer_fusable", lambda *a: False)
+    y_u, q_u, k_u, v_u = layer.pre_attention(x)
+    out_u = layer.finish(y_u, attn)
+    for a, b in ((y_f, y_u), (q_f, q_u), (k_f, k_u), (v_f, v_u), (out_f, out_u)):
+        assert a.shape == b.shape
+        assert max_abs(to_np(a), to_np(b)) <= 4e-2  # two 16-bit chains with different rounding points
