@@ -42,6 +42,25 @@ class ArtabView(ctypes.Structure):
 _VP = ctypes.POINTER(ArtabView)
 _i, _f, _p, _sz, _i64 = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int64
 
+
+class ArtabSampleEmbedArgs(ctypes.Structure):
+    """``artab_sample_embed_args`` of include/artab_attention.h, field for field."""
+
+    _fields_ = [
+        ("x_last", _p), ("ld_row", _i64),
+        ("norm_gamma", _p), ("norm_beta", _p), ("eps", _f),
+        ("w_h1", _p), ("b_h1", _p), ("w_h2", _p), ("b_h2", _p),
+        ("mean_bias", _p), ("std_bias", _p), ("weight_bias", _p),
+        ("K", _i), ("std_min", _f), ("std_max", _f),
+        ("rand_u", _p), ("rand_n", _p), ("x_mean", _p),
+        ("w_x", _p), ("b_x", _p), ("w_y", _p), ("b_y", _p),
+        ("markers", _p), ("ar_tokens", _p), ("bs", _i),
+        ("step", _p), ("Nt", _i),
+        ("preds", _p), ("emb_next", _p),
+        ("B", _i), ("D", _i), ("F", _i),
+    ]
+
+
 # name -> (restype, argtypes); every symbol declared in include/artab_attention.h
 SIGNATURES = {
     "artab_version": (_i, []),
@@ -63,6 +82,7 @@ SIGNATURES = {
     "artab_bias_gelu": (_i, [_p, _i64, _p, _p, _i64, _i, _i, _p]),
     "artab_pack_linear_weight": (_i, [_p, _p, _i, _i, _i, _p]),
     "artab_layer_pre": (_i, [_p, _i64, _p, _p, _p, _f, _p, _p, _p, _i64, _i, _i, _p]),
+    "artab_decode_sample_embed": (_i, [ctypes.POINTER(ArtabSampleEmbedArgs), _i, _p]),
     "artab_layer_post": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _f, _p, _i64, _i, _i, _i, _p]),
 }
 

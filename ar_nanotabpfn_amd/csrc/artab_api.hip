@@ -332,6 +332,26 @@ hipError_t launch_post(const FusedPostParams &P, int D, int F, hipStream_t st) {
     }
 }
 
+template <typename T, int D>
+hipError_t launch_sample_d(const SampleEmbedParams &P, int F, hipStream_t st) {
+    dim3 grid(static_cast<unsigned>((P.B + kFusedRows - 1) / kFusedRows)), block(fused_waves(D) * 64);
+    switch (F) {
+        case 128: hipLaunchKernelGGL((sample_embed_kernel<T, D, 128>), grid, block, 0, st, P); break;
+        case 256: hipLaunchKernelGGL((sample_embed_kernel<T, D, 256>), grid, block, 0, st, P); break;
+        default: hipLaunchKernelGGL((sample_embed_kernel<T, D, 512>), grid, block, 0, st, P); break;
+    }
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_sample(const SampleEmbedParams &P, int D, int F, hipStream_t st) {
+    switch (D) {
+        case 128: return launch_sample_d<T, 128>(P, F, st);
+        case 256: return launch_sample_d<T, 256>(P, F, st);
+        default: return launch_sample_d<T, 512>(P, F, st);
+    }
+}
+
 bool fused_width_ok(int n) { return n == 128 || n == 256 || n == 512; }
 bool misaligned16(const void *p) { return p && reinterpret_cast<uintptr_t>(p) % 16 != 0; }
 
@@ -837,6 +857,39 @@ int artab_layer_post(const void *attn, int64_t lda, const void *y, int64_t ldy, 
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipError_t e = dtype == ARTAB_BF16 ? launch_post<bf16_t>(P, D, F, st) : launch_post<f16_t>(P, D, F, st);
     return launch_status(e, "layer_post");
+}
+
+int artab_decode_sample_embed(const artab_sample_embed_args *a, int dtype, void *stream) {
+    if (!a) return fail(ARTAB_ERR_NULL_POINTER, "args is NULL");
+    if (dtype != ARTAB_BF16 && dtype != ARTAB_F16)
+        return fail(ARTAB_ERR_UNSUPPORTED, "decode_sample_embed supports bf16 and fp16 only (dtype code %d)", dtype);
+    if (a->B < 0 || a->Nt <= 0 || a->K <= 0 || a->bs <= 0)
+        return fail(ARTAB_ERR_BAD_SHAPE, "bad sizes B=%d Nt=%d K=%d bs=%d", a->B, a->Nt, a->K, a->bs);
+    if (!fused_width_ok(a->D) || !fused_width_ok(a->F) || a->K > kMaxMixture)
+        return fail(ARTAB_ERR_UNSUPPORTED, "decode_sample_embed needs D, F in {128, 256, 512} and K <= %d (got %d, %d, %d)",
+                    kMaxMixture, a->D, a->F, a->K);
+    if (a->B == 0) return ARTAB_OK;
+    if (!a->x_last || !a->norm_gamma || !a->norm_beta || !a->w_h1 || !a->w_h2 || !a->mean_bias || !a->std_bias ||
+        !a->weight_bias || !a->rand_u || !a->rand_n || !a->x_mean || !a->w_x || !a->b_x || !a->w_y || !a->b_y ||
+        !a->markers || !a->ar_tokens || !a->step || !a->preds || !a->emb_next)
+        return fail(ARTAB_ERR_NULL_POINTER, "decode_sample_embed: only b_h1 and b_h2 may be NULL");
+    if (misaligned16(a->x_last) || misaligned16(a->w_h1) || misaligned16(a->w_h2) || misaligned16(a->b_h1) ||
+        misaligned16(a->b_h2) || misaligned16(a->norm_gamma) || misaligned16(a->norm_beta) || misaligned16(a->w_x) ||
+        misaligned16(a->b_x) || misaligned16(a->w_y) || misaligned16(a->b_y) || misaligned16(a->markers) ||
+        misaligned16(a->ar_tokens) || misaligned16(a->emb_next) || a->ld_row % 8 || a->ld_row < a->D)
+        return fail(ARTAB_ERR_BAD_STRIDE, "decode_sample_embed: model vectors and rows must be 16-byte aligned");
+    SampleEmbedParams P;
+    P.x_last = a->x_last; P.ld_row = a->ld_row; P.norm_g = a->norm_gamma; P.norm_b = a->norm_beta; P.eps = a->eps;
+    P.w_h1 = a->w_h1; P.b_h1 = a->b_h1; P.w_h2 = a->w_h2; P.b_h2 = a->b_h2;
+    P.mean_bias = a->mean_bias; P.std_bias = a->std_bias; P.weight_bias = a->weight_bias;
+    P.K = a->K; P.std_min = a->std_min; P.std_max = a->std_max;
+    P.rand_u = a->rand_u; P.rand_n = a->rand_n; P.x_mean = a->x_mean;
+    P.w_x = a->w_x; P.b_x = a->b_x; P.w_y = a->w_y; P.b_y = a->b_y; P.markers = a->markers;
+    P.ar_tokens = a->ar_tokens; P.bs = a->bs; P.step = a->step; P.Nt = a->Nt;
+    P.preds = a->preds; P.emb = a->emb_next; P.B = a->B;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipError_t e = dtype == ARTAB_BF16 ? launch_sample<bf16_t>(P, a->D, a->F, st) : launch_sample<f16_t>(P, a->D, a->F, st);
+    return launch_status(e, "decode_sample_embed");
 }
 
 }  // extern "C"

@@ -398,4 +398,206 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_kernel(FusedPo
     unstage_tile<T, D, NT>(static_cast<T *>(P.out) + row0 * D, D, a0, LDD, valid, tid);
 }
 
+// ---- end of a decode step: final norm + mixture head + one sample per trajectory + the
+// embedding of the next step's [buffer, target] rows, in one launch.
+//
+// Replaces, for dim_y = 1, the chain  backbone.norm -> head MLP -> mixture parameters ->
+// component pick -> normal draw -> write the prediction -> embed (x_t, y_t) as the next buffer
+// row and x_{t+1} as the next target row.  The uniform and normal variates come from the
+// caller (one pair per trajectory and step), the step index from device memory, so that the
+// whole sampling loop can be replayed from one recorded graph.
+struct SampleEmbedParams {
+    const void *x_last; long ld_row;  // target row of trajectory b at x_last + b * ld_row, [D]
+    const void *norm_g, *norm_b; float eps;
+    const void *w_h1, *b_h1;          // head layer 1: packed [F, D], [F]
+    const void *w_h2, *b_h2;          // head layer 2 padded to 32 outputs: packed [32, F], [32]
+    const void *mean_bias, *std_bias, *weight_bias;  // [K]
+    int K; float std_min, std_max;
+    const float *rand_u, *rand_n;     // [Nt, B] uniform [0,1) / standard normal
+    const void *x_mean;               // [B, Nt] feature mean of every target row
+    const void *w_x, *b_x, *w_y, *b_y;  // embedder: Linear(1, D) weights as [D] vectors
+    const void *markers;              // [3, D]: target, context, buffer
+    const void *ar_tokens; int bs;    // [bs, D]
+    const int *step;                  // device-side index t of the target being sampled
+    int Nt;
+    void *preds;                      // [B, Nt]
+    void *emb;                        // [B, 2, D] rows of step t + 1
+    int B;
+};
+
+constexpr int kMaxMixture = 10;  // 3 * K outputs must fit one 32-column block
+
+template <typename T, int D, int F>
+__global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(SampleEmbedParams P) {
+    constexpr int NW = fused_waves(D), NT = NW * 64;
+    constexpr int LDD = D + 8, LDF = F + 8;
+    constexpr int NBF = (F / 32 + NW - 1) / NW;
+    constexpr int EPL = D / 64;  // elements per lane of one row in the row-wise norm
+    static_assert(F / 32 >= NW ? (F / 32) % NW == 0 : true, "unsupported widths");
+    __shared__ __attribute__((aligned(16))) T a0[kFusedRows * LDD];  // z = norm(x_last)
+    __shared__ __attribute__((aligned(16))) T a1[kFusedRows * LDF];  // gelu(head layer 1)
+    __shared__ float raw_s[kFusedRows][33];
+    __shared__ float y_s[kFusedRows];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hb = lane >> 5;
+    const int t = *P.step;
+    if (t < 0 || t >= P.Nt) return;  // uniform over the grid
+    const long row0 = static_cast<long>(blockIdx.x) * kFusedRows;
+    const int valid = static_cast<int>(min(static_cast<long>(kFusedRows), P.B - row0));
+
+    int nbf[NBF];
+#pragma unroll
+    for (int b = 0; b < NBF; ++b) nbf[b] = wave + NW * b;
+    const int nb0[1] = {0};
+    const bool ff_active = wave < F / 32;
+    WeightStream<T, D, NBF> w_1;
+    WeightStream<T, F, 1> w_2;
+    if (ff_active) w_1.start(static_cast<const T *>(P.w_h1), nbf, lane);
+    if (wave == 0) w_2.start(static_cast<const T *>(P.w_h2), nb0, lane);
+    stage_tile<T, D, NT>(a0, LDD, static_cast<const T *>(P.x_last) + row0 * P.ld_row, P.ld_row, valid, tid);
+    __syncthreads();
+
+    // ---- z = LayerNorm(x_last), one wavefront per row, in place
+    {
+        float gam[EPL], bet[EPL];
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            gam[e] = to_f32(static_cast<const T *>(P.norm_g)[lane * EPL + e]);
+            bet[e] = to_f32(static_cast<const T *>(P.norm_b)[lane * EPL + e]);
+        }
+        for (int r = wave; r < kFusedRows; r += NW) {
+            T *row = a0 + r * LDD + lane * EPL;
+            float x[EPL], sum = 0.f;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                x[e] = to_f32(row[e]);
+                sum += x[e];
+            }
+            const float mean = wave_sum(sum) / D;
+            float q = 0.f;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) q += (x[e] - mean) * (x[e] - mean);
+            const float rstd = rsqrtf(wave_sum(q) / D + P.eps);
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) row[e] = from_f32<T>((x[e] - mean) * rstd * gam[e] + bet[e]);
+        }
+    }
+    __syncthreads();
+
+    // ---- h = gelu(z W_h1^T + b_h1) -> a1
+    if (ff_active) {
+        float bias[NBF][16];
+        load_cols<T, NBF>(P.b_h1 ? static_cast<const T *>(P.b_h1) : reinterpret_cast<const T *>(kZeroVector), nbf, hb,
+                          bias);
+        f32x16 acc[NBF];
+        w_1.run(acc, a0, LDD, c, hb);
+#pragma unroll
+        for (int b = 0; b < NBF; ++b)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float v = acc[b][4 * g + e] + bias[b][4 * g + e];
+                    o[e] = 0.5f * v * (1.f + erff(v * 0.70710678118654752f));
+                }
+                store4f<T>(a1 + c * LDF + col_of(nbf[b], 4 * g, hb), o[0], o[1], o[2], o[3]);
+            }
+    }
+    __syncthreads();
+
+    // ---- raw = h W_h2^T + b_h2 (one 32-column block, first wavefront), kept in float32
+    if (wave == 0) {
+        float bias[1][16];
+        load_cols<T, 1>(P.b_h2 ? static_cast<const T *>(P.b_h2) : reinterpret_cast<const T *>(kZeroVector), nb0, hb, bias);
+        f32x16 acc[1];
+        w_2.run(acc, a1, LDF, c, hb);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) raw_s[c][col_of(0, v, hb)] = acc[0][v] + bias[0][v];
+    }
+    __syncthreads();
+
+    // ---- one sample per trajectory: component by inverse CDF of the softmax weights, then a normal
+    if (tid < kFusedRows) {
+        float y = 0.f;
+        if (tid < valid) {
+            const long row = row0 + tid;
+            const T *mb = static_cast<const T *>(P.mean_bias), *sb = static_cast<const T *>(P.std_bias),
+                    *wb = static_cast<const T *>(P.weight_bias);
+            float logit[kMaxMixture], mx = -INFINITY;
+#pragma unroll
+            for (int k = 0; k < kMaxMixture; ++k)
+                if (k < P.K) {
+                    logit[k] = raw_s[tid][3 * k + 2] + to_f32(wb[k]);
+                    mx = fmaxf(mx, logit[k]);
+                }
+            float z = 0.f;
+#pragma unroll
+            for (int k = 0; k < kMaxMixture; ++k)
+                if (k < P.K) {
+                    logit[k] = expf(logit[k] - mx);
+                    z += logit[k];
+                }
+            const float target = P.rand_u[static_cast<long>(t) * P.B + row] * z;
+            int comp = P.K - 1;
+            float cum = 0.f;
+            bool found = false;
+#pragma unroll
+            for (int k = 0; k < kMaxMixture; ++k)
+                if (k < P.K) {
+                    cum += logit[k];
+                    if (!found && cum > target) {
+                        comp = k;
+                        found = true;
+                    }
+                }
+            const float mean = raw_s[tid][3 * comp] + to_f32(mb[comp]);
+            const float sraw = raw_s[tid][3 * comp + 1] + to_f32(sb[comp]);
+            const float sp = sraw > 20.f ? sraw : log1pf(expf(sraw));
+            const float sd = fminf(sp, P.std_max) + P.std_min;
+            const T yr = from_f32<T>(mean + sd * P.rand_n[static_cast<long>(t) * P.B + row]);
+            static_cast<T *>(P.preds)[row * P.Nt + t] = yr;
+            y = to_f32(yr);
+        }
+        y_s[tid] = y;
+    }
+    __syncthreads();
+
+    // ---- embedding of step t + 1: row 0 = buffer(x_t, y_t) + ar_token[(t + 1) % bs], row 1 = target(x_{t+1})
+    {
+        const T *wx = static_cast<const T *>(P.w_x), *bx = static_cast<const T *>(P.b_x);
+        const T *wy = static_cast<const T *>(P.w_y), *by = static_cast<const T *>(P.b_y);
+        const T *mk = static_cast<const T *>(P.markers);
+        const T *tok = static_cast<const T *>(P.ar_tokens) + static_cast<long>((t + 1) % P.bs) * D;
+        const T *xm = static_cast<const T *>(P.x_mean);
+        const int tn = min(t + 1, P.Nt - 1);
+        constexpr int CPR = D / 8;
+        for (int idx = tid; idx < kFusedRows * 2 * CPR; idx += NT) {
+            const int ch = idx % CPR, which = (idx / CPR) & 1, r = idx / (2 * CPR);
+            if (r >= valid) continue;
+            const long row = row0 + r;
+            float fwx[8], fbx[8], o[8];
+            load4f<T>(wx + 8 * ch, fwx); load4f<T>(wx + 8 * ch + 4, fwx + 4);
+            load4f<T>(bx + 8 * ch, fbx); load4f<T>(bx + 8 * ch + 4, fbx + 4);
+            if (which == 0) {
+                const float xv = to_f32(xm[row * P.Nt + t]), yv = y_s[r];
+                float fwy[8], fby[8], fm[8], ft[8];
+                load4f<T>(wy + 8 * ch, fwy); load4f<T>(wy + 8 * ch + 4, fwy + 4);
+                load4f<T>(by + 8 * ch, fby); load4f<T>(by + 8 * ch + 4, fby + 4);
+                load4f<T>(mk + 2 * D + 8 * ch, fm); load4f<T>(mk + 2 * D + 8 * ch + 4, fm + 4);
+                load4f<T>(tok + 8 * ch, ft); load4f<T>(tok + 8 * ch + 4, ft + 4);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = xv * fwx[e] + fbx[e] + yv * fwy[e] + fby[e] + fm[e] + ft[e];
+            } else {
+                const float xv = to_f32(xm[row * P.Nt + tn]);
+                float fm[8];
+                load4f<T>(mk + 8 * ch, fm); load4f<T>(mk + 8 * ch + 4, fm + 4);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = xv * fwx[e] + fbx[e] + fm[e];
+            }
+            u32x4 val = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
+            *reinterpret_cast<u32x4 *>(static_cast<T *>(P.emb) + (row * 2 + which) * D + 8 * ch) = val;
+        }
+    }
+}
+
 }  // namespace artab

@@ -19,7 +19,7 @@ from torch import Tensor, nn
 
 from . import _lib
 
-__all__ = ["add_layer_norm", "bias_gelu", "layer_fusable", "pack_weight", "layer_pre", "layer_post"]
+__all__ = ["add_layer_norm", "bias_gelu", "layer_fusable", "pack_weight", "layer_pre", "layer_post", "SampleEmbedStep"]
 
 
 def _rows2d(t: Tensor) -> Tensor:
@@ -138,3 +138,78 @@ def layer_post(attn: Tensor, y: Tensor, w_o: Tensor, norm2: nn.LayerNorm, w_1: T
         )
     )
     return out
+
+
+class SampleEmbedStep:
+    """The tail of a decode step as one launch (``artab_decode_sample_embed``): final norm,
+    mixture head, one draw per trajectory, prediction write, embedding of the next
+    ``[buffer, target]`` pair.  Built once per (model, batch, targets); ``__call__`` only
+    launches, so it can be recorded into a graph.
+
+    ``x_mean [B,Nt]``: feature mean of every target row; ``rand_u``/``rand_n [Nt,B]`` float32
+    variates (refilled by the caller before each sampling run); ``step``: int32 device scalar;
+    ``preds [B,Nt]``; ``emb [B,2,D]``.
+    """
+
+    MAX_COMPONENTS = 10
+
+    @staticmethod
+    def supported(embedder, backbone, head, x: Tensor) -> bool:
+        D = backbone.norm.normalized_shape[0]
+        lin1, lin2 = head.head[0], head.head[2]
+        return (layer_fusable(x, D, lin1.out_features) and head.dim_y == 1
+                and head.num_components <= SampleEmbedStep.MAX_COMPONENTS
+                and lin2.out_features == 3 * head.num_components)
+
+    def __init__(self, embedder, backbone, head, ar_tokens: Tensor, x_mean: Tensor, rand_u: Tensor, rand_n: Tensor,
+                 step: Tensor, preds: Tensor, emb: Tensor):
+        lin1, lin2 = head.head[0], head.head[2]
+        dev, dt = emb.device, emb.dtype
+        B, Nt = preds.shape
+        D, F_ = lin1.in_features, lin1.out_features
+        assert x_mean.shape == (B, Nt) and rand_u.shape == (Nt, B) and rand_n.shape == (Nt, B)
+        assert rand_u.dtype == torch.float32 and rand_n.dtype == torch.float32 and step.dtype == torch.int32
+        assert emb.shape == (B, 2, D) and emb.is_contiguous() and preds.is_contiguous() and x_mean.is_contiguous()
+        w2 = torch.zeros((32, F_), device=dev, dtype=dt)
+        w2[: lin2.out_features] = lin2.weight.detach()
+        b2 = torch.zeros(32, device=dev, dtype=dt)
+        if lin2.bias is not None:
+            b2[: lin2.out_features] = lin2.bias.detach()
+        # everything the launch points at is kept alive here
+        self._keep = dict(
+            w_h1=pack_weight(lin1.weight), w_h2=pack_weight(w2), b_h2=b2,
+            w_x=embedder.x_embed.weight.detach().reshape(-1).contiguous(),
+            w_y=embedder.y_embed.weight.detach().reshape(-1).contiguous(),
+            ar_tokens=ar_tokens.detach().contiguous(), x_mean=x_mean, rand_u=rand_u, rand_n=rand_n, step=step,
+            preds=preds, emb=emb,
+        )
+        k = self._keep
+        self.dtype_code = _lib.dtype_code(dt)
+        self.device = dev
+        a = _lib.ArtabSampleEmbedArgs()
+        a.norm_gamma, a.norm_beta, a.eps = backbone.norm.weight.data_ptr(), backbone.norm.bias.data_ptr(), backbone.norm.eps
+        a.w_h1, a.b_h1 = k["w_h1"].data_ptr(), (lin1.bias.data_ptr() if lin1.bias is not None else None)
+        a.w_h2, a.b_h2 = k["w_h2"].data_ptr(), b2.data_ptr()
+        a.mean_bias, a.std_bias, a.weight_bias = (head.mean_bias.data_ptr(), head.std_bias.data_ptr(),
+                                                  head.weight_bias.data_ptr())
+        a.K, a.std_min, a.std_max = head.num_components, float(head.std_min), 2.0
+        a.rand_u, a.rand_n, a.x_mean = rand_u.data_ptr(), rand_n.data_ptr(), x_mean.data_ptr()
+        a.w_x, a.b_x = k["w_x"].data_ptr(), embedder.x_embed.bias.data_ptr()
+        a.w_y, a.b_y = k["w_y"].data_ptr(), embedder.y_embed.bias.data_ptr()
+        a.markers = embedder.marker_embed.weight.data_ptr()
+        a.ar_tokens, a.bs = k["ar_tokens"].data_ptr(), ar_tokens.shape[0]
+        a.step, a.Nt = step.data_ptr(), Nt
+        a.preds, a.emb_next = preds.data_ptr(), emb.data_ptr()
+        a.B, a.D, a.F = B, D, F_
+        self.args = a
+
+    def __call__(self, x_last: Tensor) -> None:
+        """``x_last [B,2,D]`` (or ``[B,1,D]``): output of the last layer; its last row per
+        trajectory is the target row."""
+        B, N, D = x_last.shape
+        if x_last.stride(2) != 1 or x_last.stride(0) % 8:
+            x_last = x_last.contiguous()
+        tgt = x_last[:, N - 1]
+        self.args.x_last, self.args.ld_row = tgt.data_ptr(), tgt.stride(0)
+        _lib.check(_lib.load().artab_decode_sample_embed(ctypes.byref(self.args), self.dtype_code,
+                                                         _lib.current_stream(self.device)))

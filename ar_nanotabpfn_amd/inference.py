@@ -25,7 +25,7 @@ from torch import Tensor
 
 from . import attention_kernels as ak
 from .attention import DecodeMask, TeacherForcingMask
-from .glue import add_layer_norm
+from .glue import SampleEmbedStep, add_layer_norm
 
 __all__ = ["ARTabPFNPredictor"]
 
@@ -60,6 +60,7 @@ class ARTabPFNPredictor:
         # Replay the decode step of sample_sequence from a recorded HIP graph (shared
         # layout on a HIP device only).  Set to False to launch every kernel from Python.
         self.use_hip_graph = True
+        self.fuse_step_tail = True   # head + draw + next embedding as one launch inside the graph
         self._graph_state = None
 
     @classmethod
@@ -285,27 +286,37 @@ class ARTabPFNPredictor:
     def _graph_step(self, st) -> None:
         """One ``[buffer, target]`` decode step driven entirely by device-side state
         (the body that is recorded): step index ``st.t``, buffer length ``st.nbuf``."""
+        if st.tail is not None:
+            # embedding of this step was left in st.emb by the previous step's tail launch
+            x_row = st.emb
+            for layer in self.backbone.layers:
+                x_row = self._layer_decode_with_cache_shared(layer, x_row, 1, n_buf_device=st.nbuf)
+            st.tail(x_row)          # norm, head, draw, preds[:, t], embedding of step t + 1
+            st.counters.add_(1)     # (t, nbuf)
+            return
         bs = self.ar_tokens.shape[0]
-        x_t = st.x_target.index_select(1, st.t)
-        x_p = st.x_target.index_select(1, st.t - 1)
-        tok = self.ar_tokens.index_select(0, torch.remainder(st.t, bs))  # ar_tokens[t % bs], inference.py:359
+        t = st.t.long()
+        x_t = st.x_target.index_select(1, t)
+        x_p = st.x_target.index_select(1, t - 1)
+        tok = self.ar_tokens.index_select(0, torch.remainder(t, bs))  # ar_tokens[t % bs], inference.py:359
         buffer_emb = self.embedder.embed_buffer(x_p, st.y_prev) + tok
         x_row = torch.cat([buffer_emb, self.embedder.embed_target(x_t)], dim=1)
         for layer in self.backbone.layers:
             x_row = self._layer_decode_with_cache_shared(layer, x_row, 1, n_buf_device=st.nbuf)
         z = add_layer_norm(x_row, None, None, self.backbone.norm)
         y = self.head.sample(z[:, -1:, :])[:, :, 0, 0]
-        st.preds.index_copy_(1, st.t, y)
+        st.preds.index_copy_(1, t, y)
         st.y_prev.copy_(y)
-        st.t.add_(1)
-        st.nbuf.add_(1)
+        st.counters.add_(1)
 
     def _sample_sequence_graph(self, x_target: Tensor) -> Tensor:
         B, Nt, F_ = x_target.shape
         device, dtype = x_target.device, x_target.dtype
         layer0 = self.backbone.layers[0]
+        params = list(self.backbone.parameters()) + list(self.embedder.parameters()) + list(self.head.parameters())
+        params.append(self.ar_tokens)
         key = (B, Nt, F_, self.context_len, dtype, str(device), layer0.k_ctx_cache.data_ptr(),
-               layer0.k_buf_cache.data_ptr(), tuple(p._version for p in self.backbone.parameters()))
+               layer0.k_buf_cache.data_ptr(), self.fuse_step_tail, tuple((p.data_ptr(), p._version) for p in params))
         st = self._graph_state
         if st is None or st.key != key:
             st = _GraphState()
@@ -313,20 +324,37 @@ class ARTabPFNPredictor:
             st.x_target = torch.empty((B, Nt, F_), device=device, dtype=dtype)
             st.y_prev = torch.zeros((B, 1), device=device, dtype=dtype)
             st.preds = torch.zeros((B, Nt), device=device, dtype=dtype)
-            st.t = torch.ones(1, device=device, dtype=torch.long)
-            st.nbuf = torch.zeros(1, device=device, dtype=torch.int32)
+            st.counters = torch.zeros(2, device=device, dtype=torch.int32)  # (step index t, buffer length)
+            st.t, st.nbuf = st.counters[0:1], st.counters[1:2]
             st.graph = None
+            st.tail = None
+            if self.fuse_step_tail and SampleEmbedStep.supported(self.embedder, self.backbone, self.head, x_target):
+                D = self.backbone.d_model
+                st.emb = torch.zeros((B, 2, D), device=device, dtype=dtype)
+                st.x_mean = torch.zeros((B, Nt), device=device, dtype=dtype)
+                st.rand_u = torch.zeros((Nt, B), device=device, dtype=torch.float32)
+                st.rand_n = torch.zeros((Nt, B), device=device, dtype=torch.float32)
+                st.tail = SampleEmbedStep(self.embedder, self.backbone, self.head, self.ar_tokens, st.x_mean,
+                                          st.rand_u, st.rand_n, st.t, st.preds, st.emb)
             self._graph_state = st
         st.x_target.copy_(x_target)
 
         # first target: no buffer row yet (N = 1), launched directly
         y0 = self.autoregressive_decode(st.x_target[:, 0:1, :], None, None, 0)
+        if st.tail is not None:
+            st.x_mean.copy_(st.x_target.mean(dim=-1))
+            self._draw_step_variates(st.rand_u, st.rand_n)
+            bs = self.ar_tokens.shape[0]
+            emb1 = torch.cat([self.embedder.embed_buffer(st.x_target[:, 0:1], y0) + self.ar_tokens[1 % bs],
+                              self.embedder.embed_target(st.x_target[:, 1:2])], dim=1)
 
         def reset():
             st.y_prev.copy_(y0)
             st.preds[:, 0:1] = y0
             st.t.fill_(1)
             st.nbuf.zero_()
+            if st.tail is not None:
+                st.emb.copy_(emb1)
 
         if st.graph is None:
             # warm-up on a side stream (workspace allocation, GEMM heuristics), then record;
@@ -349,6 +377,13 @@ class ARTabPFNPredictor:
         self.buffer_len = Nt - 1
         self.seq_len = self.context_len + self.buffer_len
         return st.preds.clone()
+
+    @staticmethod
+    def _draw_step_variates(rand_u: Tensor, rand_n: Tensor) -> None:
+        """Fresh variates for every (step, trajectory) of one sampling run, from torch's
+        generator: uniform for the component pick, normal for the draw."""
+        rand_u.uniform_()
+        rand_n.normal_()
 
     # ------------------------------------------------------------------ teacher forcing
 

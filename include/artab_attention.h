@@ -249,6 +249,52 @@ int artab_layer_post(const void *attn, int64_t lda, const void *y, int64_t ldy, 
                      const void *ln3_gamma, const void *ln3_beta, float eps3, void *out,
                      int64_t rows, int D, int F, int dtype, void *stream);
 
+/*
+ * The tail of one autoregressive decode step in a single launch: final LayerNorm of the
+ * target rows, the mixture-of-Gaussians head, one draw per trajectory, the write of the
+ * prediction, and the embedding of the next step's [buffer, target] pair.  Replaces, for
+ * dim_y = 1, ar_tabpfn/model/inference.py:278-320 (autoregressive_decode: embed -> decode ->
+ * head.sample), ar_tabpfn/model/model.py:23-76 (embedder) and :150-272 (head parameters and
+ * sampling) between two consecutive runs of the layer stack.
+ *
+ * Sampling follows the reference's law — component k with probability softmax(raw_w + weight_bias)_k,
+ * then Normal(mean_k, std_k) with std_k = min(softplus(raw_s + std_bias), std_max) + std_min —
+ * from caller-supplied variates: component = first k whose cumulative weight exceeds rand_u, and
+ * y = mean_k + std_k * rand_n.  The step index t is read from device memory so the call can sit
+ * in a recorded graph; a t outside [0, Nt) makes the launch a no-op.
+ *
+ * All model tensors are of `dtype` (bf16 / fp16); D and F (head hidden width) in {128, 256, 512};
+ * K <= 10.  w_h1 is the packed [F, D] weight of head layer 1; w_h2 the packed [32, F] weight of
+ * head layer 2 with rows >= 3K zero (output 3k + j: j = 0 mean, 1 std, 2 weight; model.py:195-196)
+ * and b_h2 its bias padded to 32 entries.
+ */
+typedef struct artab_sample_embed_args {
+    const void *x_last;      /* target row of trajectory b at x_last + b * ld_row elements, [D] */
+    int64_t ld_row;
+    const void *norm_gamma, *norm_beta; /* backbone.norm */
+    float eps;
+    const void *w_h1, *b_h1; /* head.head.0 (packed), bias [F] or NULL */
+    const void *w_h2, *b_h2; /* head.head.2 padded to 32 outputs (packed), bias [32] or NULL */
+    const void *mean_bias, *std_bias, *weight_bias; /* [K] */
+    int K;
+    float std_min, std_max;
+    const float *rand_u;     /* [Nt, B] uniform in [0, 1) */
+    const float *rand_n;     /* [Nt, B] standard normal */
+    const void *x_mean;      /* [B, Nt] mean over features of every target row */
+    const void *w_x, *b_x;   /* embedder.x_embed: weight [D, 1] as [D], bias [D] */
+    const void *w_y, *b_y;   /* embedder.y_embed */
+    const void *markers;     /* embedder.marker_embed.weight [3, D] */
+    const void *ar_tokens;   /* [bs, D] */
+    int bs;
+    const int32_t *step;     /* device: index t of the target being sampled */
+    int Nt;
+    void *preds;             /* [B, Nt]; column t is written */
+    void *emb_next;          /* [B, 2, D] contiguous: rows of step t + 1 */
+    int B, D, F;
+} artab_sample_embed_args;
+
+int artab_decode_sample_embed(const artab_sample_embed_args *args, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

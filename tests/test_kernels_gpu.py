@@ -612,3 +612,130 @@ def test_layer_fused_equals_unfused_composition(device, monkeypatch, D, F, H):
     for a, b in ((y_f, y_u), (q_f, q_u), (k_f, k_u), (v_f, v_u), (out_f, out_u)):
         assert a.shape == b.shape
         assert max_abs(to_np(a), to_np(b)) <= 4e-2  # two 16-bit chains with different rounding points
+
+
+# ----- decode-step tail: norm + head + draw + next embedding ------------------------------------------
+
+
+def _tail_model(D, F, K, bs, dtype, device, seed=0):
+    from ar_nanotabpfn_amd import model as m
+
+    torch.manual_seed(seed)
+    net = m.ARTabPFN(d_model=D, n_heads=4, n_layers=1, d_ff=F, num_features=3, buffer_size=bs, num_components=K)
+    with torch.no_grad():  # make every learned vector non-trivial
+        for p in list(net.embedder.parameters()) + list(net.head.parameters()) + [net.ar_tokens]:
+            p.add_(0.3 * torch.randn_like(p))
+        net.backbone.norm.weight.add_(0.2 * torch.randn(D))
+        net.backbone.norm.bias.add_(0.2 * torch.randn(D))
+    return net.to(device=device, dtype=dtype)
+
+
+def _tail_reference(net, x_last, x_mean, u, n, t, dtype):
+    """float64 restatement of backbone.norm -> head -> inverse-CDF pick -> draw -> embeddings,
+    with the kernel's rounding points (z and gelu output rounded to the storage dtype)."""
+    d = lambda p: p.detach().cpu().double()  # noqa: E731
+    rd = lambda v: v.to(dtype).double()  # noqa: E731
+    B, Nt = x_mean.shape
+    norm, head, emb = net.backbone.norm, net.head, net.embedder
+    z = rd(torch.nn.functional.layer_norm(x_last.double(), (x_last.shape[-1],), d(norm.weight), d(norm.bias), norm.eps))
+    h = rd(torch.nn.functional.gelu(z @ d(head.head[0].weight).t() + d(head.head[0].bias)))
+    raw = (h @ d(head.head[2].weight).t() + d(head.head[2].bias)).view(B, head.num_components, 3)
+    w = torch.softmax(raw[:, :, 2] + d(head.weight_bias), dim=1)
+    cdf = torch.cumsum(w, dim=1)
+    comp = (cdf > u[:, None]).double().argmax(dim=1)
+    margin = (cdf[:, :-1] - u[:, None]).abs().min(dim=1).values
+    rows = torch.arange(B)
+    mean = raw[rows, comp, 0] + d(head.mean_bias)[comp]
+    std = torch.nn.functional.softplus(raw[rows, comp, 1] + d(head.std_bias)[comp]).clamp(max=2.0) + head.std_min
+    y = rd(mean + std * n)
+    bs = net.ar_tokens.shape[0]
+    wx, bx = d(emb.x_embed.weight).view(-1), d(emb.x_embed.bias)
+    wy, by = d(emb.y_embed.weight).view(-1), d(emb.y_embed.bias)
+    mk = d(emb.marker_embed.weight)
+    buf = x_mean[:, t, None].double() * wx + bx + y[:, None] * wy + by + mk[2] + d(net.ar_tokens)[(t + 1) % bs]
+    tgt = x_mean[:, min(t + 1, Nt - 1), None].double() * wx + bx + mk[0]
+    return y, torch.stack([buf, tgt], dim=1), margin
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,D,F,K,t", [(70, 128, 128, 5, 3), (1024, 256, 256, 5, 1), (33, 512, 256, 10, 6),
+                                       (40, 256, 512, 3, 7)])
+def test_decode_sample_embed_matches_float64(device, dtype, B, D, F, K, t):
+    from ar_nanotabpfn_amd.glue import SampleEmbedStep
+
+    Nt, bs = 8, 5
+    net = _tail_model(D, F, K, bs, dtype, device)
+    g = torch.Generator().manual_seed(1)
+    x_last = torch.randn(B, 2, D, generator=g).to(dtype)
+    x_mean = (0.5 * torch.randn(B, Nt, generator=g)).to(dtype)
+    u = torch.rand(Nt, B, generator=g)
+    n = torch.randn(Nt, B, generator=g)
+    step = torch.tensor([t], dtype=torch.int32, device=device)
+    preds = torch.full((B, Nt), 7.0, device=device, dtype=dtype)
+    emb = torch.zeros(B, 2, D, device=device, dtype=dtype)
+    assert SampleEmbedStep.supported(net.embedder, net.backbone, net.head, emb)
+    tail = SampleEmbedStep(net.embedder, net.backbone, net.head, net.ar_tokens, x_mean.to(device), u.to(device),
+                           n.to(device), step, preds, emb)
+    tail(x_last.to(device))
+    y_ref, emb_ref, margin = _tail_reference(net, x_last[:, 1], x_mean, u[t].double(), n[t].double(), t, dtype)
+    ok = margin > 2e-2  # rows whose uniform variate sits on a component boundary may pick the neighbour
+    assert ok.float().mean() > 0.8
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    got = preds.cpu().double()
+    assert torch.all(got[:, [c for c in range(Nt) if c != t]] == 7.0)  # only column t is written
+    # the head runs on 16-bit z and h: allow a few output ulps on top of the final rounding
+    tol_y = 6 * ulp * max(1.0, float(y_ref.abs().max()))
+    assert float((got[:, t] - y_ref).abs()[ok].max()) <= tol_y
+    # embeddings are compared given the kernel's own draw
+    y_used = got[:, t]
+    emb_fix = emb_ref.clone()
+    wy = net.embedder.y_embed.weight.detach().cpu().double().view(-1)
+    emb_fix[:, 0] += (y_used - y_ref)[:, None] * wy
+    assert float((emb.cpu().double() - emb_fix).abs().max()) <= 1.02 * ulp * max(1.0, float(emb_fix.abs().max()))
+
+
+def test_decode_sample_embed_step_out_of_range_is_noop(device):
+    from ar_nanotabpfn_amd.glue import SampleEmbedStep
+
+    dtype, B, D, Nt = torch.bfloat16, 16, 128, 4
+    net = _tail_model(D, 128, 5, 3, dtype, device)
+    step = torch.tensor([Nt], dtype=torch.int32, device=device)
+    preds = torch.full((B, Nt), 7.0, device=device, dtype=dtype)
+    emb = torch.full((B, 2, D), 3.0, device=device, dtype=dtype)
+    tail = SampleEmbedStep(net.embedder, net.backbone, net.head, net.ar_tokens,
+                           torch.zeros(B, Nt, device=device, dtype=dtype), torch.rand(Nt, B, device=device),
+                           torch.randn(Nt, B, device=device), step, preds, emb)
+    tail(torch.randn(B, 2, D, device=device).to(dtype))
+    assert torch.all(preds == 7.0) and torch.all(emb == 3.0)
+    step.fill_(-1)
+    tail(torch.randn(B, 2, D, device=device).to(dtype))
+    assert torch.all(preds == 7.0) and torch.all(emb == 3.0)
+
+
+def test_decode_sample_embed_component_frequencies(device):
+    """With many trajectories sharing one head input, the picked components follow the mixture
+    weights and the draws have the mixture's mean (law of the sampler, not a bitwise check)."""
+    from ar_nanotabpfn_amd.glue import SampleEmbedStep
+
+    dtype, B, D, F, K, Nt = torch.bfloat16, 32768, 128, 128, 5, 2
+    net = _tail_model(D, F, K, 3, dtype, device, seed=3)
+    with torch.no_grad():
+        net.head.head[2].weight.mul_(0.05)  # mild logits: no component so rare that the sample variance hinges on it
+    g = torch.Generator().manual_seed(5)
+    x_row = torch.randn(1, 2, D, generator=g).to(dtype).expand(B, -1, -1).contiguous()
+    u, n = torch.rand(Nt, B, generator=g), torch.randn(Nt, B, generator=g)
+    step = torch.tensor([1], dtype=torch.int32, device=device)
+    preds = torch.zeros(B, Nt, device=device, dtype=torch.bfloat16)
+    emb = torch.zeros(B, 2, D, device=device, dtype=dtype)
+    tail = SampleEmbedStep(net.embedder, net.backbone, net.head, net.ar_tokens,
+                           torch.zeros(B, Nt, device=device, dtype=dtype), u.to(device), n.to(device), step, preds, emb)
+    tail(x_row.to(device))
+    with torch.no_grad():
+        mean, std, weight, _ = net.head._parameterize(net.backbone.norm(x_row[:1, 1:2].to(device)))
+    mean, std, weight = (v.float().cpu().view(-1) for v in (mean, std, weight))
+    assert float(weight.min()) > 0.02
+    mix_mean = float((weight * mean).sum())
+    mix_var = float((weight * (std ** 2 + mean ** 2)).sum()) - mix_mean ** 2
+    y = preds[:, 1].float().cpu()
+    assert abs(float(y.mean()) - mix_mean) <= 5 * (mix_var / B) ** 0.5 + 2e-2
+    assert abs(float(y.var()) - mix_var) <= 0.1 * mix_var + 2e-2

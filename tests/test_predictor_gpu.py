@@ -366,3 +366,72 @@ def test_predictor_errors(device):
         pred.transformer_decode(torch.zeros(2, 3, 32, device=device), commit=0)
     with pytest.raises(ValueError):  # N != 2*Nt (inference.py:855-856)
         pred._teacher_forcing_decode_shared(torch.zeros(2, 5, 32, device=device), 2)
+
+
+def test_graph_sampling_with_fused_step_tail_equals_python_loop(device, monkeypatch):
+    """The recorded step with the one-launch tail (norm + head + draw + next embedding) against the
+    Python loop of autoregressive_decode.  Both are made deterministic the same way: component 0
+    (uniform variate 0) and a fixed normal variate."""
+    from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
+    from ar_nanotabpfn_amd.model import MixtureGaussianHead
+
+    def det_sample(self, z, num_samples=1):
+        mean, std, _, _ = self._parameterize(z)
+        return (mean[:, :, 0:1] + 0.3 * std[:, :, 0:1]).permute(0, 1, 3, 2)
+
+    def det_variates(rand_u, rand_n):
+        rand_u.zero_()
+        rand_n.fill_(0.3)
+
+    monkeypatch.setattr(MixtureGaussianHead, "sample", det_sample)
+    monkeypatch.setattr(ARTabPFNPredictor, "_draw_step_variates", staticmethod(det_variates))
+    cfg = dict(d_model=128, n_heads=4, n_layers=3, d_ff=128, num_features=3, buffer_size=5, num_components=4)
+    model = _build(cfg, device, dtype=torch.bfloat16)
+    B, Nc, Nt = 48, 40, 9
+    pred = ARTabPFNPredictor.from_trained_model(model, backend="triton_shared_context")
+    for seed in (0, 1):
+        g = torch.Generator().manual_seed(seed)
+        xc = torch.randn(1, Nc, 3, generator=g).expand(B, -1, -1).to(device, torch.bfloat16)
+        yc = torch.randn(1, Nc, generator=g).expand(B, -1).to(device, torch.bfloat16)
+        xt = torch.randn(B, Nt, 3, generator=g).to(device, torch.bfloat16)
+        pred.use_hip_graph = True
+        y_graph = pred.sample_sequence(xc, yc, xt)
+        assert pred._graph_state.tail is not None
+        caches_g = [(l.k_buf_cache.clone(), l.v_buf_cache.clone()) for l in model.backbone.layers]
+        pred.use_hip_graph = False
+        y_loop = pred.sample_sequence(xc, yc, xt)
+        assert y_graph.shape == (B, Nt) and torch.isfinite(y_graph).all()
+        # small differences feed back through the sampled values: a few bf16 ulps per step
+        assert max_abs(to_np(y_graph), to_np(y_loop)) <= 6e-2
+        for (kg, vg), l in zip(caches_g, model.backbone.layers):
+            assert max_abs(to_np(kg), to_np(l.k_buf_cache)) <= 6e-2 and max_abs(to_np(vg), to_np(l.v_buf_cache)) <= 6e-2
+        pred.fuse_step_tail = False
+        pred.use_hip_graph = True
+        y_unfused = pred.sample_sequence(xc, yc, xt)
+        assert pred._graph_state.tail is None
+        assert max_abs(to_np(y_unfused), to_np(y_loop)) <= 6e-2
+        pred.fuse_step_tail = True
+
+
+def test_graph_sampling_fused_tail_law(device):
+    """Real variates: two calls differ, trajectories differ, and the first-step marginal of the
+    fused path agrees with the Python loop's in mean and spread (same context, many trajectories)."""
+    from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
+
+    cfg = dict(d_model=128, n_heads=4, n_layers=2, d_ff=128, num_features=1, buffer_size=8, num_components=5)
+    model = _build(cfg, device, dtype=torch.bfloat16)
+    xc, yc, xt, _ = _gp_dataset(1, B=1, Nc=32, Nt=4)
+    B = 4096
+    xc, yc, xt = (_t(np.repeat(a, B, axis=0), device).to(torch.bfloat16) for a in (xc, yc, xt))
+    pred = ARTabPFNPredictor.from_trained_model(model, backend="triton_shared_context")
+    torch.manual_seed(0)
+    y1 = pred.sample_sequence(xc, yc, xt).float()
+    assert pred._graph_state.tail is not None
+    y2 = pred.sample_sequence(xc, yc, xt).float()
+    pred.use_hip_graph = False
+    y3 = pred.sample_sequence(xc, yc, xt).float()
+    assert torch.isfinite(y1).all() and (y1 - y2).abs().max() > 0 and (y1[0] - y1[1]).abs().max() > 0
+    for col in range(1, 4):  # columns 1.. come from the fused tail in y1/y2, from head.sample in y3
+        s = float(y3[:, col].std())
+        assert abs(float(y1[:, col].mean() - y3[:, col].mean())) <= 6 * s / B ** 0.5 + 1e-2
+        assert abs(float(y1[:, col].std()) - s) <= 0.1 * s + 1e-2
