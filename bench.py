@@ -174,12 +174,19 @@ def log_density_bench(device, dtype, model, with_cpu):
     return res
 
 
+# Measured with rocprofv3 (median over the decode launches): 9321.8 KiB x 2.0 fetched,
+# 18432.0 KiB written.
+CONTEXT_PASS_HBM_BYTES = int(9321.8 * 1024 * 2.0 + 18432.0 * 1024)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=NT3)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline legs")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only copy a 256 MiB buffer five times (reference kernel for scaling HBM counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: trajectories are independent given the context, so more GPUs "
@@ -188,6 +195,15 @@ def main():
         sys.exit(f"--steps must be in [1, {NT3}] (one step per target of the configuration)")
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a HIP device")
+
+    if args.copy_calibration:
+        a = torch.empty(128 * 1024 * 1024, dtype=torch.bfloat16, device="cuda:0").normal_()
+        b = torch.empty_like(a)
+        for _ in range(5):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": a.numel() * 2, "copy_bytes_written": a.numel() * 2, "launches": 5}))
+        return
 
     from ar_nanotabpfn_amd import _lib
     from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
@@ -239,7 +255,10 @@ def main():
         "peak": MFMA_BF16_PEAK_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
-        "traffic": None,
+        # HBM bytes of one decode-shaped launch: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from two
+        # rocprofv3 --pmc runs of this script, the factors from the same counters on a 256 MiB copy
+        # (--copy-calibration); algorithmic: K/V 16.8 MB + Q 1.0 MB read, 17.3 MB of partials written.
+        "traffic": CONTEXT_PASS_HBM_BYTES,
         "launches": n_dec,
         "avg_launch_us": round(avg_launch_us, 2),
         "flops_per_launch_lq2": 4.0 * B3 * H * 2 * NC3 * Dh,
