@@ -3,10 +3,10 @@
 // One wavefront per (trajectory, head).  The buffer K/V rows of that pair are
 // streamed once with 16-byte loads (HBM-bound: 2 flop per byte), each group of
 // DH/8 lanes owning one key row at a time and keeping a private online-softmax
-// state per query.  The partial results of the split context pass enter the same
-// states as extra "keys" whose weight is their log-sum-exp, and one butterfly
-// reduction across the lane groups (a wavefront-wide log-sum-exp merge in
-// float32) produces the final output.  The new buffer row is read from the
+// state per query.  The lane-group states are then brought to a common maximum
+// and summed through LDS together with the partial results of the split context
+// pass, each weighted by its log-sum-exp (a wavefront-wide LSE merge in float32,
+// one output element per lane).  The new buffer row is read from the
 // projection and written to its cache slot by the same wavefront: no torch.cat,
 // no second pass.
 #pragma once
@@ -30,6 +30,7 @@ struct DecodeParams {
 
 constexpr int kDecodeWaves = 4;
 constexpr int kDecodeUnroll = 4;
+constexpr int kSplitBatch = 8;  // context partials fetched per round of the merge
 
 template <typename T>
 __device__ __forceinline__ void unpack8(const u32x4 &raw, float (&f)[8]) {
@@ -69,6 +70,25 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
         l[i] = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[i][e] = 0.f;
+    }
+
+    // maximum over the context partials' LSEs (log2 domain), requested before the key loop so
+    // that its latency hides under it
+    float M[LQ];
+#pragma unroll
+    for (int i = 0; i < LQ; ++i) M[i] = -INFINITY;
+    for (int sp0 = 0; sp0 < P.n_split; sp0 += kSplitBatch) {
+        float v[kSplitBatch][LQ];  // a batch of loads in flight, then the maxima
+#pragma unroll
+        for (int u = 0; u < kSplitBatch; ++u) {
+            const int sp = sp0 + u < P.n_split ? sp0 + u : P.n_split - 1;
+#pragma unroll
+            for (int i = 0; i < LQ; ++i) v[u][i] = P.part_lse[static_cast<long>(sp) * total_rows + pair * LQ + i];
+        }
+#pragma unroll
+        for (int u = 0; u < kSplitBatch; ++u)
+#pragma unroll
+            for (int i = 0; i < LQ; ++i) M[i] = fmaxf(M[i], v[u][i] * kLog2e);
     }
 
     const int n_buf = P.n_buf_dev ? *P.n_buf_dev : P.n_buf;
@@ -135,62 +155,68 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
         }
     }
 
-    // Context partials: split s is folded in by lane group s mod RPW.  A partial
-    // (o, lse) is a key with score lse (log2 domain) and value o.
-    for (int sp = grp; sp < P.n_split; sp += RPW) {
+    // ---- merge of the RPW lane-group states and the context partials, through LDS.
+    // (A register butterfly needs 4 dependent rounds of 20 cross-lane moves here; the LDS
+    // version is two short phases of independent accesses.)  Every wavefront has its own region;
+    // its LDS operations execute in issue order, wave_barrier keeps the compiler from moving
+    // them across the phases.
+    __shared__ float lds_m[kDecodeWaves][RPW][LQ];
+    __shared__ float lds_l[kDecodeWaves][RPW][LQ];
+    __shared__ __attribute__((aligned(16))) float lds_acc[kDecodeWaves][RPW][LQ][DH];
+    if (sub == 0) {
 #pragma unroll
-        for (int i = 0; i < LQ; ++i) {
-            const long row = pair * LQ + i;
-            const float sc = P.part_lse[static_cast<long>(sp) * total_rows + row] * kLog2e;
-            const float *po = P.part_o + (static_cast<long>(sp) * total_rows + row) * DH + 8 * sub;
-            f32x4 o0 = *reinterpret_cast<const f32x4 *>(po);
-            f32x4 o1 = *reinterpret_cast<const f32x4 *>(po + 4);
-            const float m_new = fmaxf(m[i], sc);
-            if (m_new == -INFINITY) continue;
-            const float alpha = fast_exp2(m[i] - m_new);
-            const float p = fast_exp2(sc - m_new);
-            m[i] = m_new;
-            l[i] = l[i] * alpha + p;
+        for (int i = 0; i < LQ; ++i) lds_m[wave][grp][i] = m[i];
+    }
+    __builtin_amdgcn_wave_barrier();
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                acc[i][e] = fmaf(p, o0[e], acc[i][e] * alpha);
-                acc[i][4 + e] = fmaf(p, o1[e], acc[i][4 + e] * alpha);
+    for (int g = 0; g < RPW; ++g)
+#pragma unroll
+        for (int i = 0; i < LQ; ++i) M[i] = fmaxf(M[i], lds_m[wave][g][i]);
+    // scale this group's state to the common maximum and publish it
+#pragma unroll
+    for (int i = 0; i < LQ; ++i) {
+        const float w = m[i] == -INFINITY ? 0.f : fast_exp2(m[i] - M[i]);
+        f32x4 a0 = {acc[i][0] * w, acc[i][1] * w, acc[i][2] * w, acc[i][3] * w};
+        f32x4 a1 = {acc[i][4] * w, acc[i][5] * w, acc[i][6] * w, acc[i][7] * w};
+        *reinterpret_cast<f32x4 *>(&lds_acc[wave][grp][i][8 * sub]) = a0;
+        *reinterpret_cast<f32x4 *>(&lds_acc[wave][grp][i][8 * sub + 4]) = a1;
+        if (sub == 0) lds_l[wave][grp][i] = l[i] * w;
+    }
+    __builtin_amdgcn_wave_barrier();
+    // one output element per lane and round: column (i, d)
+    for (int col = lane; col < LQ * DH; col += 64) {
+        const int i = col / DH, d = col % DH;
+        // M of row i: select without dynamic register indexing
+        float Mi = M[0];
+#pragma unroll
+        for (int ii = 1; ii < LQ; ++ii) Mi = i == ii ? M[ii] : Mi;
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int g = 0; g < RPW; ++g) {
+            num += lds_acc[wave][g][i][d];
+            den += lds_l[wave][g][i];
+        }
+        for (int sp0 = 0; sp0 < P.n_split; sp0 += kSplitBatch) {
+            float lv[kSplitBatch], ov[kSplitBatch];
+#pragma unroll
+            for (int u = 0; u < kSplitBatch; ++u) {
+                const int sp = sp0 + u < P.n_split ? sp0 + u : P.n_split - 1;
+                const long row = static_cast<long>(sp) * total_rows + pair * LQ + i;
+                lv[u] = P.part_lse[row];
+                ov[u] = P.part_o[row * DH + d];
+            }
+#pragma unroll
+            for (int u = 0; u < kSplitBatch; ++u) {
+                const float lse2 = lv[u] * kLog2e;
+                const float w = (sp0 + u < P.n_split && lse2 != -INFINITY) ? fast_exp2(lse2 - Mi) : 0.f;
+                num = fmaf(w, ov[u], num);
+                den += w;
             }
         }
+        view_row<T>(P.out, b, h, i)[d] = from_f32<T>(den > 0.f ? num / den : 0.f);
+        if (P.lse && d == 0) P.lse[pair * LQ + i] = den > 0.f ? (Mi + fast_log2(den)) * kLn2 : -INFINITY;
     }
-
-    // Butterfly merge of the RPW lane-group states (same slice `sub` across groups).
-#pragma unroll
-    for (int off = LPR; off < 64; off <<= 1) {
-#pragma unroll
-        for (int i = 0; i < LQ; ++i) {
-            const float m_o = __shfl_xor(m[i], off, 64);
-            const float l_o = __shfl_xor(l[i], off, 64);
-            const float m_new = fmaxf(m[i], m_o);
-            const float a_s = m[i] == -INFINITY ? 0.f : fast_exp2(m[i] - m_new);
-            const float a_o = m_o == -INFINITY ? 0.f : fast_exp2(m_o - m_new);
-            l[i] = l[i] * a_s + l_o * a_o;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float acc_o = __shfl_xor(acc[i][e], off, 64);
-                acc[i][e] = acc[i][e] * a_s + acc_o * a_o;
-            }
-            m[i] = m_new;
-        }
-    }
-
-    if (grp == 0) {
-#pragma unroll
-        for (int i = 0; i < LQ; ++i) {
-            const float inv = l[i] > 0.f ? 1.f / l[i] : 0.f;
-            u32x4 val;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) val[e] = pack2<T>(acc[i][2 * e] * inv, acc[i][2 * e + 1] * inv);
-            *reinterpret_cast<u32x4 *>(view_row<T>(P.out, b, h, i) + 8 * sub) = val;
-            if (P.lse && sub == 0)
-                P.lse[pair * LQ + i] = l[i] > 0.f ? (m[i] + fast_log2(l[i])) * kLn2 : -INFINITY;
-        }
-    } else if (grp == 1 && P.has_new) {
+    if (grp == 1 && P.has_new) {
         // In-place append: slot n_buf of the cache receives the new row.
         *reinterpret_cast<u32x4 *>(view_row<T>(P.kb, b, h, n_buf) + 8 * sub) =
             *reinterpret_cast<const u32x4 *>(knew_row + 8 * sub);
