@@ -247,7 +247,8 @@ static hipError_t launch_portable_dtype(const PortableParams &P, int dtype, hipS
 // per (row, 4 output elements).
 struct CombineParams {
     View out;
-    const float *part_o, *part_lse;
+    const void *part_o;  // input type
+    const float *part_lse;
     float *lse;
     long rows;
     int H, Lq, Dh, n_split;
@@ -265,10 +266,10 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineParams P) {
     float wsum = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
     for (int s = 0; s < P.n_split; ++s) {
         float w = expf(P.part_lse[s * P.rows + row] - mx);
-        f32x4 o = *reinterpret_cast<const f32x4 *>(P.part_o + (s * P.rows + row) * P.Dh + d0);
+        const T *o = static_cast<const T *>(P.part_o) + (s * P.rows + row) * P.Dh + d0;
         wsum += w;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[e] = fmaf(w, o[e], acc[e]);
+        for (int e = 0; e < 4; ++e) acc[e] = fmaf(w, to_f32(o[e]), acc[e]);
     }
     int i = static_cast<int>(row % P.Lq);
     int h = static_cast<int>((row / P.Lq) % P.H);
@@ -280,8 +281,13 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineParams P) {
     if (P.lse && d0 == 0) P.lse[row] = mx + logf(wsum);
 }
 
+// Partial outputs in the input type (16-bit on this path) followed by float32 log-sum-exps.
 static size_t split_workspace_bytes(long rows, int Dh, int n_split) {
-    return static_cast<size_t>(n_split) * static_cast<size_t>(rows) * (Dh + 1) * sizeof(float);
+    return static_cast<size_t>(n_split) * static_cast<size_t>(rows) * (Dh * 2 + sizeof(float));
+}
+
+static float *split_lse_base(void *workspace, long rows, int Dh, int n_split) {
+    return reinterpret_cast<float *>(static_cast<char *>(workspace) + static_cast<size_t>(n_split) * rows * Dh * 2);
 }
 
 }  // namespace artab
@@ -463,8 +469,8 @@ int artab_context_attention(const artab_view *q, const artab_view *k_ctx, const 
     FlashPlan pl = plan_flash(B, H, Lq, Nc, Dh, stacked, /*allow_split=*/true);
     if (pl.n_split > 1) {
         size_t need = split_workspace_bytes(rows, Dh, pl.n_split);
-        if (!workspace || workspace_bytes < need) {
-            // Without a workspace the unsplit schedule is still correct, only less parallel.
+        if (!workspace || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16) {
+            // Without a (usable) workspace the unsplit schedule is still correct, only less parallel.
             pl.n_split = 1;
             pl.kv_per_split = (Nc + 127) / 128 * 128;
         }
@@ -479,8 +485,8 @@ int artab_context_attention(const artab_view *q, const artab_view *k_ctx, const 
     F.qscale = scale * kLog2e;
     F.mode = kFlashContext;
     if (pl.n_split > 1) {
-        F.part_o = static_cast<float *>(workspace);
-        F.part_lse = F.part_o + static_cast<size_t>(pl.n_split) * rows * Dh;
+        F.part_o = workspace;
+        F.part_lse = split_lse_base(workspace, rows, Dh, pl.n_split);
     }
     {
         ProfileScope prof(st);
@@ -542,7 +548,7 @@ int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const a
         pl = plan_flash(B, H, Lq, Nc, Dh, /*stacked=*/true, /*allow_split=*/true);
         const bool direct = !need_buf && pl.n_split == 1;  // context pass writes the final output
         need_ws = direct ? 0 : split_workspace_bytes(rows, Dh, pl.n_split);
-        if (need_ws && (!workspace || workspace_bytes < need_ws)) {
+        if (need_ws && (!workspace || workspace_bytes < need_ws || reinterpret_cast<uintptr_t>(workspace) % 16)) {
             if (impl == ARTAB_IMPL_MFMA)
                 return fail(ARTAB_ERR_WORKSPACE, "decode needs %zu workspace bytes, got %zu", need_ws,
                             workspace_bytes);
@@ -576,8 +582,8 @@ int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const a
     F.qscale = scale * kLog2e;
     F.mode = kFlashContext;
     if (need_ws) {
-        F.part_o = static_cast<float *>(workspace);
-        F.part_lse = F.part_o + static_cast<size_t>(pl.n_split) * rows * Dh;
+        F.part_o = workspace;
+        F.part_lse = split_lse_base(workspace, rows, Dh, pl.n_split);
     }
     {
         ProfileScope prof(st);

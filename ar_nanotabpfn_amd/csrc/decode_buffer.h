@@ -17,7 +17,7 @@ namespace artab {
 
 struct DecodeParams {
     View q, kb, vb, knew, vnew, out;
-    const float *part_o;    // [n_split][B*H*Lq][DH] normalised context partials
+    const void *part_o;     // [n_split][B*H*Lq][DH] normalised context partials, input type
     const float *part_lse;  // [n_split][B*H*Lq] natural-log LSE of each partial
     float *lse;             // optional final LSE [B,H,Lq]
     int B, H;
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
                 const int sp = sp0 + u < P.n_split ? sp0 + u : P.n_split - 1;
                 const long row = static_cast<long>(sp) * total_rows + pair * LQ + i;
                 lv[u] = P.part_lse[row];
-                ov[u] = P.part_o[row * DH + d];
+                ov[u] = to_f32(static_cast<const T *>(P.part_o)[row * DH + d]);
             }
 #pragma unroll
             for (int u = 0; u < kSplitBatch; ++u) {

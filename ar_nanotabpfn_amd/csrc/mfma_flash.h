@@ -75,7 +75,8 @@ struct FlashParams {
     View kcache, vcache;
     int cache_batches;
     float *lse;       // [B,H,Lq] final log-sum-exp (natural log) or nullptr
-    float *part_o;    // split partials: [n_split][B*H*Lq][DH] normalised float32
+    void *part_o;     // split partials: [n_split][B*H*Lq][DH] normalised, in the input type (the
+                      // reference merges partial outputs of the input type too, triton_kernels.py:478-524)
     float *part_lse;  // [n_split][B*H*Lq] natural log
     int B, H, Lq;
     int Nc, Nb, Nt;
@@ -617,14 +618,14 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
         const float m_fin = m_run[j] == -INFINITY ? 0.f : m_run[j];
         const float lse = l_tot > 0.f ? (m_fin + fast_log2(l_tot)) * kLn2 : -INFINITY;
         if (P.part_o) {
-            float *po = P.part_o + (static_cast<long>(split) * total_rows + orow_idx[j]) * DH;
+            T *po = static_cast<T *>(P.part_o) + (static_cast<long>(split) * total_rows + orow_idx[j]) * DH;
 #pragma unroll
             for (int db = 0; db < DB; ++db)
 #pragma unroll
                 for (int gq = 0; gq < 4; ++gq) {
-                    f32x4 val = {o_acc[j][db][4 * gq] * inv, o_acc[j][db][4 * gq + 1] * inv,
-                                 o_acc[j][db][4 * gq + 2] * inv, o_acc[j][db][4 * gq + 3] * inv};
-                    *reinterpret_cast<f32x4 *>(po + 32 * db + 8 * gq + 4 * hb) = val;
+                    u32x2 val = {pack2<T>(o_acc[j][db][4 * gq] * inv, o_acc[j][db][4 * gq + 1] * inv),
+                                 pack2<T>(o_acc[j][db][4 * gq + 2] * inv, o_acc[j][db][4 * gq + 3] * inv)};
+                    *reinterpret_cast<u32x2 *>(po + 32 * db + 8 * gq + 4 * hb) = val;
                 }
             if (hb == 0) P.part_lse[static_cast<long>(split) * total_rows + orow_idx[j]] = lse;
         } else {

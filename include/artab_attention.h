@@ -18,8 +18,10 @@
  *    A batch stride of 0 means "one copy shared by every batch entry"; that is
  *    how the shared context K/V `[H, Nc, Dh]` is passed.
  *  - dtype selects the element type of q/k/v/out (and caches); log-sum-exp
- *    outputs and workspaces are always float32.  Softmax statistics and
- *    accumulation are float32 for every dtype.
+ *    outputs are always float32.  Softmax statistics and accumulation are
+ *    float32 for every dtype.  A workspace is opaque scratch, 16-byte aligned
+ *    (it holds the partial outputs of context slices in the input type, as the
+ *    reference merges them, and their float32 log-sum-exps).
  *  - `scale` <= 0 selects the default head_dim^-0.5.
  *  - Every function returns ARTAB_OK (0) or a negative artab_status; on error
  *    nothing has been launched.  artab_last_error() gives a thread-local text.
@@ -84,7 +86,7 @@ const char *artab_last_error(void);
 int artab_profile_begin(int max_records);
 int artab_profile_end(double *total_ms, int *records);
 
-/* Bytes of float32 workspace the split-context paths need for the given problem
+/* Bytes of workspace the split-context paths need for the given problem
  * (artab_context_attention, artab_decode_attention).  0 means no workspace is
  * needed.  Pure host arithmetic, no device access. */
 size_t artab_workspace_bytes(int B, int H, int Lq, int Nc, int Dh, int dtype);
