@@ -82,6 +82,10 @@ SIGNATURES = {
     "artab_bias_gelu": (_i, [_p, _i64, _p, _p, _i64, _i, _i, _p]),
     "artab_pack_linear_weight": (_i, [_p, _p, _i, _i, _i, _p]),
     "artab_layer_pre": (_i, [_p, _i64, _p, _p, _p, _f, _p, _p, _p, _i64, _i, _i, _p]),
+    "artab_layer_post_pre": (
+        _i,
+        [_p, _i64, _p, _i64, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _f, _p, _p, _p, _f, _p, _p, _p, _i64, _i, _i, _i, _p],
+    ),
     "artab_decode_sample_embed": (_i, [ctypes.POINTER(ArtabSampleEmbedArgs), _i, _p]),
     "artab_layer_post": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _f, _p, _i64, _i, _i, _i, _p]),
 }

@@ -329,6 +329,26 @@ hipError_t launch_post_d(const FusedPostParams &P, int F, hipStream_t st) {
     return hipGetLastError();
 }
 
+template <typename T, int D>
+hipError_t launch_post_pre_d(const FusedPostParams &P, const FusedPreParams &N, int F, hipStream_t st) {
+    dim3 grid(static_cast<unsigned>((P.rows + kFusedRows - 1) / kFusedRows)), block(fused_waves(D) * 64);
+    switch (F) {
+        case 128: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 128>), grid, block, 0, st, P, N); break;
+        case 256: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 256>), grid, block, 0, st, P, N); break;
+        default: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 512>), grid, block, 0, st, P, N); break;
+    }
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_post_pre(const FusedPostParams &P, const FusedPreParams &N, int D, int F, hipStream_t st) {
+    switch (D) {
+        case 128: return launch_post_pre_d<T, 128>(P, N, F, st);
+        case 256: return launch_post_pre_d<T, 256>(P, N, F, st);
+        default: return launch_post_pre_d<T, 512>(P, N, F, st);
+    }
+}
+
 template <typename T>
 hipError_t launch_post(const FusedPostParams &P, int D, int F, hipStream_t st) {
     switch (D) {
@@ -817,22 +837,54 @@ int artab_pack_linear_weight(const void *w, void *packed, int N, int K, int dtyp
     return launch_status(hipGetLastError(), "pack_linear_weight");
 }
 
+static int fill_pre(FusedPreParams &P, const void *x, int64_t ldx, const void *w_fo, const void *ln1_gamma,
+                    const void *ln1_beta, float eps1, const void *w_qkv, void *y, void *qkv, int64_t rows, int D,
+                    bool x_required) {
+    if (!fused_width_ok(D)) return fail(ARTAB_ERR_UNSUPPORTED, "layer_pre needs D in {128, 256, 512} (got %d)", D);
+    if ((x_required && !x) || !w_fo || !ln1_gamma || !ln1_beta || !w_qkv || !y || !qkv)
+        return fail(ARTAB_ERR_NULL_POINTER, "layer_pre: every pointer is required");
+    if (misaligned16(x) || misaligned16(w_fo) || misaligned16(w_qkv) || misaligned16(y) || misaligned16(qkv) ||
+        misaligned16(ln1_gamma) || misaligned16(ln1_beta) || (x_required && (ldx % 8 || ldx < D)))
+        return fail(ARTAB_ERR_BAD_STRIDE, "layer_pre operands must be 16-byte aligned with ldx %% 8 == 0, ldx >= D");
+    P.x = x; P.ldx = ldx; P.w_fo = w_fo; P.g1 = ln1_gamma; P.b1 = ln1_beta; P.w_qkv = w_qkv;
+    P.y = y; P.qkv = qkv; P.rows = rows; P.eps = eps1;
+    return ARTAB_OK;
+}
+
+static int fill_post(FusedPostParams &P, const void *attn, int64_t lda, const void *y, int64_t ldy, const void *w_o,
+                     const void *ln2_gamma, const void *ln2_beta, float eps2, const void *w_1, const void *b_1,
+                     const void *w_2, const void *b_2, const void *ln3_gamma, const void *ln3_beta, float eps3,
+                     void *out, int64_t rows, int D, int F, bool out_required) {
+    if (!fused_width_ok(D) || !fused_width_ok(F))
+        return fail(ARTAB_ERR_UNSUPPORTED, "layer_post needs D and F in {128, 256, 512} (got %d, %d)", D, F);
+    if (!attn || !y || !w_o || !ln2_gamma || !ln2_beta || !w_1 || !w_2 || !ln3_gamma || !ln3_beta ||
+        (out_required && !out))
+        return fail(ARTAB_ERR_NULL_POINTER, "layer_post: only b_1 and b_2 may be NULL");
+    if (misaligned16(attn) || misaligned16(y) || misaligned16(w_o) || misaligned16(w_1) || misaligned16(w_2) ||
+        misaligned16(b_1) || misaligned16(b_2) || misaligned16(ln2_gamma) || misaligned16(ln2_beta) ||
+        misaligned16(ln3_gamma) || misaligned16(ln3_beta) || misaligned16(out) || lda % 8 || ldy % 8 || lda < D ||
+        ldy < D)
+        return fail(ARTAB_ERR_BAD_STRIDE, "layer_post operands must be 16-byte aligned with row strides %% 8 == 0");
+    P.attn = attn; P.lda = lda; P.y = y; P.ldy = ldy; P.w_o = w_o; P.g2 = ln2_gamma; P.b2 = ln2_beta;
+    P.w_1 = w_1; P.bias_1 = b_1; P.w_2 = w_2; P.bias_2 = b_2; P.g3 = ln3_gamma; P.b3 = ln3_beta;
+    P.out = out; P.rows = rows; P.eps2 = eps2; P.eps3 = eps3;
+    return ARTAB_OK;
+}
+
+static int check_layer_dtype_rows(const char *what, int dtype, int64_t rows) {
+    if (dtype != ARTAB_BF16 && dtype != ARTAB_F16)
+        return fail(ARTAB_ERR_UNSUPPORTED, "%s supports bf16 and fp16 only (dtype code %d)", what, dtype);
+    if (rows < 0) return fail(ARTAB_ERR_BAD_SHAPE, "%s: negative row count %lld", what, (long long)rows);
+    return ARTAB_OK;
+}
+
 int artab_layer_pre(const void *x, int64_t ldx, const void *w_fo, const void *ln1_gamma, const void *ln1_beta,
                     float eps1, const void *w_qkv, void *y, void *qkv, int64_t rows, int D, int dtype,
                     void *stream) {
-    if (dtype != ARTAB_BF16 && dtype != ARTAB_F16)
-        return fail(ARTAB_ERR_UNSUPPORTED, "layer_pre supports bf16 and fp16 only (dtype code %d)", dtype);
-    if (rows < 0 || D <= 0) return fail(ARTAB_ERR_BAD_SHAPE, "bad sizes rows=%lld D=%d", (long long)rows, D);
-    if (!fused_width_ok(D)) return fail(ARTAB_ERR_UNSUPPORTED, "layer_pre needs D in {128, 256, 512} (got %d)", D);
-    if (rows == 0) return ARTAB_OK;
-    if (!x || !w_fo || !ln1_gamma || !ln1_beta || !w_qkv || !y || !qkv)
-        return fail(ARTAB_ERR_NULL_POINTER, "layer_pre: every pointer is required");
-    if (misaligned16(x) || misaligned16(w_fo) || misaligned16(w_qkv) || misaligned16(y) || misaligned16(qkv) ||
-        misaligned16(ln1_gamma) || misaligned16(ln1_beta) || ldx % 8 || ldx < D)
-        return fail(ARTAB_ERR_BAD_STRIDE, "layer_pre operands must be 16-byte aligned with ldx %% 8 == 0, ldx >= D");
+    ARTAB_TRY(check_layer_dtype_rows("layer_pre", dtype, rows));
     FusedPreParams P;
-    P.x = x; P.ldx = ldx; P.w_fo = w_fo; P.g1 = ln1_gamma; P.b1 = ln1_beta; P.w_qkv = w_qkv;
-    P.y = y; P.qkv = qkv; P.rows = rows; P.eps = eps1;
+    ARTAB_TRY(fill_pre(P, x, ldx, w_fo, ln1_gamma, ln1_beta, eps1, w_qkv, y, qkv, rows, D, true));
+    if (rows == 0) return ARTAB_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipError_t e = dtype == ARTAB_BF16 ? launch_pre<bf16_t>(P, D, st) : launch_pre<f16_t>(P, D, st);
     return launch_status(e, "layer_pre");
@@ -842,27 +894,33 @@ int artab_layer_post(const void *attn, int64_t lda, const void *y, int64_t ldy, 
                      const void *ln2_gamma, const void *ln2_beta, float eps2, const void *w_1, const void *b_1,
                      const void *w_2, const void *b_2, const void *ln3_gamma, const void *ln3_beta, float eps3,
                      void *out, int64_t rows, int D, int F, int dtype, void *stream) {
-    if (dtype != ARTAB_BF16 && dtype != ARTAB_F16)
-        return fail(ARTAB_ERR_UNSUPPORTED, "layer_post supports bf16 and fp16 only (dtype code %d)", dtype);
-    if (rows < 0 || D <= 0 || F <= 0)
-        return fail(ARTAB_ERR_BAD_SHAPE, "bad sizes rows=%lld D=%d F=%d", (long long)rows, D, F);
-    if (!fused_width_ok(D) || !fused_width_ok(F))
-        return fail(ARTAB_ERR_UNSUPPORTED, "layer_post needs D and F in {128, 256, 512} (got %d, %d)", D, F);
-    if (rows == 0) return ARTAB_OK;
-    if (!attn || !y || !w_o || !ln2_gamma || !ln2_beta || !w_1 || !w_2 || !ln3_gamma || !ln3_beta || !out)
-        return fail(ARTAB_ERR_NULL_POINTER, "layer_post: only b_1 and b_2 may be NULL");
-    if (misaligned16(attn) || misaligned16(y) || misaligned16(w_o) || misaligned16(w_1) || misaligned16(w_2) ||
-        misaligned16(b_1) || misaligned16(b_2) || misaligned16(ln2_gamma) || misaligned16(ln2_beta) ||
-        misaligned16(ln3_gamma) || misaligned16(ln3_beta) || misaligned16(out) || lda % 8 || ldy % 8 || lda < D ||
-        ldy < D)
-        return fail(ARTAB_ERR_BAD_STRIDE, "layer_post operands must be 16-byte aligned with row strides %% 8 == 0");
+    ARTAB_TRY(check_layer_dtype_rows("layer_post", dtype, rows));
     FusedPostParams P;
-    P.attn = attn; P.lda = lda; P.y = y; P.ldy = ldy; P.w_o = w_o; P.g2 = ln2_gamma; P.b2 = ln2_beta;
-    P.w_1 = w_1; P.bias_1 = b_1; P.w_2 = w_2; P.bias_2 = b_2; P.g3 = ln3_gamma; P.b3 = ln3_beta;
-    P.out = out; P.rows = rows; P.eps2 = eps2; P.eps3 = eps3;
+    ARTAB_TRY(fill_post(P, attn, lda, y, ldy, w_o, ln2_gamma, ln2_beta, eps2, w_1, b_1, w_2, b_2, ln3_gamma,
+                        ln3_beta, eps3, out, rows, D, F, true));
+    if (rows == 0) return ARTAB_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipError_t e = dtype == ARTAB_BF16 ? launch_post<bf16_t>(P, D, F, st) : launch_post<f16_t>(P, D, F, st);
     return launch_status(e, "layer_post");
+}
+
+int artab_layer_post_pre(const void *attn, int64_t lda, const void *y, int64_t ldy, const void *w_o,
+                         const void *ln2_gamma, const void *ln2_beta, float eps2, const void *w_1, const void *b_1,
+                         const void *w_2, const void *b_2, const void *ln3_gamma, const void *ln3_beta, float eps3,
+                         const void *next_w_fo, const void *next_ln1_gamma, const void *next_ln1_beta,
+                         float next_eps1, const void *next_w_qkv, void *next_y, void *next_qkv, int64_t rows, int D,
+                         int F, int dtype, void *stream) {
+    ARTAB_TRY(check_layer_dtype_rows("layer_post_pre", dtype, rows));
+    FusedPostParams P;
+    FusedPreParams N;
+    ARTAB_TRY(fill_post(P, attn, lda, y, ldy, w_o, ln2_gamma, ln2_beta, eps2, w_1, b_1, w_2, b_2, ln3_gamma,
+                        ln3_beta, eps3, nullptr, rows, D, F, false));
+    ARTAB_TRY(fill_pre(N, nullptr, 0, next_w_fo, next_ln1_gamma, next_ln1_beta, next_eps1, next_w_qkv, next_y,
+                       next_qkv, rows, D, false));
+    if (rows == 0) return ARTAB_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipError_t e = dtype == ARTAB_BF16 ? launch_post_pre<bf16_t>(P, N, D, F, st) : launch_post_pre<f16_t>(P, N, D, F, st);
+    return launch_status(e, "layer_post_pre");
 }
 
 int artab_decode_sample_embed(const artab_sample_embed_args *a, int dtype, void *stream) {

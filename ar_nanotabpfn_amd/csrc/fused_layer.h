@@ -145,6 +145,22 @@ __device__ __forceinline__ void load_cols(const T *vec, const int (&nblk)[NB], i
         for (int g = 0; g < 4; ++g) load4f<T>(vec + col_of(nblk[b], 4 * g, hb), &out[b][4 * g]);
 }
 
+// Parameter vectors (LayerNorm gamma / beta, biases) are copied to LDS when the kernel starts:
+// fetched from global memory right where they are used, each costs its phase a full memory
+// round trip (the phases are far shorter than that).  A missing vector becomes zeros.
+template <typename T, int LEN, int NT>
+__device__ __forceinline__ void stage_vector(T *dst, const void *src, int tid) {
+    static_assert(LEN % 8 == 0, "16-byte chunks");
+    for (int ch = tid; ch < LEN / 8; ch += NT) {
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (src) v = *reinterpret_cast<const u32x4 *>(static_cast<const T *>(src) + 8 * ch);
+        *reinterpret_cast<u32x4 *>(dst + 8 * ch) = v;
+    }
+}
+
+// LDS slots of the parameter vectors (each max(D, F) elements wide)
+enum VecSlot : int { kVecG1 = 0, kVecB1, kVecG2, kVecB2, kVecBias1, kVecG3, kVecB3, kVecBias2, kVecSlots };
+
 // Row statistics over all N columns of the tile: each lane holds, for its token column, the
 // values of NB blocks; sums are completed across the lane pair (hb) and the wavefronts.
 // red_a / red_b are two [NW*32] exchange arrays (two, so that back-to-back calls need no
@@ -225,31 +241,40 @@ __device__ __forceinline__ void layer_norm_to_lds(const float (&v)[NB][16], cons
         }
 }
 
-template <typename T, int D>
-__global__ __launch_bounds__(fused_waves(D) * 64) void fused_pre_kernel(FusedPreParams P) {
+// Body of the pre kernel on one 32-row tile.  a0: x tile (row stride D + 8), staged here from
+// P.x unless X_IN_LDS (then a finished tile is already there and the caller has synchronised);
+// later the staging buffer of the qkv passes.  a1: y tile.
+template <typename T, int D, int NT>
+__device__ __forceinline__ void stage_pre_vectors(const FusedPreParams &P, T *vecs, int vec_ld, int tid) {
+    stage_vector<T, D, NT>(vecs + kVecG1 * vec_ld, P.g1, tid);
+    stage_vector<T, D, NT>(vecs + kVecB1 * vec_ld, P.b1, tid);
+}
+
+template <typename T, int D, bool X_IN_LDS>
+__device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T *a1, float *red_a, float *red_b,
+                                               long row0, int valid,
+                                               WeightStream<T, D, D / 32 / fused_waves(D)> &w_a, T *vecs, int vec_ld) {
     constexpr int NW = fused_waves(D), NT = NW * 64;
     constexpr int LD = D + 8;
     constexpr int NB = D / 32 / NW;  // 32-column blocks per wavefront per D columns
     static_assert(D % (32 * NW) == 0, "D must be a multiple of 32 * wavefronts");
-    __shared__ __attribute__((aligned(16))) T a0[kFusedRows * LD];  // x tile, later qkv staging
-    __shared__ __attribute__((aligned(16))) T a1[kFusedRows * LD];  // y tile
-    __shared__ float red_a[NW * 32], red_b[NW * 32];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hb = lane >> 5;
-    const long row0 = static_cast<long>(blockIdx.x) * kFusedRows;
-    const int valid = static_cast<int>(min(static_cast<long>(kFusedRows), P.rows - row0));
 
     int nblk[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b) nblk[b] = wave + NW * b;
 
-    WeightStream<T, D, NB> w_a, w_b;
-    w_a.start(static_cast<const T *>(P.w_fo), nblk, lane);
-    stage_tile<T, D, NT>(a0, LD, static_cast<const T *>(P.x) + row0 * P.ldx, P.ldx, valid, tid);
-    float gam[NB][16], bet[NB][16];
-    load_cols<T, NB>(static_cast<const T *>(P.g1), nblk, hb, gam);
-    load_cols<T, NB>(static_cast<const T *>(P.b1), nblk, hb, bet);
+    WeightStream<T, D, NB> w_b;
+    if (!X_IN_LDS) w_a.start(static_cast<const T *>(P.w_fo), nblk, lane);  // else requested by the caller already
+    if (!X_IN_LDS) {
+        stage_tile<T, D, NT>(a0, LD, static_cast<const T *>(P.x) + row0 * P.ldx, P.ldx, valid, tid);
+        stage_pre_vectors<T, D, NT>(P, vecs, vec_ld, tid);
+    }
     w_b.start(static_cast<const T *>(P.w_qkv), nblk, lane);  // q columns
-    __syncthreads();
+    if (!X_IN_LDS) __syncthreads();
+    float gam[NB][16], bet[NB][16];
+    load_cols<T, NB>(vecs + kVecG1 * vec_ld, nblk, hb, gam);
+    load_cols<T, NB>(vecs + kVecB1 * vec_ld, nblk, hb, bet);
 
     // ---- y = LN1(x + x W_fo^T)
     {
@@ -295,21 +320,39 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_pre_kernel(FusedPre
     }
 }
 
-template <typename T, int D, int F>
-__global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_kernel(FusedPostParams P) {
+template <typename T, int D>
+__global__ __launch_bounds__(fused_waves(D) * 64) void fused_pre_kernel(FusedPreParams P) {
+    constexpr int NW = fused_waves(D), LD = D + 8;
+    __shared__ __attribute__((aligned(16))) T a0[kFusedRows * LD];
+    __shared__ __attribute__((aligned(16))) T a1[kFusedRows * LD];
+    __shared__ float red_a[NW * 32], red_b[NW * 32];
+    const long row0 = static_cast<long>(blockIdx.x) * kFusedRows;
+    const int valid = static_cast<int>(min(static_cast<long>(kFusedRows), P.rows - row0));
+    __shared__ __attribute__((aligned(16))) T vecs[kVecSlots * D];
+    WeightStream<T, D, D / 32 / NW> w_a;
+    fused_pre_body<T, D, false>(P, a0, a1, red_a, red_b, row0, valid, w_a, vecs, D);
+}
+
+// Body of the post kernel on one 32-row tile.  a0 (row stride max(D, F) + 8): attn tile, gelu
+// output, finally the finished tile (row stride D + 8); a1: y tile, then x1 = LN2(...).  With
+// WRITE_OUT the tile is stored to P.out; otherwise it is left in a0, synchronised, for the
+// caller (the next layer's pre body).
+struct NoHook {
+    __device__ __forceinline__ void operator()() const {}
+};
+
+// `before_last` runs right ahead of the last product (two of the three weight streams are
+// dead by then): the fused layer boundary uses it to request the next layer's first weights.
+template <typename T, int D, int F, bool WRITE_OUT, typename Hook>
+__device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0, T *a1, float *red_a, float *red_b,
+                                                long row0, int valid, Hook before_last, T *vecs, int vec_ld) {
     constexpr int NW = fused_waves(D), NT = NW * 64;
     constexpr int LDD = D + 8, LDF = F + 8;
-    constexpr int LDM = LDD > LDF ? LDD : LDF;
     constexpr int NBD = D / 32 / NW;
     constexpr int NBF = (F / 32 + NW - 1) / NW;  // with F/32 < NW the upper wavefronts sit the product out
     static_assert(D % (32 * NW) == 0 && F % 32 == 0, "unsupported widths");
     static_assert(F / 32 >= NW ? (F / 32) % NW == 0 : true, "unsupported widths");
-    __shared__ __attribute__((aligned(16))) T a0[kFusedRows * LDM];  // attn tile, gelu output, out staging
-    __shared__ __attribute__((aligned(16))) T a1[kFusedRows * LDD];  // y tile, then x1 = LN2(...)
-    __shared__ float red_a[NW * 32], red_b[NW * 32];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hb = lane >> 5;
-    const long row0 = static_cast<long>(blockIdx.x) * kFusedRows;
-    const int valid = static_cast<int>(min(static_cast<long>(kFusedRows), P.rows - row0));
 
     int nbd[NBD], nbf[NBF];
 #pragma unroll
@@ -324,14 +367,20 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_kernel(FusedPo
     w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
     stage_tile<T, D, NT>(a0, LDD, static_cast<const T *>(P.attn) + row0 * P.lda, P.lda, valid, tid);
     stage_tile<T, D, NT>(a1, LDD, static_cast<const T *>(P.y) + row0 * P.ldy, P.ldy, valid, tid);
+    stage_vector<T, D, NT>(vecs + kVecG2 * vec_ld, P.g2, tid);
+    stage_vector<T, D, NT>(vecs + kVecB2 * vec_ld, P.b2, tid);
+    stage_vector<T, F, NT>(vecs + kVecBias1 * vec_ld, P.bias_1, tid);
+    stage_vector<T, D, NT>(vecs + kVecG3 * vec_ld, P.g3, tid);
+    stage_vector<T, D, NT>(vecs + kVecB3 * vec_ld, P.b3, tid);
+    stage_vector<T, D, NT>(vecs + kVecBias2 * vec_ld, P.bias_2, tid);
     if (ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane);
     __syncthreads();
 
     // ---- x1 = LN2(y + attn W_o^T); each lane replaces exactly the y entries it read
     {
         float gam[NBD][16], bet[NBD][16];
-        load_cols<T, NBD>(static_cast<const T *>(P.g2), nbd, hb, gam);
-        load_cols<T, NBD>(static_cast<const T *>(P.b2), nbd, hb, bet);
+        load_cols<T, NBD>(vecs + kVecG2 * vec_ld, nbd, hb, gam);
+        load_cols<T, NBD>(vecs + kVecB2 * vec_ld, nbd, hb, bet);
         f32x16 acc[NBD];
         w_o.run(acc, a0, LDD, c, hb);
         w_2.start(static_cast<const T *>(P.w_2), nbd, lane);
@@ -352,8 +401,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_kernel(FusedPo
     // ---- h = gelu(x1 W_1^T + b_1)  -> a0
     if (ff_active) {
         float bias[NBF][16];
-        load_cols<T, NBF>(P.bias_1 ? static_cast<const T *>(P.bias_1) : reinterpret_cast<const T *>(kZeroVector), nbf,
-                          hb, bias);
+        load_cols<T, NBF>(vecs + kVecBias1 * vec_ld, nbf, hb, bias);
         f32x16 acc[NBF];
         w_1.run(acc, a1, LDD, c, hb);
 #pragma unroll
@@ -370,14 +418,14 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_kernel(FusedPo
             }
     }
     float gam[NBD][16], bet[NBD][16], bias[NBD][16];
-    load_cols<T, NBD>(static_cast<const T *>(P.g3), nbd, hb, gam);
-    load_cols<T, NBD>(static_cast<const T *>(P.b3), nbd, hb, bet);
-    load_cols<T, NBD>(P.bias_2 ? static_cast<const T *>(P.bias_2) : reinterpret_cast<const T *>(kZeroVector), nbd, hb,
-                      bias);
+    load_cols<T, NBD>(vecs + kVecG3 * vec_ld, nbd, hb, gam);
+    load_cols<T, NBD>(vecs + kVecB3 * vec_ld, nbd, hb, bet);
+    load_cols<T, NBD>(vecs + kVecBias2 * vec_ld, nbd, hb, bias);
     __syncthreads();
 
     // ---- out = LN3(x1 + h W_2^T + b_2), staged through a0 for row-contiguous stores
     {
+        before_last();
         f32x16 acc[NBD];
         w_2.run(acc, a0, LDF, c, hb);
         float v[NBD][16];
@@ -395,7 +443,44 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_kernel(FusedPo
         layer_norm_to_lds<T, NBD, NW>(v, gam, bet, nbd, a0, LDD, red_a, red_b, wave, c, hb, D, P.eps3);
     }
     __syncthreads();
-    unstage_tile<T, D, NT>(static_cast<T *>(P.out) + row0 * D, D, a0, LDD, valid, tid);
+    if (WRITE_OUT) unstage_tile<T, D, NT>(static_cast<T *>(P.out) + row0 * D, D, a0, LDD, valid, tid);
+}
+
+template <typename T, int D, int F>
+__global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_kernel(FusedPostParams P) {
+    constexpr int NW = fused_waves(D), LDD = D + 8, LDF = F + 8, LDM = LDD > LDF ? LDD : LDF;
+    __shared__ __attribute__((aligned(16))) T a0[kFusedRows * LDM];
+    __shared__ __attribute__((aligned(16))) T a1[kFusedRows * LDD];
+    __shared__ float red_a[NW * 32], red_b[NW * 32];
+    const long row0 = static_cast<long>(blockIdx.x) * kFusedRows;
+    const int valid = static_cast<int>(min(static_cast<long>(kFusedRows), P.rows - row0));
+    constexpr int VW = D > F ? D : F;
+    __shared__ __attribute__((aligned(16))) T vecs[kVecSlots * VW];
+    fused_post_body<T, D, F, true>(P, a0, a1, red_a, red_b, row0, valid, NoHook{}, vecs, VW);
+}
+
+// The post part of layer L and the pre part of layer L+1 on the same 32 rows: the layer output
+// never leaves LDS, and one launch (with its fixed cost) disappears per layer boundary.
+template <typename T, int D, int F>
+__global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_pre_kernel(FusedPostParams P, FusedPreParams N) {
+    constexpr int NW = fused_waves(D), LDD = D + 8, LDF = F + 8, LDM = LDD > LDF ? LDD : LDF;
+    __shared__ __attribute__((aligned(16))) T a0[kFusedRows * LDM];
+    __shared__ __attribute__((aligned(16))) T a1[kFusedRows * LDD];
+    __shared__ float red_a[NW * 32], red_b[NW * 32];
+    const long row0 = static_cast<long>(blockIdx.x) * kFusedRows;
+    const int valid = static_cast<int>(min(static_cast<long>(kFusedRows), P.rows - row0));
+    constexpr int NB = D / 32 / NW;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    int nblk[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) nblk[b] = wave + NW * b;
+    WeightStream<T, D, NB> next_fo;
+    constexpr int VW = D > F ? D : F;
+    __shared__ __attribute__((aligned(16))) T vecs[kVecSlots * VW];
+    stage_pre_vectors<T, D, NW * 64>(N, vecs, VW, threadIdx.x);  // visible after the first barrier below
+    fused_post_body<T, D, F, false>(P, a0, a1, red_a, red_b, row0, valid,
+                                    [&]() { next_fo.start(static_cast<const T *>(N.w_fo), nblk, lane); }, vecs, VW);
+    fused_pre_body<T, D, true>(N, a0, a1, red_a, red_b, row0, valid, next_fo, vecs, VW);
 }
 
 // ---- end of a decode step: final norm + mixture head + one sample per trajectory + the

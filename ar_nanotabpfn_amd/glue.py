@@ -19,7 +19,7 @@ from torch import Tensor, nn
 
 from . import _lib
 
-__all__ = ["add_layer_norm", "bias_gelu", "layer_fusable", "pack_weight", "layer_pre", "layer_post", "SampleEmbedStep"]
+__all__ = ["add_layer_norm", "bias_gelu", "layer_fusable", "pack_weight", "layer_pre", "layer_post", "layer_post_pre", "SampleEmbedStep"]
 
 
 def _rows2d(t: Tensor) -> Tensor:
@@ -138,6 +138,29 @@ def layer_post(attn: Tensor, y: Tensor, w_o: Tensor, norm2: nn.LayerNorm, w_1: T
         )
     )
     return out
+
+
+def layer_post_pre(attn: Tensor, y: Tensor, w_o: Tensor, norm2: nn.LayerNorm, w_1: Tensor, b_1: Optional[Tensor],
+                   w_2: Tensor, b_2: Optional[Tensor], norm3: nn.LayerNorm, next_w_fo: Tensor,
+                   next_norm1: nn.LayerNorm, next_w_qkv: Tensor):
+    """``layer_post`` of one layer and ``layer_pre`` of the next in one launch; the layer output
+    between them is not materialised.  Returns the next layer's ``(y [rows, D], qkv [rows, 3D])``."""
+    D = y.shape[-1]
+    a2, y2 = _rows16(attn), _rows16(y)
+    rows = y2.shape[0]
+    y_next = torch.empty((rows, D), device=y.device, dtype=y.dtype)
+    qkv_next = torch.empty((rows, 3 * D), device=y.device, dtype=y.dtype)
+    _lib.check(
+        _lib.load().artab_layer_post_pre(
+            _ptr(a2), a2.stride(0), _ptr(y2), y2.stride(0), _ptr(w_o), _ptr(norm2.weight), _ptr(norm2.bias),
+            float(norm2.eps), _ptr(w_1), _ptr(b_1), _ptr(w_2), _ptr(b_2),
+            _ptr(norm3.weight), _ptr(norm3.bias), float(norm3.eps),
+            _ptr(next_w_fo), _ptr(next_norm1.weight), _ptr(next_norm1.bias), float(next_norm1.eps), _ptr(next_w_qkv),
+            _ptr(y_next), _ptr(qkv_next), rows, D, w_1.shape[0] * 32,
+            _lib.dtype_code(y.dtype), _lib.current_stream(y.device),
+        )
+    )
+    return y_next, qkv_next
 
 
 class SampleEmbedStep:

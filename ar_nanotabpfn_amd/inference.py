@@ -111,6 +111,22 @@ class ARTabPFNPredictor:
         """Reset the cursors, keep the memory (inference.py:137-141)."""
         self.seq_len = self.context_len = self.buffer_len = 0
 
+    # ------------------------------------------------------------------ the layer stack
+
+    def _run_layers(self, x_row: Tensor, attend) -> Tensor:
+        """``x_row [B,N,D]`` through every layer; ``attend(layer, q, k, v) -> [B,H,N,Dh]`` is the
+        row attention of the pass at hand (it also owns the cache writes).  Between two
+        attention calls the tail of one layer and the head of the next run as one launch where
+        the fused kernels cover them (``TwoStageTransformerLayer.finish_then_pre``)."""
+        layers = list(self.backbone.layers)
+        state = layers[0].pre_attention(x_row)
+        for idx, layer in enumerate(layers):
+            y, q, k, v = state
+            attn = attend(layer, q, k, v)
+            if idx + 1 == len(layers):
+                return layer.finish(y, attn)
+            state = layer.finish_then_pre(y, attn, layers[idx + 1])
+
     # ------------------------------------------------------------------ prefill
 
     @torch.no_grad()
@@ -125,9 +141,7 @@ class ARTabPFNPredictor:
         for layer in self.backbone.layers:
             if layer.k_cache.shape[2] < Nc:
                 raise ValueError("KV cache too small for the context; call init_kv_cache with a larger max_seq_len.")
-            x_row, q, k, v = layer.pre_attention(x_row)
-            attn = ak.prefill_attention(q, k, v, layer.k_cache, layer.v_cache)
-            x_row = layer.finish(x_row, attn)
+        self._run_layers(x_row, lambda layer, q, k, v: ak.prefill_attention(q, k, v, layer.k_cache, layer.v_cache))
         self.seq_len = Nc
 
     @torch.no_grad()
@@ -141,9 +155,8 @@ class ARTabPFNPredictor:
             if layer.k_ctx_cache.shape[1] != Nc or layer.k_ctx_cache.shape[0] != H:
                 layer.k_ctx_cache = torch.zeros(H, Nc, Dh, device=x_row.device, dtype=x_row.dtype)
                 layer.v_ctx_cache = torch.zeros_like(layer.k_ctx_cache)
-            x_row, q, k, v = layer.pre_attention(x_row)
-            attn = ak.prefill_attention(q, k, v, layer.k_ctx_cache, layer.v_ctx_cache)
-            x_row = layer.finish(x_row, attn)
+        self._run_layers(
+            x_row, lambda layer, q, k, v: ak.prefill_attention(q, k, v, layer.k_ctx_cache, layer.v_ctx_cache))
         self.context_len = Nc
         self.buffer_len = 0
         self.seq_len = Nc
@@ -161,15 +174,16 @@ class ARTabPFNPredictor:
         if self.backend == _SHARED:
             if self.buffer_len + commit > self.max_buffer_len:
                 raise ValueError("Shared-context buffer cache exceeded; increase max buffer length.")
-            for layer in self.backbone.layers:
-                x_row = self._layer_decode_with_cache_shared(layer, x_row, commit)
+            if N not in (1, 2):
+                raise ValueError("Shared-context decode only supports N=1 (target) or N=2 (buffer, target).")
+            x_row = self._run_layers(x_row, lambda layer, q, k, v: self._attend_decode_shared(layer, q, k, v))
             self.buffer_len += commit
             self.seq_len = self.context_len + self.buffer_len
             return add_layer_norm(x_row, None, None, self.backbone.norm)
 
         mask = DecodeMask(num_cached=self.seq_len, num_new=N)
-        for layer in self.backbone.layers:
-            x_row = self._layer_decode_with_cache(layer, x_row, mask, cache_start=self.seq_len)
+        start = self.seq_len
+        x_row = self._run_layers(x_row, lambda layer, q, k, v: self._attend_with_cache(layer, q, k, v, mask, start))
         self.seq_len += commit
         return add_layer_norm(x_row, None, None, self.backbone.norm)
 
@@ -182,6 +196,12 @@ class ARTabPFNPredictor:
         if N not in (1, 2):
             raise ValueError("Shared-context decode only supports N=1 (target) or N=2 (buffer, target).")
         x_row, q, k_new, v_new = layer.pre_attention(x_row)
+        return layer.finish(x_row, self._attend_decode_shared(layer, q, k_new, v_new, n_buf_device))
+
+    def _attend_decode_shared(self, layer, q: Tensor, k_new: Tensor, v_new: Tensor,
+                              n_buf_device: Optional[Tensor] = None) -> Tensor:
+        """The attention call of a shared-layout decode step (inference.py:785-823)."""
+        N = q.shape[2]
         k_ctx = layer.k_ctx_cache[:, : self.context_len]
         v_ctx = layer.v_ctx_cache[:, : self.context_len]
         # with a device-side length the host value is only the bound that is validated
@@ -194,13 +214,17 @@ class ARTabPFNPredictor:
                 q, k_ctx, v_ctx, layer.k_buf_cache, layer.v_buf_cache, n_buf,
                 k_new[:, :, 0:1], v_new[:, :, 0:1], n_buf_device=n_buf_device,
             )
-        return layer.finish(x_row, attn)
+        return attn
 
     def _layer_decode_with_cache(self, layer, x_row: Tensor, mask, cache_start: int) -> Tensor:
         """One layer on the full per-dataset cache (inference.py:687-744): the new K/V are
         written at ``[cache_start, cache_start+N)`` and the queries attend under ``mask``."""
-        B, N, D = x_row.shape
         x_row, q, k_new, v_new = layer.pre_attention(x_row)
+        return layer.finish(x_row, self._attend_with_cache(layer, q, k_new, v_new, mask, cache_start))
+
+    def _attend_with_cache(self, layer, q: Tensor, k_new: Tensor, v_new: Tensor, mask, cache_start: int) -> Tensor:
+        """Cache write + attention of one layer on the per-dataset layout (inference.py:704-741)."""
+        N = q.shape[2]
         if layer.k_cache.shape[2] < cache_start + N:
             raise ValueError("KV cache exceeded; increase max_seq_len.")
         if isinstance(mask, TeacherForcingMask):
@@ -235,7 +259,7 @@ class ARTabPFNPredictor:
             new_mask = torch.where(qi == N - 1, kj < qi, kj <= qi)[None, None]
             out_n, lse_n = ak.buffer_attention(q, k_new, v_new, mask=new_mask)
             attn = ak.merge_attention_outputs(out_c, lse_c, out_n, lse_n)
-        return layer.finish(x_row, attn)
+        return attn
 
     @torch.no_grad()
     def autoregressive_decode(self, x_target: Tensor, prev_x: Optional[Tensor] = None,
@@ -288,9 +312,8 @@ class ARTabPFNPredictor:
         (the body that is recorded): step index ``st.t``, buffer length ``st.nbuf``."""
         if st.tail is not None:
             # embedding of this step was left in st.emb by the previous step's tail launch
-            x_row = st.emb
-            for layer in self.backbone.layers:
-                x_row = self._layer_decode_with_cache_shared(layer, x_row, 1, n_buf_device=st.nbuf)
+            x_row = self._run_layers(
+                st.emb, lambda layer, q, k, v: self._attend_decode_shared(layer, q, k, v, n_buf_device=st.nbuf))
             st.tail(x_row)          # norm, head, draw, preds[:, t], embedding of step t + 1
             st.counters.add_(1)     # (t, nbuf)
             return
@@ -301,8 +324,8 @@ class ARTabPFNPredictor:
         tok = self.ar_tokens.index_select(0, torch.remainder(t, bs))  # ar_tokens[t % bs], inference.py:359
         buffer_emb = self.embedder.embed_buffer(x_p, st.y_prev) + tok
         x_row = torch.cat([buffer_emb, self.embedder.embed_target(x_t)], dim=1)
-        for layer in self.backbone.layers:
-            x_row = self._layer_decode_with_cache_shared(layer, x_row, 1, n_buf_device=st.nbuf)
+        x_row = self._run_layers(
+            x_row, lambda layer, q, k, v: self._attend_decode_shared(layer, q, k, v, n_buf_device=st.nbuf))
         z = add_layer_norm(x_row, None, None, self.backbone.norm)
         y = self.head.sample(z[:, -1:, :])[:, :, 0, 0]
         st.preds.index_copy_(1, t, y)
@@ -424,16 +447,16 @@ class ARTabPFNPredictor:
         if embedding.shape[1] != 2 * num_targets:
             raise ValueError("Expected N == 2*num_targets for teacher forcing.")
         mask = TeacherForcingMask(num_cached=self.seq_len, num_targets=num_targets)
-        x_row = embedding
-        for layer in self.backbone.layers:
-            x_row = self._layer_decode_with_cache(layer, x_row, mask, cache_start=self.seq_len)
+        start = self.seq_len
+        x_row = self._run_layers(embedding, lambda layer, q, k, v: self._attend_with_cache(layer, q, k, v, mask, start))
         return add_layer_norm(x_row, None, None, self.backbone.norm)
 
     @torch.no_grad()
     def _teacher_forcing_decode_shared(self, embedding: Tensor, num_targets: int) -> Tensor:
-        x_row = embedding
-        for layer in self.backbone.layers:
-            x_row = self._layer_teacher_forcing_shared(layer, x_row, num_targets)
+        if embedding.shape[1] != 2 * num_targets:
+            raise ValueError("Expected N == 2*num_targets for teacher forcing.")
+        x_row = self._run_layers(
+            embedding, lambda layer, q, k, v: self._attend_teacher_forcing_shared(layer, q, k, v, num_targets))
         return add_layer_norm(x_row, None, None, self.backbone.norm)
 
     def _layer_teacher_forcing_shared(self, layer, x_row: Tensor, num_targets: int) -> Tensor:
@@ -443,8 +466,10 @@ class ARTabPFNPredictor:
         if N != 2 * num_targets:
             raise ValueError("Expected N == 2*num_targets for teacher forcing.")
         x_row, q, k, v = layer.pre_attention(x_row)
-        attn = ak.hybrid_teacher_forcing_attention(
+        return layer.finish(x_row, self._attend_teacher_forcing_shared(layer, q, k, v, num_targets))
+
+    def _attend_teacher_forcing_shared(self, layer, q: Tensor, k: Tensor, v: Tensor, num_targets: int) -> Tensor:
+        return ak.hybrid_teacher_forcing_attention(
             q, layer.k_ctx_cache[:, : self.context_len], layer.v_ctx_cache[:, : self.context_len],
             k[:, :, :num_targets], v[:, :, :num_targets], num_targets,
         )
-        return layer.finish(x_row, attn)

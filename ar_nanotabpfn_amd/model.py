@@ -23,7 +23,7 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from .attention import DenseMask, MultiheadAttention
-from .glue import add_layer_norm, bias_gelu, layer_fusable, layer_post, layer_pre, pack_weight
+from .glue import add_layer_norm, bias_gelu, layer_fusable, layer_post, layer_post_pre, layer_pre, pack_weight
 
 __all__ = ["Embedder", "TwoStageTransformerLayer", "TwoStageTransformer", "MixtureGaussianHead", "ARTabPFN"]
 
@@ -158,6 +158,25 @@ class TwoStageTransformerLayer(nn.Module):
                               self.norm3).view(B, N, D)
         x_row = add_layer_norm(x_row, torch.mm(attn2d, self.attn_rows.out_proj.weight.t()).view(B, N, D), None, self.norm2)
         return self.feed_forward(x_row)
+
+    def finish_then_pre(self, x_row: Tensor, attn_heads: Tensor, next_layer: "TwoStageTransformerLayer"):
+        """``next_layer.pre_attention(self.finish(x_row, attn_heads))``: ``(y, q, k, v)`` of the
+        next layer.  One launch when both layers are covered by the fused kernels and have the
+        same widths; the layer output between them is then never written to memory."""
+        same = (next_layer.ff[0].out_features == self.ff[0].out_features
+                and next_layer.attn_rows.n_heads == self.attn_rows.n_heads)
+        if not (same and self._fusable(x_row) and next_layer._fusable(x_row)):
+            return next_layer.pre_attention(self.finish(x_row, attn_heads))
+        B, H, N, Dh = attn_heads.shape
+        D = H * Dh
+        attn2d = attn_heads.transpose(1, 2).reshape(B * N, D)
+        p_o, p_1, p_2 = self.packed_weights()[2:]
+        n_fo, n_qkv = next_layer.packed_weights()[:2]
+        y, qkv = layer_post_pre(attn2d, x_row, p_o, self.norm2, p_1, self.ff[0].bias, p_2, self.ff[2].bias,
+                                self.norm3, n_fo, next_layer.norm1, n_qkv)
+        qkv = qkv.view(B, N, 3, H, Dh)
+        return (y.view(B, N, D), qkv[:, :, 0].transpose(1, 2), qkv[:, :, 1].transpose(1, 2),
+                qkv[:, :, 2].transpose(1, 2))
 
     def feed_forward(self, x_row: Tensor) -> Tensor:
         """``norm3(x + ff(x))`` with bias+GELU and bias+residual+norm fused around the two GEMMs."""

@@ -238,6 +238,10 @@ int artab_bias_gelu(const void *x, int64_t ldx, const void *bias, void *out,
  *                      out = LayerNorm3(x1 + gelu(x1 w_1^T + b_1) w_2^T + b_2)
  *                      attn [rows, D] (row stride lda), y [rows, D] (row stride ldy),
  *                      out [rows, D] contiguous; w_o, w_1, w_2 packed; b_1, b_2 may be NULL.
+ *   artab_layer_post_pre: artab_layer_post of one layer followed by artab_layer_pre of the next
+ *                      on the same rows, in one launch: the layer output stays on chip (it is
+ *                      rounded to the storage dtype exactly as if it had been stored), only the
+ *                      next layer's y [rows, D] and qkv [rows, 3D] are written.
  * Accumulation, residual sums and LayerNorm statistics are float32; the intermediates x1 and
  * gelu(...) are rounded to the storage dtype once, as operands of the next product.
  */
@@ -296,6 +300,14 @@ typedef struct artab_sample_embed_args {
 } artab_sample_embed_args;
 
 int artab_decode_sample_embed(const artab_sample_embed_args *args, int dtype, void *stream);
+
+int artab_layer_post_pre(const void *attn, int64_t lda, const void *y, int64_t ldy, const void *w_o,
+                         const void *ln2_gamma, const void *ln2_beta, float eps2,
+                         const void *w_1, const void *b_1, const void *w_2, const void *b_2,
+                         const void *ln3_gamma, const void *ln3_beta, float eps3,
+                         const void *next_w_fo, const void *next_ln1_gamma, const void *next_ln1_beta,
+                         float next_eps1, const void *next_w_qkv, void *next_y, void *next_qkv,
+                         int64_t rows, int D, int F, int dtype, void *stream);
 
 #ifdef __cplusplus
 }

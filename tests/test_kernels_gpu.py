@@ -739,3 +739,38 @@ def test_decode_sample_embed_component_frequencies(device):
     y = preds[:, 1].float().cpu()
     assert abs(float(y.mean()) - mix_mean) <= 5 * (mix_var / B) ** 0.5 + 2e-2
     assert abs(float(y.var()) - mix_var) <= 0.1 * mix_var + 2e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,D,F,H", [(33, 128, 256, 4), (2048, 256, 256, 8), (70, 512, 256, 16), (40, 256, 512, 8)])
+def test_layer_post_pre_equals_post_then_pre(device, dtype, rows, D, F, H):
+    """The one-launch layer boundary must give bit for bit what the two launches give: the
+    layer output between them is rounded to the storage type in both."""
+    from ar_nanotabpfn_amd import model as m
+
+    torch.manual_seed(1)
+    la = m.TwoStageTransformerLayer(D, H, F).to(device=device, dtype=dtype)
+    lb = m.TwoStageTransformerLayer(D, H, F).to(device=device, dtype=dtype)
+    B = rows  # one row per "batch" entry keeps the shapes general
+    y = randn((B, 1, D), 2, dtype, 1.0).to(device)
+    attn = randn((B, 1, H, D // H), 3, dtype).to(device).transpose(1, 2)
+    y2, q2, k2, v2 = la.finish_then_pre(y, attn, lb)
+    y1, q1, k1, v1 = lb.pre_attention(la.finish(y, attn))
+    for a, b in ((y1, y2), (q1, q2), (k1, k2), (v1, v2)):
+        assert a.shape == b.shape and torch.equal(a, b)
+
+
+def test_layer_post_pre_falls_back_when_not_covered(device):
+    """float32 layers (or widths outside the fused kernels) compose the same result from the
+    separate pieces."""
+    from ar_nanotabpfn_amd import model as m
+
+    torch.manual_seed(1)
+    la = m.TwoStageTransformerLayer(64, 2, 64).to(device)
+    lb = m.TwoStageTransformerLayer(64, 2, 64).to(device)
+    y = randn((8, 2, 64), 2, torch.float32).to(device)
+    attn = randn((8, 2, 2, 32), 3, torch.float32).to(device).transpose(1, 2)
+    got = la.finish_then_pre(y, attn, lb)
+    ref = lb.pre_attention(la.finish(y, attn))
+    for a, b in zip(got, ref):
+        assert torch.equal(a, b)

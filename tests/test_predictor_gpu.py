@@ -435,3 +435,43 @@ def test_graph_sampling_fused_tail_law(device):
         s = float(y3[:, col].std())
         assert abs(float(y1[:, col].mean() - y3[:, col].mean())) <= 6 * s / B ** 0.5 + 1e-2
         assert abs(float(y1[:, col].std()) - s) <= 0.1 * s + 1e-2
+
+
+def test_layer_by_layer_methods_equal_the_fused_stack(device):
+    """The reference-named per-layer methods (one layer = pre, attention, finish) against the
+    predictor's own pass over the stack, which fuses layer boundaries: teacher forcing on the
+    shared layout and one decode step, bf16."""
+    from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
+
+    cfg = dict(d_model=128, n_heads=4, n_layers=3, d_ff=128, num_features=2, buffer_size=4, num_components=3)
+    model = _build(cfg, device, dtype=torch.bfloat16)
+    B, Nc, Nt = 6, 48, 5
+    g = torch.Generator().manual_seed(3)
+    xc = torch.randn(1, Nc, 2, generator=g).expand(B, -1, -1).to(device, torch.bfloat16)
+    yc = torch.randn(1, Nc, generator=g).expand(B, -1).to(device, torch.bfloat16)
+    xt = torch.randn(B, Nt, 2, generator=g).to(device, torch.bfloat16)
+    yt = torch.randn(B, Nt, generator=g).to(device, torch.bfloat16)
+    pred = ARTabPFNPredictor.from_trained_model(model, backend="triton_shared_context")
+    pred.init_kv_cache(B, Nt, device, torch.bfloat16)
+    pred.prefill_context(xc, yc)
+    emb = pred._teacher_forcing_embedding(xt, yt)
+    z_stack = pred._teacher_forcing_decode_shared(emb, Nt)
+    x = emb
+    for layer in model.backbone.layers:
+        x = pred._layer_teacher_forcing_shared(layer, x, Nt)
+    z_layers = model.backbone.norm(x)
+    assert max_abs(to_np(z_stack), to_np(z_layers)) <= 2e-2
+
+    # one [buffer, target] decode step, twice from the same cache state
+    step = torch.cat([model.embedder.embed_buffer(xt[:, 0:1], yt[:, 0:1]) + model.ar_tokens[1],
+                      model.embedder.embed_target(xt[:, 1:2])], dim=1)
+    z1 = pred.transformer_decode(step, commit=1)
+    caches = [(l.k_buf_cache.clone(), l.v_buf_cache.clone()) for l in model.backbone.layers]
+    pred.buffer_len = 0
+    x = step
+    for layer in model.backbone.layers:
+        x = pred._layer_decode_with_cache_shared(layer, x, 1)
+    z2 = model.backbone.norm(x)
+    assert max_abs(to_np(z1), to_np(z2)) <= 2e-2
+    for (kc, vc), l in zip(caches, model.backbone.layers):
+        assert max_abs(to_np(kc[:, :, 0]), to_np(l.k_buf_cache[:, :, 0])) <= 2e-2
