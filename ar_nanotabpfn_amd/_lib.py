@@ -74,6 +74,10 @@ SIGNATURES = {
         _i,
         [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _p, _i, _i, _f, _i, _p, _sz, _i, _p],
     ),
+    "artab_decode_attention_overlapped": (
+        _i,
+        [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _p, _i, _i, _f, _i, _p, _sz, _i, _p, _p],
+    ),
     "artab_teacher_forcing_attention": (_i, [_VP, _VP, _VP, _VP, _VP, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "artab_prefill_attention": (_i, [_VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "artab_buffer_attention": (_i, [_VP, _VP, _VP, _p, _i64, _i64, _i64, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _p]),

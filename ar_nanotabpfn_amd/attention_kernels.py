@@ -219,6 +219,7 @@ def decode_attention(
     v_new: Optional[Tensor] = None,
     use_triton: bool = True,
     n_buf_device: Optional[Tensor] = None,
+    side_stream: Optional["torch.cuda.Stream"] = None,
 ) -> Tensor:
     """One decode step of row attention (inference.py:785-823) in one call.
 
@@ -231,6 +232,10 @@ def decode_attention(
     ``n_buf_device`` (one int32 on the device) makes the kernels read the committed
     length at run time, for launches recorded in a HIP graph; ``n_buf`` is then the
     upper bound that is validated against the cache capacity.
+
+    ``side_stream`` (a default-priority stream of the same device) lets the buffer pass
+    run next to the context pass (``artab_decode_attention_overlapped``); the call is
+    still ordered on the current stream.
     """
     dev = _lib.require_device(q, k_ctx, v_ctx, k_buf_cache, v_buf_cache, k_new, v_new)
     lib = _lib.load()
@@ -248,15 +253,17 @@ def decode_attention(
     qv, ov = _lib.view4(q), _lib.view4(out)
     kbv, vbv = _lib.view4(k_buf_cache), _lib.view4(v_buf_cache)
     knv, vnv = _lib.view4(k_new), _lib.view4(v_new)
-    _lib.check(
-        lib.artab_decode_attention(
-            _lib.ref(qv), _lib.ref(kv), _lib.ref(vv), _lib.ref(kbv), _lib.ref(vbv), _lib.ref(knv), _lib.ref(vnv),
-            _lib.ref(ov), B, H, Lq, Nc, int(n_buf),
-            ctypes.c_void_p(n_buf_device.data_ptr()) if n_buf_device is not None else None,
-            cap, Dh, 0.0, _lib.dtype_code(q.dtype),
-            ws_ptr, ws_bytes, _impl(use_triton), _lib.current_stream(dev),
-        )
+    args = (
+        _lib.ref(qv), _lib.ref(kv), _lib.ref(vv), _lib.ref(kbv), _lib.ref(vbv), _lib.ref(knv), _lib.ref(vnv),
+        _lib.ref(ov), B, H, Lq, Nc, int(n_buf),
+        ctypes.c_void_p(n_buf_device.data_ptr()) if n_buf_device is not None else None,
+        cap, Dh, 0.0, _lib.dtype_code(q.dtype),
+        ws_ptr, ws_bytes, _impl(use_triton), _lib.current_stream(dev),
     )
+    if side_stream is not None:
+        _lib.check(lib.artab_decode_attention_overlapped(*args, ctypes.c_void_p(side_stream.cuda_stream)))
+    else:
+        _lib.check(lib.artab_decode_attention(*args))
     return out
 
 

@@ -8,10 +8,12 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/artab_attention.h"
 #include "common.h"
 #include "decode_buffer.h"
+#include "decode_stream.h"
 #include "fused_layer.h"
 #include "glue_kernels.h"
 #include "mfma_flash.h"
@@ -235,6 +237,28 @@ static hipError_t launch_decode(const DecodeParams &P, int dtype, int Dh, int Lq
     return Lq == 1 ? launch_decode_lq<f16_t, 1>(P, Dh, stream) : launch_decode_lq<f16_t, 2>(P, Dh, stream);
 }
 
+// The streaming buffer pass: one wavefront per workgroup, two per CU.
+template <typename T>
+static hipError_t launch_stream_t(const DecodeParams &P, int Lq, hipStream_t stream) {
+    const long pairs = static_cast<long>(P.B) * P.H;
+    if (pairs == 0) return hipSuccess;
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        cus = 256;
+    const long tasks = (pairs + 15) / 16;
+    dim3 grid(static_cast<unsigned>(tasks < 2L * cus ? tasks : 2L * cus)), block(64);
+    if (Lq == 1)
+        hipLaunchKernelGGL((decode_stream_kernel<T, 1>), grid, block, kStreamLdsBytes, stream, P);
+    else
+        hipLaunchKernelGGL((decode_stream_kernel<T, 2>), grid, block, kStreamLdsBytes, stream, P);
+    return hipGetLastError();
+}
+
+static hipError_t launch_stream(const DecodeParams &P, int dtype, int Lq, hipStream_t stream) {
+    return dtype == ARTAB_BF16 ? launch_stream_t<bf16_t>(P, Lq, stream) : launch_stream_t<f16_t>(P, Lq, stream);
+}
+
 static hipError_t launch_portable_dtype(const PortableParams &P, int dtype, hipStream_t stream) {
     switch (dtype) {
         case ARTAB_BF16: return launch_portable<bf16_t>(P, stream);
@@ -303,6 +327,35 @@ using namespace artab;
 static int launch_status(hipError_t e, const char *what) {
     if (e == hipSuccess) return ARTAB_OK;
     return fail(ARTAB_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+// Event pairs for forking work onto a side stream and joining it back; a small ring per
+// device, created on first use (timing disabled).  A wait binds to the record that precedes it,
+// so re-recording an event of the ring later does not disturb earlier waits.
+static int fork_join_events(hipEvent_t *fork, hipEvent_t *join) {
+    constexpr int kDevices = 16, kRing = 8;
+    struct Ring {
+        hipEvent_t ev[2 * kRing];
+        int next = 0;
+        bool ready = false;
+    };
+    static Ring rings[kDevices];
+    static std::mutex mu;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kDevices)
+        return fail(ARTAB_ERR_UNSUPPORTED, "no current HIP device (or index above %d)", kDevices - 1);
+    std::lock_guard<std::mutex> lock(mu);
+    Ring &r = rings[dev];
+    if (!r.ready) {
+        for (int i = 0; i < 2 * kRing; ++i)
+            if (hipEventCreateWithFlags(&r.ev[i], hipEventDisableTiming) != hipSuccess)
+                return fail(ARTAB_ERR_LAUNCH, "hipEventCreateWithFlags failed");
+        r.ready = true;
+    }
+    *fork = r.ev[2 * r.next];
+    *join = r.ev[2 * r.next + 1];
+    r.next = (r.next + 1) % kRing;
+    return ARTAB_OK;
 }
 
 namespace {
@@ -451,7 +504,8 @@ size_t artab_workspace_bytes(int B, int H, int Lq, int Nc, int Dh, int dtype) {
     FlashPlan a = plan_flash(B, H, Lq, Nc, Dh, /*stacked=*/true, /*allow_split=*/true);
     FlashPlan b = plan_flash(B, H, Lq, Nc, Dh, /*stacked=*/false, /*allow_split=*/true);
     const int n_split = a.n_split > b.n_split ? a.n_split : b.n_split;
-    return split_workspace_bytes(static_cast<long>(B) * H * Lq, Dh, n_split);
+    // one slot more than the context slices: the streaming buffer pass leaves a partial of its own
+    return split_workspace_bytes(static_cast<long>(B) * H * Lq, Dh, n_split + 1);
 }
 
 int artab_context_attention(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
@@ -526,11 +580,12 @@ int artab_context_attention(const artab_view *q, const artab_view *k_ctx, const 
     return ARTAB_OK;
 }
 
-int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
-                           const artab_view *k_buf, const artab_view *v_buf, const artab_view *k_new,
-                           const artab_view *v_new, const artab_view *out, int B, int H, int Lq, int Nc,
-                           int n_buf, const int32_t *n_buf_device, int buf_capacity, int Dh, float scale,
-                           int dtype, void *workspace, size_t workspace_bytes, int impl, void *stream) {
+static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                       const artab_view *k_buf, const artab_view *v_buf, const artab_view *k_new,
+                       const artab_view *v_new, const artab_view *out, int B, int H, int Lq, int Nc,
+                       int n_buf, const int32_t *n_buf_device, int buf_capacity, int Dh, float scale,
+                       int dtype, void *workspace, size_t workspace_bytes, int impl, void *stream,
+                       void *side_stream) {
     ARTAB_TRY(check_common(B, H, Lq, Dh, dtype));
     if (Lq != 1 && Lq != 2)
         return fail(ARTAB_ERR_BAD_SHAPE, "decode supports Lq=1 (target) or Lq=2 (buffer, target); got %d", Lq);
@@ -564,10 +619,15 @@ int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const a
     const long rows = static_cast<long>(B) * H * Lq;
     FlashPlan pl;
     size_t need_ws = 0;
+    bool stream_buf = false;
     if (use_mfma) {
         pl = plan_flash(B, H, Lq, Nc, Dh, /*stacked=*/true, /*allow_split=*/true);
         const bool direct = !need_buf && pl.n_split == 1;  // context pass writes the final output
-        need_ws = direct ? 0 : split_workspace_bytes(rows, Dh, pl.n_split);
+        // the streaming buffer pass exists for head_dim 32 (the shape whose context pass leaves room
+        // for it on a SIMD); it is used when the caller offers a second stream to run it on
+        stream_buf = need_buf && Dh == 32 &&
+                     ((side_stream && side_stream != stream) || env_int("ARTAB_STREAM", 0) != 0);
+        need_ws = direct ? 0 : split_workspace_bytes(rows, Dh, pl.n_split + (stream_buf ? 1 : 0));
         if (need_ws && (!workspace || workspace_bytes < need_ws || reinterpret_cast<uintptr_t>(workspace) % 16)) {
             if (impl == ARTAB_IMPL_MFMA)
                 return fail(ARTAB_ERR_WORKSPACE, "decode needs %zu workspace bytes, got %zu", need_ws,
@@ -601,23 +661,82 @@ int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const a
     F.n_split = pl.n_split; F.kv_per_split = pl.kv_per_split;
     F.qscale = scale * kLog2e;
     F.mode = kFlashContext;
+    const int slots = pl.n_split + (stream_buf ? 1 : 0);
     if (need_ws) {
         F.part_o = workspace;
-        F.part_lse = split_lse_base(workspace, rows, Dh, pl.n_split);
+        F.part_lse = split_lse_base(workspace, rows, Dh, slots);
     }
-    {
-        ProfileScope prof(st);
-        ARTAB_TRY(launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "decode context pass"));
-    }
-    if (!need_ws) return ARTAB_OK;
-
     DecodeParams D;
     memset(&D, 0, sizeof(D));
     D.q = dv(q); D.kb = dv(k_buf); D.vb = dv(v_buf); D.knew = dv(k_new); D.vnew = dv(v_new); D.out = dv(out);
     D.part_o = F.part_o; D.part_lse = F.part_lse; D.lse = nullptr;
     D.B = B; D.H = H; D.n_split = pl.n_split; D.n_buf = n_buf; D.n_buf_dev = n_buf_device; D.has_new = has_new;
     D.qscale = scale * kLog2e;
-    return launch_status(launch_decode(D, dtype, Dh, Lq, st), "decode buffer pass");
+
+    if (!stream_buf) {
+        {
+            ProfileScope prof(st);
+            ARTAB_TRY(launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "decode context pass"));
+        }
+        if (!need_ws) return ARTAB_OK;
+        return launch_status(launch_decode(D, dtype, Dh, Lq, st), "decode buffer pass");
+    }
+
+    // Streaming schedule: the buffer pass (HBM-bound, on the matrix pipe) leaves its result as one
+    // more partial; with a side stream it runs next to the context pass (forked and joined with
+    // events, so the call stays ordered on `stream` and can be recorded into a graph).
+    D.buf_part_o = static_cast<char *>(workspace) + static_cast<size_t>(pl.n_split) * rows * Dh * 2;
+    D.buf_part_lse = F.part_lse + static_cast<size_t>(pl.n_split) * rows;
+    hipStream_t side = (side_stream && side_stream != stream) ? static_cast<hipStream_t>(side_stream) : st;
+    hipEvent_t fork = nullptr, join = nullptr;
+    if (side != st) {
+        ARTAB_TRY(fork_join_events(&fork, &join));
+        hipError_t e = hipEventRecord(fork, st);
+        if (e == hipSuccess) e = hipStreamWaitEvent(side, fork, 0);
+        if (e != hipSuccess) return launch_status(e, "decode fork");
+    }
+    hipError_t e_ctx, e_buf, e_join = hipSuccess;
+    {
+        ProfileScope prof(st);
+        e_ctx = launch_flash_dtype(F, dtype, Dh, pl.BM, st);
+    }
+    e_buf = launch_stream(D, dtype, Lq, side);
+    if (side != st) {
+        // always rejoin, so that a failed launch does not leave the side stream forked (e.g. inside a capture)
+        e_join = hipEventRecord(join, side);
+        if (e_join == hipSuccess) e_join = hipStreamWaitEvent(st, join, 0);
+    }
+    ARTAB_TRY(launch_status(e_ctx, "decode context pass"));
+    ARTAB_TRY(launch_status(e_buf, "decode buffer pass (stream)"));
+    ARTAB_TRY(launch_status(e_join, "decode join"));
+    CombineParams C;
+    C.out = dv(out); C.part_o = F.part_o; C.part_lse = F.part_lse; C.lse = nullptr;
+    C.rows = rows; C.H = H; C.Lq = Lq; C.Dh = Dh; C.n_split = slots;
+    unsigned cgrid = static_cast<unsigned>((rows * (Dh / 4) + 255) / 256);
+    if (dtype == ARTAB_BF16)
+        hipLaunchKernelGGL((combine_kernel<bf16_t>), dim3(cgrid), dim3(256), 0, st, C);
+    else
+        hipLaunchKernelGGL((combine_kernel<f16_t>), dim3(cgrid), dim3(256), 0, st, C);
+    return launch_status(hipGetLastError(), "decode combine");
+}
+
+int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                           const artab_view *k_buf, const artab_view *v_buf, const artab_view *k_new,
+                           const artab_view *v_new, const artab_view *out, int B, int H, int Lq, int Nc,
+                           int n_buf, const int32_t *n_buf_device, int buf_capacity, int Dh, float scale,
+                           int dtype, void *workspace, size_t workspace_bytes, int impl, void *stream) {
+    return decode_impl(q, k_ctx, v_ctx, k_buf, v_buf, k_new, v_new, out, B, H, Lq, Nc, n_buf, n_buf_device,
+                       buf_capacity, Dh, scale, dtype, workspace, workspace_bytes, impl, stream, nullptr);
+}
+
+int artab_decode_attention_overlapped(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                                      const artab_view *k_buf, const artab_view *v_buf, const artab_view *k_new,
+                                      const artab_view *v_new, const artab_view *out, int B, int H, int Lq, int Nc,
+                                      int n_buf, const int32_t *n_buf_device, int buf_capacity, int Dh, float scale,
+                                      int dtype, void *workspace, size_t workspace_bytes, int impl, void *stream,
+                                      void *side_stream) {
+    return decode_impl(q, k_ctx, v_ctx, k_buf, v_buf, k_new, v_new, out, B, H, Lq, Nc, n_buf, n_buf_device,
+                       buf_capacity, Dh, scale, dtype, workspace, workspace_bytes, impl, stream, side_stream);
 }
 
 int artab_teacher_forcing_attention(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,

@@ -20,6 +20,8 @@ struct DecodeParams {
     const void *part_o;     // [n_split][B*H*Lq][DH] normalised context partials, input type
     const float *part_lse;  // [n_split][B*H*Lq] natural-log LSE of each partial
     float *lse;             // optional final LSE [B,H,Lq]
+    void *buf_part_o;       // streaming variant only: the buffer pass's own partial, [B*H*Lq][DH] input type,
+    float *buf_part_lse;    // and its natural-log LSE [B*H*Lq]
     int B, H;
     int n_split;
     int n_buf;    // committed buffer rows

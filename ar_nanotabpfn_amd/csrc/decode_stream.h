@@ -1,0 +1,296 @@
+// Decode-step buffer pass on the matrix pipe, as a light background stream (gfx950, head_dim 32).
+//
+// The context pass of a decode step is bound by the vector and matrix units and leaves HBM idle;
+// the buffer pass streams B*H*n_buf*128 bytes and needs almost no arithmetic.  To run the two side
+// by side the buffer pass has to fit in what two resident context-pass wavefronts leave on a SIMD
+// (80 registers, one wavefront) and must not compete for vector-ALU issue slots.  Hence:
+//
+//  * dot products on the matrix pipe with v_mfma_f32_4x4x4 (16 independent 4x4x4 products per
+//    instruction): one block = one (trajectory, head) pair, lane 4p+i of a wavefront is
+//    (pair p, index i).  Scores S^T[key i][query j] = K[key i] . Q[query j]: A operand = 4
+//    head-dim elements of key row i (lane (p,i)), B operand = the same 4 elements of query j
+//    (lane (p,j); zero for j >= Lq), result: lane (p,j) holds the 4 keys' scores of query j.
+//    O^T[dim][query j] += V^T[dim][key] P^T[key][query j]: B operand = the lane's own four
+//    probabilities, A operand = V[key 0..3][dim] fetched with the transposing LDS read
+//    ds_read_b64_tr_b16; lane (p,j) accumulates all 32 output dims of query j.
+//    Softmax state (max, sum) is one scalar per lane.  About 35 vector instructions, 16 MFMAs
+//    (8 cycles each) and 16 LDS reads per 4 keys x 16 pairs.
+//  * loads land in LDS, not in registers: every wavefront keeps a ring of 8 KiB chunks (4 keys x
+//    16 pairs x K and V) filled by direct global->LDS loads (16 bytes per lane, lane l lands at
+//    chunk + 16 l), three chunks in flight while one is consumed, and reads a chunk back
+//    lane-locally (K) or transposed (V).
+//
+// Output per (pair, query): normalised partial result in the input type + float32 LSE, i.e. one
+// more "context slice" for the combine step; the new row is appended to the cache on the way.
+#pragma once
+
+#include "common.h"
+#include "decode_buffer.h"
+
+namespace artab {
+
+constexpr int kStreamChunks = 4;           // ring depth per wavefront
+constexpr int kStreamChunkBytes = 8192;    // 4 keys x 16 pairs x (64 B of K + 64 B of V)
+constexpr int kStreamQBytes = 4096;        // one task's queries: 4 x (64 lanes x 16 B)
+constexpr size_t kStreamLdsBytes = kStreamChunks * kStreamChunkBytes + 2 * kStreamQBytes;
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding).
+constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
+
+// 16 bytes per lane from global memory straight into LDS: lane l lands at lds + 16 l (lds is
+// wavefront-uniform).  Kept in a plain function: called directly from a kernel template the
+// builtin makes the host pass drop the kernel's launch stub.
+__device__ __forceinline__ void load_to_lds_16(const void *global_src, void *lds_dst) {
+    __builtin_amdgcn_global_load_lds(global_src, lds_dst, 16, 0, 0);
+}
+
+// LDS reads of the ring go through inline assembly: the compiler must not see an LDS read that
+// could alias the asynchronous fills, or it would drain every load before each read.
+__device__ __forceinline__ void lds_read2x128(u32x4 &a, u32x4 &b, unsigned addr) {
+    asm volatile(
+        "ds_read_b128 %0, %2\n\t"
+        "ds_read_b128 %1, %2 offset:1024\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(a), "=&v"(b)
+        : "v"(addr)
+        : "memory");
+}
+// Eight transposing reads: the V operands of the eight 4-dim groups of one 4-key chunk.
+// Address layout of a V chunk: sub-slot t (1 KiB) holds dims 8t..8t+7, so group u = 2t + half
+// sits at t * 1024 + 8 * half.
+__device__ __forceinline__ void lds_read8_tr(u32x2 (&v)[8], unsigned addr) {
+    asm volatile(
+        "ds_read_b64_tr_b16 %0, %8\n\t"
+        "ds_read_b64_tr_b16 %1, %8 offset:8\n\t"
+        "ds_read_b64_tr_b16 %2, %8 offset:1024\n\t"
+        "ds_read_b64_tr_b16 %3, %8 offset:1032\n\t"
+        "ds_read_b64_tr_b16 %4, %8 offset:2048\n\t"
+        "ds_read_b64_tr_b16 %5, %8 offset:2056\n\t"
+        "ds_read_b64_tr_b16 %6, %8 offset:3072\n\t"
+        "ds_read_b64_tr_b16 %7, %8 offset:3080\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
+        : "v"(addr)
+        : "memory");
+}
+
+template <typename T>
+struct Mfma4;
+template <>
+struct Mfma4<bf16_t> {
+    static __device__ __forceinline__ f32x4 mma(u32x2 a, u32x2 b, f32x4 c) {
+        typedef __bf16 v4bf __attribute__((ext_vector_type(4)));
+        return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(v4bf, a), __builtin_bit_cast(v4bf, b), c, 0,
+                                                      0, 0);
+    }
+};
+template <>
+struct Mfma4<f16_t> {
+    static __device__ __forceinline__ f32x4 mma(u32x2 a, u32x2 b, f32x4 c) {
+        typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+        return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(v4h, a), __builtin_bit_cast(v4h, b), c, 0, 0, 0);
+    }
+};
+
+// One wavefront per workgroup; a task = 16 consecutive (trajectory, head) pairs; tasks are dealt
+// round-robin over the grid.  Dynamic LDS: kStreamLdsBytes.
+template <typename T, int LQ>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void decode_stream_kernel(DecodeParams P) {
+    constexpr int DH = 32;
+    constexpr int S = kStreamChunks;
+    extern __shared__ __attribute__((aligned(16))) unsigned char stream_lds[];
+
+    // Every argument the loop needs, as plain values: the inline assembly clobbers memory, and
+    // anything still read through the argument block would be re-read after every such statement.
+    const View vq = P.q, vkb = P.kb, vvb = P.vb, vkn = P.knew, vvn = P.vnew;
+    const int H = P.H, has_new = P.has_new;
+    const float qscale = P.qscale;
+    T *const part_o = static_cast<T *>(P.buf_part_o);
+    float *const part_lse = P.buf_part_lse;
+    const int n_pairs = P.B * H;
+    const int n_buf = P.n_buf_dev ? *P.n_buf_dev : P.n_buf;
+    const int n_total = n_buf + (has_new ? 1 : 0);
+
+    const int lane = threadIdx.x;
+    const int pl = lane >> 2, sub = lane & 3;  // pair within the task, row / query index
+    const int n_tasks = (n_pairs + 15) / 16;
+    const int n_groups = (n_total + 3) / 4;    // 4-key chunks per task
+
+    const unsigned lds0 = static_cast<unsigned>(reinterpret_cast<uintptr_t>(stream_lds));
+    const unsigned q_lds0 = lds0 + S * kStreamChunkBytes;
+    // transposing read: within a 16-lane group lane L supplies the row of (pair L%4, key L/4)
+    const unsigned tr_off = 16u * (4u * (4u * (lane >> 4) + (lane & 3)) + ((lane & 15) >> 2));
+
+    if (n_total == 0) {  // nothing to attend to: empty partials (weight 0 in the combine)
+        for (int task = blockIdx.x; task < n_tasks; task += gridDim.x) {
+            const int pair = 16 * task + pl;
+            if (pair < n_pairs && sub < LQ) {
+                part_lse[static_cast<long>(pair) * LQ + sub] = -INFINITY;
+                u32x4 z = {0u, 0u, 0u, 0u};
+                T *po = part_o + (static_cast<long>(pair) * LQ + sub) * DH;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) *reinterpret_cast<u32x4 *>(po + 8 * e) = z;
+            }
+        }
+        return;
+    }
+
+    // This wavefront shares its SIMD with two older, compute-bound ones; without a raised
+    // priority it is only issued in their gaps.  It issues little: the priority costs them little.
+    __builtin_amdgcn_s_setprio(3);
+
+    // ---- producer: chunk `issue_g` of task `issue_task` into ring slot issue_slot
+    const int my_tasks = blockIdx.x < n_tasks ? (n_tasks - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+    const int total_chunks = my_tasks * n_groups;
+    int issued = 0, issue_task = blockIdx.x, issue_g = 0, issue_slot = 0, issue_q = 0;
+    int issue_seq = 0, seq = 0;  // how many of this wavefront's tasks the producer / consumer have finished
+    auto issue_one = [&]() {
+        int pair = 16 * issue_task + pl;
+        pair = pair < n_pairs ? pair : n_pairs - 1;  // a ragged last task re-reads the last pair; never stored
+        const int b = pair / H, h = pair % H;
+        if (issue_g == 0) {
+            // the task's queries: lane (p, j < LQ) fetches its 64-byte row in four pieces
+            const T *qrow = view_row<T>(vq, b, h, sub < LQ ? sub : 0);
+            unsigned char *qd = stream_lds + S * kStreamChunkBytes + issue_q * kStreamQBytes;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) load_to_lds_16(qrow + 8 * t, qd + 1024 * t);
+        }
+        int row = 4 * issue_g + sub;
+        row = row < n_total ? row : n_total - 1;  // keys past the end re-read the last one and are masked
+        const bool is_new = has_new && row == n_buf;
+        const T *kr = is_new ? view_row<T>(vkn, b, h, 0) : view_row<T>(vkb, b, h, row);
+        const T *vr = is_new ? view_row<T>(vvn, b, h, 0) : view_row<T>(vvb, b, h, row);
+        unsigned char *cd = stream_lds + issue_slot * kStreamChunkBytes;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) load_to_lds_16(kr + 8 * t, cd + 1024 * t);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) load_to_lds_16(vr + 8 * t, cd + 4096 + 1024 * t);
+        ++issued;
+        issue_slot = issue_slot + 1 == S ? 0 : issue_slot + 1;
+        if (++issue_g == n_groups) {
+            issue_g = 0;
+            issue_task += gridDim.x;
+            issue_q ^= 1;
+            ++issue_seq;
+        }
+    };
+    // two query slots: the producer may be at most one task ahead of the consumer
+    auto may_issue = [&]() { return issued < total_chunks && issue_seq <= seq + 1; };
+    for (int i = 0; i < S; ++i)
+        if (may_issue()) issue_one();
+
+    // ---- consumer
+    float m = -INFINITY, l = 0.f;
+    f32x4 o[8];  // output dims 4u..4u+3 of this lane's query
+#pragma unroll
+    for (int u = 0; u < 8; ++u) o[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+    int task = blockIdx.x, g = 0, slot = 0, qsel = 0;
+    for (int c = 0; c < total_chunks; ++c) {
+        // chunk c must have landed; only the chunks requested after it (8 loads each) may be pending
+        switch (issued - c - 1) {
+            case 3: __builtin_amdgcn_s_waitcnt(vmcnt_imm(24)); break;
+            case 2: __builtin_amdgcn_s_waitcnt(vmcnt_imm(16)); break;
+            case 1: __builtin_amdgcn_s_waitcnt(vmcnt_imm(8)); break;
+            default: __builtin_amdgcn_s_waitcnt(vmcnt_imm(0)); break;
+        }
+        const unsigned chunk = lds0 + static_cast<unsigned>(slot) * kStreamChunkBytes;
+        const unsigned qaddr = q_lds0 + static_cast<unsigned>(qsel) * kStreamQBytes + lane * 16u;
+
+        int pair = 16 * task + pl;
+        const bool pair_ok = pair < n_pairs;
+        pair = pair_ok ? pair : n_pairs - 1;
+        const int b = pair / H, h = pair % H;
+        const bool appends = has_new && 4 * g + sub == n_buf && pair_ok;
+        T *const kd = view_row<T>(vkb, b, h, n_buf), *const vd = view_row<T>(vvb, b, h, n_buf);
+
+        // ---- scores of 4 keys for this lane's query, head dims in two halves (register budget).
+        // Lanes that stand for no query (sub >= LQ) multiply by zero.
+        f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            u32x4 k0, k1, q0, q1;
+            lds_read2x128(k0, k1, chunk + 2048u * half + lane * 16u);
+            lds_read2x128(q0, q1, qaddr + 2048u * half);
+            if (appends) {  // in-place append: this lane holds the new K row
+                *reinterpret_cast<u32x4 *>(kd + 16 * half) = k0;
+                *reinterpret_cast<u32x4 *>(kd + 16 * half + 8) = k1;
+            }
+            if (sub >= LQ) {
+                q0 = u32x4{0u, 0u, 0u, 0u};
+                q1 = q0;
+            }
+            s = Mfma4<T>::mma(u32x2{k0[0], k0[1]}, u32x2{q0[0], q0[1]}, s);
+            s = Mfma4<T>::mma(u32x2{k0[2], k0[3]}, u32x2{q0[2], q0[3]}, s);
+            s = Mfma4<T>::mma(u32x2{k1[0], k1[1]}, u32x2{q1[0], q1[1]}, s);
+            s = Mfma4<T>::mma(u32x2{k1[2], k1[3]}, u32x2{q1[2], q1[3]}, s);
+        }
+        if (appends) {  // ... and reads its V row back lane-locally
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                u32x4 v0, v1;
+                lds_read2x128(v0, v1, chunk + 4096u + 2048u * half + lane * 16u);
+                *reinterpret_cast<u32x4 *>(vd + 16 * half) = v0;
+                *reinterpret_cast<u32x4 *>(vd + 16 * half + 8) = v1;
+            }
+        }
+        float sc[4];
+        float cm = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            sc[r] = 4 * g + r < n_total ? s[r] * qscale : -INFINITY;
+            cm = fmaxf(cm, sc[r]);
+        }
+        // online softmax; the rescale is skipped (wavefront-uniformly) while no maximum moves
+        const float m_new = fmaxf(m, cm);
+        if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
+            const float alpha = m == -INFINITY ? 0.f : fast_exp2(m - m_new);
+            l *= alpha;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) o[u] *= alpha;
+            m = m_new;
+        }
+        float p[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            p[r] = fast_exp2(sc[r] - m);  // m is finite here: key 4g is always valid
+            l += p[r];
+        }
+        const u32x2 pop = {pack2<T>(p[0], p[1]), pack2<T>(p[2], p[3])};
+        {
+            u32x2 vop[8];
+            lds_read8_tr(vop, chunk + 4096u + tr_off);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) o[u] = Mfma4<T>::mma(vop[u], pop, o[u]);
+        }
+        // the chunk has been read: refill its slot (and any the producer had to leave empty)
+        const bool task_ends = g + 1 == n_groups;
+        if (task_ends) ++seq;
+        while (may_issue() && issued - c - 1 < S) issue_one();
+
+        slot = slot + 1 == S ? 0 : slot + 1;
+        if (++g == n_groups) {
+            // ---- task done: write this lane's partial (lanes of real queries of real pairs)
+            if (pair_ok && sub < LQ) {
+                const float inv = l > 0.f ? 1.f / l : 0.f;
+                T *po = part_o + (static_cast<long>(pair) * LQ + sub) * DH;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    u32x4 val = {pack2<T>(o[2 * e][0] * inv, o[2 * e][1] * inv), pack2<T>(o[2 * e][2] * inv, o[2 * e][3] * inv),
+                                 pack2<T>(o[2 * e + 1][0] * inv, o[2 * e + 1][1] * inv),
+                                 pack2<T>(o[2 * e + 1][2] * inv, o[2 * e + 1][3] * inv)};
+                    *reinterpret_cast<u32x4 *>(po + 8 * e) = val;
+                }
+                part_lse[static_cast<long>(pair) * LQ + sub] = l > 0.f ? (m + fast_log2(l)) * kLn2 : -INFINITY;
+            }
+            m = -INFINITY;
+            l = 0.f;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) o[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+            g = 0;
+            task += gridDim.x;
+            qsel ^= 1;
+        }
+    }
+}
+
+}  // namespace artab

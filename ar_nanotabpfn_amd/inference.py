@@ -61,6 +61,10 @@ class ARTabPFNPredictor:
         # layout on a HIP device only).  Set to False to launch every kernel from Python.
         self.use_hip_graph = True
         self.fuse_step_tail = True   # head + draw + next embedding as one launch inside the graph
+        # Run the HBM-bound buffer pass of a decode step on a second stream, next to the
+        # compute-bound context pass (shared layout, HIP device).
+        self.overlap_buffer_pass = True
+        self._side_streams = {}
         self._graph_state = None
 
     @classmethod
@@ -106,6 +110,14 @@ class ARTabPFNPredictor:
             H, Dh = layer.attn_rows.n_heads, layer.attn_rows.head_dim
             zeros(layer, "k_cache", (batch_size, H, max_seq_len, Dh))
             zeros(layer, "v_cache", (batch_size, H, max_seq_len, Dh))
+
+    def _side_stream(self, device):
+        if device.type != "cuda":
+            return None
+        key = device.index if device.index is not None else torch.cuda.current_device()
+        if key not in self._side_streams:
+            self._side_streams[key] = torch.cuda.Stream(device=device)  # default priority
+        return self._side_streams[key]
 
     def clear_cache(self) -> None:
         """Reset the cursors, keep the memory (inference.py:137-141)."""
@@ -206,13 +218,14 @@ class ARTabPFNPredictor:
         v_ctx = layer.v_ctx_cache[:, : self.context_len]
         # with a device-side length the host value is only the bound that is validated
         n_buf = self.buffer_len if n_buf_device is None else self.max_buffer_len - (N - 1)
+        side = self._side_stream(q.device) if self.overlap_buffer_pass else None
         if N == 1:
             attn = ak.decode_attention(q, k_ctx, v_ctx, layer.k_buf_cache, layer.v_buf_cache, n_buf,
-                                       n_buf_device=n_buf_device)
+                                       n_buf_device=n_buf_device, side_stream=side)
         else:
             attn = ak.decode_attention(
                 q, k_ctx, v_ctx, layer.k_buf_cache, layer.v_buf_cache, n_buf,
-                k_new[:, :, 0:1], v_new[:, :, 0:1], n_buf_device=n_buf_device,
+                k_new[:, :, 0:1], v_new[:, :, 0:1], n_buf_device=n_buf_device, side_stream=side,
             )
         return attn
 
@@ -339,7 +352,7 @@ class ARTabPFNPredictor:
         params = list(self.backbone.parameters()) + list(self.embedder.parameters()) + list(self.head.parameters())
         params.append(self.ar_tokens)
         key = (B, Nt, F_, self.context_len, dtype, str(device), layer0.k_ctx_cache.data_ptr(),
-               layer0.k_buf_cache.data_ptr(), self.fuse_step_tail, tuple((p.data_ptr(), p._version) for p in params))
+               layer0.k_buf_cache.data_ptr(), self.fuse_step_tail, self.overlap_buffer_pass, tuple((p.data_ptr(), p._version) for p in params))
         st = self._graph_state
         if st is None or st.key != key:
             st = _GraphState()

@@ -138,6 +138,29 @@ int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const a
                            void *workspace, size_t workspace_bytes, int impl, void *stream);
 
 /*
+ * artab_decode_attention with the two passes side by side.  The context pass (bound by the
+ * matrix and vector units) is launched on `stream`; the buffer pass (bound by HBM) on
+ * `side_stream`, forked from and joined back into `stream` with events, so the call is ordered
+ * like the plain one from the caller's point of view and may be recorded into a graph.  For
+ * head_dim 32 on the MFMA path the buffer pass is a streaming kernel built to share a SIMD with
+ * the context pass (dot products on the matrix pipe, loads landing in LDS); it leaves its result
+ * as one more partial and a combine launch on `stream` writes `out`.  The workspace of
+ * artab_workspace_bytes covers the extra partial.  Same arguments, same results to rounding (the
+ * merge order differs).  With a NULL side_stream, side_stream == stream, another head_dim or a
+ * call the MFMA path does not cover it behaves exactly like artab_decode_attention.  Both streams
+ * must belong to the current device and have the default priority.
+ * The reference has no counterpart: it runs the two passes back to back
+ * (ar_tabpfn/model/triton_kernels.py:705-755).
+ */
+int artab_decode_attention_overlapped(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                           const artab_view *k_buf, const artab_view *v_buf,
+                           const artab_view *k_new, const artab_view *v_new,
+                           const artab_view *out,
+                           int B, int H, int Lq, int Nc, int n_buf, const int32_t *n_buf_device,
+                           int buf_capacity, int Dh, float scale, int dtype,
+                           void *workspace, size_t workspace_bytes, int impl, void *stream, void *side_stream);
+
+/*
  * Teacher-forced attention over [Buffer_0..Nt-1, Target_0..Nt-1] queries.
  * Replaces hybrid_teacher_forcing_attention (triton_kernels.py:662-702: context
  * pass + masked buffer pass :620-659 + merge) and, with a per-batch context, the

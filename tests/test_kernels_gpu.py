@@ -113,8 +113,9 @@ def test_context_attention_strided_q_view(device):
 # ----- decode step ------------------------------------------------------------------------------
 
 
-def _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, use_mfma, scale=1.0, seed=3):
+def _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, use_mfma, scale=1.0, seed=3, overlapped=False):
     ak = _ak()
+    side = torch.cuda.Stream(device=device) if overlapped else None
     q, k_ctx, v_ctx = _ctx_inputs(B, H, Lq, Nc, D, dtype, seed=seed, scale=scale)
     k_cache = randn((B, H, cap, D), seed + 10, dtype, scale)
     v_cache = randn((B, H, cap, D), seed + 11, dtype, scale)
@@ -124,6 +125,7 @@ def _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, use_mfma,
     out = ak.decode_attention(
         q.to(device), k_ctx.to(device), v_ctx.to(device), kc_d, vc_d, n_buf,
         k_new.to(device) if with_new else None, v_new.to(device) if with_new else None, use_triton=use_mfma,
+        side_stream=side,
     )
     ref, k_all, v_all = ao.decode_step_attention(
         to_np(q), to_np(k_ctx), to_np(v_ctx), to_np(k_cache[:, :, :n_buf]), to_np(v_cache[:, :, :n_buf]),
@@ -156,6 +158,69 @@ def _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, use_mfma,
 )
 def test_decode_attention_matches_oracle(device, dtype, use_mfma, B, H, Lq, Nc, D, n_buf, cap, with_new):
     _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, use_mfma)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize(
+    "B,H,Lq,Nc,D,n_buf,cap,with_new",
+    [
+        (8, 4, 1, 64, 32, 0, 16, False),  # nothing for the buffer pass to do: plain schedule
+        (8, 4, 2, 64, 32, 0, 16, True),   # the new row alone
+        (8, 4, 2, 64, 32, 3, 16, True),   # exactly one 4-key chunk
+        (8, 4, 2, 64, 32, 15, 16, True),  # last slot
+        (8, 4, 1, 64, 32, 7, 16, False),  # target only over committed buffers, ragged last chunk
+        (5, 3, 2, 200, 32, 22, 40, True),  # 15 pairs: one ragged task
+        (33, 8, 2, 100, 64, 19, 64, True),  # other head dims: register-staged buffer pass
+        (5, 2, 2, 300, 128, 70, 80, True),
+        (128, 8, 2, 8192, 32, 100, 128, True),  # split context + streamed buffer partial + combine
+        (600, 8, 2, 1024, 32, 37, 64, True),  # more tasks than workgroups: several tasks per wavefront
+        (4, 3, 2, 50, 16, 9, 12, True),  # portable-only head_dim: side stream is ignored
+    ],
+)
+def test_decode_attention_overlapped_matches_oracle(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new):
+    """Buffer pass on a side stream next to the context pass, then the combine launch."""
+    _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, True, scale=0.6, overlapped=True)
+
+
+def test_decode_attention_overlapped_device_length_in_graph(device):
+    """The overlapped call recorded into a graph (fork/join inside the capture) with the buffer
+    length in device memory: every replay appends one row and must equal the eager plain call."""
+    ak = _ak()
+    dtype, B, H, Nc, D, cap = torch.bfloat16, 64, 8, 2048, 32, 8
+    q, k_ctx, v_ctx = (t.to(device) for t in _ctx_inputs(B, H, 2, Nc, D, dtype, seed=1, scale=0.6))
+    k_cache, v_cache = randn((B, H, cap, D), 2, dtype, 0.6).to(device), randn((B, H, cap, D), 3, dtype, 0.6).to(device)
+    k_ref, v_ref = k_cache.clone(), v_cache.clone()
+    k_new, v_new = randn((B, H, 1, D), 4, dtype, 0.6).to(device), randn((B, H, 1, D), 5, dtype, 0.6).to(device)
+    nbuf = torch.zeros(1, dtype=torch.int32, device=device)
+    side = torch.cuda.Stream(device=device)
+    out_static = torch.empty_like(q)
+
+    def step():
+        out_static.copy_(ak.decode_attention(q, k_ctx, v_ctx, k_cache, v_cache, cap - 1, k_new, v_new,
+                                             n_buf_device=nbuf, side_stream=side))
+        nbuf.add_(1)
+
+    warm = torch.cuda.Stream(device=device)
+    warm.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(warm):
+        step()
+    torch.cuda.current_stream(device).wait_stream(warm)
+    nbuf.zero_()
+    k_cache.copy_(k_ref)
+    v_cache.copy_(v_ref)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    nbuf.zero_()
+    k_cache.copy_(k_ref)
+    v_cache.copy_(v_ref)
+    for n in range(6):
+        graph.replay()
+        torch.cuda.synchronize()
+        expect = ak.decode_attention(q, k_ctx, v_ctx, k_ref, v_ref, n, k_new, v_new)  # plain, eager, appends to the copy
+        assert int(nbuf.item()) == n + 1
+        assert max_abs(to_np(out_static), to_np(expect)) <= 2e-2
+        assert torch.equal(k_cache, k_ref) and torch.equal(v_cache, v_ref)
 
 
 @pytest.mark.parametrize("n_buf", [1, 2, 17, 33, 64])
