@@ -46,6 +46,20 @@ __device__ __forceinline__ void load_to_lds_16(const void *global_src, void *lds
 
 // LDS reads of the ring go through inline assembly: the compiler must not see an LDS read that
 // could alias the asynchronous fills, or it would drain every load before each read.
+// Two 16-byte pieces of this lane's K row (addr_k, +1024) and of its query row (addr_q, +1024):
+// one LDS round trip.
+__device__ __forceinline__ void lds_read_kq(u32x4 &k0, u32x4 &k1, u32x4 &q0, u32x4 &q1, unsigned addr_k,
+                                            unsigned addr_q) {
+    asm volatile(
+        "ds_read_b128 %0, %4\n\t"
+        "ds_read_b128 %2, %5\n\t"
+        "ds_read_b128 %1, %4 offset:1024\n\t"
+        "ds_read_b128 %3, %5 offset:1024\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(k0), "=&v"(k1), "=&v"(q0), "=&v"(q1)
+        : "v"(addr_k), "v"(addr_q)
+        : "memory");
+}
 __device__ __forceinline__ void lds_read2x128(u32x4 &a, u32x4 &b, unsigned addr) {
     asm volatile(
         "ds_read_b128 %0, %2\n\t"
@@ -55,21 +69,17 @@ __device__ __forceinline__ void lds_read2x128(u32x4 &a, u32x4 &b, unsigned addr)
         : "v"(addr)
         : "memory");
 }
-// Eight transposing reads: the V operands of the eight 4-dim groups of one 4-key chunk.
+// Four transposing reads: the V operands of four 4-dim groups of one 4-key chunk.
 // Address layout of a V chunk: sub-slot t (1 KiB) holds dims 8t..8t+7, so group u = 2t + half
-// sits at t * 1024 + 8 * half.
-__device__ __forceinline__ void lds_read8_tr(u32x2 (&v)[8], unsigned addr) {
+// sits at t * 1024 + 8 * half; one call covers sub-slots t and t + 1.
+__device__ __forceinline__ void lds_read4_tr(u32x2 (&v)[4], unsigned addr) {
     asm volatile(
-        "ds_read_b64_tr_b16 %0, %8\n\t"
-        "ds_read_b64_tr_b16 %1, %8 offset:8\n\t"
-        "ds_read_b64_tr_b16 %2, %8 offset:1024\n\t"
-        "ds_read_b64_tr_b16 %3, %8 offset:1032\n\t"
-        "ds_read_b64_tr_b16 %4, %8 offset:2048\n\t"
-        "ds_read_b64_tr_b16 %5, %8 offset:2056\n\t"
-        "ds_read_b64_tr_b16 %6, %8 offset:3072\n\t"
-        "ds_read_b64_tr_b16 %7, %8 offset:3080\n\t"
+        "ds_read_b64_tr_b16 %0, %4\n\t"
+        "ds_read_b64_tr_b16 %1, %4 offset:8\n\t"
+        "ds_read_b64_tr_b16 %2, %4 offset:1024\n\t"
+        "ds_read_b64_tr_b16 %3, %4 offset:1032\n\t"
         "s_waitcnt lgkmcnt(0)"
-        : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
+        : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3])
         : "v"(addr)
         : "memory");
 }
@@ -139,32 +149,48 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
     // priority it is only issued in their gaps.  It issues little: the priority costs them little.
     __builtin_amdgcn_s_setprio(3);
 
-    // ---- producer: chunk `issue_g` of task `issue_task` into ring slot issue_slot
+    // ---- producer: chunk `issue_g` of task `issue_task` into ring slot issue_slot.  Row pointers
+    // are kept per task and advanced by four rows per chunk; only a task's last chunk (clamped
+    // rows, the new row) computes addresses the long way.
     const int my_tasks = blockIdx.x < n_tasks ? (n_tasks - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
     const int total_chunks = my_tasks * n_groups;
+    const long chunk_step = 4 * vkb.sn, chunk_step_v = 4 * vvb.sn;  // elements between rows g*4 and (g+1)*4
     int issued = 0, issue_task = blockIdx.x, issue_g = 0, issue_slot = 0, issue_q = 0;
     int issue_seq = 0, seq = 0;  // how many of this wavefront's tasks the producer / consumer have finished
+    const T *p_k = nullptr, *p_v = nullptr;  // this lane's row of the chunk to be requested next
     auto issue_one = [&]() {
-        int pair = 16 * issue_task + pl;
-        pair = pair < n_pairs ? pair : n_pairs - 1;  // a ragged last task re-reads the last pair; never stored
-        const int b = pair / H, h = pair % H;
-        if (issue_g == 0) {
+        const bool first = issue_g == 0, last = issue_g + 1 == n_groups;  // wavefront-uniform
+        int p_b = 0, p_h = 0;
+        if (first || last) {  // the (trajectory, head) of this lane's pair: twice per task at most
+            int pair = 16 * issue_task + pl;
+            pair = pair < n_pairs ? pair : n_pairs - 1;  // a ragged last task re-reads the last pair; never stored
+            p_b = pair / H;
+            p_h = pair % H;
+        }
+        if (first) {
+            p_k = view_row<T>(vkb, p_b, p_h, sub);
+            p_v = view_row<T>(vvb, p_b, p_h, sub);
             // the task's queries: lane (p, j < LQ) fetches its 64-byte row in four pieces
-            const T *qrow = view_row<T>(vq, b, h, sub < LQ ? sub : 0);
+            const T *qrow = view_row<T>(vq, p_b, p_h, sub < LQ ? sub : 0);
             unsigned char *qd = stream_lds + S * kStreamChunkBytes + issue_q * kStreamQBytes;
 #pragma unroll
             for (int t = 0; t < 4; ++t) load_to_lds_16(qrow + 8 * t, qd + 1024 * t);
         }
-        int row = 4 * issue_g + sub;
-        row = row < n_total ? row : n_total - 1;  // keys past the end re-read the last one and are masked
-        const bool is_new = has_new && row == n_buf;
-        const T *kr = is_new ? view_row<T>(vkn, b, h, 0) : view_row<T>(vkb, b, h, row);
-        const T *vr = is_new ? view_row<T>(vvn, b, h, 0) : view_row<T>(vvb, b, h, row);
+        const T *kr = p_k, *vr = p_v;
+        if (last) {
+            int row = 4 * issue_g + sub;
+            row = row < n_total ? row : n_total - 1;  // keys past the end re-read the last one and are masked
+            const bool is_new = has_new && row == n_buf;
+            kr = is_new ? view_row<T>(vkn, p_b, p_h, 0) : view_row<T>(vkb, p_b, p_h, row);
+            vr = is_new ? view_row<T>(vvn, p_b, p_h, 0) : view_row<T>(vvb, p_b, p_h, row);
+        }
         unsigned char *cd = stream_lds + issue_slot * kStreamChunkBytes;
 #pragma unroll
         for (int t = 0; t < 4; ++t) load_to_lds_16(kr + 8 * t, cd + 1024 * t);
 #pragma unroll
         for (int t = 0; t < 4; ++t) load_to_lds_16(vr + 8 * t, cd + 4096 + 1024 * t);
+        p_k += chunk_step;
+        p_v += chunk_step_v;
         ++issued;
         issue_slot = issue_slot + 1 == S ? 0 : issue_slot + 1;
         if (++issue_g == n_groups) {
@@ -185,6 +211,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
 #pragma unroll
     for (int u = 0; u < 8; ++u) o[u] = f32x4{0.f, 0.f, 0.f, 0.f};
     int task = blockIdx.x, g = 0, slot = 0, qsel = 0;
+    const int new_group = has_new ? n_buf >> 2 : -1;  // the chunk that holds the row to append
     for (int c = 0; c < total_chunks; ++c) {
         // chunk c must have landed; only the chunks requested after it (8 loads each) may be pending
         switch (issued - c - 1) {
@@ -196,25 +223,13 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
         const unsigned chunk = lds0 + static_cast<unsigned>(slot) * kStreamChunkBytes;
         const unsigned qaddr = q_lds0 + static_cast<unsigned>(qsel) * kStreamQBytes + lane * 16u;
 
-        int pair = 16 * task + pl;
-        const bool pair_ok = pair < n_pairs;
-        pair = pair_ok ? pair : n_pairs - 1;
-        const int b = pair / H, h = pair % H;
-        const bool appends = has_new && 4 * g + sub == n_buf && pair_ok;
-        T *const kd = view_row<T>(vkb, b, h, n_buf), *const vd = view_row<T>(vvb, b, h, n_buf);
-
         // ---- scores of 4 keys for this lane's query, head dims in two halves (register budget).
         // Lanes that stand for no query (sub >= LQ) multiply by zero.
         f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
             u32x4 k0, k1, q0, q1;
-            lds_read2x128(k0, k1, chunk + 2048u * half + lane * 16u);
-            lds_read2x128(q0, q1, qaddr + 2048u * half);
-            if (appends) {  // in-place append: this lane holds the new K row
-                *reinterpret_cast<u32x4 *>(kd + 16 * half) = k0;
-                *reinterpret_cast<u32x4 *>(kd + 16 * half + 8) = k1;
-            }
+            lds_read_kq(k0, k1, q0, q1, chunk + 2048u * half + lane * 16u, qaddr + 2048u * half);
             if (sub >= LQ) {
                 q0 = u32x4{0u, 0u, 0u, 0u};
                 q1 = q0;
@@ -224,24 +239,34 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
             s = Mfma4<T>::mma(u32x2{k1[0], k1[1]}, u32x2{q1[0], q1[1]}, s);
             s = Mfma4<T>::mma(u32x2{k1[2], k1[3]}, u32x2{q1[2], q1[3]}, s);
         }
-        if (appends) {  // ... and reads its V row back lane-locally
+        if (g == new_group) {
+            // in-place append (once per task): the lane that holds the new row copies it from the
+            // chunk, lane-locally, into slot n_buf of the cache
+            const int pair = 16 * task + pl;
+            if (4 * g + sub == n_buf && pair < n_pairs) {
+                const int b = pair / H, h = pair % H;
+                T *kd = view_row<T>(vkb, b, h, n_buf), *vd = view_row<T>(vvb, b, h, n_buf);
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                u32x4 v0, v1;
-                lds_read2x128(v0, v1, chunk + 4096u + 2048u * half + lane * 16u);
-                *reinterpret_cast<u32x4 *>(vd + 16 * half) = v0;
-                *reinterpret_cast<u32x4 *>(vd + 16 * half + 8) = v1;
+                for (int half = 0; half < 2; ++half) {
+                    u32x4 k0, k1, v0, v1;
+                    lds_read2x128(k0, k1, chunk + 2048u * half + lane * 16u);
+                    lds_read2x128(v0, v1, chunk + 4096u + 2048u * half + lane * 16u);
+                    *reinterpret_cast<u32x4 *>(kd + 16 * half) = k0;
+                    *reinterpret_cast<u32x4 *>(kd + 16 * half + 8) = k1;
+                    *reinterpret_cast<u32x4 *>(vd + 16 * half) = v0;
+                    *reinterpret_cast<u32x4 *>(vd + 16 * half + 8) = v1;
+                }
             }
         }
         float sc[4];
-        float cm = -INFINITY;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            sc[r] = 4 * g + r < n_total ? s[r] * qscale : -INFINITY;
-            cm = fmaxf(cm, sc[r]);
+        for (int r = 0; r < 4; ++r) sc[r] = s[r] * qscale;
+        if (g + 1 == n_groups) {  // only a task's last chunk can hold keys past the end
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sc[r] = 4 * g + r < n_total ? sc[r] : -INFINITY;
         }
         // online softmax; the rescale is skipped (wavefront-uniformly) while no maximum moves
-        const float m_new = fmaxf(m, cm);
+        const float m_new = fmaxf(fmaxf(m, fmaxf(sc[0], sc[1])), fmaxf(sc[2], sc[3]));
         if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
             const float alpha = m == -INFINITY ? 0.f : fast_exp2(m - m_new);
             l *= alpha;
@@ -251,26 +276,25 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
         }
         float p[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            p[r] = fast_exp2(sc[r] - m);  // m is finite here: key 4g is always valid
-            l += p[r];
-        }
+        for (int r = 0; r < 4; ++r) p[r] = fast_exp2(sc[r] - m);  // m is finite here: key 4g is always valid
+        l += (p[0] + p[1]) + (p[2] + p[3]);
         const u32x2 pop = {pack2<T>(p[0], p[1]), pack2<T>(p[2], p[3])};
-        {
-            u32x2 vop[8];
-            lds_read8_tr(vop, chunk + 4096u + tr_off);
 #pragma unroll
-            for (int u = 0; u < 8; ++u) o[u] = Mfma4<T>::mma(vop[u], pop, o[u]);
+        for (int half = 0; half < 2; ++half) {
+            u32x2 vop[4];
+            lds_read4_tr(vop, chunk + 4096u + 2048u * half + tr_off);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) o[4 * half + u] = Mfma4<T>::mma(vop[u], pop, o[4 * half + u]);
         }
         // the chunk has been read: refill its slot (and any the producer had to leave empty)
-        const bool task_ends = g + 1 == n_groups;
-        if (task_ends) ++seq;
+        if (g + 1 == n_groups) ++seq;
         while (may_issue() && issued - c - 1 < S) issue_one();
 
         slot = slot + 1 == S ? 0 : slot + 1;
         if (++g == n_groups) {
             // ---- task done: write this lane's partial (lanes of real queries of real pairs)
-            if (pair_ok && sub < LQ) {
+            const int pair = 16 * task + pl;
+            if (pair < n_pairs && sub < LQ) {
                 const float inv = l > 0.f ? 1.f / l : 0.f;
                 T *po = part_o + (static_cast<long>(pair) * LQ + sub) * DH;
 #pragma unroll
