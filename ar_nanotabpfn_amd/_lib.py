@@ -43,6 +43,12 @@ _VP = ctypes.POINTER(ArtabView)
 _i, _f, _p, _sz, _i64 = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int64
 
 
+class ArtabAttentionPartials(ctypes.Structure):
+    """``artab_attention_partials`` of include/artab_attention.h."""
+
+    _fields_ = [("part_o", _p), ("part_lse", _p), ("n_slots", _i), ("B", _i), ("H", _i), ("Lq", _i), ("Dh", _i)]
+
+
 class ArtabSampleEmbedArgs(ctypes.Structure):
     """``artab_sample_embed_args`` of include/artab_attention.h, field for field."""
 
@@ -78,6 +84,11 @@ SIGNATURES = {
         _i,
         [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _p, _i, _i, _f, _i, _p, _sz, _i, _p, _p],
     ),
+    "artab_decode_attention_partials": (
+        _i,
+        [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _p, _i, _i, _f, _i, _p, _sz, _i, _p, _p,
+         ctypes.POINTER(ArtabAttentionPartials)],
+    ),
     "artab_teacher_forcing_attention": (_i, [_VP, _VP, _VP, _VP, _VP, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "artab_prefill_attention": (_i, [_VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "artab_buffer_attention": (_i, [_VP, _VP, _VP, _p, _i64, _i64, _i64, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _p]),
@@ -89,6 +100,12 @@ SIGNATURES = {
     "artab_layer_post_pre": (
         _i,
         [_p, _i64, _p, _i64, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _f, _p, _p, _p, _f, _p, _p, _p, _i64, _i, _i, _i, _p],
+    ),
+    "artab_layer_post_from_partials": (
+        _i, [ctypes.POINTER(ArtabAttentionPartials), _p, _i64, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _f, _p, _i64, _i, _i, _i, _p]),
+    "artab_layer_post_pre_from_partials": (
+        _i,
+        [ctypes.POINTER(ArtabAttentionPartials), _p, _i64, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _f, _p, _p, _p, _f, _p, _p, _p, _i64, _i, _i, _i, _p],
     ),
     "artab_decode_sample_embed": (_i, [ctypes.POINTER(ArtabSampleEmbedArgs), _i, _p]),
     "artab_layer_post": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _f, _p, _i64, _i, _i, _i, _p]),

@@ -23,6 +23,7 @@ from torch import Tensor
 from . import _lib
 
 __all__ = [
+    "AttentionPartials",
     "hip_available",
     "triton_available",
     "context_attention",
@@ -220,7 +221,8 @@ def decode_attention(
     use_triton: bool = True,
     n_buf_device: Optional[Tensor] = None,
     side_stream: Optional["torch.cuda.Stream"] = None,
-) -> Tensor:
+    leave_partials: bool = False,
+):
     """One decode step of row attention (inference.py:785-823) in one call.
 
     ``q [B,H,Lq,D]`` with Lq in {1,2}; ``k_buf_cache``/``v_buf_cache`` are the
@@ -236,6 +238,10 @@ def decode_attention(
     ``side_stream`` (a default-priority stream of the same device) lets the buffer pass
     run next to the context pass (``artab_decode_attention_overlapped``); the call is
     still ordered on the current stream.
+
+    ``leave_partials=True`` skips the final merge where the schedule produces partial results
+    and returns an ``AttentionPartials`` for ``glue.layer_post`` / ``layer_post_pre`` to merge
+    while they load their input; where it does not, the merged tensor is returned as usual.
     """
     dev = _lib.require_device(q, k_ctx, v_ctx, k_buf_cache, v_buf_cache, k_new, v_new)
     lib = _lib.load()
@@ -260,11 +266,29 @@ def decode_attention(
         cap, Dh, 0.0, _lib.dtype_code(q.dtype),
         ws_ptr, ws_bytes, _impl(use_triton), _lib.current_stream(dev),
     )
-    if side_stream is not None:
-        _lib.check(lib.artab_decode_attention_overlapped(*args, ctypes.c_void_p(side_stream.cuda_stream)))
+    side = ctypes.c_void_p(side_stream.cuda_stream) if side_stream is not None else None
+    if leave_partials:
+        desc = _lib.ArtabAttentionPartials()
+        _lib.check(lib.artab_decode_attention_partials(*args, side, ctypes.byref(desc)))
+        if desc.n_slots > 0:
+            return AttentionPartials(desc, q.dtype, q.device)
+    elif side_stream is not None:
+        _lib.check(lib.artab_decode_attention_overlapped(*args, side))
     else:
         _lib.check(lib.artab_decode_attention(*args))
     return out
+
+
+class AttentionPartials:
+    """Unmerged attention result of a decode step (``artab_attention_partials``): it points into
+    the device's split workspace and is valid until the next attention call on that device."""
+
+    def __init__(self, desc, dtype, device):
+        self.desc, self.dtype, self.device = desc, dtype, device
+
+    @property
+    def shape(self):  # of the merged [B,H,Lq,Dh] result
+        return (self.desc.B, self.desc.H, self.desc.Lq, self.desc.Dh)
 
 
 def teacher_forcing_attention(

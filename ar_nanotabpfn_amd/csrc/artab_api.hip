@@ -585,7 +585,8 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
                        const artab_view *v_new, const artab_view *out, int B, int H, int Lq, int Nc,
                        int n_buf, const int32_t *n_buf_device, int buf_capacity, int Dh, float scale,
                        int dtype, void *workspace, size_t workspace_bytes, int impl, void *stream,
-                       void *side_stream) {
+                       void *side_stream, artab_attention_partials *leave_partials = nullptr) {
+    if (leave_partials) memset(leave_partials, 0, sizeof(*leave_partials));
     ARTAB_TRY(check_common(B, H, Lq, Dh, dtype));
     if (Lq != 1 && Lq != 2)
         return fail(ARTAB_ERR_BAD_SHAPE, "decode supports Lq=1 (target) or Lq=2 (buffer, target); got %d", Lq);
@@ -709,6 +710,11 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
     ARTAB_TRY(launch_status(e_ctx, "decode context pass"));
     ARTAB_TRY(launch_status(e_buf, "decode buffer pass (stream)"));
     ARTAB_TRY(launch_status(e_join, "decode join"));
+    if (leave_partials) {  // the caller's next kernel merges them (artab_layer_post*_from_partials)
+        leave_partials->part_o = F.part_o; leave_partials->part_lse = F.part_lse; leave_partials->n_slots = slots;
+        leave_partials->B = B; leave_partials->H = H; leave_partials->Lq = Lq; leave_partials->Dh = Dh;
+        return ARTAB_OK;
+    }
     CombineParams C;
     C.out = dv(out); C.part_o = F.part_o; C.part_lse = F.part_lse; C.lse = nullptr;
     C.rows = rows; C.H = H; C.Lq = Lq; C.Dh = Dh; C.n_split = slots;
@@ -727,6 +733,17 @@ int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const a
                            int dtype, void *workspace, size_t workspace_bytes, int impl, void *stream) {
     return decode_impl(q, k_ctx, v_ctx, k_buf, v_buf, k_new, v_new, out, B, H, Lq, Nc, n_buf, n_buf_device,
                        buf_capacity, Dh, scale, dtype, workspace, workspace_bytes, impl, stream, nullptr);
+}
+
+int artab_decode_attention_partials(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                                    const artab_view *k_buf, const artab_view *v_buf, const artab_view *k_new,
+                                    const artab_view *v_new, const artab_view *out, int B, int H, int Lq, int Nc,
+                                    int n_buf, const int32_t *n_buf_device, int buf_capacity, int Dh, float scale,
+                                    int dtype, void *workspace, size_t workspace_bytes, int impl, void *stream,
+                                    void *side_stream, artab_attention_partials *partials) {
+    if (!partials) return fail(ARTAB_ERR_NULL_POINTER, "partials descriptor is NULL");
+    return decode_impl(q, k_ctx, v_ctx, k_buf, v_buf, k_new, v_new, out, B, H, Lq, Nc, n_buf, n_buf_device,
+                       buf_capacity, Dh, scale, dtype, workspace, workspace_bytes, impl, stream, side_stream, partials);
 }
 
 int artab_decode_attention_overlapped(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
@@ -973,9 +990,23 @@ static int fill_pre(FusedPreParams &P, const void *x, int64_t ldx, const void *w
 static int fill_post(FusedPostParams &P, const void *attn, int64_t lda, const void *y, int64_t ldy, const void *w_o,
                      const void *ln2_gamma, const void *ln2_beta, float eps2, const void *w_1, const void *b_1,
                      const void *w_2, const void *b_2, const void *ln3_gamma, const void *ln3_beta, float eps3,
-                     void *out, int64_t rows, int D, int F, bool out_required) {
+                     void *out, int64_t rows, int D, int F, bool out_required,
+                     const artab_attention_partials *parts = nullptr) {
     if (!fused_width_ok(D) || !fused_width_ok(F))
         return fail(ARTAB_ERR_UNSUPPORTED, "layer_post needs D and F in {128, 256, 512} (got %d, %d)", D, F);
+    if (parts) {
+        if (!parts->part_o || !parts->part_lse) return fail(ARTAB_ERR_NULL_POINTER, "partials are NULL");
+        if (parts->n_slots < 1 || parts->H < 1 || parts->Lq < 1 || parts->B < 0 || parts->Dh < 8 || parts->Dh % 8 ||
+            parts->H * parts->Dh != D || static_cast<int64_t>(parts->B) * parts->Lq != rows)
+            return fail(ARTAB_ERR_BAD_SHAPE,
+                        "partials (B=%d H=%d Lq=%d Dh=%d, %d slots) do not describe %lld rows of width %d", parts->B,
+                        parts->H, parts->Lq, parts->Dh, parts->n_slots, (long long)rows, D);
+        if (misaligned16(parts->part_o)) return fail(ARTAB_ERR_BAD_STRIDE, "partials must be 16-byte aligned");
+        P.part_o = parts->part_o; P.part_lse = parts->part_lse; P.n_slots = parts->n_slots;
+        P.part_rows = static_cast<long>(parts->B) * parts->H * parts->Lq; P.H = parts->H; P.Lq = parts->Lq;
+        attn = parts->part_o;  // placeholder for the checks below
+        lda = D;
+    }
     if (!attn || !y || !w_o || !ln2_gamma || !ln2_beta || !w_1 || !w_2 || !ln3_gamma || !ln3_beta ||
         (out_required && !out))
         return fail(ARTAB_ERR_NULL_POINTER, "layer_post: only b_1 and b_2 may be NULL");
@@ -1001,7 +1032,7 @@ int artab_layer_pre(const void *x, int64_t ldx, const void *w_fo, const void *ln
                     float eps1, const void *w_qkv, void *y, void *qkv, int64_t rows, int D, int dtype,
                     void *stream) {
     ARTAB_TRY(check_layer_dtype_rows("layer_pre", dtype, rows));
-    FusedPreParams P;
+    FusedPreParams P{};
     ARTAB_TRY(fill_pre(P, x, ldx, w_fo, ln1_gamma, ln1_beta, eps1, w_qkv, y, qkv, rows, D, true));
     if (rows == 0) return ARTAB_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -1014,7 +1045,7 @@ int artab_layer_post(const void *attn, int64_t lda, const void *y, int64_t ldy, 
                      const void *w_2, const void *b_2, const void *ln3_gamma, const void *ln3_beta, float eps3,
                      void *out, int64_t rows, int D, int F, int dtype, void *stream) {
     ARTAB_TRY(check_layer_dtype_rows("layer_post", dtype, rows));
-    FusedPostParams P;
+    FusedPostParams P{};
     ARTAB_TRY(fill_post(P, attn, lda, y, ldy, w_o, ln2_gamma, ln2_beta, eps2, w_1, b_1, w_2, b_2, ln3_gamma,
                         ln3_beta, eps3, out, rows, D, F, true));
     if (rows == 0) return ARTAB_OK;
@@ -1023,23 +1054,65 @@ int artab_layer_post(const void *attn, int64_t lda, const void *y, int64_t ldy, 
     return launch_status(e, "layer_post");
 }
 
-int artab_layer_post_pre(const void *attn, int64_t lda, const void *y, int64_t ldy, const void *w_o,
-                         const void *ln2_gamma, const void *ln2_beta, float eps2, const void *w_1, const void *b_1,
-                         const void *w_2, const void *b_2, const void *ln3_gamma, const void *ln3_beta, float eps3,
-                         const void *next_w_fo, const void *next_ln1_gamma, const void *next_ln1_beta,
-                         float next_eps1, const void *next_w_qkv, void *next_y, void *next_qkv, int64_t rows, int D,
-                         int F, int dtype, void *stream) {
+static int layer_post_pre_impl(const artab_attention_partials *parts, const void *attn, int64_t lda, const void *y,
+                               int64_t ldy, const void *w_o, const void *ln2_gamma, const void *ln2_beta, float eps2,
+                               const void *w_1, const void *b_1, const void *w_2, const void *b_2,
+                               const void *ln3_gamma, const void *ln3_beta, float eps3, const void *next_w_fo,
+                               const void *next_ln1_gamma, const void *next_ln1_beta, float next_eps1,
+                               const void *next_w_qkv, void *next_y, void *next_qkv, int64_t rows, int D, int F,
+                               int dtype, void *stream) {
     ARTAB_TRY(check_layer_dtype_rows("layer_post_pre", dtype, rows));
-    FusedPostParams P;
-    FusedPreParams N;
+    FusedPostParams P{};
+    FusedPreParams N{};
     ARTAB_TRY(fill_post(P, attn, lda, y, ldy, w_o, ln2_gamma, ln2_beta, eps2, w_1, b_1, w_2, b_2, ln3_gamma,
-                        ln3_beta, eps3, nullptr, rows, D, F, false));
+                        ln3_beta, eps3, nullptr, rows, D, F, false, parts));
     ARTAB_TRY(fill_pre(N, nullptr, 0, next_w_fo, next_ln1_gamma, next_ln1_beta, next_eps1, next_w_qkv, next_y,
                        next_qkv, rows, D, false));
     if (rows == 0) return ARTAB_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipError_t e = dtype == ARTAB_BF16 ? launch_post_pre<bf16_t>(P, N, D, F, st) : launch_post_pre<f16_t>(P, N, D, F, st);
     return launch_status(e, "layer_post_pre");
+}
+
+int artab_layer_post_pre(const void *attn, int64_t lda, const void *y, int64_t ldy, const void *w_o,
+                         const void *ln2_gamma, const void *ln2_beta, float eps2, const void *w_1, const void *b_1,
+                         const void *w_2, const void *b_2, const void *ln3_gamma, const void *ln3_beta, float eps3,
+                         const void *next_w_fo, const void *next_ln1_gamma, const void *next_ln1_beta,
+                         float next_eps1, const void *next_w_qkv, void *next_y, void *next_qkv, int64_t rows, int D,
+                         int F, int dtype, void *stream) {
+    return layer_post_pre_impl(nullptr, attn, lda, y, ldy, w_o, ln2_gamma, ln2_beta, eps2, w_1, b_1, w_2, b_2,
+                               ln3_gamma, ln3_beta, eps3, next_w_fo, next_ln1_gamma, next_ln1_beta, next_eps1,
+                               next_w_qkv, next_y, next_qkv, rows, D, F, dtype, stream);
+}
+
+int artab_layer_post_pre_from_partials(const artab_attention_partials *parts, const void *y, int64_t ldy,
+                                       const void *w_o, const void *ln2_gamma, const void *ln2_beta, float eps2,
+                                       const void *w_1, const void *b_1, const void *w_2, const void *b_2,
+                                       const void *ln3_gamma, const void *ln3_beta, float eps3,
+                                       const void *next_w_fo, const void *next_ln1_gamma,
+                                       const void *next_ln1_beta, float next_eps1, const void *next_w_qkv,
+                                       void *next_y, void *next_qkv, int64_t rows, int D, int F, int dtype,
+                                       void *stream) {
+    if (!parts) return fail(ARTAB_ERR_NULL_POINTER, "partials descriptor is NULL");
+    return layer_post_pre_impl(parts, nullptr, 0, y, ldy, w_o, ln2_gamma, ln2_beta, eps2, w_1, b_1, w_2, b_2,
+                               ln3_gamma, ln3_beta, eps3, next_w_fo, next_ln1_gamma, next_ln1_beta, next_eps1,
+                               next_w_qkv, next_y, next_qkv, rows, D, F, dtype, stream);
+}
+
+int artab_layer_post_from_partials(const artab_attention_partials *parts, const void *y, int64_t ldy,
+                                   const void *w_o, const void *ln2_gamma, const void *ln2_beta, float eps2,
+                                   const void *w_1, const void *b_1, const void *w_2, const void *b_2,
+                                   const void *ln3_gamma, const void *ln3_beta, float eps3, void *out, int64_t rows,
+                                   int D, int F, int dtype, void *stream) {
+    if (!parts) return fail(ARTAB_ERR_NULL_POINTER, "partials descriptor is NULL");
+    ARTAB_TRY(check_layer_dtype_rows("layer_post", dtype, rows));
+    FusedPostParams P{};
+    ARTAB_TRY(fill_post(P, nullptr, 0, y, ldy, w_o, ln2_gamma, ln2_beta, eps2, w_1, b_1, w_2, b_2, ln3_gamma,
+                        ln3_beta, eps3, out, rows, D, F, true, parts));
+    if (rows == 0) return ARTAB_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipError_t e = dtype == ARTAB_BF16 ? launch_post<bf16_t>(P, D, F, st) : launch_post<f16_t>(P, D, F, st);
+    return launch_status(e, "layer_post");
 }
 
 int artab_decode_sample_embed(const artab_sample_embed_args *a, int dtype, void *stream) {

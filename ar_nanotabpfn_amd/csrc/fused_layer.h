@@ -45,7 +45,12 @@ struct FusedPreParams {
 };
 
 struct FusedPostParams {
-    const void *attn; long lda;  // [rows, D]
+    const void *attn; long lda;  // [rows, D]; unused when the attention arrives as partials:
+    const void *part_o;          // [n_slots][part_rows][D / H] partial outputs (input type), or NULL
+    const float *part_lse;       // [n_slots][part_rows] their natural-log LSEs
+    int n_slots;                 // partials per (trajectory, head, query)
+    long part_rows;              // B * H * Lq
+    int H, Lq;                   // token row r = b * Lq + i  <->  partial row (b * H + h) * Lq + i
     const void *y;    long ldy;  // [rows, D] residual stream (output of the pre kernel)
     const void *w_o;             // [D, D] packed
     const void *g2, *b2;         // LayerNorm 2
@@ -143,6 +148,71 @@ __device__ __forceinline__ void load_cols(const T *vec, const int (&nblk)[NB], i
     for (int b = 0; b < NB; ++b)
 #pragma unroll
         for (int g = 0; g < 4; ++g) load4f<T>(vec + col_of(nblk[b], 4 * g, hb), &out[b][4 * g]);
+}
+
+// The attention tile of 32 token rows built from partial results (context slices + buffer pass)
+// instead of a finished matrix: out = sum_s w_s o_s / sum_s w_s with w_s = exp(lse_s - max lse),
+// the same arithmetic, in the same order, as the stand-alone combine launch, rounded once to the
+// storage type on its way into LDS.  One item = 8 output dims of one (row, head).
+constexpr int kMergeBatch = 9;  // partials fetched per round (8 context slices + the buffer pass)
+
+template <typename T, int D, int NT>
+__device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const FusedPostParams &P, long row0,
+                                                       int valid, int tid) {
+    const int dh = D / P.H;          // head dim, a multiple of 8
+    constexpr int CPR = D / 8;       // 16-byte chunks per token row
+    for (int idx = tid; idx < kFusedRows * CPR; idx += NT) {
+        const int r = idx / CPR, ch = idx % CPR;
+        u32x4 packed = {0u, 0u, 0u, 0u};
+        if (r < valid) {
+            const long tok = row0 + r;
+            const long b = tok / P.Lq;
+            const int i = static_cast<int>(tok % P.Lq);
+            const int h = (8 * ch) / dh, d0 = (8 * ch) % dh;
+            const long prow = (b * P.H + h) * P.Lq + i;
+            const T *po = static_cast<const T *>(P.part_o) + prow * dh + d0;
+            const float *pl = P.part_lse + prow;
+            const long o_step = P.part_rows * dh;
+            float mx = -INFINITY;
+            for (int s0 = 0; s0 < P.n_slots; s0 += kMergeBatch) {
+                float lv[kMergeBatch];
+#pragma unroll
+                for (int u = 0; u < kMergeBatch; ++u) {
+                    const int sl = s0 + u < P.n_slots ? s0 + u : P.n_slots - 1;
+                    lv[u] = pl[sl * P.part_rows];
+                }
+#pragma unroll
+                for (int u = 0; u < kMergeBatch; ++u) mx = fmaxf(mx, lv[u]);
+            }
+            float wsum = 0.f, acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            for (int s0 = 0; s0 < P.n_slots; s0 += kMergeBatch) {
+                float lv[kMergeBatch];
+                u32x4 ov[kMergeBatch];
+#pragma unroll
+                for (int u = 0; u < kMergeBatch; ++u) {
+                    const int sl = s0 + u < P.n_slots ? s0 + u : P.n_slots - 1;
+                    lv[u] = pl[sl * P.part_rows];
+                    ov[u] = *reinterpret_cast<const u32x4 *>(po + sl * o_step);
+                }
+#pragma unroll
+                for (int u = 0; u < kMergeBatch; ++u) {
+                    if (s0 + u < P.n_slots) {
+                        const float w = expf(lv[u] - mx);
+                        wsum += w;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            acc[2 * e] = fmaf(w, unpack_lo<T>(ov[u][e]), acc[2 * e]);
+                            acc[2 * e + 1] = fmaf(w, unpack_hi<T>(ov[u][e]), acc[2 * e + 1]);
+                        }
+                    }
+                }
+            }
+            const float inv = 1.f / wsum;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) packed[e] = pack2<T>(acc[2 * e] * inv, acc[2 * e + 1] * inv);
+        }
+        *reinterpret_cast<u32x4 *>(dst + r * lds_ld + 8 * ch) = packed;
+    }
 }
 
 // Parameter vectors (LayerNorm gamma / beta, biases) are copied to LDS when the kernel starts:
@@ -365,7 +435,7 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
     WeightStream<T, D, NBF> w_1;
     WeightStream<T, F, NBD> w_2;
     w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
-    stage_tile<T, D, NT>(a0, LDD, static_cast<const T *>(P.attn) + row0 * P.lda, P.lda, valid, tid);
+    if (!P.part_o) stage_tile<T, D, NT>(a0, LDD, static_cast<const T *>(P.attn) + row0 * P.lda, P.lda, valid, tid);
     stage_tile<T, D, NT>(a1, LDD, static_cast<const T *>(P.y) + row0 * P.ldy, P.ldy, valid, tid);
     stage_vector<T, D, NT>(vecs + kVecG2 * vec_ld, P.g2, tid);
     stage_vector<T, D, NT>(vecs + kVecB2 * vec_ld, P.b2, tid);
@@ -373,6 +443,7 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
     stage_vector<T, D, NT>(vecs + kVecG3 * vec_ld, P.g3, tid);
     stage_vector<T, D, NT>(vecs + kVecB3 * vec_ld, P.b3, tid);
     stage_vector<T, D, NT>(vecs + kVecBias2 * vec_ld, P.bias_2, tid);
+    if (P.part_o) stage_merged_attention<T, D, NT>(a0, LDD, P, row0, valid, tid);
     if (ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane);
     __syncthreads();
 

@@ -126,9 +126,20 @@ def layer_post(attn: Tensor, y: Tensor, w_o: Tensor, norm2: nn.LayerNorm, w_1: T
 
     ``attn`` and ``y`` are ``[rows, D]``-shaped (any leading dims); returns ``[rows, D]``."""
     D = y.shape[-1]
-    a2, y2 = _rows16(attn), _rows16(y)
+    y2 = _rows16(y)
     rows = y2.shape[0]
     out = torch.empty((rows, D), device=y.device, dtype=y.dtype)
+    if hasattr(attn, "desc"):  # unmerged partials: merged while the kernel loads its input
+        _lib.check(
+            _lib.load().artab_layer_post_from_partials(
+                ctypes.byref(attn.desc), _ptr(y2), y2.stride(0), _ptr(w_o), _ptr(norm2.weight), _ptr(norm2.bias),
+                float(norm2.eps), _ptr(w_1), _ptr(b_1), _ptr(w_2), _ptr(b_2),
+                _ptr(norm3.weight), _ptr(norm3.bias), float(norm3.eps), _ptr(out), rows, D, w_1.shape[0] * 32,
+                _lib.dtype_code(y.dtype), _lib.current_stream(y.device),
+            )
+        )
+        return out
+    a2 = _rows16(attn)
     _lib.check(
         _lib.load().artab_layer_post(
             _ptr(a2), a2.stride(0), _ptr(y2), y2.stride(0), _ptr(w_o), _ptr(norm2.weight), _ptr(norm2.bias),
@@ -146,10 +157,23 @@ def layer_post_pre(attn: Tensor, y: Tensor, w_o: Tensor, norm2: nn.LayerNorm, w_
     """``layer_post`` of one layer and ``layer_pre`` of the next in one launch; the layer output
     between them is not materialised.  Returns the next layer's ``(y [rows, D], qkv [rows, 3D])``."""
     D = y.shape[-1]
-    a2, y2 = _rows16(attn), _rows16(y)
+    y2 = _rows16(y)
     rows = y2.shape[0]
     y_next = torch.empty((rows, D), device=y.device, dtype=y.dtype)
     qkv_next = torch.empty((rows, 3 * D), device=y.device, dtype=y.dtype)
+    if hasattr(attn, "desc"):  # unmerged partials
+        _lib.check(
+            _lib.load().artab_layer_post_pre_from_partials(
+                ctypes.byref(attn.desc), _ptr(y2), y2.stride(0), _ptr(w_o), _ptr(norm2.weight), _ptr(norm2.bias),
+                float(norm2.eps), _ptr(w_1), _ptr(b_1), _ptr(w_2), _ptr(b_2),
+                _ptr(norm3.weight), _ptr(norm3.bias), float(norm3.eps),
+                _ptr(next_w_fo), _ptr(next_norm1.weight), _ptr(next_norm1.bias), float(next_norm1.eps),
+                _ptr(next_w_qkv), _ptr(y_next), _ptr(qkv_next), rows, D, w_1.shape[0] * 32,
+                _lib.dtype_code(y.dtype), _lib.current_stream(y.device),
+            )
+        )
+        return y_next, qkv_next
+    a2 = _rows16(attn)
     _lib.check(
         _lib.load().artab_layer_post_pre(
             _ptr(a2), a2.stride(0), _ptr(y2), y2.stride(0), _ptr(w_o), _ptr(norm2.weight), _ptr(norm2.bias),

@@ -64,6 +64,9 @@ class ARTabPFNPredictor:
         # Run the HBM-bound buffer pass of a decode step on a second stream, next to the
         # compute-bound context pass (shared layout, HIP device).
         self.overlap_buffer_pass = True
+        # Leave the attention partials of a decode step unmerged; the layer kernel that follows
+        # merges them while loading its input.
+        self.merge_in_layer = True
         self._side_streams = {}
         self._graph_state = None
 
@@ -219,13 +222,16 @@ class ARTabPFNPredictor:
         # with a device-side length the host value is only the bound that is validated
         n_buf = self.buffer_len if n_buf_device is None else self.max_buffer_len - (N - 1)
         side = self._side_stream(q.device) if self.overlap_buffer_pass else None
+        # where the layer's fused kernel can merge the partial results itself, leave them unmerged
+        partials = self.merge_in_layer and layer.fused_for(q)
         if N == 1:
             attn = ak.decode_attention(q, k_ctx, v_ctx, layer.k_buf_cache, layer.v_buf_cache, n_buf,
-                                       n_buf_device=n_buf_device, side_stream=side)
+                                       n_buf_device=n_buf_device, side_stream=side, leave_partials=partials)
         else:
             attn = ak.decode_attention(
                 q, k_ctx, v_ctx, layer.k_buf_cache, layer.v_buf_cache, n_buf,
                 k_new[:, :, 0:1], v_new[:, :, 0:1], n_buf_device=n_buf_device, side_stream=side,
+                leave_partials=partials,
             )
         return attn
 
@@ -352,7 +358,7 @@ class ARTabPFNPredictor:
         params = list(self.backbone.parameters()) + list(self.embedder.parameters()) + list(self.head.parameters())
         params.append(self.ar_tokens)
         key = (B, Nt, F_, self.context_len, dtype, str(device), layer0.k_ctx_cache.data_ptr(),
-               layer0.k_buf_cache.data_ptr(), self.fuse_step_tail, self.overlap_buffer_pass, tuple((p.data_ptr(), p._version) for p in params))
+               layer0.k_buf_cache.data_ptr(), self.fuse_step_tail, self.overlap_buffer_pass, self.merge_in_layer, tuple((p.data_ptr(), p._version) for p in params))
         st = self._graph_state
         if st is None or st.key != key:
             st = _GraphState()

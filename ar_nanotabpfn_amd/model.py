@@ -131,6 +131,10 @@ class TwoStageTransformerLayer(nn.Module):
     def _fusable(self, x_row: Tensor) -> bool:
         return layer_fusable(x_row, x_row.shape[-1], self.ff[0].out_features)
 
+    def fused_for(self, t: Tensor) -> bool:
+        """Whether tensors of ``t``'s dtype and device go through this layer's fused kernels."""
+        return layer_fusable(t, self.norm1.normalized_shape[0], self.ff[0].out_features)
+
     def pre_attention(self, x_row: Tensor):
         """Everything before the row-attention call: ``(y, q, k, v)`` with ``y`` the normed
         feature stage ``[B,N,D]`` and q, k, v ``[B,H,N,Dh]`` views of one ``[B,N,3D]`` tensor.
@@ -151,11 +155,14 @@ class TwoStageTransformerLayer(nn.Module):
         (inference.py:825-831); one launch where the fused kernel covers the layer."""
         B, H, N, Dh = attn_heads.shape
         D = H * Dh
-        attn2d = attn_heads.transpose(1, 2).reshape(B * N, D)
+        # unmerged partials (attention_kernels.AttentionPartials) go to the kernel as they are
+        attn2d = attn_heads if hasattr(attn_heads, "desc") else attn_heads.transpose(1, 2).reshape(B * N, D)
         if self._fusable(x_row):
             p_o, p_1, p_2 = self.packed_weights()[2:]
             return layer_post(attn2d, x_row, p_o, self.norm2, p_1, self.ff[0].bias, p_2, self.ff[2].bias,
                               self.norm3).view(B, N, D)
+        if hasattr(attn_heads, "desc"):
+            raise ValueError("attention partials need a layer the fused kernels cover")
         x_row = add_layer_norm(x_row, torch.mm(attn2d, self.attn_rows.out_proj.weight.t()).view(B, N, D), None, self.norm2)
         return self.feed_forward(x_row)
 
@@ -169,7 +176,7 @@ class TwoStageTransformerLayer(nn.Module):
             return next_layer.pre_attention(self.finish(x_row, attn_heads))
         B, H, N, Dh = attn_heads.shape
         D = H * Dh
-        attn2d = attn_heads.transpose(1, 2).reshape(B * N, D)
+        attn2d = attn_heads if hasattr(attn_heads, "desc") else attn_heads.transpose(1, 2).reshape(B * N, D)
         p_o, p_1, p_2 = self.packed_weights()[2:]
         n_fo, n_qkv = next_layer.packed_weights()[:2]
         y, qkv = layer_post_pre(attn2d, x_row, p_o, self.norm2, p_1, self.ff[0].bias, p_2, self.ff[2].bias,

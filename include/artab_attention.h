@@ -161,6 +161,39 @@ int artab_decode_attention_overlapped(const artab_view *q, const artab_view *k_c
                            void *workspace, size_t workspace_bytes, int impl, void *stream, void *side_stream);
 
 /*
+ * The attention result of a decode step left unmerged: the partial outputs of the context slices
+ * and of the buffer pass with their log-sum-exps, as they lie in the caller's workspace.
+ *   part_o    [n_slots][B*H*Lq][Dh]  normalised partial outputs, input type
+ *   part_lse  [n_slots][B*H*Lq]      natural-log LSE of each partial (-inf = no key)
+ * row (b*H + h)*Lq + i belongs to trajectory b, head h, query i.  The merged value is
+ * sum_s w_s o_s / sum_s w_s with w_s = exp(lse_s - max_s lse_s) (triton_kernels.py:478-524).
+ * The descriptor stays valid until the workspace is written again.
+ */
+typedef struct artab_attention_partials {
+    const void *part_o;
+    const float *part_lse;
+    int n_slots;
+    int B, H, Lq, Dh;
+} artab_attention_partials;
+
+/*
+ * artab_decode_attention_overlapped without its last launch: the partials are not merged into
+ * `out` but described in *partials for artab_layer_post_from_partials /
+ * artab_layer_post_pre_from_partials, whose kernels merge them while they load their input — one
+ * launch and one round trip of the attention output less per layer.  When the call does not
+ * produce partials (another head_dim, no buffer rows and an unsplit context, the portable path)
+ * it writes `out` as usual and sets partials->n_slots to 0; `out` is therefore always required.
+ */
+int artab_decode_attention_partials(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                           const artab_view *k_buf, const artab_view *v_buf,
+                           const artab_view *k_new, const artab_view *v_new,
+                           const artab_view *out,
+                           int B, int H, int Lq, int Nc, int n_buf, const int32_t *n_buf_device,
+                           int buf_capacity, int Dh, float scale, int dtype,
+                           void *workspace, size_t workspace_bytes, int impl, void *stream, void *side_stream,
+                           artab_attention_partials *partials);
+
+/*
  * Teacher-forced attention over [Buffer_0..Nt-1, Target_0..Nt-1] queries.
  * Replaces hybrid_teacher_forcing_attention (triton_kernels.py:662-702: context
  * pass + masked buffer pass :620-659 + merge) and, with a per-batch context, the
@@ -331,6 +364,26 @@ int artab_layer_post_pre(const void *attn, int64_t lda, const void *y, int64_t l
                          const void *next_w_fo, const void *next_ln1_gamma, const void *next_ln1_beta,
                          float next_eps1, const void *next_w_qkv, void *next_y, void *next_qkv,
                          int64_t rows, int D, int F, int dtype, void *stream);
+
+/*
+ * artab_layer_post / artab_layer_post_pre with the attention input given as unmerged partials
+ * (artab_decode_attention_partials): token row r = b*Lq + i, columns [h*Dh, (h+1)*Dh) of the
+ * attention matrix are merged from partial row (b*H + h)*Lq + i while the tile is loaded, rounded
+ * once to the storage type exactly as the stand-alone merge would.  rows = B*Lq, D = H*Dh.
+ */
+int artab_layer_post_from_partials(const artab_attention_partials *partials, const void *y, int64_t ldy,
+                                   const void *w_o, const void *ln2_gamma, const void *ln2_beta, float eps2,
+                                   const void *w_1, const void *b_1, const void *w_2, const void *b_2,
+                                   const void *ln3_gamma, const void *ln3_beta, float eps3, void *out,
+                                   int64_t rows, int D, int F, int dtype, void *stream);
+int artab_layer_post_pre_from_partials(const artab_attention_partials *partials, const void *y, int64_t ldy,
+                                       const void *w_o, const void *ln2_gamma, const void *ln2_beta, float eps2,
+                                       const void *w_1, const void *b_1, const void *w_2, const void *b_2,
+                                       const void *ln3_gamma, const void *ln3_beta, float eps3,
+                                       const void *next_w_fo, const void *next_ln1_gamma,
+                                       const void *next_ln1_beta, float next_eps1, const void *next_w_qkv,
+                                       void *next_y, void *next_qkv,
+                                       int64_t rows, int D, int F, int dtype, void *stream);
 
 #ifdef __cplusplus
 }

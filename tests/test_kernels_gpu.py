@@ -839,3 +839,44 @@ def test_layer_post_pre_falls_back_when_not_covered(device):
     ref = lb.pre_attention(la.finish(y, attn))
     for a, b in zip(got, ref):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,Lq,Nc,n_buf,cap", [(64, 4, 2, 4096, 9, 16), (33, 8, 2, 2048, 0, 8), (40, 8, 1, 4096, 5, 8)])
+def test_decode_partials_merged_in_layer_kernel(device, dtype, B, H, Lq, Nc, n_buf, cap):
+    """decode_attention(leave_partials=True) + the layer kernels that merge the partials while
+    loading, against the merged attention output fed to the same kernels: the merge is the same
+    arithmetic rounded at the same point, so the results must agree bit for bit."""
+    from ar_nanotabpfn_amd import attention_kernels as ak
+    from ar_nanotabpfn_amd import model as m
+
+    D, Dh, F = 32 * H, 32, 256
+    torch.manual_seed(2)
+    la = m.TwoStageTransformerLayer(D, H, F).to(device=device, dtype=dtype)
+    lb = m.TwoStageTransformerLayer(D, H, F).to(device=device, dtype=dtype)
+    q, k_ctx, v_ctx = (t.to(device) for t in _ctx_inputs(B, H, Lq, Nc, Dh, dtype, seed=5, scale=0.6))
+    k_cache, v_cache = randn((B, H, cap, Dh), 6, dtype, 0.6).to(device), randn((B, H, cap, Dh), 7, dtype, 0.6).to(device)
+    k_new = randn((B, H, 1, Dh), 8, dtype, 0.6).to(device) if Lq == 2 else None
+    v_new = randn((B, H, 1, Dh), 9, dtype, 0.6).to(device) if Lq == 2 else None
+    y = randn((B, Lq, D), 10, dtype, 1.0).to(device)
+    side = torch.cuda.Stream(device=device)
+
+    kc, vc = k_cache.clone(), v_cache.clone()
+    merged = ak.decode_attention(q, k_ctx, v_ctx, kc, vc, n_buf, k_new, v_new, side_stream=side)
+    ref_post = la.finish(y, merged)
+    ref_mid = la.finish_then_pre(y, merged, lb)
+
+    kc2, vc2 = k_cache.clone(), v_cache.clone()
+    parts = ak.decode_attention(q, k_ctx, v_ctx, kc2, vc2, n_buf, k_new, v_new, side_stream=side, leave_partials=True)
+    if n_buf + (Lq - 1) == 0:
+        assert isinstance(parts, torch.Tensor)  # nothing to merge: the finished tensor comes back
+        return
+    assert isinstance(parts, ak.AttentionPartials) and parts.shape == (B, H, Lq, Dh)
+    got_post = la.finish(y, parts)
+    parts = ak.decode_attention(q, k_ctx, v_ctx, k_cache.clone(), v_cache.clone(), n_buf, k_new, v_new,
+                                side_stream=side, leave_partials=True)
+    got_mid = la.finish_then_pre(y, parts, lb)
+    assert torch.equal(kc, kc2) and torch.equal(vc, vc2)
+    assert torch.equal(got_post, ref_post)
+    for a, b in zip(got_mid, ref_mid):
+        assert torch.equal(a, b)
