@@ -174,9 +174,9 @@ def log_density_bench(device, dtype, model, with_cpu):
     return res
 
 
-# Measured with rocprofv3 (median over the decode launches): 9321.8 KiB x 2.0 fetched,
-# 18432.0 KiB written.
-CONTEXT_PASS_HBM_BYTES = int(9321.8 * 1024 * 2.0 + 18432.0 * 1024)
+# Measured with rocprofv3 (median over the decode launches): 9308.5 KiB x 2.0 fetched,
+# 10240.0 KiB written (the partial outputs leave in 16-bit, their LSE in fp32).
+CONTEXT_PASS_HBM_BYTES = int(9308.5 * 1024 * 2.0 + 10240.0 * 1024)
 
 
 def main():
@@ -232,6 +232,14 @@ def main():
     run_decode(pred, x_context, y_context, x_target, args.steps, device, dtype)
     tot, cnt = ctypes.c_double(0.0), ctypes.c_int(0)
     lib.artab_profile_end(ctypes.byref(tot), ctypes.byref(cnt))
+    # the same launches with the buffer pass after the context pass instead of beside it: the
+    # context-pass kernel with the chip to itself
+    pred.overlap_buffer_pass = False
+    lib.artab_profile_begin(CFG3["n_layers"] * (args.steps + 1) + 64)
+    run_decode(pred, x_context, y_context, x_target, args.steps, device, dtype)
+    tot_alone, cnt_alone = ctypes.c_double(0.0), ctypes.c_int(0)
+    lib.artab_profile_end(ctypes.byref(tot_alone), ctypes.byref(cnt_alone))
+    pred.overlap_buffer_pass = True
     pred.use_hip_graph = True
     # the first L launches are the prefill's dense passes, the first decode step has Lq=1
     H, Dh, L = CFG3["n_heads"], CFG3["d_model"] // CFG3["n_heads"], CFG3["n_layers"]
@@ -245,6 +253,7 @@ def main():
     ptot, pcnt = ctypes.c_double(0.0), ctypes.c_int(0)
     lib.artab_profile_end(ctypes.byref(ptot), ctypes.byref(pcnt))
     dec_kernel_ms = tot.value - ptot.value
+    alone_ms = tot_alone.value - ptot.value
     avg_launch_us = dec_kernel_ms * 1e3 / max(n_dec, 1)
     achieved = flops_total / (dec_kernel_ms * 1e-3) / 1e12 if dec_kernel_ms > 0 else 0.0
     prefill_flops = 4.0 * H * NC3 * NC3 * Dh * L
@@ -257,10 +266,14 @@ def main():
         "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
         # HBM bytes of one decode-shaped launch: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 from two
         # rocprofv3 --pmc runs of this script, the factors from the same counters on a 256 MiB copy
-        # (--copy-calibration); algorithmic: K/V 16.8 MB + Q 1.0 MB read, 17.3 MB of partials written.
+        # (--copy-calibration); algorithmic: K/V 16.8 MB + Q 1.0 MB read, 8.9 MB of partials written.
         "traffic": CONTEXT_PASS_HBM_BYTES,
         "launches": n_dec,
         "avg_launch_us": round(avg_launch_us, 2),
+        # In the timed schedule the buffer pass of the same layer runs beside this kernel and takes
+        # issue slots from it; these two are the kernel without that neighbour.
+        "avg_launch_us_alone": round(alone_ms * 1e3 / max(n_dec, 1), 2),
+        "frac_alone": round(flops_total / (alone_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4) if alone_ms > 0 else None,
         "flops_per_launch_lq2": 4.0 * B3 * H * 2 * NC3 * Dh,
         "prefill_tflops": round(prefill_flops / (ptot.value * 1e-3) / 1e12, 2) if ptot.value > 0 else None,
     }
