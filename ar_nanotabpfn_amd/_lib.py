@@ -101,6 +101,7 @@ SIGNATURES = {
         _i,
         [_p, _i64, _p, _i64, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _f, _p, _p, _p, _f, _p, _p, _p, _i64, _i, _i, _i, _p],
     ),
+    "artab_merge_attention_partials": (_i, [ctypes.POINTER(ArtabAttentionPartials), _VP, _i, _p]),
     "artab_layer_post_from_partials": (
         _i, [ctypes.POINTER(ArtabAttentionPartials), _p, _i64, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _f, _p, _i64, _i, _i, _i, _p]),
     "artab_layer_post_pre_from_partials": (

@@ -290,6 +290,16 @@ class AttentionPartials:
     def shape(self):  # of the merged [B,H,Lq,Dh] result
         return (self.desc.B, self.desc.H, self.desc.Lq, self.desc.Dh)
 
+    def merged(self) -> Tensor:
+        """The merged ``[B,H,Lq,Dh]`` tensor (``artab_merge_attention_partials``), for callers whose
+        next step is not one of the layer kernels that merge on load."""
+        B, H, Lq, Dh = self.shape
+        out = torch.empty((B, Lq, H, Dh), device=self.device, dtype=self.dtype).transpose(1, 2)
+        ov = _lib.view4(out)
+        _lib.check(_lib.load().artab_merge_attention_partials(
+            ctypes.byref(self.desc), _lib.ref(ov), _lib.dtype_code(self.dtype), _lib.current_stream(self.device)))
+        return out
+
 
 def teacher_forcing_attention(
     q: Tensor, k_ctx: Tensor, v_ctx: Tensor, k_buf: Tensor, v_buf: Tensor, num_targets: int,

@@ -360,55 +360,81 @@ static int fork_join_events(hipEvent_t *fork, hipEvent_t *join) {
 
 namespace {
 
+// Token rows per workgroup of the layer kernels: 16 while that still leaves the launch within a
+// few workgroups per CU (everything a workgroup does per row is bound by its one CU), else 32
+// (half the weight traffic per row).
+inline int fused_tile_rows(long rows) {
+    if (const char *e = getenv("ARTAB_TILE_ROWS")) {  // tuning / test hook
+        const int v = atoi(e);
+        if (v == kFusedRows || v == kFusedRowsSmall) return v;
+    }
+    return rows <= kFusedSmallMaxRows ? kFusedRowsSmall : kFusedRows;
+}
+
+template <typename T, int TR>
+hipError_t launch_pre_r(const FusedPreParams &P, int D, hipStream_t st) {
+    dim3 grid(static_cast<unsigned>((P.rows + TR - 1) / TR)), block(fused_waves(D) * 64);
+    switch (D) {
+        case 128: hipLaunchKernelGGL((fused_pre_kernel<T, 128, TR>), grid, block, 0, st, P); break;
+        case 256: hipLaunchKernelGGL((fused_pre_kernel<T, 256, TR>), grid, block, 0, st, P); break;
+        default: hipLaunchKernelGGL((fused_pre_kernel<T, 512, TR>), grid, block, 0, st, P); break;
+    }
+    return hipGetLastError();
+}
 template <typename T>
 hipError_t launch_pre(const FusedPreParams &P, int D, hipStream_t st) {
-    dim3 grid(static_cast<unsigned>((P.rows + kFusedRows - 1) / kFusedRows)), block(fused_waves(D) * 64);
-    switch (D) {
-        case 128: hipLaunchKernelGGL((fused_pre_kernel<T, 128>), grid, block, 0, st, P); break;
-        case 256: hipLaunchKernelGGL((fused_pre_kernel<T, 256>), grid, block, 0, st, P); break;
-        default: hipLaunchKernelGGL((fused_pre_kernel<T, 512>), grid, block, 0, st, P); break;
-    }
-    return hipGetLastError();
+    return fused_tile_rows(P.rows) == kFusedRowsSmall ? launch_pre_r<T, kFusedRowsSmall>(P, D, st)
+                                                      : launch_pre_r<T, kFusedRows>(P, D, st);
 }
 
-template <typename T, int D>
+template <typename T, int D, int TR>
 hipError_t launch_post_d(const FusedPostParams &P, int F, hipStream_t st) {
-    dim3 grid(static_cast<unsigned>((P.rows + kFusedRows - 1) / kFusedRows)), block(fused_waves(D) * 64);
+    dim3 grid(static_cast<unsigned>((P.rows + TR - 1) / TR)), block(fused_waves(D) * 64);
     switch (F) {
-        case 128: hipLaunchKernelGGL((fused_post_kernel<T, D, 128>), grid, block, 0, st, P); break;
-        case 256: hipLaunchKernelGGL((fused_post_kernel<T, D, 256>), grid, block, 0, st, P); break;
-        default: hipLaunchKernelGGL((fused_post_kernel<T, D, 512>), grid, block, 0, st, P); break;
+        case 128: hipLaunchKernelGGL((fused_post_kernel<T, D, 128, TR>), grid, block, 0, st, P); break;
+        case 256: hipLaunchKernelGGL((fused_post_kernel<T, D, 256, TR>), grid, block, 0, st, P); break;
+        default: hipLaunchKernelGGL((fused_post_kernel<T, D, 512, TR>), grid, block, 0, st, P); break;
     }
     return hipGetLastError();
 }
 
-template <typename T, int D>
+template <typename T, int D, int TR>
 hipError_t launch_post_pre_d(const FusedPostParams &P, const FusedPreParams &N, int F, hipStream_t st) {
-    dim3 grid(static_cast<unsigned>((P.rows + kFusedRows - 1) / kFusedRows)), block(fused_waves(D) * 64);
+    dim3 grid(static_cast<unsigned>((P.rows + TR - 1) / TR)), block(fused_waves(D) * 64);
     switch (F) {
-        case 128: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 128>), grid, block, 0, st, P, N); break;
-        case 256: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 256>), grid, block, 0, st, P, N); break;
-        default: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 512>), grid, block, 0, st, P, N); break;
+        case 128: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 128, TR>), grid, block, 0, st, P, N); break;
+        case 256: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 256, TR>), grid, block, 0, st, P, N); break;
+        default: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 512, TR>), grid, block, 0, st, P, N); break;
     }
     return hipGetLastError();
 }
 
+template <typename T, int TR>
+hipError_t launch_post_pre_r(const FusedPostParams &P, const FusedPreParams &N, int D, int F, hipStream_t st) {
+    switch (D) {
+        case 128: return launch_post_pre_d<T, 128, TR>(P, N, F, st);
+        case 256: return launch_post_pre_d<T, 256, TR>(P, N, F, st);
+        default: return launch_post_pre_d<T, 512, TR>(P, N, F, st);
+    }
+}
 template <typename T>
 hipError_t launch_post_pre(const FusedPostParams &P, const FusedPreParams &N, int D, int F, hipStream_t st) {
-    switch (D) {
-        case 128: return launch_post_pre_d<T, 128>(P, N, F, st);
-        case 256: return launch_post_pre_d<T, 256>(P, N, F, st);
-        default: return launch_post_pre_d<T, 512>(P, N, F, st);
-    }
+    return fused_tile_rows(P.rows) == kFusedRowsSmall ? launch_post_pre_r<T, kFusedRowsSmall>(P, N, D, F, st)
+                                                      : launch_post_pre_r<T, kFusedRows>(P, N, D, F, st);
 }
 
+template <typename T, int TR>
+hipError_t launch_post_r(const FusedPostParams &P, int D, int F, hipStream_t st) {
+    switch (D) {
+        case 128: return launch_post_d<T, 128, TR>(P, F, st);
+        case 256: return launch_post_d<T, 256, TR>(P, F, st);
+        default: return launch_post_d<T, 512, TR>(P, F, st);
+    }
+}
 template <typename T>
 hipError_t launch_post(const FusedPostParams &P, int D, int F, hipStream_t st) {
-    switch (D) {
-        case 128: return launch_post_d<T, 128>(P, F, st);
-        case 256: return launch_post_d<T, 256>(P, F, st);
-        default: return launch_post_d<T, 512>(P, F, st);
-    }
+    return fused_tile_rows(P.rows) == kFusedRowsSmall ? launch_post_r<T, kFusedRowsSmall>(P, D, F, st)
+                                                      : launch_post_r<T, kFusedRows>(P, D, F, st);
 }
 
 template <typename T, int D>
@@ -726,6 +752,27 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
     return launch_status(hipGetLastError(), "decode combine");
 }
 
+int artab_merge_attention_partials(const artab_attention_partials *partials, const artab_view *out, int dtype,
+                                   void *stream) {
+    if (!partials || !out || !out->data) return fail(ARTAB_ERR_NULL_POINTER, "merge partials: null argument");
+    if (dtype != ARTAB_BF16 && dtype != ARTAB_F16)
+        return fail(ARTAB_ERR_UNSUPPORTED, "merge partials: partial outputs exist in bf16/fp16 only");
+    if (partials->n_slots < 1 || !partials->part_o || !partials->part_lse || partials->B < 1 || partials->H < 1 ||
+        partials->Lq < 1 || partials->Dh < 4 || partials->Dh % 4)
+        return fail(ARTAB_ERR_BAD_SHAPE, "merge partials: empty or malformed descriptor");
+    CombineParams C;
+    C.out = dv(out); C.part_o = partials->part_o; C.part_lse = partials->part_lse; C.lse = nullptr;
+    C.rows = static_cast<long>(partials->B) * partials->H * partials->Lq;
+    C.H = partials->H; C.Lq = partials->Lq; C.Dh = partials->Dh; C.n_split = partials->n_slots;
+    unsigned grid = static_cast<unsigned>((C.rows * (C.Dh / 4) + 255) / 256);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == ARTAB_BF16)
+        hipLaunchKernelGGL((combine_kernel<bf16_t>), dim3(grid), dim3(256), 0, st, C);
+    else
+        hipLaunchKernelGGL((combine_kernel<f16_t>), dim3(grid), dim3(256), 0, st, C);
+    return launch_status(hipGetLastError(), "merge partials");
+}
+
 int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
                            const artab_view *k_buf, const artab_view *v_buf, const artab_view *k_new,
                            const artab_view *v_new, const artab_view *out, int B, int H, int Lq, int Nc,
@@ -1002,6 +1049,8 @@ static int fill_post(FusedPostParams &P, const void *attn, int64_t lda, const vo
                         "partials (B=%d H=%d Lq=%d Dh=%d, %d slots) do not describe %lld rows of width %d", parts->B,
                         parts->H, parts->Lq, parts->Dh, parts->n_slots, (long long)rows, D);
         if (misaligned16(parts->part_o)) return fail(ARTAB_ERR_BAD_STRIDE, "partials must be 16-byte aligned");
+        if (static_cast<int64_t>(parts->B) * parts->H * parts->Lq >= (int64_t{1} << 31))
+            return fail(ARTAB_ERR_BAD_SHAPE, "partials: B*H*Lq must stay below 2^31");  // the kernel indexes rows in 32 bits
         P.part_o = parts->part_o; P.part_lse = parts->part_lse; P.n_slots = parts->n_slots;
         P.part_rows = static_cast<long>(parts->B) * parts->H * parts->Lq; P.H = parts->H; P.Lq = parts->Lq;
         attn = parts->part_o;  // placeholder for the checks below

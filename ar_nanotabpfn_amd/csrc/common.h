@@ -99,6 +99,33 @@ __device__ __forceinline__ float wave_sum(float x) {
     return x;
 }
 
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding).
+constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
+
+// 16 bytes per lane from global memory straight into LDS: lane l lands at lds + 16 l (lds is
+// wavefront-uniform; lanes switched off write nothing and leave their 16 bytes untouched).
+// Kept in a plain function: called directly from a kernel template the builtin makes the host
+// pass drop the kernel's launch stub.
+__device__ __forceinline__ void load_to_lds_16(const void *global_src, void *lds_dst) {
+    __builtin_amdgcn_global_load_lds(global_src, lds_dst, 16, 0, 0);
+}
+
+// A 64-byte row per lane in four 16-byte pieces, piece t of lane l landing at lds + 1024 t + 16 l.
+// The instruction's immediate offset moves the global AND the LDS address, hence the 1008 = 1024 - 16
+// per piece on the LDS side: no per-piece address arithmetic in vector registers.
+__device__ __forceinline__ void load_row64_to_lds(const void *global_src, unsigned char *lds_dst) {
+    __builtin_amdgcn_global_load_lds(global_src, lds_dst, 16, 0, 0);
+    __builtin_amdgcn_global_load_lds(global_src, lds_dst + 1008, 16, 16, 0);
+    __builtin_amdgcn_global_load_lds(global_src, lds_dst + 2016, 16, 32, 0);
+    __builtin_amdgcn_global_load_lds(global_src, lds_dst + 3024, 16, 48, 0);
+}
+
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 // Visible-key limit of teacher-forcing query row i among Nt buffer keys: buffer
 // query i (< Nt) sees keys [0, i]; target query i (>= Nt) sees keys [0, i - Nt).
 __host__ __device__ __forceinline__ int tf_limit(int i, int Nt) { return i < Nt ? i + 1 : i - Nt; }

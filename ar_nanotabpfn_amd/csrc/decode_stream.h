@@ -34,16 +34,6 @@ constexpr int kStreamChunkBytes = 8192;    // 4 keys x 16 pairs x (64 B of K + 6
 constexpr int kStreamQBytes = 4096;        // one task's queries: 4 x (64 lanes x 16 B)
 constexpr size_t kStreamLdsBytes = kStreamChunks * kStreamChunkBytes + 2 * kStreamQBytes;
 
-// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding).
-constexpr int vmcnt_imm(int n) { return (n & 15) | (7 << 4) | (15 << 8) | ((n >> 4) << 14); }
-
-// 16 bytes per lane from global memory straight into LDS: lane l lands at lds + 16 l (lds is
-// wavefront-uniform).  Kept in a plain function: called directly from a kernel template the
-// builtin makes the host pass drop the kernel's launch stub.
-__device__ __forceinline__ void load_to_lds_16(const void *global_src, void *lds_dst) {
-    __builtin_amdgcn_global_load_lds(global_src, lds_dst, 16, 0, 0);
-}
-
 // LDS reads of the ring go through inline assembly: the compiler must not see an LDS read that
 // could alias the asynchronous fills, or it would drain every load before each read.
 // Two 16-byte pieces of this lane's K row (addr_k, +1024) and of its query row (addr_q, +1024):
@@ -68,6 +58,9 @@ __device__ __forceinline__ void lds_read2x128(u32x4 &a, u32x4 &b, unsigned addr)
         : "=&v"(a), "=&v"(b)
         : "v"(addr)
         : "memory");
+}
+__device__ __forceinline__ void lds_write128(unsigned addr, u32x4 v) {
+    asm volatile("ds_write_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : : "v"(addr), "v"(v) : "memory");
 }
 // Four transposing reads: the V operands of four 4-dim groups of one 4-key chunk.
 // Address layout of a V chunk: sub-slot t (1 KiB) holds dims 8t..8t+7, so group u = 2t + half
@@ -170,11 +163,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
         if (first) {
             p_k = view_row<T>(vkb, p_b, p_h, sub);
             p_v = view_row<T>(vvb, p_b, p_h, sub);
-            // the task's queries: lane (p, j < LQ) fetches its 64-byte row in four pieces
-            const T *qrow = view_row<T>(vq, p_b, p_h, sub < LQ ? sub : 0);
+            // the task's queries: lane (p, j < LQ) fetches its 64-byte row in four pieces; the
+            // pieces of the other lanes stay zero (cleared once, below)
             unsigned char *qd = stream_lds + S * kStreamChunkBytes + issue_q * kStreamQBytes;
-#pragma unroll
-            for (int t = 0; t < 4; ++t) load_to_lds_16(qrow + 8 * t, qd + 1024 * t);
+            if (sub < LQ) load_row64_to_lds(view_row<T>(vq, p_b, p_h, sub), qd);
         }
         const T *kr = p_k, *vr = p_v;
         if (last) {
@@ -185,10 +177,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
             vr = is_new ? view_row<T>(vvn, p_b, p_h, 0) : view_row<T>(vvb, p_b, p_h, row);
         }
         unsigned char *cd = stream_lds + issue_slot * kStreamChunkBytes;
-#pragma unroll
-        for (int t = 0; t < 4; ++t) load_to_lds_16(kr + 8 * t, cd + 1024 * t);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) load_to_lds_16(vr + 8 * t, cd + 4096 + 1024 * t);
+        load_row64_to_lds(kr, cd);
+        load_row64_to_lds(vr, cd + 4096);
         p_k += chunk_step;
         p_v += chunk_step_v;
         ++issued;
@@ -200,13 +190,20 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
             ++issue_seq;
         }
     };
+    // Lanes that stand for no query (sub >= LQ) contribute zeros to the score product: their
+    // pieces of both query slots are cleared once and never written again.
+    if (sub >= LQ) {
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int t = 0; t < 8; ++t) lds_write128(q_lds0 + 1024u * t + lane * 16u, zero);
+    }
     // two query slots: the producer may be at most one task ahead of the consumer
     auto may_issue = [&]() { return issued < total_chunks && issue_seq <= seq + 1; };
     for (int i = 0; i < S; ++i)
         if (may_issue()) issue_one();
 
     // ---- consumer
-    float m = -INFINITY, l = 0.f;
+    float m = -INFINITY, mq = 0.f, l = 0.f;  // running maximum of the raw scores, and times qscale
     f32x4 o[8];  // output dims 4u..4u+3 of this lane's query
 #pragma unroll
     for (int u = 0; u < 8; ++u) o[u] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -223,17 +220,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
         const unsigned chunk = lds0 + static_cast<unsigned>(slot) * kStreamChunkBytes;
         const unsigned qaddr = q_lds0 + static_cast<unsigned>(qsel) * kStreamQBytes + lane * 16u;
 
-        // ---- scores of 4 keys for this lane's query, head dims in two halves (register budget).
-        // Lanes that stand for no query (sub >= LQ) multiply by zero.
+        // ---- scores of 4 keys for this lane's query, head dims in two halves (register budget)
         f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
             u32x4 k0, k1, q0, q1;
             lds_read_kq(k0, k1, q0, q1, chunk + 2048u * half + lane * 16u, qaddr + 2048u * half);
-            if (sub >= LQ) {
-                q0 = u32x4{0u, 0u, 0u, 0u};
-                q1 = q0;
-            }
             s = Mfma4<T>::mma(u32x2{k0[0], k0[1]}, u32x2{q0[0], q0[1]}, s);
             s = Mfma4<T>::mma(u32x2{k0[2], k0[3]}, u32x2{q0[2], q0[3]}, s);
             s = Mfma4<T>::mma(u32x2{k1[0], k1[1]}, u32x2{q1[0], q1[1]}, s);
@@ -258,25 +250,24 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
                 }
             }
         }
-        float sc[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) sc[r] = s[r] * qscale;
+        float sc[4] = {s[0], s[1], s[2], s[3]};  // raw dot products; qscale (> 0) enters with the exponent
         if (g + 1 == n_groups) {  // only a task's last chunk can hold keys past the end
 #pragma unroll
             for (int r = 0; r < 4; ++r) sc[r] = 4 * g + r < n_total ? sc[r] : -INFINITY;
         }
         // online softmax; the rescale is skipped (wavefront-uniformly) while no maximum moves
-        const float m_new = fmaxf(fmaxf(m, fmaxf(sc[0], sc[1])), fmaxf(sc[2], sc[3]));
+        const float m_new = max3(max3(m, sc[0], sc[1]), sc[2], sc[3]);
         if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
-            const float alpha = m == -INFINITY ? 0.f : fast_exp2(m - m_new);
+            const float alpha = m == -INFINITY ? 0.f : fast_exp2((m - m_new) * qscale);
             l *= alpha;
 #pragma unroll
             for (int u = 0; u < 8; ++u) o[u] *= alpha;
             m = m_new;
+            mq = m_new * qscale;
         }
         float p[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) p[r] = fast_exp2(sc[r] - m);  // m is finite here: key 4g is always valid
+        for (int r = 0; r < 4; ++r) p[r] = fast_exp2(fmaf(sc[r], qscale, -mq));  // m is finite here: key 4g is always valid
         l += (p[0] + p[1]) + (p[2] + p[3]);
         const u32x2 pop = {pack2<T>(p[0], p[1]), pack2<T>(p[2], p[3])};
 #pragma unroll
@@ -304,9 +295,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
                                  pack2<T>(o[2 * e + 1][2] * inv, o[2 * e + 1][3] * inv)};
                     *reinterpret_cast<u32x4 *>(po + 8 * e) = val;
                 }
-                part_lse[static_cast<long>(pair) * LQ + sub] = l > 0.f ? (m + fast_log2(l)) * kLn2 : -INFINITY;
+                part_lse[static_cast<long>(pair) * LQ + sub] = l > 0.f ? (mq + fast_log2(l)) * kLn2 : -INFINITY;
             }
             m = -INFINITY;
+            mq = 0.f;
             l = 0.f;
 #pragma unroll
             for (int u = 0; u < 8; ++u) o[u] = f32x4{0.f, 0.f, 0.f, 0.f};

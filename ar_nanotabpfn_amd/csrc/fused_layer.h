@@ -8,8 +8,9 @@
 //   fused_post_kernel:  x1 = LN2(y + attn W_o^T);  h = gelu(x1 W_1^T + b_1);
 //                       out = LN3(x1 + h W_2^T + b_2)
 //
-// One workgroup owns 32 token rows and all columns.  Products are computed transposed
-// with v_mfma_f32_32x32x16 (C^T[n, m] = sum_k W[n, k] A[m, k]): the weight rows are the
+// One workgroup owns 32 (or, for few rows, 16) token rows and all columns.  Products are
+// computed transposed with v_mfma_f32_32x32x16 / v_mfma_f32_16x16x32
+// (C^T[n, m] = sum_k W[n, k] A[m, k]): the weight rows are the
 // A operand, read straight from global memory in a pre-packed operand order (weights are
 // constants, packed once), so every wavefront load is one contiguous KiB; the
 // activation rows are the B operand, staged once in LDS and re-read per 16 contraction
@@ -23,7 +24,12 @@
 
 namespace artab {
 
-constexpr int kFusedRows = 32;  // token rows per workgroup
+constexpr int kFusedRows = 32;       // token rows per workgroup ...
+constexpr int kFusedRowsSmall = 16;  // ... or, when that leaves most of the chip idle, 16: a decode step has
+                                     // 2048 rows = 64 workgroups of 32, and everything a workgroup does
+                                     // per row (merge, LayerNorm, epilogues) is bound by its one CU's
+                                     // instruction issue
+constexpr long kFusedSmallMaxRows = 8192;  // up to here the 16-row tiles are used
 
 // Stands in for an absent bias vector (1024 16-bit zeros; widths go up to 512).
 static __device__ const unsigned int kZeroVector[512] = {0u};
@@ -79,17 +85,78 @@ __global__ void pack_weight_kernel(const T *w, T *packed, int N, int K) {
     *reinterpret_cast<u32x4 *>(packed + chunk * 8) = *reinterpret_cast<const u32x4 *>(src);
 }
 
+// Tile shapes.  TR = 32: v_mfma_f32_32x32x16, a lane owns token lane%32 and, per block of 32
+// output features, 16 of them in four groups of four consecutive ones (group g of half
+// s = lane/32 starts at 8g + 4s).  TR = 16: v_mfma_f32_16x16x32, token lane%16, blocks of 16
+// features, one group of four starting at 4s with s = lane/16.  Both read the same packed weights:
+// the A operand of the 16x16x32 shape for feature block nb and 32-wide contraction step KS is
+// W[16 nb + lane%16][32 KS + 8 s ..], which the 32x32x16 packing holds at block nb/2, 16-wide step
+// 2 KS + s/2, lane 16 (nb%2) + lane%16 + 32 (s%2) — runs of 256 contiguous bytes.
+template <typename T>
+struct Mfma16;
+template <>
+struct Mfma16<bf16_t> {
+    static __device__ __forceinline__ f32x4 mma(bf16x8 a, bf16x8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <>
+struct Mfma16<f16_t> {
+    static __device__ __forceinline__ f32x4 mma(f16x8 a, f16x8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+template <typename T, int TR>
+struct Tile;
+template <typename T>
+struct Tile<T, 32> {
+    typedef f32x16 acc_t;
+    typedef typename MfmaOps<T>::vec vec;
+    static constexpr int kBlock = 32, kGroups = 4, kVals = 16, kStepK = 16;
+    static constexpr long kStepStride = 512;  // packed elements from one contraction step to the next
+    static __device__ __forceinline__ int token(int lane) { return lane & 31; }
+    static __device__ __forceinline__ int sub(int lane) { return lane >> 5; }
+    static __device__ __forceinline__ int col(int nb, int g, int s) { return 32 * nb + 8 * g + 4 * s; }
+    static __device__ __forceinline__ long weight_offset(int nb, int K, int lane) {
+        return (static_cast<long>(nb) * (K / 16) * 64 + lane) * 8;
+    }
+    static __device__ __forceinline__ acc_t mma(vec a, vec b, acc_t c) { return MfmaOps<T>::mma(a, b, c); }
+    // sum over the lanes that hold the same token
+    static __device__ __forceinline__ float over_token(float x) { return x + __shfl_xor(x, 32, 64); }
+};
+template <typename T>
+struct Tile<T, 16> {
+    typedef f32x4 acc_t;
+    typedef typename MfmaOps<T>::vec vec;
+    static constexpr int kBlock = 16, kGroups = 1, kVals = 4, kStepK = 32;
+    static constexpr long kStepStride = 1024;
+    static __device__ __forceinline__ int token(int lane) { return lane & 15; }
+    static __device__ __forceinline__ int sub(int lane) { return lane >> 4; }
+    static __device__ __forceinline__ int col(int nb, int, int s) { return 16 * nb + 4 * s; }
+    static __device__ __forceinline__ long weight_offset(int nb, int K, int lane) {
+        const int s = lane >> 4, c = lane & 15;
+        return ((static_cast<long>(nb >> 1) * (K / 16) + (s >> 1)) * 64 + 16 * (nb & 1) + c + 32 * (s & 1)) * 8;
+    }
+    static __device__ __forceinline__ acc_t mma(vec a, vec b, acc_t c) { return Mfma16<T>::mma(a, b, c); }
+    static __device__ __forceinline__ float over_token(float x) {
+        x += __shfl_xor(x, 16, 64);
+        return x + __shfl_xor(x, 32, 64);
+    }
+};
+
 // One transposed product: acc[b][v] = sum_k W[32*nblk[b] + row(v)][k] * A[c][k] for NB blocks of
 // 32 output columns; A is the [32, K] activation tile in LDS (row stride ld), W the packed weight.
 // The weight fragments are fetched explicitly ahead of their use — start() issues the first PF
 // contraction steps and can be called long before run(), e.g. ahead of the previous product's
 // epilogue, so that the memory round trips of chained products overlap.  (Left to itself the
 // compiler issues each load right before the MFMA that needs it: one round trip per step.)
-template <typename T, int K, int NB>
+template <typename T, int K, int NB, int TR = 32>
 struct WeightStream {
-    typedef MfmaOps<T> Ops;
-    typedef typename Ops::vec vec;
-    static constexpr int KS = K / 16;
+    typedef Tile<T, TR> TL;
+    typedef typename TL::vec vec;
+    typedef typename TL::acc_t acc_t;
+    static constexpr int KS = K / TL::kStepK;
     static constexpr int PFW = NB >= 4 ? 4 : (NB == 2 ? 8 : 16);
     static constexpr int PF = PFW < KS ? PFW : KS;
     const T *wl[NB];
@@ -97,27 +164,28 @@ struct WeightStream {
 
     __device__ __forceinline__ void start(const T *wp, const int (&nblk)[NB], int lane) {
 #pragma unroll
-        for (int b = 0; b < NB; ++b) wl[b] = wp + static_cast<long>(nblk[b]) * KS * 512 + lane * 8;
+        for (int b = 0; b < NB; ++b) wl[b] = wp + TL::weight_offset(nblk[b], K, lane);
 #pragma unroll
         for (int p = 0; p < PF; ++p)
 #pragma unroll
-            for (int b = 0; b < NB; ++b) wf[p][b] = *reinterpret_cast<const vec *>(wl[b] + p * 512);
+            for (int b = 0; b < NB; ++b) wf[p][b] = *reinterpret_cast<const vec *>(wl[b] + p * TL::kStepStride);
         __builtin_amdgcn_sched_barrier(0);  // the prefetch stays where it was written
     }
 
-    __device__ __forceinline__ void run(f32x16 (&acc)[NB], const T *a_lds, int ld, int c, int hb) {
+    __device__ __forceinline__ void run(acc_t (&acc)[NB], const T *a_lds, int ld, int c, int hb) {
 #pragma unroll
         for (int b = 0; b < NB; ++b)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[b][v] = 0.f;
+            for (int v = 0; v < TL::kVals; ++v) acc[b][v] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            const vec af = *reinterpret_cast<const vec *>(a_lds + c * ld + 16 * ks + 8 * hb);
+            const vec af = *reinterpret_cast<const vec *>(a_lds + c * ld + TL::kStepK * ks + 8 * hb);
 #pragma unroll
-            for (int b = 0; b < NB; ++b) acc[b] = Ops::mma(wf[ks % PF][b], af, acc[b]);
+            for (int b = 0; b < NB; ++b) acc[b] = TL::mma(wf[ks % PF][b], af, acc[b]);
             if (ks + PF < KS) {
 #pragma unroll
-                for (int b = 0; b < NB; ++b) wf[ks % PF][b] = *reinterpret_cast<const vec *>(wl[b] + (ks + PF) * 512);
+                for (int b = 0; b < NB; ++b)
+                    wf[ks % PF][b] = *reinterpret_cast<const vec *>(wl[b] + (ks + PF) * TL::kStepStride);
             }
         }
     }
@@ -142,37 +210,124 @@ __device__ __forceinline__ void store4f(T *p, float a, float b, float c, float d
 
 // The entries of a length-N vector (bias, gamma, beta) at this lane's accumulator columns;
 // a missing bias is read from a zero vector the caller substitutes.
-template <typename T, int NB>
-__device__ __forceinline__ void load_cols(const T *vec, const int (&nblk)[NB], int hb, float (&out)[NB][16]) {
+template <typename T, int NB, int TR = 32>
+__device__ __forceinline__ void load_cols(const T *vec, const int (&nblk)[NB], int hb,
+                                          float (&out)[NB][Tile<T, TR>::kVals]) {
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) load4f<T>(vec + col_of(nblk[b], 4 * g, hb), &out[b][4 * g]);
+        for (int g = 0; g < Tile<T, TR>::kGroups; ++g)
+            load4f<T>(vec + Tile<T, TR>::col(nblk[b], g, hb), &out[b][4 * g]);
 }
 
 // The attention tile of 32 token rows built from partial results (context slices + buffer pass)
 // instead of a finished matrix: out = sum_s w_s o_s / sum_s w_s with w_s = exp(lse_s - max lse),
 // the same arithmetic, in the same order, as the stand-alone combine launch, rounded once to the
 // storage type on its way into LDS.  One item = 8 output dims of one (row, head).
+// Partial row and first dim of item (token row `tok`, 16-byte chunk `ch`): token = b*Lq + i, the
+// chunk lies in head h at dim d0, and the partial row is (b*H + h)*Lq + i.  Decode has Lq in
+// {1, 2} and a power-of-two head dim: those take shifts; anything else 32-bit divisions (a
+// 64-bit division per item cost more than the loads it addressed).
+struct PartialIndex {
+    int lq, heads, dh, dh_shift;  // dh_shift < 0: head dim is not a power of two
+    __device__ __forceinline__ PartialIndex(int Lq, int H, int Dh)
+        : lq(Lq), heads(H), dh(Dh), dh_shift((Dh & (Dh - 1)) == 0 ? __builtin_ctz(static_cast<unsigned>(Dh)) : -1) {}
+    __device__ __forceinline__ void locate(unsigned tok, int ch, unsigned &prow, int &d0) const {
+        unsigned b, i;
+        if (lq == 1) {
+            b = tok; i = 0;
+        } else if (lq == 2) {
+            b = tok >> 1; i = tok & 1u;
+        } else {
+            b = tok / static_cast<unsigned>(lq); i = tok - b * static_cast<unsigned>(lq);
+        }
+        unsigned h;
+        if (dh_shift >= 0) {
+            h = static_cast<unsigned>(8 * ch) >> dh_shift; d0 = (8 * ch) & (dh - 1);
+        } else {
+            h = static_cast<unsigned>(8 * ch) / static_cast<unsigned>(dh); d0 = 8 * ch - static_cast<int>(h) * dh;
+        }
+        prow = (b * static_cast<unsigned>(heads) + h) * static_cast<unsigned>(lq) + i;
+    }
+};
+
 constexpr int kMergeBatch = 9;  // partials fetched per round (8 context slices + the buffer pass)
 
-template <typename T, int D, int NT>
+template <typename T, int D, int NT, int TR>
 __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const FusedPostParams &P, long row0,
                                                        int valid, int tid) {
     const int dh = D / P.H;          // head dim, a multiple of 8
+    const PartialIndex where(P.Lq, P.H, dh);
+    const unsigned tok0 = static_cast<unsigned>(row0);  // the launcher keeps rows below 2^31
     constexpr int CPR = D / 8;       // 16-byte chunks per token row
-    for (int idx = tid; idx < kFusedRows * CPR; idx += NT) {
+    constexpr int ITEMS = TR * CPR / NT;
+    static_assert(TR * CPR % NT == 0, "whole items per thread");
+    const long o_step = P.part_rows * dh;
+    if (P.n_slots <= kMergeBatch) {
+        // Common case: every slot of two items is requested before anything is used, so the
+        // thread pays one memory round trip per pair of items (rows beyond `valid` read the
+        // last valid row and are zeroed afterwards: no divergent loads).
+        constexpr int G = ITEMS % 2 == 0 ? 2 : 1;
+#pragma unroll
+        for (int it0 = 0; it0 < ITEMS; it0 += G) {
+            float lv[G][kMergeBatch];
+            u32x4 ov[G][kMergeBatch];
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const int idx = tid + (it0 + g) * NT;
+                const int r = idx / CPR, ch = idx % CPR;
+                unsigned prow;
+                int d0;
+                where.locate(tok0 + (r < valid ? r : valid - 1), ch, prow, d0);
+                const T *po = static_cast<const T *>(P.part_o) + static_cast<long>(prow) * dh + d0;
+                const float *pl = P.part_lse + prow;
+#pragma unroll
+                for (int u = 0; u < kMergeBatch; ++u) {
+                    const int sl = u < P.n_slots ? u : P.n_slots - 1;
+                    lv[g][u] = pl[sl * P.part_rows];
+                    ov[g][u] = *reinterpret_cast<const u32x4 *>(po + sl * o_step);
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const int idx = tid + (it0 + g) * NT;
+                const int r = idx / CPR, ch = idx % CPR;
+                float mx = -INFINITY;
+#pragma unroll
+                for (int u = 0; u < kMergeBatch; ++u) mx = fmaxf(mx, lv[g][u]);  // repeats of the last slot change nothing
+                float wsum = 0.f, acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int u = 0; u < kMergeBatch; ++u) {
+                    if (u < P.n_slots) {
+                        const float w = expf(lv[g][u] - mx);
+                        wsum += w;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            acc[2 * e] = fmaf(w, unpack_lo<T>(ov[g][u][e]), acc[2 * e]);
+                            acc[2 * e + 1] = fmaf(w, unpack_hi<T>(ov[g][u][e]), acc[2 * e + 1]);
+                        }
+                    }
+                }
+                const float inv = 1.f / wsum;
+                u32x4 packed = {0u, 0u, 0u, 0u};
+                if (r < valid) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) packed[e] = pack2<T>(acc[2 * e] * inv, acc[2 * e + 1] * inv);
+                }
+                *reinterpret_cast<u32x4 *>(dst + r * lds_ld + 8 * ch) = packed;
+            }
+        }
+        return;
+    }
+    for (int idx = tid; idx < TR * CPR; idx += NT) {
         const int r = idx / CPR, ch = idx % CPR;
         u32x4 packed = {0u, 0u, 0u, 0u};
         if (r < valid) {
-            const long tok = row0 + r;
-            const long b = tok / P.Lq;
-            const int i = static_cast<int>(tok % P.Lq);
-            const int h = (8 * ch) / dh, d0 = (8 * ch) % dh;
-            const long prow = (b * P.H + h) * P.Lq + i;
-            const T *po = static_cast<const T *>(P.part_o) + prow * dh + d0;
+            unsigned prow;
+            int d0;
+            where.locate(tok0 + r, ch, prow, d0);
+            const T *po = static_cast<const T *>(P.part_o) + static_cast<long>(prow) * dh + d0;
             const float *pl = P.part_lse + prow;
-            const long o_step = P.part_rows * dh;
             float mx = -INFINITY;
             for (int s0 = 0; s0 < P.n_slots; s0 += kMergeBatch) {
                 float lv[kMergeBatch];
@@ -218,73 +373,112 @@ __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const
 // Parameter vectors (LayerNorm gamma / beta, biases) are copied to LDS when the kernel starts:
 // fetched from global memory right where they are used, each costs its phase a full memory
 // round trip (the phases are far shorter than that).  A missing vector becomes zeros.
-template <typename T, int LEN, int NT>
-__device__ __forceinline__ void stage_vector(T *dst, const void *src, int tid) {
-    static_assert(LEN % 8 == 0, "16-byte chunks");
-    for (int ch = tid; ch < LEN / 8; ch += NT) {
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (src) v = *reinterpret_cast<const u32x4 *>(static_cast<const T *>(src) + 8 * ch);
-        *reinterpret_cast<u32x4 *>(dst + 8 * ch) = v;
+// Tiles and vectors are copied without registers: each wavefront sends whole rows (one vector) from global
+// memory straight into LDS, so every load of a kernel's prologue is in flight at once instead of
+// one round trip per copy.  The caller waits (vmcnt 0) before the barrier that publishes them.
+template <typename T, int W, int NT, int TR>
+__device__ __forceinline__ void dma_tile(T *dst, int lds_ld, const T *src, long ld, int valid, int tid) {
+    constexpr int NW = NT / 64, CPR = W / 8;
+    static_assert(CPR <= 64, "a row is at most one wavefront of 16-byte pieces");
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+#pragma unroll
+    for (int r = wave; r < TR; r += NW) {
+        if (lane < CPR) {
+            if (r < valid) {
+                load_to_lds_16(src + r * ld + 8 * lane, dst + r * lds_ld);
+            } else {
+                const u32x4 zero = {0u, 0u, 0u, 0u};
+                *reinterpret_cast<u32x4 *>(dst + r * lds_ld + 8 * lane) = zero;
+            }
+        }
     }
 }
+// `turn` spreads the vectors of a prologue over the wavefronts.
+template <typename T, int LEN, int NT>
+__device__ __forceinline__ void dma_vector(T *dst, const void *src, int tid, int turn) {
+    constexpr int NW = NT / 64;
+    static_assert(LEN % 8 == 0 && LEN / 8 <= 64, "at most one wavefront of 16-byte pieces");
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    if (wave == turn % NW && lane < LEN / 8) {
+        if (src) {
+            load_to_lds_16(static_cast<const T *>(src) + 8 * lane, dst);
+        } else {
+            const u32x4 zero = {0u, 0u, 0u, 0u};
+            *reinterpret_cast<u32x4 *>(dst + 8 * lane) = zero;
+        }
+    }
+}
+__device__ __forceinline__ void wait_all_loads() { __builtin_amdgcn_s_waitcnt(vmcnt_imm(0)); }
 
 // LDS slots of the parameter vectors (each max(D, F) elements wide)
 enum VecSlot : int { kVecG1 = 0, kVecB1, kVecG2, kVecB2, kVecBias1, kVecG3, kVecB3, kVecBias2, kVecSlots };
 
-// Row statistics over all N columns of the tile: each lane holds, for its token column, the
-// values of NB blocks; sums are completed across the lane pair (hb) and the wavefronts.
-// red_a / red_b are two [NW*32] exchange arrays (two, so that back-to-back calls need no
-// trailing barrier).
-template <int NB, int NW>
-__device__ __forceinline__ void row_mean_rstd(const float (&v)[NB][16], float *red_a, float *red_b, int wave, int c,
-                                              int hb, int N, float eps, float &mean, float &rstd) {
+// Row statistics over all N = NB*32*NW columns of the tile: each lane holds, for its token column,
+// the values of NB blocks.  A wavefront first reduces its own NB*32 values per row to (mean, sum of
+// squared deviations) in registers; the wavefronts' pairs are combined after ONE exchange through
+// red_a / red_b ([NW*32] each) by the pairwise update of Chan et al., which is as robust as the
+// two-pass form.  Callers separate two calls by a barrier (the one that publishes the normalised
+// tile does).
+template <typename T, int NB, int NW, int TR>
+__device__ __forceinline__ void row_mean_rstd(const float (&v)[NB][Tile<T, TR>::kVals], float *red_a, float *red_b,
+                                              int wave, int c, int hb, int N, float eps, float &mean, float &rstd) {
+    typedef Tile<T, TR> TL;
+    constexpr float kLocal = NB * TL::kBlock;
     float s = 0.f;
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s += v[b][e];
-    s += __shfl_xor(s, 32, 64);
-    if (hb == 0) red_a[wave * 32 + c] = s;
-    __syncthreads();
-    float tot = 0.f;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) tot += red_a[w * 32 + c];
-    mean = tot / N;
+        for (int e = 0; e < TL::kVals; ++e) s += v[b][e];
+    s = TL::over_token(s);
+    const float lmean = s * (1.f / kLocal);
     float q = 0.f;
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const float d = v[b][e] - mean;
+        for (int e = 0; e < TL::kVals; ++e) {
+            const float d = v[b][e] - lmean;
             q += d * d;
         }
-    q += __shfl_xor(q, 32, 64);
-    if (hb == 0) red_b[wave * 32 + c] = q;
+    q = TL::over_token(q);
+    if (hb == 0) {
+        red_a[wave * TR + c] = lmean;
+        red_b[wave * TR + c] = q;
+    }
     __syncthreads();
-    float var = 0.f;
+    float lm[NW], tot = 0.f;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) var += red_b[w * 32 + c];
-    rstd = rsqrtf(var / N + eps);
+    for (int w = 0; w < NW; ++w) {
+        lm[w] = red_a[w * TR + c];
+        tot += lm[w];
+    }
+    mean = tot * (1.f / NW);
+    float m2 = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+        const float d = lm[w] - mean;
+        m2 += red_b[w * TR + c] + kLocal * d * d;
+    }
+    rstd = rsqrtf(m2 / N + eps);
 }
 
-// Cooperative copy of a [32, W] tile between global memory (row stride ld) and LDS (row stride
+// Cooperative copy of a [TR, W] tile between global memory (row stride ld) and LDS (row stride
 // lds_ld) with 16-byte accesses along rows.  Loading zero-fills rows beyond `valid`.
-template <typename T, int W, int NT>
+template <typename T, int W, int NT, int TR = 32>
 __device__ __forceinline__ void stage_tile(T *dst, int lds_ld, const T *src, long ld, int valid, int tid) {
     constexpr int CPR = W / 8;
 #pragma unroll
-    for (int idx = tid; idx < kFusedRows * CPR; idx += NT) {
+    for (int idx = tid; idx < TR * CPR; idx += NT) {
         const int r = idx / CPR, ch = idx % CPR;
         u32x4 val = {0u, 0u, 0u, 0u};
         if (r < valid) val = *reinterpret_cast<const u32x4 *>(src + r * ld + 8 * ch);
         *reinterpret_cast<u32x4 *>(dst + r * lds_ld + 8 * ch) = val;
     }
 }
-template <typename T, int W, int NT>
+template <typename T, int W, int NT, int TR>
 __device__ __forceinline__ void unstage_tile(T *dst, long ld, const T *src, int lds_ld, int valid, int tid) {
     constexpr int CPR = W / 8;
 #pragma unroll
-    for (int idx = tid; idx < kFusedRows * CPR; idx += NT) {
+    for (int idx = tid; idx < TR * CPR; idx += NT) {
         const int r = idx / CPR, ch = idx % CPR;
         if (r < valid)
             *reinterpret_cast<u32x4 *>(dst + r * ld + 8 * ch) = *reinterpret_cast<const u32x4 *>(src + r * lds_ld + 8 * ch);
@@ -293,117 +487,127 @@ __device__ __forceinline__ void unstage_tile(T *dst, long ld, const T *src, int 
 
 // LayerNorm over the tile rows of v (statistics across all wavefronts), result written as T
 // into the LDS tile `dst` at this lane's (row c, accumulator columns).
-template <typename T, int NB, int NW>
-__device__ __forceinline__ void layer_norm_to_lds(const float (&v)[NB][16], const float (&gam)[NB][16],
-                                                  const float (&bet)[NB][16], const int (&nblk)[NB], T *dst, int ld,
-                                                  float *red_a, float *red_b, int wave, int c, int hb, int N,
-                                                  float eps) {
+template <typename T, int NB, int NW, int TR>
+__device__ __forceinline__ void layer_norm_to_lds(const float (&v)[NB][Tile<T, TR>::kVals],
+                                                  const float (&gam)[NB][Tile<T, TR>::kVals],
+                                                  const float (&bet)[NB][Tile<T, TR>::kVals], const int (&nblk)[NB],
+                                                  T *dst, int ld, float *red_a, float *red_b, int wave, int c, int hb,
+                                                  int N, float eps) {
+    typedef Tile<T, TR> TL;
     float mean, rstd;
-    row_mean_rstd<NB, NW>(v, red_a, red_b, wave, c, hb, N, eps, mean, rstd);
+    row_mean_rstd<T, NB, NW, TR>(v, red_a, red_b, wave, c, hb, N, eps, mean, rstd);
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
+        for (int g = 0; g < TL::kGroups; ++g) {
             float o[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) o[e] = (v[b][4 * g + e] - mean) * rstd * gam[b][4 * g + e] + bet[b][4 * g + e];
-            store4f<T>(dst + c * ld + col_of(nblk[b], 4 * g, hb), o[0], o[1], o[2], o[3]);
+            store4f<T>(dst + c * ld + TL::col(nblk[b], g, hb), o[0], o[1], o[2], o[3]);
         }
 }
 
-// Body of the pre kernel on one 32-row tile.  a0: x tile (row stride D + 8), staged here from
+// Body of the pre kernel on one TR-row tile.  a0: x tile (row stride D + 8), staged here from
 // P.x unless X_IN_LDS (then a finished tile is already there and the caller has synchronised);
 // later the staging buffer of the qkv passes.  a1: y tile.
 template <typename T, int D, int NT>
 __device__ __forceinline__ void stage_pre_vectors(const FusedPreParams &P, T *vecs, int vec_ld, int tid) {
-    stage_vector<T, D, NT>(vecs + kVecG1 * vec_ld, P.g1, tid);
-    stage_vector<T, D, NT>(vecs + kVecB1 * vec_ld, P.b1, tid);
+    dma_vector<T, D, NT>(vecs + kVecG1 * vec_ld, P.g1, tid, 6);
+    dma_vector<T, D, NT>(vecs + kVecB1 * vec_ld, P.b1, tid, 7);
 }
 
-template <typename T, int D, bool X_IN_LDS>
+// 32/16-feature blocks per wavefront for N output features
+template <typename T, int TR>
+constexpr int fused_blocks(int N, int NW) { return (N / Tile<T, TR>::kBlock + NW - 1) / NW; }
+
+template <typename T, int D, int TR, bool X_IN_LDS>
 __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T *a1, float *red_a, float *red_b,
                                                long row0, int valid,
-                                               WeightStream<T, D, D / 32 / fused_waves(D)> &w_a, T *vecs, int vec_ld) {
+                                               WeightStream<T, D, fused_blocks<T, TR>(D, fused_waves(D)), TR> &w_a,
+                                               T *vecs, int vec_ld) {
+    typedef Tile<T, TR> TL;
     constexpr int NW = fused_waves(D), NT = NW * 64;
     constexpr int LD = D + 8;
-    constexpr int NB = D / 32 / NW;  // 32-column blocks per wavefront per D columns
-    static_assert(D % (32 * NW) == 0, "D must be a multiple of 32 * wavefronts");
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hb = lane >> 5;
+    constexpr int NB = fused_blocks<T, TR>(D, NW);  // feature blocks per wavefront per D columns
+    constexpr int VB = TL::kVals, GB = TL::kGroups;
+    static_assert(D % (TL::kBlock * NW) == 0, "D must be a multiple of block width * wavefronts");
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = TL::token(lane), hb = TL::sub(lane);
 
     int nblk[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b) nblk[b] = wave + NW * b;
 
-    WeightStream<T, D, NB> w_b;
-    if (!X_IN_LDS) w_a.start(static_cast<const T *>(P.w_fo), nblk, lane);  // else requested by the caller already
-    if (!X_IN_LDS) {
-        stage_tile<T, D, NT>(a0, LD, static_cast<const T *>(P.x) + row0 * P.ldx, P.ldx, valid, tid);
+    WeightStream<T, D, NB, TR> w_b;
+    if (!X_IN_LDS) {  // else requested by the caller already
+        w_a.start(static_cast<const T *>(P.w_fo), nblk, lane);
+        dma_tile<T, D, NT, TR>(a0, LD, static_cast<const T *>(P.x) + row0 * P.ldx, P.ldx, valid, tid);
         stage_pre_vectors<T, D, NT>(P, vecs, vec_ld, tid);
+        wait_all_loads();
+        __syncthreads();
     }
     w_b.start(static_cast<const T *>(P.w_qkv), nblk, lane);  // q columns
-    if (!X_IN_LDS) __syncthreads();
-    float gam[NB][16], bet[NB][16];
-    load_cols<T, NB>(vecs + kVecG1 * vec_ld, nblk, hb, gam);
-    load_cols<T, NB>(vecs + kVecB1 * vec_ld, nblk, hb, bet);
+    float gam[NB][VB], bet[NB][VB];
+    load_cols<T, NB, TR>(vecs + kVecG1 * vec_ld, nblk, hb, gam);
+    load_cols<T, NB, TR>(vecs + kVecB1 * vec_ld, nblk, hb, bet);
 
     // ---- y = LN1(x + x W_fo^T)
     {
-        f32x16 acc[NB];
+        typename TL::acc_t acc[NB];
         w_a.run(acc, a0, LD, c, hb);
-        float v[NB][16];
+        float v[NB][VB];
 #pragma unroll
         for (int b = 0; b < NB; ++b)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
+            for (int g = 0; g < GB; ++g) {
                 float r[4];
-                load4f<T>(a0 + c * LD + col_of(nblk[b], 4 * g, hb), r);
+                load4f<T>(a0 + c * LD + TL::col(nblk[b], g, hb), r);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[b][4 * g + e] = acc[b][4 * g + e] + r[e];
             }
-        layer_norm_to_lds<T, NB, NW>(v, gam, bet, nblk, a1, LD, red_a, red_b, wave, c, hb, D, P.eps);
+        layer_norm_to_lds<T, NB, NW, TR>(v, gam, bet, nblk, a1, LD, red_a, red_b, wave, c, hb, D, P.eps);
     }
     __syncthreads();  // y complete in a1; a0 no longer read
-    unstage_tile<T, D, NT>(static_cast<T *>(P.y) + row0 * D, D, a1, LD, valid, tid);
+    unstage_tile<T, D, NT, TR>(static_cast<T *>(P.y) + row0 * D, D, a1, LD, valid, tid);
 
     // ---- qkv = y W_qkv^T, three passes of D columns, each staged through a0 for row-contiguous
     // stores; the weights of the next pass are requested before the current one is computed
 #pragma unroll
     for (int part = 0; part < 3; ++part) {
-        WeightStream<T, D, NB> &cur = (part & 1) ? w_a : w_b, &nxt = (part & 1) ? w_b : w_a;
+        WeightStream<T, D, NB, TR> &cur = (part & 1) ? w_a : w_b, &nxt = (part & 1) ? w_b : w_a;
         if (part < 2) {
             int nb2[NB];
 #pragma unroll
-            for (int b = 0; b < NB; ++b) nb2[b] = (part + 1) * (D / 32) + nblk[b];
+            for (int b = 0; b < NB; ++b) nb2[b] = (part + 1) * (D / TL::kBlock) + nblk[b];
             nxt.start(static_cast<const T *>(P.w_qkv), nb2, lane);
         }
-        f32x16 acc[NB];
+        typename TL::acc_t acc[NB];
         cur.run(acc, a1, LD, c, hb);
         if (part) __syncthreads();  // the previous pass has been copied out of a0
 #pragma unroll
         for (int b = 0; b < NB; ++b)
 #pragma unroll
-            for (int g = 0; g < 4; ++g)
-                store4f<T>(a0 + c * LD + col_of(nblk[b], 4 * g, hb), acc[b][4 * g], acc[b][4 * g + 1],
+            for (int g = 0; g < GB; ++g)
+                store4f<T>(a0 + c * LD + TL::col(nblk[b], g, hb), acc[b][4 * g], acc[b][4 * g + 1],
                            acc[b][4 * g + 2], acc[b][4 * g + 3]);
         __syncthreads();
-        unstage_tile<T, D, NT>(static_cast<T *>(P.qkv) + row0 * (3 * D) + part * D, 3 * D, a0, LD, valid, tid);
+        unstage_tile<T, D, NT, TR>(static_cast<T *>(P.qkv) + row0 * (3 * D) + part * D, 3 * D, a0, LD, valid, tid);
     }
 }
 
-template <typename T, int D>
+template <typename T, int D, int TR>
 __global__ __launch_bounds__(fused_waves(D) * 64) void fused_pre_kernel(FusedPreParams P) {
     constexpr int NW = fused_waves(D), LD = D + 8;
-    __shared__ __attribute__((aligned(16))) T a0[kFusedRows * LD];
-    __shared__ __attribute__((aligned(16))) T a1[kFusedRows * LD];
-    __shared__ float red_a[NW * 32], red_b[NW * 32];
-    const long row0 = static_cast<long>(blockIdx.x) * kFusedRows;
-    const int valid = static_cast<int>(min(static_cast<long>(kFusedRows), P.rows - row0));
+    __shared__ __attribute__((aligned(16))) T a0[TR * LD];
+    __shared__ __attribute__((aligned(16))) T a1[TR * LD];
+    __shared__ float red_a[NW * TR], red_b[NW * TR];
+    const long row0 = static_cast<long>(blockIdx.x) * TR;
+    const int valid = static_cast<int>(min(static_cast<long>(TR), P.rows - row0));
     __shared__ __attribute__((aligned(16))) T vecs[kVecSlots * D];
-    WeightStream<T, D, D / 32 / NW> w_a;
-    fused_pre_body<T, D, false>(P, a0, a1, red_a, red_b, row0, valid, w_a, vecs, D);
+    WeightStream<T, D, fused_blocks<T, TR>(D, NW), TR> w_a;
+    fused_pre_body<T, D, TR, false>(P, a0, a1, red_a, red_b, row0, valid, w_a, vecs, D);
 }
 
-// Body of the post kernel on one 32-row tile.  a0 (row stride max(D, F) + 8): attn tile, gelu
+// Body of the post kernel on one TR-row tile.  a0 (row stride max(D, F) + 8): attn tile, gelu
 // output, finally the finished tile (row stride D + 8); a1: y tile, then x1 = LN2(...).  With
 // WRITE_OUT the tile is stored to P.out; otherwise it is left in a0, synchronised, for the
 // caller (the next layer's pre body).
@@ -413,145 +617,150 @@ struct NoHook {
 
 // `before_last` runs right ahead of the last product (two of the three weight streams are
 // dead by then): the fused layer boundary uses it to request the next layer's first weights.
-template <typename T, int D, int F, bool WRITE_OUT, typename Hook>
+template <typename T, int D, int F, int TR, bool WRITE_OUT, typename Hook>
 __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0, T *a1, float *red_a, float *red_b,
                                                 long row0, int valid, Hook before_last, T *vecs, int vec_ld) {
+    typedef Tile<T, TR> TL;
     constexpr int NW = fused_waves(D), NT = NW * 64;
     constexpr int LDD = D + 8, LDF = F + 8;
-    constexpr int NBD = D / 32 / NW;
-    constexpr int NBF = (F / 32 + NW - 1) / NW;  // with F/32 < NW the upper wavefronts sit the product out
-    static_assert(D % (32 * NW) == 0 && F % 32 == 0, "unsupported widths");
-    static_assert(F / 32 >= NW ? (F / 32) % NW == 0 : true, "unsupported widths");
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hb = lane >> 5;
+    constexpr int NBD = fused_blocks<T, TR>(D, NW);
+    constexpr int NBF = fused_blocks<T, TR>(F, NW);  // with fewer blocks than wavefronts the upper ones sit the product out
+    constexpr int VB = TL::kVals, GB = TL::kGroups;
+    static_assert(D % (TL::kBlock * NW) == 0 && F % TL::kBlock == 0, "unsupported widths");
+    static_assert(F / TL::kBlock >= NW ? (F / TL::kBlock) % NW == 0 : true, "unsupported widths");
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = TL::token(lane), hb = TL::sub(lane);
 
     int nbd[NBD], nbf[NBF];
 #pragma unroll
     for (int b = 0; b < NBD; ++b) nbd[b] = wave + NW * b;
 #pragma unroll
     for (int b = 0; b < NBF; ++b) nbf[b] = wave + NW * b;
-    const bool ff_active = wave < F / 32;  // wavefront-uniform
+    const bool ff_active = wave < F / TL::kBlock;  // wavefront-uniform
 
-    WeightStream<T, D, NBD> w_o;
-    WeightStream<T, D, NBF> w_1;
-    WeightStream<T, F, NBD> w_2;
+    WeightStream<T, D, NBD, TR> w_o;
+    WeightStream<T, D, NBF, TR> w_1;
+    WeightStream<T, F, NBD, TR> w_2;
+    // prologue: everything this tile needs from memory is requested before anything is waited for
+    dma_tile<T, D, NT, TR>(a1, LDD, static_cast<const T *>(P.y) + row0 * P.ldy, P.ldy, valid, tid);
+    if (!P.part_o)
+        dma_tile<T, D, NT, TR>(a0, LDD, static_cast<const T *>(P.attn) + row0 * P.lda, P.lda, valid, tid);
+    dma_vector<T, D, NT>(vecs + kVecG2 * vec_ld, P.g2, tid, 0);
+    dma_vector<T, D, NT>(vecs + kVecB2 * vec_ld, P.b2, tid, 1);
+    dma_vector<T, F, NT>(vecs + kVecBias1 * vec_ld, P.bias_1, tid, 2);
+    dma_vector<T, D, NT>(vecs + kVecG3 * vec_ld, P.g3, tid, 3);
+    dma_vector<T, D, NT>(vecs + kVecB3 * vec_ld, P.b3, tid, 4);
+    dma_vector<T, D, NT>(vecs + kVecBias2 * vec_ld, P.bias_2, tid, 5);
+    if (P.part_o) stage_merged_attention<T, D, NT, TR>(a0, LDD, P, row0, valid, tid);
     w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
-    if (!P.part_o) stage_tile<T, D, NT>(a0, LDD, static_cast<const T *>(P.attn) + row0 * P.lda, P.lda, valid, tid);
-    stage_tile<T, D, NT>(a1, LDD, static_cast<const T *>(P.y) + row0 * P.ldy, P.ldy, valid, tid);
-    stage_vector<T, D, NT>(vecs + kVecG2 * vec_ld, P.g2, tid);
-    stage_vector<T, D, NT>(vecs + kVecB2 * vec_ld, P.b2, tid);
-    stage_vector<T, F, NT>(vecs + kVecBias1 * vec_ld, P.bias_1, tid);
-    stage_vector<T, D, NT>(vecs + kVecG3 * vec_ld, P.g3, tid);
-    stage_vector<T, D, NT>(vecs + kVecB3 * vec_ld, P.b3, tid);
-    stage_vector<T, D, NT>(vecs + kVecBias2 * vec_ld, P.bias_2, tid);
-    if (P.part_o) stage_merged_attention<T, D, NT>(a0, LDD, P, row0, valid, tid);
-    if (ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane);
+    wait_all_loads();
     __syncthreads();
+    if (ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane);
 
     // ---- x1 = LN2(y + attn W_o^T); each lane replaces exactly the y entries it read
     {
-        float gam[NBD][16], bet[NBD][16];
-        load_cols<T, NBD>(vecs + kVecG2 * vec_ld, nbd, hb, gam);
-        load_cols<T, NBD>(vecs + kVecB2 * vec_ld, nbd, hb, bet);
-        f32x16 acc[NBD];
+        float gam[NBD][VB], bet[NBD][VB];
+        load_cols<T, NBD, TR>(vecs + kVecG2 * vec_ld, nbd, hb, gam);
+        load_cols<T, NBD, TR>(vecs + kVecB2 * vec_ld, nbd, hb, bet);
+        typename TL::acc_t acc[NBD];
         w_o.run(acc, a0, LDD, c, hb);
         w_2.start(static_cast<const T *>(P.w_2), nbd, lane);
-        float v[NBD][16];
+        float v[NBD][VB];
 #pragma unroll
         for (int b = 0; b < NBD; ++b)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
+            for (int g = 0; g < GB; ++g) {
                 float r[4];
-                load4f<T>(a1 + c * LDD + col_of(nbd[b], 4 * g, hb), r);
+                load4f<T>(a1 + c * LDD + TL::col(nbd[b], g, hb), r);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[b][4 * g + e] = acc[b][4 * g + e] + r[e];
             }
-        layer_norm_to_lds<T, NBD, NW>(v, gam, bet, nbd, a1, LDD, red_a, red_b, wave, c, hb, D, P.eps2);
+        layer_norm_to_lds<T, NBD, NW, TR>(v, gam, bet, nbd, a1, LDD, red_a, red_b, wave, c, hb, D, P.eps2);
     }
     __syncthreads();  // x1 complete in a1; every wavefront is done reading a0
 
     // ---- h = gelu(x1 W_1^T + b_1)  -> a0
     if (ff_active) {
-        float bias[NBF][16];
-        load_cols<T, NBF>(vecs + kVecBias1 * vec_ld, nbf, hb, bias);
-        f32x16 acc[NBF];
+        float bias[NBF][VB];
+        load_cols<T, NBF, TR>(vecs + kVecBias1 * vec_ld, nbf, hb, bias);
+        typename TL::acc_t acc[NBF];
         w_1.run(acc, a1, LDD, c, hb);
 #pragma unroll
         for (int b = 0; b < NBF; ++b)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
+            for (int g = 0; g < GB; ++g) {
                 float o[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const float t = acc[b][4 * g + e] + bias[b][4 * g + e];
                     o[e] = 0.5f * t * (1.f + erff(t * 0.70710678118654752f));
                 }
-                store4f<T>(a0 + c * LDF + col_of(nbf[b], 4 * g, hb), o[0], o[1], o[2], o[3]);
+                store4f<T>(a0 + c * LDF + TL::col(nbf[b], g, hb), o[0], o[1], o[2], o[3]);
             }
     }
-    float gam[NBD][16], bet[NBD][16], bias[NBD][16];
-    load_cols<T, NBD>(vecs + kVecG3 * vec_ld, nbd, hb, gam);
-    load_cols<T, NBD>(vecs + kVecB3 * vec_ld, nbd, hb, bet);
-    load_cols<T, NBD>(vecs + kVecBias2 * vec_ld, nbd, hb, bias);
+    float gam[NBD][VB], bet[NBD][VB], bias[NBD][VB];
+    load_cols<T, NBD, TR>(vecs + kVecG3 * vec_ld, nbd, hb, gam);
+    load_cols<T, NBD, TR>(vecs + kVecB3 * vec_ld, nbd, hb, bet);
+    load_cols<T, NBD, TR>(vecs + kVecBias2 * vec_ld, nbd, hb, bias);
     __syncthreads();
 
     // ---- out = LN3(x1 + h W_2^T + b_2), staged through a0 for row-contiguous stores
     {
         before_last();
-        f32x16 acc[NBD];
+        typename TL::acc_t acc[NBD];
         w_2.run(acc, a0, LDF, c, hb);
-        float v[NBD][16];
+        float v[NBD][VB];
 #pragma unroll
         for (int b = 0; b < NBD; ++b)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
+            for (int g = 0; g < GB; ++g) {
                 float r[4];
-                load4f<T>(a1 + c * LDD + col_of(nbd[b], 4 * g, hb), r);
+                load4f<T>(a1 + c * LDD + TL::col(nbd[b], g, hb), r);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[b][4 * g + e] = acc[b][4 * g + e] + r[e] + bias[b][4 * g + e];
             }
-        // the barriers inside the statistics also order every wavefront's last read of a0
-        // (the product above) before the first write of the result into it
-        layer_norm_to_lds<T, NBD, NW>(v, gam, bet, nbd, a0, LDD, red_a, red_b, wave, c, hb, D, P.eps3);
+        // every wavefront must be done with its last read of a0 (the product above) before the
+        // result is written into it: the barrier inside the statistics orders exactly that
+        layer_norm_to_lds<T, NBD, NW, TR>(v, gam, bet, nbd, a0, LDD, red_a, red_b, wave, c, hb, D, P.eps3);
     }
     __syncthreads();
-    if (WRITE_OUT) unstage_tile<T, D, NT>(static_cast<T *>(P.out) + row0 * D, D, a0, LDD, valid, tid);
+    if (WRITE_OUT) unstage_tile<T, D, NT, TR>(static_cast<T *>(P.out) + row0 * D, D, a0, LDD, valid, tid);
 }
 
-template <typename T, int D, int F>
+template <typename T, int D, int F, int TR>
 __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_kernel(FusedPostParams P) {
     constexpr int NW = fused_waves(D), LDD = D + 8, LDF = F + 8, LDM = LDD > LDF ? LDD : LDF;
-    __shared__ __attribute__((aligned(16))) T a0[kFusedRows * LDM];
-    __shared__ __attribute__((aligned(16))) T a1[kFusedRows * LDD];
-    __shared__ float red_a[NW * 32], red_b[NW * 32];
-    const long row0 = static_cast<long>(blockIdx.x) * kFusedRows;
-    const int valid = static_cast<int>(min(static_cast<long>(kFusedRows), P.rows - row0));
+    __shared__ __attribute__((aligned(16))) T a0[TR * LDM];
+    __shared__ __attribute__((aligned(16))) T a1[TR * LDD];
+    __shared__ float red_a[NW * TR], red_b[NW * TR];
+    const long row0 = static_cast<long>(blockIdx.x) * TR;
+    const int valid = static_cast<int>(min(static_cast<long>(TR), P.rows - row0));
     constexpr int VW = D > F ? D : F;
     __shared__ __attribute__((aligned(16))) T vecs[kVecSlots * VW];
-    fused_post_body<T, D, F, true>(P, a0, a1, red_a, red_b, row0, valid, NoHook{}, vecs, VW);
+    fused_post_body<T, D, F, TR, true>(P, a0, a1, red_a, red_b, row0, valid, NoHook{}, vecs, VW);
 }
 
-// The post part of layer L and the pre part of layer L+1 on the same 32 rows: the layer output
+// The post part of layer L and the pre part of layer L+1 on the same rows: the layer output
 // never leaves LDS, and one launch (with its fixed cost) disappears per layer boundary.
-template <typename T, int D, int F>
+template <typename T, int D, int F, int TR>
 __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_pre_kernel(FusedPostParams P, FusedPreParams N) {
     constexpr int NW = fused_waves(D), LDD = D + 8, LDF = F + 8, LDM = LDD > LDF ? LDD : LDF;
-    __shared__ __attribute__((aligned(16))) T a0[kFusedRows * LDM];
-    __shared__ __attribute__((aligned(16))) T a1[kFusedRows * LDD];
-    __shared__ float red_a[NW * 32], red_b[NW * 32];
-    const long row0 = static_cast<long>(blockIdx.x) * kFusedRows;
-    const int valid = static_cast<int>(min(static_cast<long>(kFusedRows), P.rows - row0));
-    constexpr int NB = D / 32 / NW;
+    __shared__ __attribute__((aligned(16))) T a0[TR * LDM];
+    __shared__ __attribute__((aligned(16))) T a1[TR * LDD];
+    __shared__ float red_a[NW * TR], red_b[NW * TR];
+    const long row0 = static_cast<long>(blockIdx.x) * TR;
+    const int valid = static_cast<int>(min(static_cast<long>(TR), P.rows - row0));
+    constexpr int NB = fused_blocks<T, TR>(D, NW);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     int nblk[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b) nblk[b] = wave + NW * b;
-    WeightStream<T, D, NB> next_fo;
+    WeightStream<T, D, NB, TR> next_fo;
     constexpr int VW = D > F ? D : F;
     __shared__ __attribute__((aligned(16))) T vecs[kVecSlots * VW];
     stage_pre_vectors<T, D, NW * 64>(N, vecs, VW, threadIdx.x);  // visible after the first barrier below
-    fused_post_body<T, D, F, false>(P, a0, a1, red_a, red_b, row0, valid,
-                                    [&]() { next_fo.start(static_cast<const T *>(N.w_fo), nblk, lane); }, vecs, VW);
-    fused_pre_body<T, D, true>(N, a0, a1, red_a, red_b, row0, valid, next_fo, vecs, VW);
+    fused_post_body<T, D, F, TR, false>(P, a0, a1, red_a, red_b, row0, valid,
+                                        [&]() { next_fo.start(static_cast<const T *>(N.w_fo), nblk, lane); }, vecs, VW);
+    fused_pre_body<T, D, TR, true>(N, a0, a1, red_a, red_b, row0, valid, next_fo, vecs, VW);
 }
 
 // ---- end of a decode step: final norm + mixture head + one sample per trajectory + the

@@ -366,6 +366,15 @@ int artab_layer_post_pre(const void *attn, int64_t lda, const void *y, int64_t l
                          int64_t rows, int D, int F, int dtype, void *stream);
 
 /*
+ * Merge of a partial descriptor into `out` [B,H,Lq,Dh] on its own: merge_attention_outputs
+ * (triton_kernels.py:478-524) over n_slots operands instead of two — m = max lse, w = exp(lse - m),
+ * out = sum(w * out_s) / sum(w) in float32, rounded once to the storage type.  For callers of
+ * artab_decode_attention_partials whose next step is not one of the layer kernels.
+ */
+int artab_merge_attention_partials(const artab_attention_partials *partials, const artab_view *out, int dtype,
+                                   void *stream);
+
+/*
  * artab_layer_post / artab_layer_post_pre with the attention input given as unmerged partials
  * (artab_decode_attention_partials): token row r = b*Lq + i, columns [h*Dh, (h+1)*Dh) of the
  * attention matrix are merged from partial row (b*H + h)*Lq + i while the tile is loaded, rounded

@@ -223,6 +223,62 @@ def test_decode_attention_overlapped_device_length_in_graph(device):
         assert torch.equal(k_cache, k_ref) and torch.equal(v_cache, v_ref)
 
 
+def _full_size_decode(device, B, H, Nc, n_buf, cap, seed):
+    """One decode step at a BASELINE shape (Dh=32, Lq=2, bf16).  Inputs are drawn on the device
+    (the buffer cache alone is up to 0.5 GB); the oracle sees a sample of the trajectories, every
+    head of them; the cache is compared whole and bit-exact; the three schedules of the step
+    (buffer pass after the context pass, beside it, merge left to the caller) must agree on every
+    row to within the rounding of the 16-bit partial outputs."""
+    ak = _ak()
+    dtype, D, Lq = torch.bfloat16, 32, 2
+    g = torch.Generator(device=device).manual_seed(seed)
+
+    def draw(*shape):
+        return (torch.randn(*shape, generator=g, device=device, dtype=torch.float32) * 0.6).to(dtype)
+
+    q, k_ctx, v_ctx = draw(B, H, Lq, D), draw(H, Nc, D), draw(H, Nc, D)
+    k_cache, v_cache = draw(B, H, cap, D), draw(B, H, cap, D)
+    k_new, v_new = draw(B, H, 1, D), draw(B, H, 1, D)
+    exp_k, exp_v = k_cache.clone(), v_cache.clone()
+    exp_k[:, :, n_buf] = k_new[:, :, 0]
+    exp_v[:, :, n_buf] = v_new[:, :, 0]
+    side = torch.cuda.Stream(device=device)
+
+    outs = []
+    for kwargs in (dict(), dict(side_stream=side), dict(side_stream=side, leave_partials=True)):
+        kc, vc = k_cache.clone(), v_cache.clone()
+        out = ak.decode_attention(q, k_ctx, v_ctx, kc, vc, n_buf, k_new, v_new, **kwargs)
+        if hasattr(out, "desc"):  # unmerged partial slots: the stand-alone merge of the library
+            assert out.desc.n_slots >= 2
+            out = out.merged()
+        torch.cuda.synchronize()
+        assert torch.equal(kc, exp_k) and torch.equal(vc, exp_v)
+        outs.append(out.float())
+    for other in outs[1:]:
+        assert float((outs[0] - other).abs().max()) <= 2e-2
+
+    sample = sorted({0, 1, B // 2 - 1, B // 2, B - 2, B - 1, (7 * seed + 13) % B, (31 * seed + 5) % B})
+    idx = torch.tensor(sample, device=device)
+    ref, _, _ = ao.decode_step_attention(
+        to_np(q[idx]), to_np(k_ctx), to_np(v_ctx), to_np(k_cache[idx][:, :, :n_buf]), to_np(v_cache[idx][:, :, :n_buf]),
+        to_np(k_new[idx]), to_np(v_new[idx]),
+    )
+    for out in outs:
+        assert max_abs(to_np(out[idx]), ref) <= 2e-2
+
+
+@pytest.mark.parametrize("n_buf", [0, 37, 255])
+def test_decode_attention_config3_full_size(device, n_buf):
+    """BASELINE configs[3] layer-step: B=1024 trajectories, 8 heads, N_ctx=16384, buffer up to 256."""
+    _full_size_decode(device, 1024, 8, 16384, n_buf, 256, seed=3 + n_buf)
+
+
+@pytest.mark.parametrize("n_buf", [1, 130, 255])
+def test_decode_attention_config4_full_size(device, n_buf):
+    """BASELINE configs[4] layer-step: B=2048 trajectories, 16 heads, N_ctx=4096, buffer up to 256."""
+    _full_size_decode(device, 2048, 16, 4096, n_buf, 256, seed=4 + n_buf)
+
+
 @pytest.mark.parametrize("n_buf", [1, 2, 17, 33, 64])
 def test_decode_attention_config1_shape(device, n_buf):
     """BASELINE configs[1]: H=8, Dh=64, Nc=1024, B=256, entries ~N(0,1)/8, N_buf swept."""
@@ -566,9 +622,17 @@ def _mk_norm(D, seed, dtype):
     return norm.to(dtype)
 
 
+@pytest.fixture(params=[16, 32])
+def tile_rows(request, monkeypatch):
+    """Both tile shapes of the layer kernels (token rows per workgroup): the library picks by row
+    count, ARTAB_TILE_ROWS forces one."""
+    monkeypatch.setenv("ARTAB_TILE_ROWS", str(request.param))
+    return request.param
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("rows,D", [(1, 128), (33, 128), (2048, 256), (70, 512)])
-def test_layer_pre_matches_float64(device, dtype, rows, D):
+def test_layer_pre_matches_float64(device, tile_rows, dtype, rows, D):
     """y = LN1(x + x Wfo^T), qkv = y Wqkv^T against float64 on the same bits; the reference
     chain rounds y to the storage dtype before the second product, as the kernel does."""
     from ar_nanotabpfn_amd.glue import layer_pre, pack_weight
@@ -590,7 +654,7 @@ def test_layer_pre_matches_float64(device, dtype, rows, D):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("rows,D,F,with_bias", [(1, 128, 256, True), (33, 128, 128, False), (2048, 256, 256, True),
                                                (70, 512, 256, True), (40, 256, 512, True), (5, 512, 512, False)])
-def test_layer_post_matches_float64(device, dtype, rows, D, F, with_bias):
+def test_layer_post_matches_float64(device, tile_rows, dtype, rows, D, F, with_bias):
     """x1 = LN2(y + attn Wo^T); out = LN3(x1 + gelu(x1 W1^T + b1) W2^T + b2) against float64
     with the kernel's two intermediate roundings."""
     from ar_nanotabpfn_amd.glue import layer_post, pack_weight
@@ -808,7 +872,7 @@ def test_decode_sample_embed_component_frequencies(device):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("rows,D,F,H", [(33, 128, 256, 4), (2048, 256, 256, 8), (70, 512, 256, 16), (40, 256, 512, 8)])
-def test_layer_post_pre_equals_post_then_pre(device, dtype, rows, D, F, H):
+def test_layer_post_pre_equals_post_then_pre(device, tile_rows, dtype, rows, D, F, H):
     """The one-launch layer boundary must give bit for bit what the two launches give: the
     layer output between them is rounded to the storage type in both."""
     from ar_nanotabpfn_amd import model as m
@@ -843,7 +907,7 @@ def test_layer_post_pre_falls_back_when_not_covered(device):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,H,Lq,Nc,n_buf,cap", [(64, 4, 2, 4096, 9, 16), (33, 8, 2, 2048, 0, 8), (40, 8, 1, 4096, 5, 8)])
-def test_decode_partials_merged_in_layer_kernel(device, dtype, B, H, Lq, Nc, n_buf, cap):
+def test_decode_partials_merged_in_layer_kernel(device, tile_rows, dtype, B, H, Lq, Nc, n_buf, cap):
     """decode_attention(leave_partials=True) + the layer kernels that merge the partials while
     loading, against the merged attention output fed to the same kernels: the merge is the same
     arithmetic rounded at the same point, so the results must agree bit for bit."""
