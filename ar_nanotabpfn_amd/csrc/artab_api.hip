@@ -247,7 +247,9 @@ static hipError_t launch_stream_t(const DecodeParams &P, int Lq, hipStream_t str
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
         cus = 256;
     const long tasks = (pairs + 15) / 16;
-    dim3 grid(static_cast<unsigned>(tasks < 2L * cus ? tasks : 2L * cus)), block(64);
+    long per_cu = 2;  // what fits beside two workgroups of the context pass
+    if (const char *e = getenv("ARTAB_STREAM_PER_CU")) per_cu = atol(e) >= 1 && atol(e) <= 4 ? atol(e) : per_cu;  // tuning hook
+    dim3 grid(static_cast<unsigned>(tasks < per_cu * cus ? tasks : per_cu * cus)), block(64);
     if (Lq == 1)
         hipLaunchKernelGGL((decode_stream_kernel<T, 1>), grid, block, kStreamLdsBytes, stream, P);
     else
