@@ -23,6 +23,8 @@ Prints one JSON line:
                  teacher-forced evaluation on the GPU vs the same on the host CPU
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+       python bench.py --kernel-shapes   (instead: one decode layer-step at the shapes of
+                                          configs[1], [3] and [4], timings on stderr)
 """
 
 from __future__ import annotations
@@ -179,6 +181,62 @@ def log_density_bench(device, dtype, model, with_cpu):
 CONTEXT_PASS_HBM_BYTES = int(9308.5 * 1024 * 2.0 + 10240.0 * 1024)
 
 
+def kernel_shapes(device):
+    """One decode layer-step (context pass + buffer pass + merge + append) at the attention shapes
+    of configs[1], configs[3] and configs[4]: HIP-event time per call over replays of a recorded graph
+    of ten calls (the cross-queue dependencies of the two-stream schedule are part of it)."""
+    from ar_nanotabpfn_amd import attention_kernels as ak
+
+    dt = torch.bfloat16
+    side = torch.cuda.Stream(device=device)
+    out = []
+    for name, B, H, Lq, Nc, Dh, cap, n_bufs, scale in (
+        ("configs[1]", 256, 8, 1, 1024, 64, 64, (1, 16, 64), 0.125),
+        ("configs[3]", 1024, 8, 2, 16384, 32, 256, (1, 128, 255), 0.6),
+        ("configs[4]", 2048, 16, 2, 4096, 32, 256, (1, 128, 255), 0.6),
+    ):
+        g = torch.Generator(device=device).manual_seed(0)
+
+        def draw(*shape):
+            return (torch.randn(*shape, generator=g, device=device) * scale).to(dt)
+
+        q, kc, vc = draw(B, H, Lq, Dh), draw(H, Nc, Dh), draw(H, Nc, Dh)
+        kb, vb = draw(B, H, cap, Dh), draw(B, H, cap, Dh)
+        kn, vn = (draw(B, H, 1, Dh), draw(B, H, 1, Dh)) if Lq == 2 else (None, None)
+        for n in n_bufs:
+            nn = min(n, cap - (1 if Lq == 2 else 0))
+            for label, kw in (("sequential", {}), ("two streams", dict(side_stream=side))):
+                def call():
+                    return ak.decode_attention(q, kc, vc, kb, vb, nn, kn, vn, **kw)
+                # ten calls recorded into one graph: the replay is free of host launch time
+                warm = torch.cuda.Stream(device=device)
+                warm.wait_stream(torch.cuda.current_stream(device))
+                with torch.cuda.stream(warm):
+                    for _ in range(3):
+                        call()
+                torch.cuda.current_stream(device).wait_stream(warm)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    for _ in range(10):
+                        call()
+                graph.replay()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                graph.replay()
+                graph.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) / 20 * 1e3
+                flops = 4.0 * B * H * Lq * (Nc + nn + (Lq - 1)) * Dh
+                byts = 2.0 * Dh * 2 * (H * Nc + B * H * (nn + (Lq - 1))) + 2.0 * 2 * B * H * Lq * Dh
+                out.append(dict(config=name, n_buf=nn, schedule=label, us=round(us, 1),
+                                tflops=round(flops / us / 1e6, 1), gbps=round(byts / us / 1e3, 1)))
+                log(f"[shape] {name} n_buf={nn:3d} {label:11s} {us:8.1f} us  {flops / us / 1e6:7.1f} TFLOP/s  "
+                    f"{byts / us / 1e3:7.1f} GB/s")
+    print(json.dumps({"kernel_shapes": out}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -187,6 +245,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline legs")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only copy a 256 MiB buffer five times (reference kernel for scaling HBM counters)")
+    ap.add_argument("--kernel-shapes", action="store_true",
+                    help="only time one decode layer-step at the attention shapes of configs[1], [3], [4]")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: trajectories are independent given the context, so more GPUs "
@@ -209,6 +269,9 @@ def main():
     from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
 
     lib = _lib.load()  # fails loudly when the extension is not built
+    if args.kernel_shapes:
+        kernel_shapes(torch.device("cuda:0"))
+        return
     device, dtype = torch.device("cuda:0"), torch.bfloat16
     model = build_model(device, dtype)
     x_context, y_context, x_target = decode_inputs(device, dtype)
