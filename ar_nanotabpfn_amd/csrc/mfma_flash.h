@@ -158,6 +158,8 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
     const int row0_w = row0_wg + wave * ROWS_W;
 
     // ---- Q fragments (B operand of S^T), pre-scaled by scale*log2e.
+    // The loads are only requested here; they are scaled into qreg once the first K/V tiles have
+    // been requested too, so that the kernel's first memory round trips overlap.
     vec qreg[QB][KS];
     long orow_idx[QB];  // (b*H + h)*Lq + i of this lane's query per block, or -1
     int qi[QB];         // query index i within its batch entry
@@ -167,23 +169,46 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
         int r = row0_w + 32 * j + c;
         bool valid = r < P.G;
         long flat = static_cast<long>(g) * P.G + (valid ? r : 0);
-        long b = flat / P.Lq;
-        int i = static_cast<int>(flat % P.Lq);
+        long b;
+        int i;
+        if (P.Lq == 1) {  // decode: no 64-bit division on the way to the first load
+            b = flat; i = 0;
+        } else if (P.Lq == 2) {
+            b = flat >> 1; i = static_cast<int>(flat & 1);
+        } else {
+            b = flat / P.Lq; i = static_cast<int>(flat % P.Lq);
+        }
         qb[j] = b;
         qi[j] = valid ? i : -1;
         orow_idx[j] = valid ? (b * P.H + h) * P.Lq + i : -1;
-        const T *qrow = view_row<T>(P.q, b, h, i);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            u32x4 raw = {0u, 0u, 0u, 0u};
-            if (valid) raw = *reinterpret_cast<const u32x4 *>(qrow + 16 * ks + 8 * hb);
-            u32x4 sc;
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                sc[e] = pack2<T>(unpack_lo<T>(raw[e]) * P.qscale, unpack_hi<T>(raw[e]) * P.qscale);
-            qreg[j][ks] = __builtin_bit_cast(vec, sc);
-        }
     }
+    // Raw query fragments of this lane (addresses recomputed from qb/qi: nothing extra stays live
+    // across the key loop), and their scaled, rounded form in qreg.
+    auto request_q = [&](u32x4(&qraw)[QB][KS]) {
+#pragma unroll
+        for (int j = 0; j < QB; ++j) {
+            const T *qrow = view_row<T>(P.q, qb[j], h, qi[j] >= 0 ? qi[j] : 0) + 8 * hb;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                qraw[j][ks] = u32x4{0u, 0u, 0u, 0u};
+                if (qi[j] >= 0) qraw[j][ks] = *reinterpret_cast<const u32x4 *>(qrow + 16 * ks);
+            }
+        }
+    };
+    bool q_scaled = false;
+    auto scale_q = [&](const u32x4(&qraw)[QB][KS]) {
+        q_scaled = true;
+#pragma unroll
+        for (int j = 0; j < QB; ++j)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                u32x4 sc;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    sc[e] = pack2<T>(unpack_lo<T>(qraw[j][ks][e]) * P.qscale, unpack_hi<T>(qraw[j][ks][e]) * P.qscale);
+                qreg[j][ks] = __builtin_bit_cast(vec, sc);
+            }
+    };
 
     // ---- prefill: this tile's own K/V rows go to the cache.
     if (P.mode == kFlashPrefill && P.kcache.p && g < P.cache_batches) {
@@ -256,8 +281,9 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
         }
     };
 
-    // Load tile `it` (the one the running pointers are at) and advance them.
-    auto fetch = [&](int it) {
+    // Load tile `it` (the one the running pointers are at) into the given staging registers and
+    // advance the pointers.
+    auto fetch_into = [&](int it, u32x4(&kst)[NCH], u32x4(&vst)[NCH]) {
         if (it == 0 || it == ctx_tiles) seek(it);
         if (fetch_rows_left >= BN) {
 #pragma unroll
@@ -286,7 +312,7 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
         }
     };
 
-    auto stash = [&](int buf) {
+    auto stash_from = [&](int buf, const u32x4(&kst)[NCH], const u32x4(&vst)[NCH]) {
 #pragma unroll
         for (int x = 0; x < NCH; ++x) {
             if (NCH * NT == CHUNKS || tid + x * NT < CHUNKS) {
@@ -295,6 +321,8 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
             }
         }
     };
+    auto fetch = [&](int it) { fetch_into(it, kst, vst); };
+    auto stash = [&](int buf) { stash_from(buf, kst, vst); };
 
     // ---- per-lane LDS read offsets (elements).
     const int k_rd = c * KPAD + 8 * hb;                                       // + 32*sb*KPAD + 16*ks
@@ -318,6 +346,11 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
                 for (int v = 0; v < 16; ++v) o_acc[j][db][v] = 0.f;
         }
 
+        if (!q_scaled) {  // else the fast pass has left qreg ready
+            u32x4 qraw[QB][KS];
+            request_q(qraw);
+            scale_q(qraw);
+        }
         if (n_tiles > 0) {
             fetch(0);
             stash(0);
@@ -448,14 +481,15 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) o_acc[j][db][v] = 0.f;
         }
-        if (n_tiles > 0) {
-            fetch(0);
-            stash(0);
-        }
-        if (n_tiles > 1) {
-            fetch(1);
-            stash(1);
-        }
+        // the first two tiles and the queries are requested together: one memory round trip
+        // before the loop instead of three
+        u32x4 kst1[NCH], vst1[NCH], qraw[QB][KS];
+        request_q(qraw);
+        if (n_tiles > 0) fetch(0);
+        if (n_tiles > 1) fetch_into(1, kst1, vst1);
+        scale_q(qraw);
+        if (n_tiles > 0) stash(0);
+        if (n_tiles > 1) stash_from(1, kst1, vst1);
         __syncthreads();
         if (n_tiles == 0) return;
 
