@@ -207,6 +207,27 @@ def check(status: int) -> None:
 
 
 _workspaces = {}
+_retired_workspaces = []  # outgrown scratch tensors: recorded graphs may still point at them
+_workspace_tag = 0
+
+
+class workspace_tag:
+    """Calls made inside ``with workspace_tag(i):`` use scratch tensor ``i`` of their device.
+    Launch sequences that run concurrently on different streams (each ordered in itself) must not
+    share one: give each its own tag."""
+
+    def __init__(self, tag: int):
+        self.tag = int(tag)
+
+    def __enter__(self):
+        global _workspace_tag
+        self.prev, _workspace_tag = _workspace_tag, self.tag
+        return self
+
+    def __exit__(self, *exc):
+        global _workspace_tag
+        _workspace_tag = self.prev
+        return False
 
 
 def workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
@@ -214,9 +235,11 @@ def workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
     reused between calls: consecutive launches on one stream are ordered)."""
     if nbytes <= 0:
         return None
-    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device(), _workspace_tag)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() * 4 < nbytes:
+        if ws is not None:
+            _retired_workspaces.append(ws)
         ws = torch.empty((nbytes + 3) // 4, device=device, dtype=torch.float32)
         _workspaces[key] = ws
     return ws

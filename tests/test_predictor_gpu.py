@@ -328,6 +328,43 @@ def test_graph_replayed_sampling_equals_python_loop(device, dtype, monkeypatch):
     assert pred_g._graph_state is not None and pred_g._graph_state.graph is not None
 
 
+def test_graph_sampling_in_concurrent_groups_equals_one_group(device, monkeypatch):
+    """Trajectories sampled as several groups, each replaying its own recorded step on its own
+    stream with its own scratch memory, against all of them in one group: same values, same
+    caches (deterministic head; bf16; the groups are uneven on purpose)."""
+    from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
+    from ar_nanotabpfn_amd.model import MixtureGaussianHead
+
+    def det_sample(self, z, num_samples=1):
+        mean, std, weight, _ = self._parameterize(z)
+        idx = weight.argmax(dim=2, keepdim=True)
+        return torch.gather(mean, 2, idx).permute(0, 1, 3, 2) + 0.1 * torch.gather(std, 2, idx).permute(0, 1, 3, 2)
+
+    monkeypatch.setattr(MixtureGaussianHead, "sample", det_sample)
+    cfg = dict(d_model=128, n_heads=4, n_layers=3, d_ff=128, num_features=3, buffer_size=5, num_components=4)
+    model = _build(cfg, device, dtype=torch.bfloat16)
+    B, Nc, Nt = 70, 2100, 9  # long enough for a split context (partials in per-group scratch)
+    g = torch.Generator().manual_seed(5)
+    xc = torch.randn(1, Nc, 3, generator=g).expand(B, -1, -1).to(device, torch.bfloat16)
+    yc = torch.randn(1, Nc, generator=g).expand(B, -1).to(device, torch.bfloat16)
+    xt = torch.randn(B, Nt, 3, generator=g).to(device, torch.bfloat16)
+    results = {}
+    for chains in (1, 3):
+        pred = ARTabPFNPredictor.from_trained_model(model, backend="triton_shared_context")
+        pred.fuse_step_tail = False  # the deterministic head stands in for the sampler
+        pred.decode_chains, pred.min_chain_batch = chains, 8
+        for _ in range(2):  # second call: recorded graphs are reused
+            y = pred.sample_sequence(xc, yc, xt)
+        assert len(pred._graph_state.chains) == chains
+        results[chains] = (y, [(l.k_buf_cache.clone(), l.v_buf_cache.clone()) for l in model.backbone.layers])
+    y1, c1 = results[1]
+    y3, c3 = results[3]
+    assert y3.shape == (B, Nt) and torch.isfinite(y3).all()
+    assert max_abs(to_np(y1), to_np(y3)) <= 2e-2
+    for (k1, v1), (k3, v3) in zip(c1, c3):
+        assert max_abs(to_np(k1), to_np(k3)) <= 2e-2 and max_abs(to_np(v1), to_np(v3)) <= 2e-2
+
+
 def test_graph_sampling_with_random_head_is_finite_and_varied(device):
     """The real sampler (multinomial + normal draws) inside the recorded graph: every
     replay must draw fresh numbers."""
