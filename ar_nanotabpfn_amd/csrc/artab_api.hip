@@ -668,6 +668,28 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
                     "MFMA decode needs bf16/f16, head_dim in {32,64,128}, aligned rows and a shared context");
     }
 
+    // Per-trajectory context stored in front of the buffer rows of the same cache (the
+    // per-dataset layout, inference.py:687-744): context and buffer are one run of rows per
+    // (trajectory, head), which the buffer kernel streams as it is (HBM-bound, no context pass).
+    if (!use_mfma && impl != ARTAB_IMPL_PORTABLE && !shared_ctx && mfma_shape_ok(dtype, Dh) && aligned &&
+        k_buf && v_buf && k_buf->data && v_buf->data) {
+        const size_t esz = static_cast<size_t>(elem_size(dtype));
+        auto follows = [&](const artab_view *ctx, const artab_view *buf) {
+            return ctx->stride_b == buf->stride_b && ctx->stride_h == buf->stride_h && ctx->stride_n == buf->stride_n &&
+                   static_cast<const char *>(buf->data) ==
+                       static_cast<const char *>(ctx->data) + static_cast<size_t>(Nc) * ctx->stride_n * esz;
+        };
+        if (follows(k_ctx, k_buf) && follows(v_ctx, v_buf)) {
+            DecodeParams D;
+            memset(&D, 0, sizeof(D));
+            D.q = dv(q); D.kb = dv(k_ctx); D.vb = dv(v_ctx); D.knew = dv(k_new); D.vnew = dv(v_new); D.out = dv(out);
+            D.B = B; D.H = H; D.n_split = 0; D.n_buf = n_buf; D.n_buf_dev = n_buf_device; D.n_base = Nc;
+            D.has_new = has_new;
+            D.qscale = scale * kLog2e;
+            return launch_status(launch_decode(D, dtype, Dh, Lq, st), "decode over a per-trajectory cache");
+        }
+    }
+
     if (!use_mfma) {
         PortableParams P;
         memset(&P, 0, sizeof(P));

@@ -26,6 +26,8 @@ struct DecodeParams {
     int n_split;
     int n_buf;    // committed buffer rows
     const int *n_buf_dev;  // when set, the committed length is read from here at run time
+    int n_base;   // rows of kb/vb that precede the counted ones (a per-trajectory context stored in
+                  // front of the buffer rows); 0 for a shared context
     int has_new;  // 1: row n_buf comes from knew/vnew, is attended and appended
     float qscale; // scale * log2(e)
 };
@@ -93,7 +95,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
             for (int i = 0; i < LQ; ++i) M[i] = fmaxf(M[i], v[u][i] * kLog2e);
     }
 
-    const int n_buf = P.n_buf_dev ? *P.n_buf_dev : P.n_buf;
+    const int n_buf = P.n_base + (P.n_buf_dev ? *P.n_buf_dev : P.n_buf);
     const int n_total = n_buf + (P.has_new ? 1 : 0);
     const T *knew_row = P.has_new ? view_row<T>(P.knew, b, h, 0) : nullptr;
     const T *vnew_row = P.has_new ? view_row<T>(P.vnew, b, h, 0) : nullptr;

@@ -279,6 +279,36 @@ def test_decode_attention_config4_full_size(device, n_buf):
     _full_size_decode(device, 2048, 16, 4096, n_buf, 256, seed=4 + n_buf)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("B,H,Lq,Nc,D,n_buf,cap", [(6, 4, 2, 70, 32, 0, 90), (6, 4, 2, 70, 32, 9, 90), (5, 2, 1, 33, 64, 4, 40),
+                                                   (5, 2, 1, 33, 64, 0, 40),
+                                                   (3, 2, 2, 257, 128, 30, 300), (64, 8, 2, 512, 32, 100, 640)])
+def test_decode_attention_per_trajectory_cache(device, dtype, B, H, Lq, Nc, D, n_buf, cap):
+    """Per-dataset layout (inference.py:687-744): every trajectory has its own context, stored in
+    front of its buffer rows in one cache [B,H,cap,D].  The context view and the buffer view are
+    then one run of rows, which the streaming buffer kernel reads as it is (16-bit types); the new
+    row is appended at slot Nc + n_buf."""
+    ak = _ak()
+    cache_k, cache_v = randn((B, H, cap, D), 21, dtype, 0.7), randn((B, H, cap, D), 22, dtype, 0.7)
+    q = randn((B, H, Lq, D), 23, dtype, 0.7)
+    k_new = randn((B, H, 1, D), 24, dtype, 0.7) if Lq == 2 else None
+    v_new = randn((B, H, 1, D), 25, dtype, 0.7) if Lq == 2 else None
+    kc_d, vc_d = cache_k.to(device), cache_v.to(device)
+    out = ak.decode_attention(
+        q.to(device), kc_d[:, :, :Nc], vc_d[:, :, :Nc], kc_d[:, :, Nc:], vc_d[:, :, Nc:], n_buf,
+        k_new.to(device) if Lq == 2 else None, v_new.to(device) if Lq == 2 else None)
+    keys = torch.cat([cache_k[:, :, : Nc + n_buf]] + ([k_new] if Lq == 2 else []), dim=2)
+    vals = torch.cat([cache_v[:, :, : Nc + n_buf]] + ([v_new] if Lq == 2 else []), dim=2)
+    ref, _ = ao.context_attention(to_np(q), to_np(keys), to_np(vals))
+    tol = out_tol(dtype) if dtype != torch.float32 else 2e-5
+    assert max_abs(to_np(out), ref) <= tol
+    exp_k, exp_v = cache_k.clone(), cache_v.clone()
+    if Lq == 2:
+        exp_k[:, :, Nc + n_buf] = k_new[:, :, 0]
+        exp_v[:, :, Nc + n_buf] = v_new[:, :, 0]
+    assert torch.equal(kc_d.cpu(), exp_k) and torch.equal(vc_d.cpu(), exp_v)
+
+
 @pytest.mark.parametrize("n_buf", [1, 2, 17, 33, 64])
 def test_decode_attention_config1_shape(device, n_buf):
     """BASELINE configs[1]: H=8, Dh=64, Nc=1024, B=256, entries ~N(0,1)/8, N_buf swept."""
