@@ -297,3 +297,40 @@ class ARTabPFN(nn.Module):
             "the training forward (context/buffer/target row mask with a backward pass) is not part of this "
             "inference package; use ARTabPFNPredictor.from_trained_model(model)"
         )
+
+    # ---- checkpoints written by the reference's training loop (train.py:336-343): a dict
+    # {"step": int, "model": state_dict}.  With `compile_model` the embedder and the head were
+    # wrapped by torch.compile before the state_dict was taken (train.py:233-235), which puts an
+    # "_orig_mod." segment into their keys.
+
+    @staticmethod
+    def clean_state_dict(state_dict):
+        """The state_dict with every ``_orig_mod.`` path segment removed."""
+        return {k.replace("_orig_mod.", ""): v for k, v in state_dict.items()}
+
+    @classmethod
+    def from_checkpoint(cls, checkpoint, n_heads: int, num_features: int = 10, map_location="cpu"):
+        """Build the model a reference checkpoint was trained with and load it.
+
+        ``checkpoint`` is a path (read with ``torch.load(..., weights_only=True)``), the loaded
+        ``{"step", "model"}`` dict, or a bare state_dict.  Every size except the number of heads is
+        read off the tensors.  Returns ``(model, step)``; ``step`` is None for a bare state_dict.
+        """
+        if not isinstance(checkpoint, dict):
+            checkpoint = torch.load(checkpoint, map_location=map_location, weights_only=True)
+        step = checkpoint.get("step") if "model" in checkpoint else None
+        sd = cls.clean_state_dict(checkpoint["model"] if "model" in checkpoint else checkpoint)
+        try:
+            d_model = sd["embedder.x_embed.weight"].shape[0]
+            d_ff = sd["backbone.layers.0.ff.0.weight"].shape[0]
+            buffer_size = sd["ar_tokens"].shape[0]
+            num_components = sd["head.mean_bias"].shape[0]
+        except KeyError as err:
+            raise ValueError(f"not an AR-TabPFN state_dict: missing {err}") from None
+        n_layers = 1 + max(int(k.split(".")[2]) for k in sd if k.startswith("backbone.layers."))
+        if d_model % n_heads:
+            raise ValueError(f"d_model {d_model} is not divisible by n_heads {n_heads}")
+        model = cls(d_model=d_model, n_heads=n_heads, n_layers=n_layers, d_ff=d_ff, num_features=num_features,
+                    buffer_size=buffer_size, num_components=num_components)
+        model.load_state_dict(sd, strict=True)
+        return model, step

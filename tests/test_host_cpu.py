@@ -120,6 +120,37 @@ def test_model_tree_and_state_dict_keys():
         m()
 
 
+def test_reference_checkpoint_format_loads(tmp_path):
+    """The reference's training loop saves {"step", "model"} (train.py:336-343); with compile_model
+    the embedder and the head carry an "_orig_mod." segment in their keys (train.py:233-235).
+    from_checkpoint reads the sizes off the tensors, strips the segment and loads strictly."""
+    from ar_nanotabpfn_amd.model import ARTabPFN
+
+    torch.manual_seed(3)
+    src = ARTabPFN(d_model=64, n_heads=4, n_layers=3, d_ff=96, num_features=2, buffer_size=7, num_components=4)
+    sd = {}
+    for k, v in src.state_dict().items():
+        top, rest = k.split(".", 1) if "." in k else (k, "")
+        sd[f"{top}._orig_mod.{rest}" if top in ("embedder", "head") else k] = v.clone()
+    assert any("_orig_mod" in k for k in sd)
+    path = tmp_path / "step_10.pt"
+    torch.save({"step": 10, "model": sd}, path)
+
+    model, step = ARTabPFN.from_checkpoint(str(path), n_heads=4, num_features=2)
+    assert step == 10
+    assert (model.d_model, model.buffer_size, len(model.backbone.layers)) == (64, 7, 3)
+    assert model.head.mean_bias.shape[0] == 4 and model.backbone.layers[0].ff[0].out_features == 96
+    for (ka, va), (kb, vb) in zip(src.state_dict().items(), model.state_dict().items()):
+        assert ka == kb and torch.equal(va, vb)
+    # a bare state_dict works too; a foreign one is refused
+    model2, step2 = ARTabPFN.from_checkpoint(src.state_dict(), n_heads=4)
+    assert step2 is None and torch.equal(model2.ar_tokens, src.ar_tokens)
+    with pytest.raises(ValueError):
+        ARTabPFN.from_checkpoint({"w": torch.zeros(1)}, n_heads=4)
+    with pytest.raises(ValueError):
+        ARTabPFN.from_checkpoint(src.state_dict(), n_heads=5)
+
+
 def test_embedder_mean_over_features_and_markers():
     from ar_nanotabpfn_amd.model import Embedder
 
