@@ -439,24 +439,29 @@ hipError_t launch_post(const FusedPostParams &P, int D, int F, hipStream_t st) {
                                                       : launch_post_r<T, kFusedRows>(P, D, F, st);
 }
 
-template <typename T, int D>
+template <typename T, int D, int TR>
 hipError_t launch_sample_d(const SampleEmbedParams &P, int F, hipStream_t st) {
-    dim3 grid(static_cast<unsigned>((P.B + kFusedRows - 1) / kFusedRows)), block(fused_waves(D) * 64);
+    dim3 grid(static_cast<unsigned>((P.B + TR - 1) / TR)), block(fused_waves(D) * 64);
     switch (F) {
-        case 128: hipLaunchKernelGGL((sample_embed_kernel<T, D, 128>), grid, block, 0, st, P); break;
-        case 256: hipLaunchKernelGGL((sample_embed_kernel<T, D, 256>), grid, block, 0, st, P); break;
-        default: hipLaunchKernelGGL((sample_embed_kernel<T, D, 512>), grid, block, 0, st, P); break;
+        case 128: hipLaunchKernelGGL((sample_embed_kernel<T, D, 128, TR>), grid, block, 0, st, P); break;
+        case 256: hipLaunchKernelGGL((sample_embed_kernel<T, D, 256, TR>), grid, block, 0, st, P); break;
+        default: hipLaunchKernelGGL((sample_embed_kernel<T, D, 512, TR>), grid, block, 0, st, P); break;
     }
     return hipGetLastError();
 }
 
+template <typename T, int TR>
+hipError_t launch_sample_r(const SampleEmbedParams &P, int D, int F, hipStream_t st) {
+    switch (D) {
+        case 128: return launch_sample_d<T, 128, TR>(P, F, st);
+        case 256: return launch_sample_d<T, 256, TR>(P, F, st);
+        default: return launch_sample_d<T, 512, TR>(P, F, st);
+    }
+}
 template <typename T>
 hipError_t launch_sample(const SampleEmbedParams &P, int D, int F, hipStream_t st) {
-    switch (D) {
-        case 128: return launch_sample_d<T, 128>(P, F, st);
-        case 256: return launch_sample_d<T, 256>(P, F, st);
-        default: return launch_sample_d<T, 512>(P, F, st);
-    }
+    return fused_tile_rows(P.B) == kFusedRowsSmall ? launch_sample_r<T, kFusedRowsSmall>(P, D, F, st)
+                                                   : launch_sample_r<T, kFusedRows>(P, D, F, st);
 }
 
 bool fused_width_ok(int n) { return n == 128 || n == 256 || n == 512; }

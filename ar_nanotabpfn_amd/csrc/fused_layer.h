@@ -792,33 +792,38 @@ struct SampleEmbedParams {
 
 constexpr int kMaxMixture = 10;  // 3 * K outputs must fit one 32-column block
 
-template <typename T, int D, int F>
+template <typename T, int D, int F, int TR>
 __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(SampleEmbedParams P) {
+    typedef Tile<T, TR> TL;
     constexpr int NW = fused_waves(D), NT = NW * 64;
     constexpr int LDD = D + 8, LDF = F + 8;
-    constexpr int NBF = (F / 32 + NW - 1) / NW;
+    constexpr int NBF = fused_blocks<T, TR>(F, NW);
+    constexpr int NB2 = 32 / TL::kBlock;  // the second head layer is padded to 32 outputs: first wavefront
+    constexpr int VB = TL::kVals, GB = TL::kGroups;
     constexpr int EPL = D / 64;  // elements per lane of one row in the row-wise norm
-    static_assert(F / 32 >= NW ? (F / 32) % NW == 0 : true, "unsupported widths");
-    __shared__ __attribute__((aligned(16))) T a0[kFusedRows * LDD];  // z = norm(x_last)
-    __shared__ __attribute__((aligned(16))) T a1[kFusedRows * LDF];  // gelu(head layer 1)
-    __shared__ float raw_s[kFusedRows][33];
-    __shared__ float y_s[kFusedRows];
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hb = lane >> 5;
+    static_assert(F / TL::kBlock >= NW ? (F / TL::kBlock) % NW == 0 : true, "unsupported widths");
+    __shared__ __attribute__((aligned(16))) T a0[TR * LDD];  // z = norm(x_last)
+    __shared__ __attribute__((aligned(16))) T a1[TR * LDF];  // gelu(head layer 1)
+    __shared__ float raw_s[TR][33];
+    __shared__ float y_s[TR];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = TL::token(lane), hb = TL::sub(lane);
     const int t = *P.step;
     if (t < 0 || t >= P.Nt) return;  // uniform over the grid
-    const long row0 = static_cast<long>(blockIdx.x) * kFusedRows;
-    const int valid = static_cast<int>(min(static_cast<long>(kFusedRows), P.B - row0));
+    const long row0 = static_cast<long>(blockIdx.x) * TR;
+    const int valid = static_cast<int>(min(static_cast<long>(TR), P.B - row0));
 
     int nbf[NBF];
 #pragma unroll
     for (int b = 0; b < NBF; ++b) nbf[b] = wave + NW * b;
-    const int nb0[1] = {0};
-    const bool ff_active = wave < F / 32;
-    WeightStream<T, D, NBF> w_1;
-    WeightStream<T, F, 1> w_2;
+    int nb0[NB2];
+#pragma unroll
+    for (int b = 0; b < NB2; ++b) nb0[b] = b;
+    const bool ff_active = wave < F / TL::kBlock;
+    WeightStream<T, D, NBF, TR> w_1;
+    WeightStream<T, F, NB2, TR> w_2;
     if (ff_active) w_1.start(static_cast<const T *>(P.w_h1), nbf, lane);
     if (wave == 0) w_2.start(static_cast<const T *>(P.w_h2), nb0, lane);
-    stage_tile<T, D, NT>(a0, LDD, static_cast<const T *>(P.x_last) + row0 * P.ld_row, P.ld_row, valid, tid);
+    stage_tile<T, D, NT, TR>(a0, LDD, static_cast<const T *>(P.x_last) + row0 * P.ld_row, P.ld_row, valid, tid);
     __syncthreads();
 
     // ---- z = LayerNorm(x_last), one wavefront per row, in place
@@ -829,7 +834,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
             gam[e] = to_f32(static_cast<const T *>(P.norm_g)[lane * EPL + e]);
             bet[e] = to_f32(static_cast<const T *>(P.norm_b)[lane * EPL + e]);
         }
-        for (int r = wave; r < kFusedRows; r += NW) {
+        for (int r = wave; r < TR; r += NW) {
             T *row = a0 + r * LDD + lane * EPL;
             float x[EPL], sum = 0.f;
 #pragma unroll
@@ -850,39 +855,45 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
 
     // ---- h = gelu(z W_h1^T + b_h1) -> a1
     if (ff_active) {
-        float bias[NBF][16];
-        load_cols<T, NBF>(P.b_h1 ? static_cast<const T *>(P.b_h1) : reinterpret_cast<const T *>(kZeroVector), nbf, hb,
-                          bias);
-        f32x16 acc[NBF];
+        float bias[NBF][VB];
+        load_cols<T, NBF, TR>(P.b_h1 ? static_cast<const T *>(P.b_h1) : reinterpret_cast<const T *>(kZeroVector), nbf,
+                              hb, bias);
+        typename TL::acc_t acc[NBF];
         w_1.run(acc, a0, LDD, c, hb);
 #pragma unroll
         for (int b = 0; b < NBF; ++b)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
+            for (int g = 0; g < GB; ++g) {
                 float o[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const float v = acc[b][4 * g + e] + bias[b][4 * g + e];
                     o[e] = 0.5f * v * (1.f + erff(v * 0.70710678118654752f));
                 }
-                store4f<T>(a1 + c * LDF + col_of(nbf[b], 4 * g, hb), o[0], o[1], o[2], o[3]);
+                store4f<T>(a1 + c * LDF + TL::col(nbf[b], g, hb), o[0], o[1], o[2], o[3]);
             }
     }
     __syncthreads();
 
-    // ---- raw = h W_h2^T + b_h2 (one 32-column block, first wavefront), kept in float32
+    // ---- raw = h W_h2^T + b_h2 (32 output columns, first wavefront), kept in float32
     if (wave == 0) {
-        float bias[1][16];
-        load_cols<T, 1>(P.b_h2 ? static_cast<const T *>(P.b_h2) : reinterpret_cast<const T *>(kZeroVector), nb0, hb, bias);
-        f32x16 acc[1];
+        float bias[NB2][VB];
+        load_cols<T, NB2, TR>(P.b_h2 ? static_cast<const T *>(P.b_h2) : reinterpret_cast<const T *>(kZeroVector), nb0,
+                              hb, bias);
+        typename TL::acc_t acc[NB2];
         w_2.run(acc, a1, LDF, c, hb);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) raw_s[c][col_of(0, v, hb)] = acc[0][v] + bias[0][v];
+        for (int b = 0; b < NB2; ++b)
+#pragma unroll
+            for (int g = 0; g < GB; ++g)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    raw_s[c][TL::col(b, g, hb) + e] = acc[b][4 * g + e] + bias[b][4 * g + e];
     }
     __syncthreads();
 
     // ---- one sample per trajectory: component by inverse CDF of the softmax weights, then a normal
-    if (tid < kFusedRows) {
+    if (tid < TR) {
         float y = 0.f;
         if (tid < valid) {
             const long row = row0 + tid;
@@ -936,7 +947,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
         const T *xm = static_cast<const T *>(P.x_mean);
         const int tn = min(t + 1, P.Nt - 1);
         constexpr int CPR = D / 8;
-        for (int idx = tid; idx < kFusedRows * 2 * CPR; idx += NT) {
+        for (int idx = tid; idx < TR * 2 * CPR; idx += NT) {
             const int ch = idx % CPR, which = (idx / CPR) & 1, r = idx / (2 * CPR);
             if (r >= valid) continue;
             const long row = row0 + r;

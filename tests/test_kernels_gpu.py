@@ -819,7 +819,7 @@ def _tail_reference(net, x_last, x_mean, u, n, t, dtype):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,D,F,K,t", [(70, 128, 128, 5, 3), (1024, 256, 256, 5, 1), (33, 512, 256, 10, 6),
                                        (40, 256, 512, 3, 7)])
-def test_decode_sample_embed_matches_float64(device, dtype, B, D, F, K, t):
+def test_decode_sample_embed_matches_float64(device, tile_rows, dtype, B, D, F, K, t):
     from ar_nanotabpfn_amd.glue import SampleEmbedStep
 
     Nt, bs = 8, 5
