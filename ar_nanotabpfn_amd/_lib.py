@@ -64,6 +64,7 @@ class ArtabSampleEmbedArgs(ctypes.Structure):
         ("step", _p), ("Nt", _i),
         ("preds", _p), ("emb_next", _p),
         ("B", _i), ("D", _i), ("F", _i),
+        ("advance", _p), ("n_advance", _i), ("ticket", _p),
     ]
 
 
@@ -135,8 +136,8 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes
-    if lib.artab_version() != 1:
-        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.artab_version()} != 1; rebuild the extension")
+    if lib.artab_version() != 2:
+        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.artab_version()} != 2; rebuild the extension")
     _lib = lib
     return lib
 

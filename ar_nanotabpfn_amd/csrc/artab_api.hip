@@ -1221,6 +1221,9 @@ int artab_decode_sample_embed(const artab_sample_embed_args *a, int dtype, void 
     P.w_x = a->w_x; P.b_x = a->b_x; P.w_y = a->w_y; P.b_y = a->b_y; P.markers = a->markers;
     P.ar_tokens = a->ar_tokens; P.bs = a->bs; P.step = a->step; P.Nt = a->Nt;
     P.preds = a->preds; P.emb = a->emb_next; P.B = a->B;
+    if (a->advance && (a->n_advance < 1 || a->n_advance > 8 || !a->ticket))
+        return fail(ARTAB_ERR_BAD_SHAPE, "advance needs 1..8 counters and a ticket word");
+    P.advance = a->advance; P.n_advance = a->advance ? a->n_advance : 0; P.ticket = a->ticket;
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipError_t e = dtype == ARTAB_BF16 ? launch_sample<bf16_t>(P, a->D, a->F, st) : launch_sample<f16_t>(P, a->D, a->F, st);
     return launch_status(e, "decode_sample_embed");

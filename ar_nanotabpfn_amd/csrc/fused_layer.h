@@ -788,6 +788,8 @@ struct SampleEmbedParams {
     void *preds;                      // [B, Nt]
     void *emb;                        // [B, 2, D] rows of step t + 1
     int B;
+    int *advance; int n_advance;      // loop counters to increment once per launch, or nullptr
+    unsigned *ticket;                 // zero between launches: counts finished workgroups
 };
 
 constexpr int kMaxMixture = 10;  // 3 * K outputs must fit one 32-column block
@@ -972,6 +974,19 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
             }
             u32x4 val = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
             *reinterpret_cast<u32x4 *>(static_cast<T *>(P.emb) + (row * 2 + which) * D + 8 * ch) = val;
+        }
+    }
+
+    // ---- the caller's loop counters: every workgroup read the step index when it started, so
+    // the one that takes the last ticket may move them on
+    if (P.advance) {
+        __syncthreads();
+        if (tid == 0) {
+            __threadfence();
+            if (atomicAdd(P.ticket, 1u) == gridDim.x - 1) {
+                for (int i = 0; i < P.n_advance; ++i) P.advance[i] += 1;
+                *P.ticket = 0u;
+            }
         }
     }
 }

@@ -209,7 +209,7 @@ class SampleEmbedStep:
                 and lin2.out_features == 3 * head.num_components)
 
     def __init__(self, embedder, backbone, head, ar_tokens: Tensor, x_mean: Tensor, rand_u: Tensor, rand_n: Tensor,
-                 step: Tensor, preds: Tensor, emb: Tensor):
+                 step: Tensor, preds: Tensor, emb: Tensor, advance: Optional[Tensor] = None):
         lin1, lin2 = head.head[0], head.head[2]
         dev, dt = emb.device, emb.dtype
         B, Nt = preds.shape
@@ -248,6 +248,14 @@ class SampleEmbedStep:
         a.step, a.Nt = step.data_ptr(), Nt
         a.preds, a.emb_next = preds.data_ptr(), emb.data_ptr()
         a.B, a.D, a.F = B, D, F_
+        # ``advance``: contiguous int32 loop counters that the launch increments itself (the last
+        # workgroup to finish does it), instead of a separate add launched by the caller
+        self.advances = advance is not None
+        if advance is not None:
+            assert advance.dtype == torch.int32 and advance.is_contiguous() and 1 <= advance.numel() <= 8
+            k["advance"] = advance
+            k["ticket"] = torch.zeros(1, device=dev, dtype=torch.int32)
+            a.advance, a.n_advance, a.ticket = advance.data_ptr(), advance.numel(), k["ticket"].data_ptr()
         self.args = a
 
     def __call__(self, x_last: Tensor) -> None:

@@ -345,8 +345,7 @@ class ARTabPFNPredictor:
             x_row = self._run_layers(
                 st.emb, lambda layer, q, k, v: self._attend_decode_shared(layer, q, k, v, n_buf_device=st.nbuf,
                                                                           rows=st.rows, chain=st.chain))
-            st.tail(x_row)          # norm, head, draw, preds[:, t], embedding of step t + 1
-            st.counters.add_(1)     # (t, nbuf)
+            st.tail(x_row)          # norm, head, draw, preds[:, t], embedding of step t + 1, (t, nbuf) += 1
             return
         bs = self.ar_tokens.shape[0]
         t = st.t.long()
@@ -410,7 +409,7 @@ class ARTabPFNPredictor:
                     st.rand_u = torch.zeros((Nt, Bc), device=device, dtype=torch.float32)
                     st.rand_n = torch.zeros((Nt, Bc), device=device, dtype=torch.float32)
                     st.tail = SampleEmbedStep(self.embedder, self.backbone, self.head, self.ar_tokens, st.x_mean,
-                                              st.rand_u, st.rand_n, st.t, st.preds, st.emb)
+                                              st.rand_u, st.rand_n, st.t, st.preds, st.emb, advance=st.counters)
                 gs.chains.append(st)
             gs.tail = gs.chains[0].tail
             self._graph_state = gs

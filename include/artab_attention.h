@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define ARTAB_VERSION 1
+#define ARTAB_VERSION 2
 
 typedef enum artab_dtype {
     ARTAB_BF16 = 0,
@@ -353,6 +353,13 @@ typedef struct artab_sample_embed_args {
     void *preds;             /* [B, Nt]; column t is written */
     void *emb_next;          /* [B, 2, D] contiguous: rows of step t + 1 */
     int B, D, F;
+    /* Optional: the caller's device-side loop counters.  When `advance` is given, the last
+     * workgroup to finish adds 1 to advance[0] .. advance[n_advance-1] (step index, buffer
+     * length, ...), which saves the caller a launch per step.  `ticket` is one uint32 of device
+     * memory that is zero before the first call; the kernel leaves it zero. */
+    int32_t *advance;
+    int n_advance;
+    uint32_t *ticket;
 } artab_sample_embed_args;
 
 int artab_decode_sample_embed(const artab_sample_embed_args *args, int dtype, void *stream);

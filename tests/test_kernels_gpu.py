@@ -871,6 +871,33 @@ def test_decode_sample_embed_step_out_of_range_is_noop(device):
     assert torch.all(preds == 7.0) and torch.all(emb == 3.0)
 
 
+def test_decode_sample_embed_advances_loop_counters(device, tile_rows):
+    """With ``advance`` the launch moves the caller's loop counters on by one, once, whatever the
+    number of workgroups, writes column t of every call, and leaves its ticket word at zero; an
+    out-of-range step index neither samples nor advances."""
+    from ar_nanotabpfn_amd.glue import SampleEmbedStep
+
+    dtype, B, D, Nt = torch.bfloat16, 200, 128, 6
+    net = _tail_model(D, 128, 5, 3, dtype, device)
+    counters = torch.tensor([1, 0, 40], dtype=torch.int32, device=device)  # (t, n_buf, anything else)
+    preds = torch.full((B, Nt), 7.0, device=device, dtype=dtype)
+    emb = torch.zeros((B, 2, D), device=device, dtype=dtype)
+    tail = SampleEmbedStep(net.embedder, net.backbone, net.head, net.ar_tokens,
+                           torch.zeros(B, Nt, device=device, dtype=dtype), torch.rand(Nt, B, device=device),
+                           torch.randn(Nt, B, device=device), counters[0:1], preds, emb, advance=counters)
+    x = torch.randn(B, 2, D, device=device).to(dtype)
+    for n in range(1, Nt):
+        tail(x)
+        torch.cuda.synchronize()
+        assert counters.tolist() == [1 + n, n, 40 + n]
+        assert int(tail._keep["ticket"].item()) == 0
+        assert torch.all(preds[:, n] != 7.0) and (n + 1 == Nt or torch.all(preds[:, n + 1 :] == 7.0))
+    before = preds.clone()
+    tail(x)  # t == Nt: out of range
+    torch.cuda.synchronize()
+    assert counters.tolist() == [Nt, Nt - 1, 40 + Nt - 1] and torch.equal(preds, before)
+
+
 def test_decode_sample_embed_component_frequencies(device):
     """With many trajectories sharing one head input, the picked components follow the mixture
     weights and the draws have the mixture's mean (law of the sampler, not a bitwise check)."""
