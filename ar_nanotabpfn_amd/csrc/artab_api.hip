@@ -741,6 +741,7 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
     // Streaming schedule: the buffer pass (HBM-bound, on the matrix pipe) leaves its result as one
     // more partial; with a side stream it runs next to the context pass (forked and joined with
     // events, so the call stays ordered on `stream` and can be recorded into a graph).
+    D.deep_rows = env_int("ARTAB_STREAM_DEEP", kStreamDeepRows);  // tuning hook
     D.buf_part_o = static_cast<char *>(workspace) + static_cast<size_t>(pl.n_split) * rows * Dh * 2;
     D.buf_part_lse = F.part_lse + static_cast<size_t>(pl.n_split) * rows;
     hipStream_t side = (side_stream && side_stream != stream) ? static_cast<hipStream_t>(side_stream) : st;

@@ -30,6 +30,7 @@
 namespace artab {
 
 constexpr int kStreamChunks = 4;           // ring depth per wavefront
+constexpr int kStreamDeepRows = 224;       // buffers longer than this use the whole ring
 constexpr int kStreamChunkBytes = 8192;    // 4 keys x 16 pairs x (64 B of K + 64 B of V)
 constexpr int kStreamQBytes = 4096;        // one task's queries: 4 x (64 lanes x 16 B)
 constexpr size_t kStreamLdsBytes = kStreamChunks * kStreamChunkBytes + 2 * kStreamQBytes;
@@ -199,7 +200,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
     }
     // two query slots: the producer may be at most one task ahead of the consumer
     auto may_issue = [&]() { return issued < total_chunks && issue_seq <= seq + 1; };
-    for (int i = 0; i < S; ++i)
+    // Chunks kept in flight.  The loads hold the CU's outstanding-miss slots that the context pass
+    // next door needs for its own tiles; a buffer that is finished before that pass anyway uses
+    // half the ring and disturbs it less (measured at B=1024, H=8: 950 -> 974 steps/s; a quarter of
+    // the ring is too little: 933).  A long one is on the critical path itself.
+    const int depth = n_total > P.deep_rows ? S : S / 2;
+    for (int i = 0; i < depth; ++i)
         if (may_issue()) issue_one();
 
     // ---- consumer
@@ -279,7 +285,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
         }
         // the chunk has been read: refill its slot (and any the producer had to leave empty)
         if (g + 1 == n_groups) ++seq;
-        while (may_issue() && issued - c - 1 < S) issue_one();
+        while (may_issue() && issued - c - 1 < depth) issue_one();
 
         slot = slot + 1 == S ? 0 : slot + 1;
         if (++g == n_groups) {
