@@ -73,6 +73,9 @@ class ARTabPFNPredictor:
         # 2 groups 846 steps/s against 948 for one — a context pass that shares the CUs with another
         # group's buffer pass slows down by as much as the overlap saves — so the default is one.
         self.decode_chains = 1
+        # Decode steps recorded into one graph (a replay boundary costs about 5 us on the device); a
+        # one-step graph covers the remainder.
+        self.steps_per_graph = 4
         self.min_chain_batch = 256   # groups smaller than this are not worth their fixed costs
         self._side_streams = {}
         self._graph_state = None
@@ -380,7 +383,7 @@ class ARTabPFNPredictor:
         chain_rows = self._chain_rows(B)
         key = (B, Nt, F_, self.context_len, dtype, str(device), layer0.k_ctx_cache.data_ptr(),
                layer0.k_buf_cache.data_ptr(), self.fuse_step_tail, self.overlap_buffer_pass, self.merge_in_layer,
-               len(chain_rows), tuple((p.data_ptr(), p._version) for p in params))
+               len(chain_rows), int(self.steps_per_graph), tuple((p.data_ptr(), p._version) for p in params))
         gs = self._graph_state
         if gs is None or gs.key != key:
             gs = _GraphState()
@@ -401,6 +404,7 @@ class ARTabPFNPredictor:
                 st.counters = torch.zeros(2, device=device, dtype=torch.int32)  # (step index t, buffer length)
                 st.t, st.nbuf = st.counters[0:1], st.counters[1:2]
                 st.graph = None
+                st.graph_many = None   # steps_per_graph steps in one graph
                 st.tail = None
                 if fused_tail:
                     D = self.backbone.d_model
@@ -456,20 +460,31 @@ class ARTabPFNPredictor:
                 with torch.cuda.graph(graph):
                     self._graph_step(st)
                 st.graph = graph
+                if self.steps_per_graph > 1 and Nt - 1 >= self.steps_per_graph:
+                    reset(st)
+                    many = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(many):
+                        for _ in range(self.steps_per_graph):
+                            self._graph_step(st)
+                    st.graph_many = many
         gs.graph = gs.chains[0].graph
         for st in gs.chains:
             reset(st)
+        k = self.steps_per_graph if gs.chains[0].graph_many is not None else 1
+        n_many, n_single = (Nt - 1) // k if k > 1 else 0, (Nt - 1) % k if k > 1 else Nt - 1
         if len(gs.chains) == 1:
-            for _ in range(Nt - 1):
+            for _ in range(n_many):
+                gs.chains[0].graph_many.replay()
+            for _ in range(n_single):
                 gs.chains[0].graph.replay()
         else:
             # every group replays its own step on its own stream; they meet again at the end
             for st in gs.chains:
                 st.stream.wait_stream(current)
-            for _ in range(Nt - 1):
+            for i in range(n_many + n_single):
                 for st in gs.chains:
                     with torch.cuda.stream(st.stream):
-                        st.graph.replay()
+                        (st.graph_many if i < n_many else st.graph).replay()
             for st in gs.chains:
                 current.wait_stream(st.stream)
         self.buffer_len = Nt - 1
