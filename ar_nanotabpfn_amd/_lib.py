@@ -19,6 +19,8 @@ LIB_PATH = os.path.join(_HERE, "libartab_attention.so")
 ARTAB_BF16, ARTAB_F16, ARTAB_F32 = 0, 1, 2
 IMPL_AUTO, IMPL_PORTABLE, IMPL_MFMA = 0, 1, 2
 
+ORDER_WAIT = 1            # artab_attention_partials.order_flags
+ORDER_CONSUMER_WAITS = 2  # flags of artab_decode_attention_partials_ordered
 ARTAB_ERR_NULL_POINTER = -1
 ARTAB_ERR_BAD_SHAPE = -2
 ARTAB_ERR_BAD_STRIDE = -3
@@ -46,7 +48,8 @@ _i, _f, _p, _sz, _i64 = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_
 class ArtabAttentionPartials(ctypes.Structure):
     """``artab_attention_partials`` of include/artab_attention.h."""
 
-    _fields_ = [("part_o", _p), ("part_lse", _p), ("n_slots", _i), ("B", _i), ("H", _i), ("Lq", _i), ("Dh", _i)]
+    _fields_ = [("part_o", _p), ("part_lse", _p), ("n_slots", _i), ("B", _i), ("H", _i), ("Lq", _i), ("Dh", _i),
+                ("order_state", _p), ("order_timeout_us", ctypes.c_uint64), ("order_flags", _i)]
 
 
 class ArtabSampleEmbedArgs(ctypes.Structure):
@@ -90,6 +93,13 @@ SIGNATURES = {
         [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _p, _i, _i, _f, _i, _p, _sz, _i, _p, _p,
          ctypes.POINTER(ArtabAttentionPartials)],
     ),
+    "artab_decode_attention_partials_ordered": (
+        _i,
+        [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _p, _i, _i, _f, _i, _p, _sz, _i, _p, _p,
+         ctypes.POINTER(ArtabAttentionPartials), _p, ctypes.c_uint64, _i],
+    ),
+    "artab_order_signal": (_i, [_p, _i, _p]),
+    "artab_order_wait": (_i, [_p, _i, ctypes.c_uint64, _p]),
     "artab_teacher_forcing_attention": (_i, [_VP, _VP, _VP, _VP, _VP, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "artab_prefill_attention": (_i, [_VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "artab_buffer_attention": (_i, [_VP, _VP, _VP, _p, _i64, _i64, _i64, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _p]),
@@ -136,8 +146,8 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes
-    if lib.artab_version() != 2:
-        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.artab_version()} != 2; rebuild the extension")
+    if lib.artab_version() != 3:
+        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.artab_version()} != 3; rebuild the extension")
     _lib = lib
     return lib
 

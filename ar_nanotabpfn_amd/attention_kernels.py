@@ -24,6 +24,8 @@ from . import _lib
 
 __all__ = [
     "AttentionPartials",
+    "QueueOrder",
+    "concurrent_stream",
     "hip_available",
     "triton_available",
     "context_attention",
@@ -222,6 +224,7 @@ def decode_attention(
     n_buf_device: Optional[Tensor] = None,
     side_stream: Optional["torch.cuda.Stream"] = None,
     leave_partials: bool = False,
+    order: Optional["QueueOrder"] = None,
 ):
     """One decode step of row attention (inference.py:785-823) in one call.
 
@@ -238,6 +241,12 @@ def decode_attention(
     ``side_stream`` (a default-priority stream of the same device) lets the buffer pass
     run next to the context pass (``artab_decode_attention_overlapped``); the call is
     still ordered on the current stream.
+
+    ``order`` (with ``side_stream`` and ``leave_partials``) orders the two streams through the
+    counters of a ``QueueOrder`` instead of two events per call
+    (``artab_decode_attention_partials_ordered``): the caller makes ``side_stream`` wait for the
+    current stream before the first such call and the current stream for ``side_stream`` after
+    the last, and checks ``order.failed()`` before using the results.
 
     ``leave_partials=True`` skips the final merge where the schedule produces partial results
     and returns an ``AttentionPartials`` for ``glue.layer_post`` / ``layer_post_pre`` to merge
@@ -267,6 +276,16 @@ def decode_attention(
         ws_ptr, ws_bytes, _impl(use_triton), _lib.current_stream(dev),
     )
     side = ctypes.c_void_p(side_stream.cuda_stream) if side_stream is not None else None
+    if order is not None:
+        if not leave_partials or side_stream is None:
+            raise ValueError("counter-ordered decode needs side_stream and leave_partials=True")
+        desc = _lib.ArtabAttentionPartials()
+        flags = _lib.ORDER_CONSUMER_WAITS if order.consumer_waits else 0
+        _lib.check(lib.artab_decode_attention_partials_ordered(
+            *args, side, ctypes.byref(desc), ctypes.c_void_p(order.state.data_ptr()), int(order.timeout_us), flags))
+        parts = AttentionPartials(desc, q.dtype, q.device)
+        parts.order = order
+        return parts
     if leave_partials:
         desc = _lib.ArtabAttentionPartials()
         _lib.check(lib.artab_decode_attention_partials(*args, side, ctypes.byref(desc)))
@@ -279,12 +298,80 @@ def decode_attention(
     return out
 
 
+class QueueOrder:
+    """Counters in device memory that order two streams without events (``artab_order_*``):
+    ``state`` holds counter "main" at int32 index 0, counter "side" at 32 and ``failed`` at 64."""
+
+    MAIN, SIDE = 0, 1
+
+    def __init__(self, device, timeout_us: int = 2_000_000):
+        self.state = torch.zeros(128, device=device, dtype=torch.int32)
+        if self.state.data_ptr() % 128:
+            raise RuntimeError("queue-order state is not 128-byte aligned")
+        self.timeout_us = int(timeout_us)
+        # Let the consumer of an ordered attention call's partials (``glue.layer_post_pre`` /
+        # ``layer_post``, ``AttentionPartials.merged``) wait for the side stream itself instead of
+        # a wait launch inside the call.
+        self.consumer_waits = True
+
+    def signal(self, queue: int, stream: "torch.cuda.Stream") -> None:
+        _lib.check(_lib.load().artab_order_signal(
+            ctypes.c_void_p(self.state.data_ptr()), int(queue), ctypes.c_void_p(stream.cuda_stream)))
+
+    def wait(self, queue: int, stream: "torch.cuda.Stream", timeout_us: Optional[int] = None) -> None:
+        _lib.check(_lib.load().artab_order_wait(
+            ctypes.c_void_p(self.state.data_ptr()), int(queue),
+            int(self.timeout_us if timeout_us is None else timeout_us), ctypes.c_void_p(stream.cuda_stream)))
+
+    def failed(self) -> int:
+        """Number of waits that gave up (synchronises with the device)."""
+        return int(self.state[64].item())
+
+    def reset(self) -> None:
+        self.state.zero_()
+
+    def streams_run_concurrently(self, main: "torch.cuda.Stream", side: "torch.cuda.Stream",
+                                 timeout_us: int = 50_000) -> bool:
+        """One round of the protocol on the two streams: ``side`` waits for a signal that is launched
+        on ``main`` after it.  False when the wait timed out, i.e. the two streams are served by one
+        hardware queue (or a tool serialises launches) and counters cannot order them."""
+        side.wait_stream(main)
+        self.wait(self.SIDE, side, timeout_us)
+        self.signal(self.MAIN, main)
+        self.signal(self.SIDE, side)
+        self.wait(self.MAIN, main, timeout_us)
+        main.wait_stream(side)
+        main.synchronize()
+        ok = self.failed() == 0
+        self.reset()
+        main.synchronize()
+        return ok
+
+
+def concurrent_stream(device, main: Optional["torch.cuda.Stream"] = None, tries: int = 8):
+    """A default-priority stream that runs side by side with ``main`` (default: the current
+    stream), and whether that was confirmed.  The runtime serves its streams from a few hardware
+    queues; two streams that land on the same one execute one after the other, which silently
+    serialises the two passes of a decode step (and makes counter ordering impossible).  Candidates
+    are probed with one round of the ``QueueOrder`` protocol (50 ms when it fails); call this
+    outside graph capture."""
+    main = torch.cuda.current_stream(device) if main is None else main
+    probe = QueueOrder(device)
+    side = None
+    for _ in range(max(1, tries)):
+        side = torch.cuda.Stream(device=device)
+        if side.cuda_stream != main.cuda_stream and probe.streams_run_concurrently(main, side):
+            return side, True
+    return side, False
+
+
 class AttentionPartials:
     """Unmerged attention result of a decode step (``artab_attention_partials``): it points into
     the device's split workspace and is valid until the next attention call on that device."""
 
     def __init__(self, desc, dtype, device):
         self.desc, self.dtype, self.device = desc, dtype, device
+        self.order = None  # the QueueOrder of an ordered call
 
     @property
     def shape(self):  # of the merged [B,H,Lq,Dh] result

@@ -18,6 +18,7 @@
 #include "glue_kernels.h"
 #include "mfma_flash.h"
 #include "portable_kernels.h"
+#include "queue_order.h"
 
 namespace artab {
 
@@ -613,12 +614,44 @@ int artab_context_attention(const artab_view *q, const artab_view *k_ctx, const 
     return ARTAB_OK;
 }
 
+static int order_signal(uint32_t *state, int queue, hipStream_t st) {
+    hipLaunchKernelGGL(order_signal_kernel, dim3(1), dim3(64), 0, st,
+                       state + (queue == ARTAB_ORDER_SIDE ? kOrderSide : kOrderMain));
+    return launch_status(hipGetLastError(), "queue-order signal");
+}
+
+static int order_wait(uint32_t *state, int queue, uint64_t timeout_us, hipStream_t st) {
+    if (timeout_us == 0) timeout_us = 2000000;  // 2 s
+    hipLaunchKernelGGL(order_gate_kernel, dim3(1), dim3(64), 0, st, state, queue == ARTAB_ORDER_SIDE ? 1 : 0,
+                       static_cast<unsigned long long>(timeout_us) * 100ull);  // 100 MHz wall clock
+    return launch_status(hipGetLastError(), "queue-order wait");
+}
+
+static int check_order_args(const uint32_t *state, int queue) {
+    if (!state) return fail(ARTAB_ERR_NULL_POINTER, "queue-order state is NULL");
+    if (reinterpret_cast<uintptr_t>(state) % 128) return fail(ARTAB_ERR_BAD_STRIDE, "queue-order state must be 128-byte aligned");
+    if (queue != ARTAB_ORDER_MAIN && queue != ARTAB_ORDER_SIDE)
+        return fail(ARTAB_ERR_BAD_SHAPE, "queue must be ARTAB_ORDER_MAIN or ARTAB_ORDER_SIDE, got %d", queue);
+    return ARTAB_OK;
+}
+
+int artab_order_signal(uint32_t *state, int queue, void *stream) {
+    ARTAB_TRY(check_order_args(state, queue));
+    return order_signal(state, queue, static_cast<hipStream_t>(stream));
+}
+
+int artab_order_wait(uint32_t *state, int queue, uint64_t timeout_us, void *stream) {
+    ARTAB_TRY(check_order_args(state, queue));
+    return order_wait(state, queue, timeout_us, static_cast<hipStream_t>(stream));
+}
+
 static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
                        const artab_view *k_buf, const artab_view *v_buf, const artab_view *k_new,
                        const artab_view *v_new, const artab_view *out, int B, int H, int Lq, int Nc,
                        int n_buf, const int32_t *n_buf_device, int buf_capacity, int Dh, float scale,
                        int dtype, void *workspace, size_t workspace_bytes, int impl, void *stream,
-                       void *side_stream, artab_attention_partials *leave_partials = nullptr) {
+                       void *side_stream, artab_attention_partials *leave_partials = nullptr,
+                       uint32_t *order_state = nullptr, uint64_t order_timeout_us = 0, int order_flags = 0) {
     if (leave_partials) memset(leave_partials, 0, sizeof(*leave_partials));
     ARTAB_TRY(check_common(B, H, Lq, Dh, dtype));
     if (Lq != 1 && Lq != 2)
@@ -661,6 +694,9 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
         // for it on a SIMD); it is used when the caller offers a second stream to run it on
         stream_buf = need_buf && Dh == 32 &&
                      ((side_stream && side_stream != stream) || env_int("ARTAB_STREAM", 0) != 0);
+        if (order_state && !(stream_buf && side_stream && side_stream != stream))
+            return fail(ARTAB_ERR_UNSUPPORTED,
+                        "counter-ordered decode needs the streaming buffer pass (head_dim 32, buffer rows) and a second stream");
         need_ws = direct ? 0 : split_workspace_bytes(rows, Dh, pl.n_split + (stream_buf ? 1 : 0));
         if (need_ws && (!workspace || workspace_bytes < need_ws || reinterpret_cast<uintptr_t>(workspace) % 16)) {
             if (impl == ARTAB_IMPL_MFMA)
@@ -672,6 +708,8 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
         return fail(ARTAB_ERR_UNSUPPORTED,
                     "MFMA decode needs bf16/f16, head_dim in {32,64,128}, aligned rows and a shared context");
     }
+    if (order_state && !use_mfma)
+        return fail(ARTAB_ERR_UNSUPPORTED, "counter-ordered decode needs the matrix-core path with its workspace");
 
     // Per-trajectory context stored in front of the buffer rows of the same cache (the
     // per-dataset layout, inference.py:687-744): context and buffer are one run of rows per
@@ -745,6 +783,38 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
     D.buf_part_o = static_cast<char *>(workspace) + static_cast<size_t>(pl.n_split) * rows * Dh * 2;
     D.buf_part_lse = F.part_lse + static_cast<size_t>(pl.n_split) * rows;
     hipStream_t side = (side_stream && side_stream != stream) ? static_cast<hipStream_t>(side_stream) : st;
+    if (order_state) {
+        // Ordered by the two counters: the caller has forked `side` from `stream` once (and joins
+        // it once, after its last call); no event per layer.
+        hipStreamCaptureStatus cap_main = hipStreamCaptureStatusNone, cap_side = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &cap_main) != hipSuccess || hipStreamIsCapturing(side, &cap_side) != hipSuccess)
+            return fail(ARTAB_ERR_LAUNCH, "hipStreamIsCapturing failed");
+        if (cap_main != cap_side)
+            return fail(ARTAB_ERR_UNSUPPORTED,
+                        "counter-ordered decode: one stream is being captured and the other is not; make the side "
+                        "stream wait for the main one before the first call");
+        F.started = order_state + kOrderMain;  // q and the new K/V row are ready once the context pass starts
+        ARTAB_TRY(order_wait(order_state, ARTAB_ORDER_SIDE, order_timeout_us, side));
+        hipError_t e_ctx, e_buf;
+        {
+            ProfileScope prof(st);
+            e_ctx = launch_flash_dtype(F, dtype, Dh, pl.BM, st);
+        }
+        e_buf = launch_stream(D, dtype, Lq, side);
+        ARTAB_TRY(launch_status(e_ctx, "decode context pass"));
+        ARTAB_TRY(launch_status(e_buf, "decode buffer pass (stream)"));
+        ARTAB_TRY(order_signal(order_state, ARTAB_ORDER_SIDE, side));    // the buffer pass's partial is ready
+        if (order_flags & ARTAB_ORDER_CONSUMER_WAITS) {
+            leave_partials->order_state = order_state;
+            leave_partials->order_timeout_us = order_timeout_us;
+            leave_partials->order_flags = ARTAB_ORDER_WAIT;
+        } else {
+            ARTAB_TRY(order_wait(order_state, ARTAB_ORDER_MAIN, order_timeout_us, st));
+        }
+        leave_partials->part_o = F.part_o; leave_partials->part_lse = F.part_lse; leave_partials->n_slots = slots;
+        leave_partials->B = B; leave_partials->H = H; leave_partials->Lq = Lq; leave_partials->Dh = Dh;
+        return ARTAB_OK;
+    }
     hipEvent_t fork = nullptr, join = nullptr;
     if (side != st) {
         ARTAB_TRY(fork_join_events(&fork, &join));
@@ -796,6 +866,10 @@ int artab_merge_attention_partials(const artab_attention_partials *partials, con
     C.H = partials->H; C.Lq = partials->Lq; C.Dh = partials->Dh; C.n_split = partials->n_slots;
     unsigned grid = static_cast<unsigned>((C.rows * (C.Dh / 4) + 255) / 256);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (partials->order_flags & ARTAB_ORDER_WAIT) {
+        ARTAB_TRY(check_order_args(partials->order_state, ARTAB_ORDER_MAIN));
+        ARTAB_TRY(order_wait(partials->order_state, ARTAB_ORDER_MAIN, partials->order_timeout_us, st));
+    }
     if (dtype == ARTAB_BF16)
         hipLaunchKernelGGL((combine_kernel<bf16_t>), dim3(grid), dim3(256), 0, st, C);
     else
@@ -821,6 +895,22 @@ int artab_decode_attention_partials(const artab_view *q, const artab_view *k_ctx
     if (!partials) return fail(ARTAB_ERR_NULL_POINTER, "partials descriptor is NULL");
     return decode_impl(q, k_ctx, v_ctx, k_buf, v_buf, k_new, v_new, out, B, H, Lq, Nc, n_buf, n_buf_device,
                        buf_capacity, Dh, scale, dtype, workspace, workspace_bytes, impl, stream, side_stream, partials);
+}
+
+int artab_decode_attention_partials_ordered(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                                            const artab_view *k_buf, const artab_view *v_buf, const artab_view *k_new,
+                                            const artab_view *v_new, const artab_view *out, int B, int H, int Lq,
+                                            int Nc, int n_buf, const int32_t *n_buf_device, int buf_capacity, int Dh,
+                                            float scale, int dtype, void *workspace, size_t workspace_bytes, int impl,
+                                            void *stream, void *side_stream, artab_attention_partials *partials,
+                                            uint32_t *order_state, uint64_t timeout_us, int flags) {
+    if (!partials) return fail(ARTAB_ERR_NULL_POINTER, "partials descriptor is NULL");
+    ARTAB_TRY(check_order_args(order_state, ARTAB_ORDER_MAIN));
+    if (flags & ~ARTAB_ORDER_CONSUMER_WAITS)
+        return fail(ARTAB_ERR_BAD_SHAPE, "unknown ordering flags 0x%x", flags);
+    return decode_impl(q, k_ctx, v_ctx, k_buf, v_buf, k_new, v_new, out, B, H, Lq, Nc, n_buf, n_buf_device,
+                       buf_capacity, Dh, scale, dtype, workspace, workspace_bytes, impl, stream, side_stream, partials,
+                       order_state, timeout_us, flags);
 }
 
 int artab_decode_attention_overlapped(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
@@ -1100,6 +1190,31 @@ static int fill_post(FusedPostParams &P, const void *attn, int64_t lda, const vo
     return ARTAB_OK;
 }
 
+// Ordering that a partial descriptor asks of its consumer.  The wait goes into the kernel when its grid leaves half of the compute units
+// free — a waiting workgroup must not keep the buffer pass it waits for off the chip — and into a
+// launch of its own otherwise.
+static int apply_partials_order(const artab_attention_partials *parts, FusedPostParams &P, int64_t rows,
+                                hipStream_t st) {
+    if (!parts || !(parts->order_flags & ARTAB_ORDER_WAIT)) return ARTAB_OK;
+    ARTAB_TRY(check_order_args(parts->order_state, ARTAB_ORDER_MAIN));
+    if (rows == 0) return fail(ARTAB_ERR_BAD_SHAPE, "ordered partials with no rows");
+    {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            cus = 0;
+        const int64_t grid = (rows + fused_tile_rows(rows) - 1) / fused_tile_rows(rows);
+        const uint64_t us = parts->order_timeout_us ? parts->order_timeout_us : 2000000;
+        if (grid * 2 <= cus && env_int("ARTAB_ORDER_GATE_LAUNCH", 0) == 0) {
+            P.order_wait = parts->order_state;
+            P.order_limit = us * 100ull;  // 100 MHz wall clock
+        } else {
+            ARTAB_TRY(order_wait(parts->order_state, ARTAB_ORDER_MAIN, us, st));
+        }
+    }
+    return ARTAB_OK;
+}
+
 static int check_layer_dtype_rows(const char *what, int dtype, int64_t rows) {
     if (dtype != ARTAB_BF16 && dtype != ARTAB_F16)
         return fail(ARTAB_ERR_UNSUPPORTED, "%s supports bf16 and fp16 only (dtype code %d)", what, dtype);
@@ -1147,8 +1262,9 @@ static int layer_post_pre_impl(const artab_attention_partials *parts, const void
                         ln3_beta, eps3, nullptr, rows, D, F, false, parts));
     ARTAB_TRY(fill_pre(N, nullptr, 0, next_w_fo, next_ln1_gamma, next_ln1_beta, next_eps1, next_w_qkv, next_y,
                        next_qkv, rows, D, false));
-    if (rows == 0) return ARTAB_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    ARTAB_TRY(apply_partials_order(parts, P, rows, st));
+    if (rows == 0) return ARTAB_OK;
     hipError_t e = dtype == ARTAB_BF16 ? launch_post_pre<bf16_t>(P, N, D, F, st) : launch_post_pre<f16_t>(P, N, D, F, st);
     return launch_status(e, "layer_post_pre");
 }
@@ -1188,8 +1304,9 @@ int artab_layer_post_from_partials(const artab_attention_partials *parts, const 
     FusedPostParams P{};
     ARTAB_TRY(fill_post(P, nullptr, 0, y, ldy, w_o, ln2_gamma, ln2_beta, eps2, w_1, b_1, w_2, b_2, ln3_gamma,
                         ln3_beta, eps3, out, rows, D, F, true, parts));
-    if (rows == 0) return ARTAB_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    ARTAB_TRY(apply_partials_order(parts, P, rows, st));
+    if (rows == 0) return ARTAB_OK;
     hipError_t e = dtype == ARTAB_BF16 ? launch_post<bf16_t>(P, D, F, st) : launch_post<f16_t>(P, D, F, st);
     return launch_status(e, "layer_post");
 }

@@ -20,6 +20,7 @@
 #pragma once
 
 #include "common.h"
+#include "queue_order.h"
 #include "mfma_flash.h"
 
 namespace artab {
@@ -66,6 +67,8 @@ struct FusedPostParams {
     void *out;                   // [rows, D] contiguous
     long rows;
     float eps2, eps3;
+    unsigned *order_wait;        // queue-order state: wait for the side counter before the partials are read
+    unsigned long long order_limit;  // ... for at most this many ticks of the 100 MHz wall clock
 };
 
 // Packed weight layout.  A torch.nn.Linear weight W [N, K] (row-major) is stored as
@@ -650,7 +653,13 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
     dma_vector<T, D, NT>(vecs + kVecG3 * vec_ld, P.g3, tid, 3);
     dma_vector<T, D, NT>(vecs + kVecB3 * vec_ld, P.b3, tid, 4);
     dma_vector<T, D, NT>(vecs + kVecBias2 * vec_ld, P.bias_2, tid, 5);
-    if (P.part_o) stage_merged_attention<T, D, NT, TR>(a0, LDD, P, row0, valid, tid);
+    if (P.part_o) {
+        if (P.order_wait) {  // the buffer pass's partial comes from the other queue
+            if (tid == 0) order_wait_device(P.order_wait, 0, P.order_limit);
+            __syncthreads();
+        }
+        stage_merged_attention<T, D, NT, TR>(a0, LDD, P, row0, valid, tid);
+    }
     w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
     wait_all_loads();
     __syncthreads();

@@ -87,6 +87,9 @@ struct FlashParams {
     float qscale;  // softmax scale * log2(e), folded into Q
     int mode;
     int force_robust;  // 1: skip the fast path (testing the online-softmax path)
+    unsigned *started;  // optional counter that the first thread of the grid advances at once: "the
+                        // launches ahead of this one on its queue are complete" for a watcher on
+                        // another queue (queue_order.h); the kernel's own work does not depend on it
 };
 
 // Probability mass (sum of 2^s over a row) the fast path accepts.
@@ -134,6 +137,9 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
     __shared__ __attribute__((aligned(16))) T k_lds[3][BN * KPAD];
     __shared__ __attribute__((aligned(16))) T v_lds[3][BN * VPAD];
     __shared__ int redo_flag;
+
+    if (P.started && blockIdx.x == 0 && threadIdx.x == 0)
+        __hip_atomic_fetch_add(P.started, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
     // ---- workgroup -> (kv-sharing group, q tile, context split); XCD-aware: the
     // hardware deals consecutive workgroup ids round-robin over the 8 XCDs, so all

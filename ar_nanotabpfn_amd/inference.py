@@ -77,6 +77,10 @@ class ARTabPFNPredictor:
         # one-step graph covers the remainder.
         self.steps_per_graph = 4
         self.min_chain_batch = 256   # groups smaller than this are not worth their fixed costs
+        # Order the two streams of the recorded step through counters in device memory instead of
+        # two events per layer (``attention_kernels.QueueOrder``); used when the two streams are found
+        # to run concurrently, otherwise (and when set to False) the events are used.
+        self.counter_ordering = True
         self._side_streams = {}
         self._graph_state = None
 
@@ -128,9 +132,21 @@ class ARTabPFNPredictor:
         if device.type != "cuda":
             return None
         key = (device.index if device.index is not None else torch.cuda.current_device(), tag)
-        if key not in self._side_streams:
-            self._side_streams[key] = torch.cuda.Stream(device=device)  # default priority
-        return self._side_streams[key]
+        current = torch.cuda.current_stream(device)
+        side = self._side_streams.get(key)
+        if side is None or side.cuda_stream == current.cuda_stream:
+            # torch hands out streams from a small pool, round-robin, and the runtime serves them from a
+            # few hardware queues: a "new" stream can be the one that is current, or share its queue,
+            # and the two passes would silently run one after the other.  Probe for one that does not.
+            if torch.cuda.is_current_stream_capturing():
+                for _ in range(8):
+                    side = torch.cuda.Stream(device=device)  # default priority
+                    if side.cuda_stream != current.cuda_stream:
+                        break
+            else:
+                side, _ = ak.concurrent_stream(device, current)
+            self._side_streams[key] = side
+        return side
 
     def clear_cache(self) -> None:
         """Reset the cursors, keep the memory (inference.py:137-141)."""
@@ -225,7 +241,7 @@ class ARTabPFNPredictor:
 
     def _attend_decode_shared(self, layer, q: Tensor, k_new: Tensor, v_new: Tensor,
                               n_buf_device: Optional[Tensor] = None, rows: Optional[slice] = None,
-                              chain: int = 0) -> Tensor:
+                              chain: int = 0, order=None) -> Tensor:
         """The attention call of a shared-layout decode step (inference.py:785-823).  ``rows``
         restricts it to a group of trajectories (a slice of the batch axis of the buffer cache)."""
         N = q.shape[2]
@@ -245,7 +261,7 @@ class ARTabPFNPredictor:
             attn = ak.decode_attention(
                 q, k_ctx, v_ctx, k_buf, v_buf, n_buf,
                 k_new[:, :, 0:1], v_new[:, :, 0:1], n_buf_device=n_buf_device, side_stream=side,
-                leave_partials=partials,
+                leave_partials=partials, order=order,
             )
         return attn
 
@@ -347,7 +363,8 @@ class ARTabPFNPredictor:
             # embedding of this step was left in st.emb by the previous step's tail launch
             x_row = self._run_layers(
                 st.emb, lambda layer, q, k, v: self._attend_decode_shared(layer, q, k, v, n_buf_device=st.nbuf,
-                                                                          rows=st.rows, chain=st.chain))
+                                                                          rows=st.rows, chain=st.chain,
+                                                                          order=st.order_active))
             st.tail(x_row)          # norm, head, draw, preds[:, t], embedding of step t + 1, (t, nbuf) += 1
             return
         bs = self.ar_tokens.shape[0]
@@ -359,7 +376,8 @@ class ARTabPFNPredictor:
         x_row = torch.cat([buffer_emb, self.embedder.embed_target(x_t)], dim=1)
         x_row = self._run_layers(
             x_row, lambda layer, q, k, v: self._attend_decode_shared(layer, q, k, v, n_buf_device=st.nbuf,
-                                                                      rows=st.rows, chain=st.chain))
+                                                                      rows=st.rows, chain=st.chain,
+                                                                      order=st.order_active))
         z = add_layer_norm(x_row, None, None, self.backbone.norm)
         y = self.head.sample(z[:, -1:, :])[:, :, 0, 0]
         st.preds.index_copy_(1, t, y)
@@ -383,7 +401,7 @@ class ARTabPFNPredictor:
         chain_rows = self._chain_rows(B)
         key = (B, Nt, F_, self.context_len, dtype, str(device), layer0.k_ctx_cache.data_ptr(),
                layer0.k_buf_cache.data_ptr(), self.fuse_step_tail, self.overlap_buffer_pass, self.merge_in_layer,
-               len(chain_rows), int(self.steps_per_graph), tuple((p.data_ptr(), p._version) for p in params))
+               len(chain_rows), int(self.steps_per_graph), bool(self.counter_ordering), tuple((p.data_ptr(), p._version) for p in params))
         gs = self._graph_state
         if gs is None or gs.key != key:
             gs = _GraphState()
@@ -406,6 +424,12 @@ class ARTabPFNPredictor:
                 st.graph = None
                 st.graph_many = None   # steps_per_graph steps in one graph
                 st.tail = None
+                st.order = st.order_active = None
+                if self._counter_ordering_applies(x_target):
+                    order = ak.QueueOrder(device)
+                    if order.streams_run_concurrently(torch.cuda.current_stream(device),
+                                                      self._side_stream(device, idx)):
+                        st.order = order
                 if fused_tail:
                     D = self.backbone.d_model
                     st.emb = torch.zeros((Bc, 2, D), device=device, dtype=dtype)
@@ -456,17 +480,10 @@ class ARTabPFNPredictor:
                         self._graph_step(st)
                 current.wait_stream(warm)
                 reset(st)
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph):
-                    self._graph_step(st)
-                st.graph = graph
+                st.graph = self._record_steps(st, 1)
                 if self.steps_per_graph > 1 and Nt - 1 >= self.steps_per_graph:
                     reset(st)
-                    many = torch.cuda.CUDAGraph()
-                    with torch.cuda.graph(many):
-                        for _ in range(self.steps_per_graph):
-                            self._graph_step(st)
-                    st.graph_many = many
+                    st.graph_many = self._record_steps(st, self.steps_per_graph)
         gs.graph = gs.chains[0].graph
         for st in gs.chains:
             reset(st)
@@ -487,11 +504,49 @@ class ARTabPFNPredictor:
                         (st.graph_many if i < n_many else st.graph).replay()
             for st in gs.chains:
                 current.wait_stream(st.stream)
+        if any(st.order is not None and st.order.failed() for st in gs.chains):
+            # a wait on the counters timed out: the recorded streams did not run side by side.
+            # The step's results are void; record it again with events and sample afresh.
+            for st in gs.chains:
+                if st.order is not None:
+                    st.order.reset()
+            self.counter_ordering = False
+            self._graph_state = None
+            return self._sample_sequence_graph(x_target)
         self.buffer_len = Nt - 1
         self.seq_len = self.context_len + self.buffer_len
         if len(gs.chains) == 1:
             return gs.chains[0].preds.clone()
         return torch.cat([st.preds for st in gs.chains], dim=0)
+
+    def _counter_ordering_applies(self, x: Tensor) -> bool:
+        """Whether every layer's decode call takes the schedule that the counters can order: the
+        streaming buffer pass beside the context pass, partials merged by the fused layer kernel."""
+        if not (self.counter_ordering and self.overlap_buffer_pass and self.merge_in_layer and self.fuse_step_tail):
+            return False
+        return all(layer.attn_rows.head_dim == 32 and layer.fused_for(x) for layer in self.backbone.layers)
+
+    def _record_steps(self, st, n_steps: int) -> "torch.cuda.CUDAGraph":
+        """Record ``n_steps`` decode steps of one trajectory group into a HIP graph.  With counter
+        ordering the side stream joins the recording once and rejoins at the end; the per-layer
+        dependencies between the two streams are the counters' waits."""
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            if st.order is None:
+                for _ in range(n_steps):
+                    self._graph_step(st)
+            else:
+                main = torch.cuda.current_stream()
+                side = self._side_stream(main.device, st.chain)
+                side.wait_stream(main)
+                st.order_active = st.order
+                try:
+                    for _ in range(n_steps):
+                        self._graph_step(st)
+                finally:
+                    st.order_active = None
+                    main.wait_stream(side)
+        return graph
 
     @staticmethod
     def _draw_step_variates(rand_u: Tensor, rand_n: Tensor) -> None:

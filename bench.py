@@ -243,6 +243,8 @@ def main():
     ap.add_argument("--steps", type=int, default=NT3)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline legs")
+    ap.add_argument("--event-ordering", action="store_true",
+                    help="order the two streams of the recorded step with events instead of device-side counters")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only copy a 256 MiB buffer five times (reference kernel for scaling HBM counters)")
     ap.add_argument("--kernel-shapes", action="store_true",
@@ -276,6 +278,8 @@ def main():
     model = build_model(device, dtype)
     x_context, y_context, x_target = decode_inputs(device, dtype)
     pred = ARTabPFNPredictor.from_trained_model(model, backend="triton_shared_context")
+    if args.event_ordering:
+        pred.counter_ordering = False
 
     torch.manual_seed(0)
     if args.warmup:
@@ -362,6 +366,8 @@ def main():
             "B": B3, "N_ctx": NC3, "N_targets": NT3, "layers": L, "heads": H, "head_dim": Dh,
         },
         "trajectory_steps_per_sec": round(value * B3, 1),
+        "stream_ordering": ("counters" if getattr(pred._graph_state.chains[0], "order", None) is not None else "events")
+        if pred._graph_state is not None else None,
         "prefill_ms": round(prefill_ms, 3),
         "roofline": roofline,
     }

@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define ARTAB_VERSION 2
+#define ARTAB_VERSION 3
 
 typedef enum artab_dtype {
     ARTAB_BF16 = 0,
@@ -174,6 +174,10 @@ typedef struct artab_attention_partials {
     const float *part_lse;
     int n_slots;
     int B, H, Lq, Dh;
+    /* Set by artab_decode_attention_partials_ordered, zero otherwise (see there): */
+    uint32_t *order_state;      /* counters the consumer of these partials has to honour */
+    uint64_t order_timeout_us;
+    int order_flags;            /* ARTAB_ORDER_WAIT or 0 */
 } artab_attention_partials;
 
 /*
@@ -192,6 +196,60 @@ int artab_decode_attention_partials(const artab_view *q, const artab_view *k_ctx
                            int buf_capacity, int Dh, float scale, int dtype,
                            void *workspace, size_t workspace_bytes, int impl, void *stream, void *side_stream,
                            artab_attention_partials *partials);
+
+/*
+ * Ordering of the two streams of a decode step through device memory instead of events.  No
+ * counterpart in the reference, whose decode step is a sequence of launches on one stream
+ * (ar_tabpfn/model/inference.py:746-833); it exists because an event dependency between two
+ * hardware queues costs 5-6 us on the waiting queue and a layer has two of them.
+ *
+ * `state` is ARTAB_ORDER_STATE_BYTES of device memory, 128-byte aligned, zero before the first
+ * use: counter "main" (uint32 index 0), counter "side" (index 32), and `failed` (index 64).
+ *   artab_order_signal(state, queue, stream)  one-thread launch on `stream`: counter[queue] += 1,
+ *                                             after everything launched on `stream` before it.
+ *   artab_order_wait(state, ARTAB_ORDER_SIDE, ...)  one-wavefront launch that holds `stream` until
+ *                                             counter[main] >= counter[side] + 1;
+ *   artab_order_wait(state, ARTAB_ORDER_MAIN, ...)  ... until counter[side] >= counter[main].
+ * A wait gives up after timeout_us (0 = 2 s), adds 1 to `failed` and lets its stream continue;
+ * while `failed` is non-zero every wait falls through.  The host must check `failed` before it
+ * uses results ordered this way (a non-zero value means the two streams did not run
+ * concurrently: they share a hardware queue, or a tool serialises launches) and fall back to
+ * artab_decode_attention_partials.
+ *
+ * artab_decode_attention_partials_ordered is artab_decode_attention_partials with its two event
+ * dependencies replaced by
+ *   stream:       context pass (signals main as it starts)          wait(main)
+ *   side_stream:  wait(side)    buffer pass     signal(side)
+ * The caller makes side_stream wait for `stream` once before the first call of a sequence (so
+ * that a graph capture covers both) and `stream` for side_stream once after the last; between
+ * them no event is recorded.  Only the streaming schedule is supported (head_dim 32, bf16/fp16,
+ * buffer rows or n_buf_device, side_stream != stream): anything else returns
+ * ARTAB_ERR_UNSUPPORTED before a launch is made.
+ *
+ * On `stream` the signal costs no launch: the first thread of the context pass advances the main
+ * counter (everything launched on `stream` before it is complete by then).  With
+ * flags = ARTAB_ORDER_CONSUMER_WAITS the wait costs none either: the descriptor carries
+ * order_state, order_timeout_us and order_flags = ARTAB_ORDER_WAIT, and whoever consumes the
+ * partials (artab_layer_post_from_partials, artab_layer_post_pre_from_partials,
+ * artab_merge_attention_partials) waits before reading them — inside its own workgroups when its
+ * grid leaves half of the compute units free, else with a wait launch of its own.
+ */
+#define ARTAB_ORDER_STATE_BYTES 512
+#define ARTAB_ORDER_MAIN 0
+#define ARTAB_ORDER_SIDE 1
+#define ARTAB_ORDER_WAIT 1            /* artab_attention_partials.order_flags */
+#define ARTAB_ORDER_CONSUMER_WAITS 2  /* flags of artab_decode_attention_partials_ordered */
+int artab_order_signal(uint32_t *state, int queue, void *stream);
+int artab_order_wait(uint32_t *state, int queue, uint64_t timeout_us, void *stream);
+int artab_decode_attention_partials_ordered(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                           const artab_view *k_buf, const artab_view *v_buf,
+                           const artab_view *k_new, const artab_view *v_new,
+                           const artab_view *out,
+                           int B, int H, int Lq, int Nc, int n_buf, const int32_t *n_buf_device,
+                           int buf_capacity, int Dh, float scale, int dtype,
+                           void *workspace, size_t workspace_bytes, int impl, void *stream, void *side_stream,
+                           artab_attention_partials *partials,
+                                            uint32_t *order_state, uint64_t timeout_us, int flags);
 
 /*
  * Teacher-forced attention over [Buffer_0..Nt-1, Target_0..Nt-1] queries.

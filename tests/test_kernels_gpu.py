@@ -1001,3 +1001,146 @@ def test_decode_partials_merged_in_layer_kernel(device, tile_rows, dtype, B, H, 
     assert torch.equal(got_post, ref_post)
     for a, b in zip(got_mid, ref_mid):
         assert torch.equal(a, b)
+
+
+def test_queue_order_wait_gives_up_after_its_time_limit(device):
+    """A wait whose signal never comes (forced from the host: nothing is launched on the other
+    stream) ends after its time limit, counts itself in `failed`, and every later wait falls
+    through at once; the streams stay usable."""
+    import time
+
+    ak = _ak()
+    order = ak.QueueOrder(device)
+    main = torch.cuda.current_stream(device)
+    order.wait(order.SIDE, main, timeout_us=2000)      # needs counter main >= 1: never signalled
+    main.synchronize()
+    assert order.failed() == 1
+    t0 = time.time()
+    for _ in range(20):
+        order.wait(order.SIDE, main, timeout_us=10_000_000)  # falls through: `failed` is set
+    main.synchronize()
+    assert time.time() - t0 < 5.0 and order.failed() == 21
+    order.reset()
+    order.wait(order.MAIN, main, timeout_us=2000)      # counter side >= counter main (0 >= 0): no wait
+    order.signal(order.MAIN, main)
+    order.signal(order.SIDE, main)
+    order.wait(order.MAIN, main, timeout_us=2000)      # 1 >= 1
+    main.synchronize()
+    assert order.failed() == 0
+    assert order.state[0].item() == 1 and order.state[32].item() == 1
+
+
+def test_queue_order_argument_checks(device):
+    ak = _ak()
+    order = ak.QueueOrder(device)
+    main = torch.cuda.current_stream(device)
+    with pytest.raises(ValueError):
+        order.signal(2, main)
+    q, k_ctx, v_ctx = (t.to(device) for t in _ctx_inputs(4, 2, 2, 64, 64, torch.bfloat16, seed=1))
+    kc = torch.zeros((4, 2, 8, 64), device=device, dtype=torch.bfloat16)
+    kn = torch.zeros((4, 2, 1, 64), device=device, dtype=torch.bfloat16)
+    side = torch.cuda.Stream(device=device)
+    with pytest.raises(ValueError):  # needs a side stream and partials
+        ak.decode_attention(q, k_ctx, v_ctx, kc, kc.clone(), 0, kn, kn.clone(), order=order)
+    with pytest.raises(RuntimeError):  # head_dim 64 has no streaming buffer pass: refused before any launch
+        ak.decode_attention(q, k_ctx, v_ctx, kc, kc.clone(), 0, kn, kn.clone(), side_stream=side,
+                            leave_partials=True, order=order)
+    main.synchronize()
+    assert order.failed() == 0 and order.state[0].item() == 0
+
+
+@pytest.mark.parametrize("absorb", [False, True])
+@pytest.mark.parametrize("B,H,Nc,cap", [(64, 8, 2048, 8), (600, 8, 1024, 12)])
+def test_decode_attention_ordered_by_counters_equals_event_ordered(device, B, H, Nc, cap, absorb):
+    """A run of decode steps whose two streams are ordered by device-side counters (one fork
+    before the first call, one join after the last) against the same steps ordered by two events
+    per call: same partials (bit for bit after the merge), same cache, no wait timed out."""
+    ak = _ak()
+    dtype, D = torch.bfloat16, 32
+    q0, k_ctx, v_ctx = (t.to(device) for t in _ctx_inputs(B, H, 2, Nc, D, dtype, seed=1, scale=0.6))
+    k_ref, v_ref = torch.zeros((B, H, cap, D), device=device, dtype=dtype), torch.zeros((B, H, cap, D), device=device, dtype=dtype)
+    k_ord, v_ord = k_ref.clone(), v_ref.clone()
+    main = torch.cuda.current_stream(device)
+    side, concurrent = ak.concurrent_stream(device, main)
+    if not concurrent:
+        pytest.skip("no second stream runs side by side with the current one here: counters cannot order them")
+    order = ak.QueueOrder(device)
+    order.consumer_waits = absorb  # True: the merge launch waits for the side counter itself
+    steps = cap - 1
+    qs = [(q0 * (1.0 + 0.1 * s)).to(dtype) for s in range(steps)]
+    news = [(randn((B, H, 1, D), 10 + s, dtype, 0.6).to(device), randn((B, H, 1, D), 40 + s, dtype, 0.6).to(device))
+            for s in range(steps)]
+    expect = []
+    for s in range(steps):
+        expect.append(ak.decode_attention(qs[s], k_ctx, v_ctx, k_ref, v_ref, s, *news[s], side_stream=side))
+    torch.cuda.synchronize()
+    got = []
+    side.wait_stream(main)
+    for s in range(steps):
+        parts = ak.decode_attention(qs[s], k_ctx, v_ctx, k_ord, v_ord, s, *news[s], side_stream=side,
+                                    leave_partials=True, order=order)
+        got.append(parts.merged())  # on the main stream, behind the wait on the side counter
+    main.wait_stream(side)
+    torch.cuda.synchronize()
+    assert order.failed() == 0
+    assert order.state[0].item() == steps and order.state[32].item() == steps
+    for s in range(steps):
+        assert torch.equal(got[s], expect[s]), f"step {s}"
+    assert torch.equal(k_ord, k_ref) and torch.equal(v_ord, v_ref)
+
+
+@pytest.mark.parametrize("gate_launch", [0, 1])
+@pytest.mark.parametrize("B,H,Nc,cap", [(64, 4, 4096, 8), (200, 8, 1024, 6)])
+def test_layer_kernels_wait_for_the_side_queue_themselves(device, monkeypatch, tile_rows, gate_launch, B, H, Nc, cap):
+    """Three layers of a decode step whose streams are ordered by counters, with the main
+    stream's wait done by the layer kernels themselves (they wait for the buffer pass before
+    they read the partials), repeated for several steps, against the event-ordered launches: bit
+    for bit.  gate_launch=1 forces the wait into a launch of its own (what a grid larger than half
+    the chip gets)."""
+    from ar_nanotabpfn_amd import attention_kernels as ak
+    from ar_nanotabpfn_amd import model as m
+
+    monkeypatch.setenv("ARTAB_ORDER_GATE_LAUNCH", str(gate_launch))
+    dtype, Dh, F, n_layers = torch.bfloat16, 32, 128, 3
+    D = H * Dh
+    torch.manual_seed(3)
+    layers = [m.TwoStageTransformerLayer(D, H, F).to(device=device, dtype=dtype) for _ in range(n_layers)]
+    ctx = [tuple(x.to(device) for x in _ctx_inputs(1, H, 1, Nc, Dh, dtype, seed=20 + i, scale=0.6)[1:]) for i in range(n_layers)]
+    main = torch.cuda.current_stream(device)
+    side, concurrent = ak.concurrent_stream(device, main)
+    if not concurrent:
+        pytest.skip("no second stream runs side by side with the current one here: counters cannot order them")
+    order = ak.QueueOrder(device)
+    steps = cap - 1
+    xs = [randn((B, 2, D), 50 + s, dtype, 1.0).to(device) for s in range(steps)]
+
+    def run(ordered):
+        caches = [(torch.zeros((B, H, cap, Dh), device=device, dtype=dtype), torch.zeros((B, H, cap, Dh), device=device, dtype=dtype))
+                  for _ in range(n_layers)]
+        outs = []
+        if ordered:
+            side.wait_stream(main)
+        for s in range(steps):
+            state = layers[0].pre_attention(xs[s])
+            for i, layer in enumerate(layers):
+                y, q, k, v = state
+                attn = ak.decode_attention(q, ctx[i][0], ctx[i][1], caches[i][0], caches[i][1], s, k[:, :, 0:1], v[:, :, 0:1],
+                                           side_stream=side, leave_partials=True, order=order if ordered else None)
+                assert isinstance(attn, ak.AttentionPartials)
+                if i + 1 == n_layers:
+                    outs.append(layer.finish(y, attn))
+                else:
+                    state = layer.finish_then_pre(y, attn, layers[i + 1])
+        if ordered:
+            main.wait_stream(side)
+        torch.cuda.synchronize()
+        return outs, caches
+
+    ref_out, ref_caches = run(False)
+    got_out, got_caches = run(True)
+    assert order.failed() == 0
+    assert order.state[0].item() == steps * n_layers and order.state[32].item() == steps * n_layers
+    for s in range(steps):
+        assert torch.equal(got_out[s], ref_out[s]), f"step {s}"
+    for (k0, v0), (k1, v1) in zip(ref_caches, got_caches):
+        assert torch.equal(k0, k1) and torch.equal(v0, v1)
