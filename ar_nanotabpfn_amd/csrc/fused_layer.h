@@ -653,6 +653,8 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
     dma_vector<T, D, NT>(vecs + kVecG3 * vec_ld, P.g3, tid, 3);
     dma_vector<T, D, NT>(vecs + kVecB3 * vec_ld, P.b3, tid, 4);
     dma_vector<T, D, NT>(vecs + kVecBias2 * vec_ld, P.bias_2, tid, 5);
+    // the first weights travel while the partials are waited for, fetched and merged
+    w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
     if (P.part_o) {
         if (P.order_wait) {  // the buffer pass's partial comes from the other queue
             if (tid == 0) order_wait_device(P.order_wait, 0, P.order_limit);
@@ -660,7 +662,6 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
         }
         stage_merged_attention<T, D, NT, TR>(a0, LDD, P, row0, valid, tid);
     }
-    w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
     wait_all_loads();
     __syncthreads();
     if (ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane);

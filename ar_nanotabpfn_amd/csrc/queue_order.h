@@ -47,17 +47,19 @@ __device__ __forceinline__ unsigned order_load(const unsigned *p) {
 // Wait of one queue for the other (see the file comment); called by one thread.
 __device__ __forceinline__ void order_wait_device(unsigned *state, int side, unsigned long long limit_ticks) {
     // a queue's own counter is written by earlier launches of the same queue only: stable here
-    const unsigned own = order_load(state + (side ? kOrderSide : kOrderMain));
-    const unsigned target = side ? own + 1u : own;
     const unsigned *other = state + (side ? kOrderMain : kOrderSide);
     unsigned *failed = state + kOrderFailed;
+    const unsigned own = order_load(state + (side ? kOrderSide : kOrderMain));
+    unsigned seen = order_load(other);  // both requests travel together: one round trip when nothing is pending
+    const unsigned target = side ? own + 1u : own;
     const unsigned long long t0 = wall_clock64();
-    while (static_cast<int>(order_load(other) - target) < 0) {
+    while (static_cast<int>(seen - target) < 0) {
         if (order_load(failed) != 0u || wall_clock64() - t0 > limit_ticks) {
             atomicAdd(failed, 1u);
             break;
         }
         __builtin_amdgcn_s_sleep(8);
+        seen = order_load(other);
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 }
