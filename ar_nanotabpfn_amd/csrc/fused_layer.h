@@ -148,12 +148,25 @@ struct Tile<T, 16> {
     }
 };
 
+struct NoHook {
+    __device__ __forceinline__ void operator()() const {}
+};
+
 // One transposed product: acc[b][v] = sum_k W[32*nblk[b] + row(v)][k] * A[c][k] for NB blocks of
 // 32 output columns; A is the [32, K] activation tile in LDS (row stride ld), W the packed weight.
 // The weight fragments are fetched explicitly ahead of their use — start() issues the first PF
-// contraction steps and can be called long before run(), e.g. ahead of the previous product's
-// epilogue, so that the memory round trips of chained products overlap.  (Left to itself the
-// compiler issues each load right before the MFMA that needs it: one round trip per step.)
+// contraction steps and is called long before run(), so that the memory round trips of chained
+// products overlap.  (Left to itself the compiler issues each load right before the MFMA that
+// needs it: one round trip per step.)  The memory pipeline of a compute
+// unit takes about 1.75 us for one 128 KiB matrix and its request queue holds much less than a
+// matrix: a wavefront that asks for the next matrix while the current one is still on its way
+// blocks at the request until there is room, and does nothing else meanwhile.  Hence the rule
+// every caller follows: request a matrix when the one before it has arrived — run() waits for
+// its own fragments and then calls `on_arrival`, which requests the next stream — so that the
+// pipeline always has one matrix to work on and no wavefront queues up behind it.  The rule is
+// for matrices that fit the prefetch window (kWhole; widths up to 256): a deeper one is
+// requested piecemeal inside its product, the next stream is then requested ahead of that
+// product as before, and run() calls `on_arrival` without waiting.
 template <typename T, int K, int NB, int TR = 32>
 struct WeightStream {
     typedef Tile<T, TR> TL;
@@ -162,33 +175,57 @@ struct WeightStream {
     static constexpr int KS = K / TL::kStepK;
     static constexpr int PFW = NB >= 4 ? 4 : (NB == 2 ? 8 : 16);
     static constexpr int PF = PFW < KS ? PFW : KS;
+    static constexpr bool kWhole = PF >= KS;  // start() requests the whole matrix
     const T *wl[NB];
     vec wf[PF][NB];
+    int rot;  // contraction step this workgroup starts with
 
     __device__ __forceinline__ void start(const T *wp, const int (&nblk)[NB], int lane) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) wl[b] = wp + TL::weight_offset(nblk[b], K, lane);
+        // Every workgroup streams the same matrix at about the same time, and the 16 of an XCD
+        // would ask its L2 for the same lines at the same moment (measured: 1.5 us of a 19 us layer
+        // kernel).  Each starts its contraction at a different step instead; a sum does not care.
+        // Workgroup ids are dealt round-robin over the 8 XCDs, so id / 8 counts within an XCD.
+        static_assert((KS & (KS - 1)) == 0, "contraction steps must be a power of two");
+        rot = (blockIdx.x >> 3) & (KS - 1);
 #pragma unroll
         for (int p = 0; p < PF; ++p)
 #pragma unroll
-            for (int b = 0; b < NB; ++b) wf[p][b] = *reinterpret_cast<const vec *>(wl[b] + p * TL::kStepStride);
+            for (int b = 0; b < NB; ++b)
+                wf[p][b] = *reinterpret_cast<const vec *>(wl[b] + ((p + rot) & (KS - 1)) * TL::kStepStride);
         __builtin_amdgcn_sched_barrier(0);  // the prefetch stays where it was written
     }
 
-    __device__ __forceinline__ void run(acc_t (&acc)[NB], const T *a_lds, int ld, int c, int hb) {
+    template <typename Hook = NoHook>
+    __device__ __forceinline__ void run(acc_t (&acc)[NB], const T *a_lds, int ld, int c, int hb,
+                                        Hook on_arrival = Hook{}) {
+        if (kWhole) {
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // this stream is all that is in flight: it has arrived
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        on_arrival();
 #pragma unroll
         for (int b = 0; b < NB; ++b)
 #pragma unroll
             for (int v = 0; v < TL::kVals; ++v) acc[b][v] = 0.f;
+        multiply(acc, a_lds, ld, c, hb);
+    }
+
+    // acc += W A^T over the whole contraction, without waiting for anything but the fragments used
+    // (a matrix deeper than the prefetch window is requested step by step as fragments are used up)
+    __device__ __forceinline__ void multiply(acc_t (&acc)[NB], const T *a_lds, int ld, int c, int hb) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            const vec af = *reinterpret_cast<const vec *>(a_lds + c * ld + TL::kStepK * ks + 8 * hb);
+            const vec af =
+                *reinterpret_cast<const vec *>(a_lds + c * ld + TL::kStepK * ((ks + rot) & (KS - 1)) + 8 * hb);
 #pragma unroll
             for (int b = 0; b < NB; ++b) acc[b] = TL::mma(wf[ks % PF][b], af, acc[b]);
             if (ks + PF < KS) {
 #pragma unroll
                 for (int b = 0; b < NB; ++b)
-                    wf[ks % PF][b] = *reinterpret_cast<const vec *>(wl[b] + (ks + PF) * TL::kStepStride);
+                    wf[ks % PF][b] =
+                        *reinterpret_cast<const vec *>(wl[b] + ((ks + PF + rot) & (KS - 1)) * TL::kStepStride);
             }
         }
     }
@@ -256,9 +293,11 @@ struct PartialIndex {
 
 constexpr int kMergeBatch = 9;  // partials fetched per round (8 context slices + the buffer pass)
 
-template <typename T, int D, int NT, int TR>
+// `on_arrival` runs once every load issued so far (the caller's and the partials') has come back
+// and before the merge arithmetic: the place to request the next weight stream.
+template <typename T, int D, int NT, int TR, typename Hook>
 __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const FusedPostParams &P, long row0,
-                                                       int valid, int tid) {
+                                                       int valid, int tid, Hook on_arrival) {
     const int dh = D / P.H;          // head dim, a multiple of 8
     const PartialIndex where(P.Lq, P.H, dh);
     const unsigned tok0 = static_cast<unsigned>(row0);  // the launcher keeps rows below 2^31
@@ -291,6 +330,11 @@ __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const
                     ov[g][u] = *reinterpret_cast<const u32x4 *>(po + sl * o_step);
                 }
             }
+            if (it0 + G >= ITEMS) {  // the last round of loads
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+                __builtin_amdgcn_sched_barrier(0);
+                on_arrival();
+            }
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 const int idx = tid + (it0 + g) * NT;
@@ -322,6 +366,8 @@ __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const
         }
         return;
     }
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    on_arrival();
     for (int idx = tid; idx < TR * CPR; idx += NT) {
         const int r = idx / CPR, ch = idx % CPR;
         u32x4 packed = {0u, 0u, 0u, 0u};
@@ -548,7 +594,8 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
         wait_all_loads();
         __syncthreads();
     }
-    w_b.start(static_cast<const T *>(P.w_qkv), nblk, lane);  // q columns
+    constexpr bool kWhole = WeightStream<T, D, NB, TR>::kWhole;
+    if (!kWhole) w_b.start(static_cast<const T *>(P.w_qkv), nblk, lane);  // q columns
     float gam[NB][VB], bet[NB][VB];
     load_cols<T, NB, TR>(vecs + kVecG1 * vec_ld, nblk, hb, gam);
     load_cols<T, NB, TR>(vecs + kVecB1 * vec_ld, nblk, hb, bet);
@@ -556,7 +603,9 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
     // ---- y = LN1(x + x W_fo^T)
     {
         typename TL::acc_t acc[NB];
-        w_a.run(acc, a0, LD, c, hb);
+        w_a.run(acc, a0, LD, c, hb, [&]() {
+            if (kWhole) w_b.start(static_cast<const T *>(P.w_qkv), nblk, lane);  // q columns
+        });
         float v[NB][VB];
 #pragma unroll
         for (int b = 0; b < NB; ++b)
@@ -577,14 +626,15 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
 #pragma unroll
     for (int part = 0; part < 3; ++part) {
         WeightStream<T, D, NB, TR> &cur = (part & 1) ? w_a : w_b, &nxt = (part & 1) ? w_b : w_a;
-        if (part < 2) {
-            int nb2[NB];
-#pragma unroll
-            for (int b = 0; b < NB; ++b) nb2[b] = (part + 1) * (D / TL::kBlock) + nblk[b];
-            nxt.start(static_cast<const T *>(P.w_qkv), nb2, lane);
-        }
         typename TL::acc_t acc[NB];
-        cur.run(acc, a1, LD, c, hb);
+        cur.run(acc, a1, LD, c, hb, [&]() {
+            if (part < 2) {
+                int nb2[NB];
+#pragma unroll
+                for (int b = 0; b < NB; ++b) nb2[b] = (part + 1) * (D / TL::kBlock) + nblk[b];
+                nxt.start(static_cast<const T *>(P.w_qkv), nb2, lane);
+            }
+        });
         if (part) __syncthreads();  // the previous pass has been copied out of a0
 #pragma unroll
         for (int b = 0; b < NB; ++b)
@@ -614,12 +664,9 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_pre_kernel(FusedPre
 // output, finally the finished tile (row stride D + 8); a1: y tile, then x1 = LN2(...).  With
 // WRITE_OUT the tile is stored to P.out; otherwise it is left in a0, synchronised, for the
 // caller (the next layer's pre body).
-struct NoHook {
-    __device__ __forceinline__ void operator()() const {}
-};
-
-// `before_last` runs right ahead of the last product (two of the three weight streams are
-// dead by then): the fused layer boundary uses it to request the next layer's first weights.
+// `before_last` runs when the last product's weights have arrived (two of the three weight
+// streams are dead by then): the fused layer boundary uses it to request the next layer's first
+// weights.
 template <typename T, int D, int F, int TR, bool WRITE_OUT, typename Hook>
 __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0, T *a1, float *red_a, float *red_b,
                                                 long row0, int valid, Hook before_last, T *vecs, int vec_ld) {
@@ -653,18 +700,30 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
     dma_vector<T, D, NT>(vecs + kVecG3 * vec_ld, P.g3, tid, 3);
     dma_vector<T, D, NT>(vecs + kVecB3 * vec_ld, P.b3, tid, 4);
     dma_vector<T, D, NT>(vecs + kVecBias2 * vec_ld, P.bias_2, tid, 5);
+    // whole-matrix streams follow the request-on-arrival rule of WeightStream
+    constexpr bool kWhole = WeightStream<T, D, NBD, TR>::kWhole && WeightStream<T, D, NBF, TR>::kWhole &&
+                            WeightStream<T, F, NBD, TR>::kWhole;
     // the first weights travel while the partials are waited for, fetched and merged
-    w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
+    if (kWhole) w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
     if (P.part_o) {
         if (P.order_wait) {  // the buffer pass's partial comes from the other queue
             if (tid == 0) order_wait_device(P.order_wait, 0, P.order_limit);
             __syncthreads();
         }
-        stage_merged_attention<T, D, NT, TR>(a0, LDD, P, row0, valid, tid);
+        stage_merged_attention<T, D, NT, TR>(a0, LDD, P, row0, valid, tid, [&]() {
+            if (kWhole && ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane);
+        });
+        if (!kWhole) {
+            w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
+            wait_all_loads();
+        }
+    } else {
+        if (!kWhole) w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
+        wait_all_loads();
+        if (kWhole && ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane);
     }
-    wait_all_loads();
     __syncthreads();
-    if (ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane);
+    if (!kWhole && ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane);
 
     // ---- x1 = LN2(y + attn W_o^T); each lane replaces exactly the y entries it read
     {
@@ -672,8 +731,15 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
         load_cols<T, NBD, TR>(vecs + kVecG2 * vec_ld, nbd, hb, gam);
         load_cols<T, NBD, TR>(vecs + kVecB2 * vec_ld, nbd, hb, bet);
         typename TL::acc_t acc[NBD];
-        w_o.run(acc, a0, LDD, c, hb);
-        w_2.start(static_cast<const T *>(P.w_2), nbd, lane);
+        {   // W_o arrived with the prologue; W_1 is on its way and must not be waited for here
+            WeightStream<T, D, NBD, TR> &w = w_o;
+#pragma unroll
+            for (int b = 0; b < NBD; ++b)
+#pragma unroll
+                for (int q = 0; q < TL::kVals; ++q) acc[b][q] = 0.f;
+            w.multiply(acc, a0, LDD, c, hb);
+        }
+        if (!kWhole) w_2.start(static_cast<const T *>(P.w_2), nbd, lane);
         float v[NBD][VB];
 #pragma unroll
         for (int b = 0; b < NBD; ++b)
@@ -693,7 +759,9 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
         float bias[NBF][VB];
         load_cols<T, NBF, TR>(vecs + kVecBias1 * vec_ld, nbf, hb, bias);
         typename TL::acc_t acc[NBF];
-        w_1.run(acc, a1, LDD, c, hb);
+        w_1.run(acc, a1, LDD, c, hb, [&]() {
+            if (kWhole) w_2.start(static_cast<const T *>(P.w_2), nbd, lane);
+        });
 #pragma unroll
         for (int b = 0; b < NBF; ++b)
 #pragma unroll
@@ -706,6 +774,8 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
                 }
                 store4f<T>(a0 + c * LDF + TL::col(nbf[b], g, hb), o[0], o[1], o[2], o[3]);
             }
+    } else if (kWhole) {
+        w_2.start(static_cast<const T *>(P.w_2), nbd, lane);
     }
     float gam[NBD][VB], bet[NBD][VB], bias[NBD][VB];
     load_cols<T, NBD, TR>(vecs + kVecG3 * vec_ld, nbd, hb, gam);
@@ -715,9 +785,8 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
 
     // ---- out = LN3(x1 + h W_2^T + b_2), staged through a0 for row-contiguous stores
     {
-        before_last();
         typename TL::acc_t acc[NBD];
-        w_2.run(acc, a0, LDF, c, hb);
+        w_2.run(acc, a0, LDF, c, hb, before_last);
         float v[NBD][VB];
 #pragma unroll
         for (int b = 0; b < NBD; ++b)
