@@ -12,12 +12,12 @@
 // Each queue advances its own counter behind the producing kernel — with a one-thread "signal"
 // launch, or by the first thread of the next kernel of that queue (the context pass does this for
 // the main queue): on an in-order queue the producer has finished and released its writes before
-// either starts, so a relaxed increment is enough and the producer itself pays nothing.  (Signalling
-// from inside the producer was tried and lost: every workgroup has to write back its XCD's L2
-// before it may count itself in, which cost more than the launch it saved.)  A queue waits for the
-// other one with a one-wavefront "gate" launch placed in front of the consumer.  The counters only ever grow and every step advances both by the same amount,
-// so a gate needs no argument that changes from step to step and the launches can be recorded in a
-// graph:
+// either starts, so a relaxed increment is enough and the producer itself pays nothing.
+// (Signalling from inside the producer was tried and lost: every workgroup has to write back its
+// XCD's L2 before it may count itself in, which cost more than the launch it saved.)  A queue
+// waits for the other one with a one-wavefront "gate" launch placed in front of the consumer.
+// The counters only ever grow and every step advances both by the same amount, so a gate needs no
+// argument that changes from step to step and the launches can be recorded in a graph:
 //
 //   side gate:  wait until ready[main] >= ready[side] + 1   (queries of my next buffer pass exist)
 //   main gate:  wait until ready[side] >= ready[main]       (every buffer pass asked for is done)
@@ -26,11 +26,13 @@
 // need to get onto the chip.  A gate launch is one wavefront with a handful of registers and is
 // always safe.  A consumer may also wait inside its own workgroups (order_wait_device, one launch
 // less on its queue) when its grid leaves at least half of the compute units free of them, so
-// that the other queue's kernel can always be placed; the host decides.  Every wait is bounded: after `limit_ticks` of the 100 MHz wall
-// clock a gate gives up, records it in `failed`, and lets its queue continue (the results are then
-// wrong and the host must discard them); once `failed` is set every later gate falls through at
-// once, so a broken schedule (both "queues" mapped to one hardware queue, a tool that serialises
-// launches) costs one time limit in all.
+// that the other queue's kernel can always be placed; the host decides.
+//
+// Every wait is bounded: after `limit_ticks` of the 100 MHz wall clock a gate gives up, records it
+// in `failed`, and lets its queue continue (the results are then wrong and the host must discard
+// them); once `failed` is set every later gate falls through at once, so a broken schedule (both
+// "queues" mapped to one hardware queue, a tool that serialises launches) costs one time limit in
+// all.
 #pragma once
 
 #include "common.h"
