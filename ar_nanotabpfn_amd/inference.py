@@ -81,6 +81,9 @@ class ARTabPFNPredictor:
         # two events per layer (``attention_kernels.QueueOrder``); used when the two streams are found
         # to run concurrently, otherwise (and when set to False) the events are used.
         self.counter_ordering = True
+        # In the sampling loop the last layer finishes the target row only: the buffer row's output
+        # of that layer is read by nobody (its K/V were cached before the attention call).
+        self.target_only_last_layer = True
         self._side_streams = {}
         self._graph_state = None
 
@@ -154,19 +157,27 @@ class ARTabPFNPredictor:
 
     # ------------------------------------------------------------------ the layer stack
 
-    def _run_layers(self, x_row: Tensor, attend) -> Tensor:
+    def _run_layers(self, x_row: Tensor, attend, last_layer_rows: Optional[slice] = None) -> Tensor:
         """``x_row [B,N,D]`` through every layer; ``attend(layer, q, k, v) -> [B,H,N,Dh]`` is the
         row attention of the pass at hand (it also owns the cache writes).  Between two
         attention calls the tail of one layer and the head of the next run as one launch where
-        the fused kernels cover them (``TwoStageTransformerLayer.finish_then_pre``)."""
+        the fused kernels cover them (``TwoStageTransformerLayer.finish_then_pre``).
+
+        ``last_layer_rows`` names the rows whose output the caller will read.  A row's output of
+        the last layer feeds nothing but that read (its K/V for the caches come from the
+        projection in front of the attention call, which still sees every row), so the last layer
+        runs its queries and everything behind them for those rows only; the result is then
+        ``[B, len(rows), D]``.  A decode step reads the target row alone (inference.py:318-320):
+        half the queries of the last context pass."""
         layers = list(self.backbone.layers)
         state = layers[0].pre_attention(x_row)
         for idx, layer in enumerate(layers):
             y, q, k, v = state
-            attn = attend(layer, q, k, v)
             if idx + 1 == len(layers):
-                return layer.finish(y, attn)
-            state = layer.finish_then_pre(y, attn, layers[idx + 1])
+                if last_layer_rows is not None:
+                    y, q = y[:, last_layer_rows], q[:, :, last_layer_rows]
+                return layer.finish(y, attend(layer, q, k, v))
+            state = layer.finish_then_pre(y, attend(layer, q, k, v), layers[idx + 1])
 
     # ------------------------------------------------------------------ prefill
 
@@ -244,17 +255,19 @@ class ARTabPFNPredictor:
                               chain: int = 0, order=None) -> Tensor:
         """The attention call of a shared-layout decode step (inference.py:785-823).  ``rows``
         restricts it to a group of trajectories (a slice of the batch axis of the buffer cache)."""
-        N = q.shape[2]
+        # k_new / v_new hold every new row of the step — [target] or [buffer, target] — even when q
+        # has been cut down to the rows whose output is read
+        has_buffer_row = k_new.shape[2] == 2
         k_ctx = layer.k_ctx_cache[:, : self.context_len]
         v_ctx = layer.v_ctx_cache[:, : self.context_len]
         k_buf = layer.k_buf_cache if rows is None else layer.k_buf_cache[rows]
         v_buf = layer.v_buf_cache if rows is None else layer.v_buf_cache[rows]
         # with a device-side length the host value is only the bound that is validated
-        n_buf = self.buffer_len if n_buf_device is None else self.max_buffer_len - (N - 1)
+        n_buf = self.buffer_len if n_buf_device is None else self.max_buffer_len - (1 if has_buffer_row else 0)
         side = self._side_stream(q.device, chain) if self.overlap_buffer_pass else None
         # where the layer's fused kernel can merge the partial results itself, leave them unmerged
         partials = self.merge_in_layer and layer.fused_for(q)
-        if N == 1:
+        if not has_buffer_row:
             attn = ak.decode_attention(q, k_ctx, v_ctx, k_buf, v_buf, n_buf,
                                        n_buf_device=n_buf_device, side_stream=side, leave_partials=partials)
         else:
@@ -364,7 +377,8 @@ class ARTabPFNPredictor:
             x_row = self._run_layers(
                 st.emb, lambda layer, q, k, v: self._attend_decode_shared(layer, q, k, v, n_buf_device=st.nbuf,
                                                                           rows=st.rows, chain=st.chain,
-                                                                          order=st.order_active))
+                                                                          order=st.order_active),
+                last_layer_rows=self._last_layer_rows())
             st.tail(x_row)          # norm, head, draw, preds[:, t], embedding of step t + 1, (t, nbuf) += 1
             return
         bs = self.ar_tokens.shape[0]
@@ -377,12 +391,17 @@ class ARTabPFNPredictor:
         x_row = self._run_layers(
             x_row, lambda layer, q, k, v: self._attend_decode_shared(layer, q, k, v, n_buf_device=st.nbuf,
                                                                       rows=st.rows, chain=st.chain,
-                                                                      order=st.order_active))
+                                                                      order=st.order_active),
+            last_layer_rows=self._last_layer_rows())
         z = add_layer_norm(x_row, None, None, self.backbone.norm)
         y = self.head.sample(z[:, -1:, :])[:, :, 0, 0]
         st.preds.index_copy_(1, t, y)
         st.y_prev.copy_(y)
         st.counters.add_(1)
+
+    def _last_layer_rows(self) -> Optional[slice]:
+        """Rows of a ``[buffer, target]`` step that the last layer has to finish: the target."""
+        return slice(1, 2) if self.target_only_last_layer else None
 
     def _chain_rows(self, B: int):
         """Batch slices of the trajectory groups that are sampled side by side."""
@@ -401,7 +420,8 @@ class ARTabPFNPredictor:
         chain_rows = self._chain_rows(B)
         key = (B, Nt, F_, self.context_len, dtype, str(device), layer0.k_ctx_cache.data_ptr(),
                layer0.k_buf_cache.data_ptr(), self.fuse_step_tail, self.overlap_buffer_pass, self.merge_in_layer,
-               len(chain_rows), int(self.steps_per_graph), bool(self.counter_ordering), tuple((p.data_ptr(), p._version) for p in params))
+               len(chain_rows), int(self.steps_per_graph), bool(self.counter_ordering),
+               bool(self.target_only_last_layer), tuple((p.data_ptr(), p._version) for p in params))
         gs = self._graph_state
         if gs is None or gs.key != key:
             gs = _GraphState()

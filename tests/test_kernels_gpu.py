@@ -151,6 +151,7 @@ def _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, use_mfma,
         (8, 4, 2, 64, 32, 5, 16, True),
         (8, 4, 2, 64, 32, 15, 16, True),  # last slot
         (8, 4, 1, 64, 32, 7, 16, False),  # target only over committed buffers
+        (8, 4, 1, 64, 32, 6, 16, True),   # target query alone, with the step's buffer row appended (last layer of a step)
         (33, 8, 2, 100, 64, 19, 64, True),
         (5, 2, 2, 300, 128, 70, 80, True),
         (4, 3, 2, 50, 16, 9, 12, True),  # portable-only head_dim
@@ -169,6 +170,8 @@ def test_decode_attention_matches_oracle(device, dtype, use_mfma, B, H, Lq, Nc, 
         (8, 4, 2, 64, 32, 3, 16, True),   # exactly one 4-key chunk
         (8, 4, 2, 64, 32, 15, 16, True),  # last slot
         (8, 4, 1, 64, 32, 7, 16, False),  # target only over committed buffers, ragged last chunk
+        (8, 4, 1, 64, 32, 6, 16, True),   # target query alone, buffer row appended by the streaming pass
+        (70, 8, 1, 4096, 32, 11, 16, True),  # the same with a split context
         (5, 3, 2, 200, 32, 22, 40, True),  # 15 pairs: one ragged task
         (33, 8, 2, 100, 64, 19, 64, True),  # other head dims: register-staged buffer pass
         (5, 2, 2, 300, 128, 70, 80, True),

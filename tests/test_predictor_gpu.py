@@ -590,3 +590,36 @@ def test_graph_sampling_falls_back_to_events_when_a_counter_wait_times_out(devic
     torch.manual_seed(3)
     y_again = pred.sample_sequence(xc, yc, xt)
     assert torch.equal(y_ref, y_again)
+
+
+def test_graph_sampling_target_only_last_layer_changes_nothing_that_is_read(device):
+    """The sampling loop lets the last layer finish the target row only.  Against the same loop
+    with both rows finished: predictions agree to bf16 rounding (the target query of the last
+    context pass is tiled and split differently when it stands alone) and the caches — which
+    take the buffer row's K/V from in front of the attention call — are the same in every layer
+    but for the propagation of those roundings through the next step's buffer row."""
+    from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
+
+    cfg = dict(d_model=128, n_heads=4, n_layers=3, d_ff=128, num_features=3, buffer_size=5, num_components=4)
+    model = _build(cfg, device, dtype=torch.bfloat16)
+    B, Nc, Nt = 70, 2100, 9
+    g = torch.Generator().manual_seed(8)
+    xc = torch.randn(1, Nc, 3, generator=g).expand(B, -1, -1).to(device, torch.bfloat16)
+    yc = torch.randn(1, Nc, generator=g).expand(B, -1).to(device, torch.bfloat16)
+    xt = torch.randn(B, Nt, 3, generator=g).to(device, torch.bfloat16)
+    results = {}
+    for cut in (False, True):
+        pred = ARTabPFNPredictor.from_trained_model(model, backend="triton_shared_context")
+        pred.target_only_last_layer = cut
+        torch.manual_seed(21)
+        y = pred.sample_sequence(xc, yc, xt)
+        results[cut] = (y, [(l.k_buf_cache.clone(), l.v_buf_cache.clone()) for l in model.backbone.layers])
+    (y0, c0), (y1, c1) = results[False], results[True]
+    assert y1.shape == (B, Nt) and torch.isfinite(y1).all()
+    # step 1 (first replayed step) starts from identical state: only the last context pass differs
+    assert max_abs(to_np(y0[:, :2]), to_np(y1[:, :2])) <= 2e-2
+    # later steps feed earlier samples back; a sampled value moves with the rounding of its mean
+    assert max_abs(to_np(y0), to_np(y1)) <= 0.25
+    for (k0, v0), (k1, v1) in zip(c0, c1):
+        assert max_abs(to_np(k0[:, :, :1]), to_np(k1[:, :, :1])) <= 2e-2  # the row appended by step 1
+        assert max_abs(to_np(v0[:, :, :1]), to_np(v1[:, :, :1])) <= 2e-2
