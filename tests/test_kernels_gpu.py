@@ -229,9 +229,9 @@ def test_decode_attention_overlapped_device_length_in_graph(device):
 def _full_size_decode(device, B, H, Nc, n_buf, cap, seed):
     """One decode step at a BASELINE shape (Dh=32, Lq=2, bf16).  Inputs are drawn on the device
     (the buffer cache alone is up to 0.5 GB); the oracle sees a sample of the trajectories, every
-    head of them; the cache is compared whole and bit-exact; the three schedules of the step
-    (buffer pass after the context pass, beside it, merge left to the caller) must agree on every
-    row to within the rounding of the 16-bit partial outputs."""
+    head of them; the cache is compared whole and bit-exact; the schedules of the step (buffer
+    pass after the context pass, beside it, merge left to the caller, streams ordered by counters)
+    must agree on every row to within the rounding of the 16-bit partial outputs."""
     ak = _ak()
     dtype, D, Lq = torch.bfloat16, 32, 2
     g = torch.Generator(device=device).manual_seed(seed)
@@ -259,6 +259,22 @@ def _full_size_decode(device, B, H, Nc, n_buf, cap, seed):
         outs.append(out.float())
     for other in outs[1:]:
         assert float((outs[0] - other).abs().max()) <= 2e-2
+    # fourth schedule: the two streams ordered by device-side counters (one fork, one join) —
+    # the same launches as the third, so the merged result must be the same bit for bit
+    main = torch.cuda.current_stream(device)
+    side2, concurrent = ak.concurrent_stream(device, main)
+    if concurrent:
+        order = ak.QueueOrder(device)
+        kc, vc = k_cache.clone(), v_cache.clone()
+        side2.wait_stream(main)
+        parts = ak.decode_attention(q, k_ctx, v_ctx, kc, vc, n_buf, k_new, v_new, side_stream=side2,
+                                    leave_partials=True, order=order)
+        out = parts.merged()
+        main.wait_stream(side2)
+        torch.cuda.synchronize()
+        assert order.failed() == 0
+        assert torch.equal(kc, exp_k) and torch.equal(vc, exp_v)
+        assert torch.equal(out.float(), outs[2])
 
     sample = sorted({0, 1, B // 2 - 1, B // 2, B - 2, B - 1, (7 * seed + 13) % B, (31 * seed + 5) % B})
     idx = torch.tensor(sample, device=device)
