@@ -904,17 +904,61 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
     WeightStream<T, F, NB2, TR> w_2;
     if (ff_active) w_1.start(static_cast<const T *>(P.w_h1), nbf, lane);
     if (wave == 0) w_2.start(static_cast<const T *>(P.w_h2), nb0, lane);
+    // Everything small that a later phase reads from memory is requested here, in one round trip
+    // with the weights and the input tile: fetched where it is used, each costs its phase (all far
+    // shorter than a memory access) a round trip of its own.
+    float gam[EPL], bet[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+        gam[e] = to_f32(static_cast<const T *>(P.norm_g)[lane * EPL + e]);
+        bet[e] = to_f32(static_cast<const T *>(P.norm_b)[lane * EPL + e]);
+    }
+    float bias1[NBF][VB], bias2[NB2][VB];
+    if (ff_active)
+        load_cols<T, NBF, TR>(P.b_h1 ? static_cast<const T *>(P.b_h1) : reinterpret_cast<const T *>(kZeroVector), nbf,
+                              hb, bias1);
+    if (wave == 0)
+        load_cols<T, NB2, TR>(P.b_h2 ? static_cast<const T *>(P.b_h2) : reinterpret_cast<const T *>(kZeroVector), nb0,
+                              hb, bias2);
+    float my_u = 0.f, my_n = 0.f;  // this trajectory's variates (threads 0 .. valid-1)
+    if (tid < valid) {
+        my_u = P.rand_u[static_cast<long>(t) * P.B + row0 + tid];
+        my_n = P.rand_n[static_cast<long>(t) * P.B + row0 + tid];
+    }
+    // the model vectors of the embedding: a thread handles the same 8 columns in every item
+    constexpr int CPR_E = D / 8;
+    const int ch_e = tid % CPR_E;
+    static_assert(NT % CPR_E == 0, "a thread's embedding items share their column chunk");
+    u32x4 e_wx, e_bx, e_wy, e_by, e_mb, e_mt, e_tok;
+    {
+        const T *tok = static_cast<const T *>(P.ar_tokens) + static_cast<long>((t + 1) % P.bs) * D;
+        const T *mk = static_cast<const T *>(P.markers);
+        e_wx = *reinterpret_cast<const u32x4 *>(static_cast<const T *>(P.w_x) + 8 * ch_e);
+        e_bx = *reinterpret_cast<const u32x4 *>(static_cast<const T *>(P.b_x) + 8 * ch_e);
+        e_wy = *reinterpret_cast<const u32x4 *>(static_cast<const T *>(P.w_y) + 8 * ch_e);
+        e_by = *reinterpret_cast<const u32x4 *>(static_cast<const T *>(P.b_y) + 8 * ch_e);
+        e_mb = *reinterpret_cast<const u32x4 *>(mk + 2 * D + 8 * ch_e);  // marker "buffer"
+        e_mt = *reinterpret_cast<const u32x4 *>(mk + 8 * ch_e);          // marker "target"
+        e_tok = *reinterpret_cast<const u32x4 *>(tok + 8 * ch_e);
+    }
+    constexpr int E_ITEMS = TR * 2 * CPR_E / NT;  // (trajectory, row, 8-column chunk) items per thread
+    static_assert(TR * 2 * CPR_E % NT == 0, "whole embedding items per thread");
+    float e_xv[E_ITEMS];  // feature mean of the row an item embeds: x_t for the buffer row, x_{t+1} for the target row
+    {
+        const T *xm = static_cast<const T *>(P.x_mean);
+        const int tn = min(t + 1, P.Nt - 1);
+#pragma unroll
+        for (int k = 0; k < E_ITEMS; ++k) {
+            const int idx = tid + k * NT;
+            const int which = (idx / CPR_E) & 1, r = idx / (2 * CPR_E);
+            e_xv[k] = r < valid ? to_f32(xm[(row0 + r) * P.Nt + (which == 0 ? t : tn)]) : 0.f;
+        }
+    }
     stage_tile<T, D, NT, TR>(a0, LDD, static_cast<const T *>(P.x_last) + row0 * P.ld_row, P.ld_row, valid, tid);
     __syncthreads();
 
     // ---- z = LayerNorm(x_last), one wavefront per row, in place
     {
-        float gam[EPL], bet[EPL];
-#pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-            gam[e] = to_f32(static_cast<const T *>(P.norm_g)[lane * EPL + e]);
-            bet[e] = to_f32(static_cast<const T *>(P.norm_b)[lane * EPL + e]);
-        }
         for (int r = wave; r < TR; r += NW) {
             T *row = a0 + r * LDD + lane * EPL;
             float x[EPL], sum = 0.f;
@@ -936,9 +980,6 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
 
     // ---- h = gelu(z W_h1^T + b_h1) -> a1
     if (ff_active) {
-        float bias[NBF][VB];
-        load_cols<T, NBF, TR>(P.b_h1 ? static_cast<const T *>(P.b_h1) : reinterpret_cast<const T *>(kZeroVector), nbf,
-                              hb, bias);
         typename TL::acc_t acc[NBF];
         w_1.run(acc, a0, LDD, c, hb);
 #pragma unroll
@@ -948,7 +989,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
                 float o[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const float v = acc[b][4 * g + e] + bias[b][4 * g + e];
+                    const float v = acc[b][4 * g + e] + bias1[b][4 * g + e];
                     o[e] = 0.5f * v * (1.f + erff(v * 0.70710678118654752f));
                 }
                 store4f<T>(a1 + c * LDF + TL::col(nbf[b], g, hb), o[0], o[1], o[2], o[3]);
@@ -958,9 +999,6 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
 
     // ---- raw = h W_h2^T + b_h2 (32 output columns, first wavefront), kept in float32
     if (wave == 0) {
-        float bias[NB2][VB];
-        load_cols<T, NB2, TR>(P.b_h2 ? static_cast<const T *>(P.b_h2) : reinterpret_cast<const T *>(kZeroVector), nb0,
-                              hb, bias);
         typename TL::acc_t acc[NB2];
         w_2.run(acc, a1, LDF, c, hb);
 #pragma unroll
@@ -969,7 +1007,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
             for (int g = 0; g < GB; ++g)
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    raw_s[c][TL::col(b, g, hb) + e] = acc[b][4 * g + e] + bias[b][4 * g + e];
+                    raw_s[c][TL::col(b, g, hb) + e] = acc[b][4 * g + e] + bias2[b][4 * g + e];
     }
     __syncthreads();
 
@@ -994,7 +1032,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
                     logit[k] = expf(logit[k] - mx);
                     z += logit[k];
                 }
-            const float target = P.rand_u[static_cast<long>(t) * P.B + row] * z;
+            const float target = my_u * z;
             int comp = P.K - 1;
             float cum = 0.f;
             bool found = false;
@@ -1011,7 +1049,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
             const float sraw = raw_s[tid][3 * comp + 1] + to_f32(sb[comp]);
             const float sp = sraw > 20.f ? sraw : log1pf(expf(sraw));
             const float sd = fminf(sp, P.std_max) + P.std_min;
-            const T yr = from_f32<T>(mean + sd * P.rand_n[static_cast<long>(t) * P.B + row]);
+            const T yr = from_f32<T>(mean + sd * my_n);
             static_cast<T *>(P.preds)[row * P.Nt + t] = yr;
             y = to_f32(yr);
         }
@@ -1021,38 +1059,27 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
 
     // ---- embedding of step t + 1: row 0 = buffer(x_t, y_t) + ar_token[(t + 1) % bs], row 1 = target(x_{t+1})
     {
-        const T *wx = static_cast<const T *>(P.w_x), *bx = static_cast<const T *>(P.b_x);
-        const T *wy = static_cast<const T *>(P.w_y), *by = static_cast<const T *>(P.b_y);
-        const T *mk = static_cast<const T *>(P.markers);
-        const T *tok = static_cast<const T *>(P.ar_tokens) + static_cast<long>((t + 1) % P.bs) * D;
-        const T *xm = static_cast<const T *>(P.x_mean);
-        const int tn = min(t + 1, P.Nt - 1);
-        constexpr int CPR = D / 8;
-        for (int idx = tid; idx < TR * 2 * CPR; idx += NT) {
-            const int ch = idx % CPR, which = (idx / CPR) & 1, r = idx / (2 * CPR);
+        float fwx[8], fbx[8], fwy[8], fby[8], fmb[8], fmt[8], ftk[8];
+        unpack8<T>(e_wx, fwx); unpack8<T>(e_bx, fbx); unpack8<T>(e_wy, fwy); unpack8<T>(e_by, fby);
+        unpack8<T>(e_mb, fmb); unpack8<T>(e_mt, fmt); unpack8<T>(e_tok, ftk);
+#pragma unroll
+        for (int k = 0; k < E_ITEMS; ++k) {
+            const int idx = tid + k * NT;
+            const int which = (idx / CPR_E) & 1, r = idx / (2 * CPR_E);
             if (r >= valid) continue;
             const long row = row0 + r;
-            float fwx[8], fbx[8], o[8];
-            load4f<T>(wx + 8 * ch, fwx); load4f<T>(wx + 8 * ch + 4, fwx + 4);
-            load4f<T>(bx + 8 * ch, fbx); load4f<T>(bx + 8 * ch + 4, fbx + 4);
+            const float xv = e_xv[k];
+            float o[8];
             if (which == 0) {
-                const float xv = to_f32(xm[row * P.Nt + t]), yv = y_s[r];
-                float fwy[8], fby[8], fm[8], ft[8];
-                load4f<T>(wy + 8 * ch, fwy); load4f<T>(wy + 8 * ch + 4, fwy + 4);
-                load4f<T>(by + 8 * ch, fby); load4f<T>(by + 8 * ch + 4, fby + 4);
-                load4f<T>(mk + 2 * D + 8 * ch, fm); load4f<T>(mk + 2 * D + 8 * ch + 4, fm + 4);
-                load4f<T>(tok + 8 * ch, ft); load4f<T>(tok + 8 * ch + 4, ft + 4);
+                const float yv = y_s[r];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) o[e] = xv * fwx[e] + fbx[e] + yv * fwy[e] + fby[e] + fm[e] + ft[e];
+                for (int e = 0; e < 8; ++e) o[e] = xv * fwx[e] + fbx[e] + yv * fwy[e] + fby[e] + fmb[e] + ftk[e];
             } else {
-                const float xv = to_f32(xm[row * P.Nt + tn]);
-                float fm[8];
-                load4f<T>(mk + 8 * ch, fm); load4f<T>(mk + 8 * ch + 4, fm + 4);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) o[e] = xv * fwx[e] + fbx[e] + fm[e];
+                for (int e = 0; e < 8; ++e) o[e] = xv * fwx[e] + fbx[e] + fmt[e];
             }
             u32x4 val = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
-            *reinterpret_cast<u32x4 *>(static_cast<T *>(P.emb) + (row * 2 + which) * D + 8 * ch) = val;
+            *reinterpret_cast<u32x4 *>(static_cast<T *>(P.emb) + (row * 2 + which) * D + 8 * ch_e) = val;
         }
     }
 
