@@ -150,6 +150,7 @@ struct Tile<T, 16> {
 
 struct NoHook {
     __device__ __forceinline__ void operator()() const {}
+    __device__ __forceinline__ void operator()(int) const {}
 };
 
 // One transposed product: acc[b][v] = sum_k W[32*nblk[b] + row(v)][k] * A[c][k] for NB blocks of
@@ -180,7 +181,32 @@ struct WeightStream {
     vec wf[PF][NB];
     int rot;  // contraction step this workgroup starts with
 
+    // start() = begin() + request(0 .. PF-1).  The requests of a wavefront are accepted at the pace
+    // of the CU's address unit (64 B/clk: 1 us for a 128 KiB matrix over the eight wavefronts) and
+    // the wavefront waits at each; run() can spread the requests of the NEXT stream over the steps
+    // of its own product (`per_step`), so that its MFMAs execute while the requests queue.
     __device__ __forceinline__ void start(const T *wp, const int (&nblk)[NB], int lane) {
+        begin(wp, nblk, lane);
+#pragma unroll
+        for (int p = 0; p < PF; ++p) request(p);
+        __builtin_amdgcn_sched_barrier(0);  // the prefetch stays where it was written
+    }
+
+    __device__ __forceinline__ void request(int p) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+            wf[p][b] = *reinterpret_cast<const vec *>(wl[b] + ((p + rot) & (KS - 1)) * TL::kStepStride);
+    }
+
+    // The requests that fall to step `ks` of a product of `n_steps` steps when this stream's PF
+    // requests are spread evenly over it.
+    __device__ __forceinline__ void request_share(int ks, int n_steps) {
+#pragma unroll
+        for (int p = 0; p < PF; ++p)
+            if (p * n_steps / PF == ks) request(p);
+    }
+
+    __device__ __forceinline__ void begin(const T *wp, const int (&nblk)[NB], int lane) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) wl[b] = wp + TL::weight_offset(nblk[b], K, lane);
         // Every workgroup streams the same matrix at about the same time, and the 16 of an XCD
@@ -189,32 +215,40 @@ struct WeightStream {
         // Workgroup ids are dealt round-robin over the 8 XCDs, so id / 8 counts within an XCD.
         static_assert((KS & (KS - 1)) == 0, "contraction steps must be a power of two");
         rot = (blockIdx.x >> 3) & (KS - 1);
-#pragma unroll
-        for (int p = 0; p < PF; ++p)
-#pragma unroll
-            for (int b = 0; b < NB; ++b)
-                wf[p][b] = *reinterpret_cast<const vec *>(wl[b] + ((p + rot) & (KS - 1)) * TL::kStepStride);
-        __builtin_amdgcn_sched_barrier(0);  // the prefetch stays where it was written
     }
 
-    template <typename Hook = NoHook>
+    // `on_arrival` runs once this stream's fragments are there (kWhole) — the place to begin() the
+    // next stream —, `per_step(ks)` behind the MFMAs of every contraction step — the place for the
+    // next stream's request_share(ks, KS).  For a stream deeper than its prefetch window both run
+    // up front, which is start() of the next stream ahead of this product.
+    template <typename Hook = NoHook, typename StepHook = NoHook>
     __device__ __forceinline__ void run(acc_t (&acc)[NB], const T *a_lds, int ld, int c, int hb,
-                                        Hook on_arrival = Hook{}) {
+                                        Hook on_arrival = Hook{}, StepHook per_step = StepHook{}) {
         if (kWhole) {
             __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // this stream is all that is in flight: it has arrived
             __builtin_amdgcn_sched_barrier(0);
         }
         on_arrival();
+        if (!kWhole) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) per_step(ks);
+            __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int b = 0; b < NB; ++b)
 #pragma unroll
             for (int v = 0; v < TL::kVals; ++v) acc[b][v] = 0.f;
-        multiply(acc, a_lds, ld, c, hb);
+        if (kWhole)
+            multiply(acc, a_lds, ld, c, hb, per_step);
+        else
+            multiply(acc, a_lds, ld, c, hb);
     }
 
     // acc += W A^T over the whole contraction, without waiting for anything but the fragments used
     // (a matrix deeper than the prefetch window is requested step by step as fragments are used up)
-    __device__ __forceinline__ void multiply(acc_t (&acc)[NB], const T *a_lds, int ld, int c, int hb) {
+    template <typename StepHook = NoHook>
+    __device__ __forceinline__ void multiply(acc_t (&acc)[NB], const T *a_lds, int ld, int c, int hb,
+                                             StepHook per_step = StepHook{}) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             const vec af =
@@ -227,6 +261,7 @@ struct WeightStream {
                     wf[ks % PF][b] =
                         *reinterpret_cast<const vec *>(wl[b] + ((ks + PF + rot) & (KS - 1)) * TL::kStepStride);
             }
+            per_step(ks);
         }
     }
 };
@@ -603,9 +638,9 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
     // ---- y = LN1(x + x W_fo^T)
     {
         typename TL::acc_t acc[NB];
-        w_a.run(acc, a0, LD, c, hb, [&]() {
-            if (kWhole) w_b.start(static_cast<const T *>(P.w_qkv), nblk, lane);  // q columns
-        });
+        w_a.run(acc, a0, LD, c, hb,
+                [&]() { if (kWhole) w_b.begin(static_cast<const T *>(P.w_qkv), nblk, lane); },  // q columns
+                [&](int ks) { if (kWhole) w_b.request_share(ks, WeightStream<T, D, NB, TR>::KS); });
         float v[NB][VB];
 #pragma unroll
         for (int b = 0; b < NB; ++b)
@@ -627,14 +662,18 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
     for (int part = 0; part < 3; ++part) {
         WeightStream<T, D, NB, TR> &cur = (part & 1) ? w_a : w_b, &nxt = (part & 1) ? w_b : w_a;
         typename TL::acc_t acc[NB];
-        cur.run(acc, a1, LD, c, hb, [&]() {
-            if (part < 2) {
-                int nb2[NB];
+        cur.run(acc, a1, LD, c, hb,
+                [&]() {
+                    if (part < 2) {
+                        int nb2[NB];
 #pragma unroll
-                for (int b = 0; b < NB; ++b) nb2[b] = (part + 1) * (D / TL::kBlock) + nblk[b];
-                nxt.start(static_cast<const T *>(P.w_qkv), nb2, lane);
-            }
-        });
+                        for (int b = 0; b < NB; ++b) nb2[b] = (part + 1) * (D / TL::kBlock) + nblk[b];
+                        nxt.begin(static_cast<const T *>(P.w_qkv), nb2, lane);
+                    }
+                },
+                [&](int ks) {
+                    if (part < 2) nxt.request_share(ks, WeightStream<T, D, NB, TR>::KS);
+                });
         if (part) __syncthreads();  // the previous pass has been copied out of a0
 #pragma unroll
         for (int b = 0; b < NB; ++b)
@@ -667,9 +706,10 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_pre_kernel(FusedPre
 // `before_last` runs when the last product's weights have arrived (two of the three weight
 // streams are dead by then): the fused layer boundary uses it to request the next layer's first
 // weights.
-template <typename T, int D, int F, int TR, bool WRITE_OUT, typename Hook>
+template <typename T, int D, int F, int TR, bool WRITE_OUT, typename Hook, typename StepHook>
 __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0, T *a1, float *red_a, float *red_b,
-                                                long row0, int valid, Hook before_last, T *vecs, int vec_ld) {
+                                                long row0, int valid, Hook before_last, StepHook last_steps, T *vecs,
+                                                int vec_ld) {
     typedef Tile<T, TR> TL;
     constexpr int NW = fused_waves(D), NT = NW * 64;
     constexpr int LDD = D + 8, LDF = F + 8;
@@ -759,9 +799,9 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
         float bias[NBF][VB];
         load_cols<T, NBF, TR>(vecs + kVecBias1 * vec_ld, nbf, hb, bias);
         typename TL::acc_t acc[NBF];
-        w_1.run(acc, a1, LDD, c, hb, [&]() {
-            if (kWhole) w_2.start(static_cast<const T *>(P.w_2), nbd, lane);
-        });
+        w_1.run(acc, a1, LDD, c, hb,
+                [&]() { if (kWhole) w_2.begin(static_cast<const T *>(P.w_2), nbd, lane); },
+                [&](int ks) { if (kWhole) w_2.request_share(ks, WeightStream<T, D, NBF, TR>::KS); });
 #pragma unroll
         for (int b = 0; b < NBF; ++b)
 #pragma unroll
@@ -786,7 +826,7 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
     // ---- out = LN3(x1 + h W_2^T + b_2), staged through a0 for row-contiguous stores
     {
         typename TL::acc_t acc[NBD];
-        w_2.run(acc, a0, LDF, c, hb, before_last);
+        w_2.run(acc, a0, LDF, c, hb, before_last, last_steps);
         float v[NBD][VB];
 #pragma unroll
         for (int b = 0; b < NBD; ++b)
@@ -815,7 +855,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_kernel(FusedPo
     const int valid = static_cast<int>(min(static_cast<long>(TR), P.rows - row0));
     constexpr int VW = D > F ? D : F;
     __shared__ __attribute__((aligned(16))) T vecs[kVecSlots * VW];
-    fused_post_body<T, D, F, TR, true>(P, a0, a1, red_a, red_b, row0, valid, NoHook{}, vecs, VW);
+    fused_post_body<T, D, F, TR, true>(P, a0, a1, red_a, red_b, row0, valid, NoHook{}, NoHook{}, vecs, VW);
 }
 
 // The post part of layer L and the pre part of layer L+1 on the same rows: the layer output
@@ -837,8 +877,9 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_pre_kernel(Fus
     constexpr int VW = D > F ? D : F;
     __shared__ __attribute__((aligned(16))) T vecs[kVecSlots * VW];
     stage_pre_vectors<T, D, NW * 64>(N, vecs, VW, threadIdx.x);  // visible after the first barrier below
-    fused_post_body<T, D, F, TR, false>(P, a0, a1, red_a, red_b, row0, valid,
-                                        [&]() { next_fo.start(static_cast<const T *>(N.w_fo), nblk, lane); }, vecs, VW);
+    fused_post_body<T, D, F, TR, false>(
+        P, a0, a1, red_a, red_b, row0, valid, [&]() { next_fo.begin(static_cast<const T *>(N.w_fo), nblk, lane); },
+        [&](int ks) { next_fo.request_share(ks, WeightStream<T, F, NB, TR>::KS); }, vecs, VW);
     fused_pre_body<T, D, TR, true>(N, a0, a1, red_a, red_b, row0, valid, next_fo, vecs, VW);
 }
 
