@@ -217,17 +217,15 @@ struct WeightStream {
         rot = (blockIdx.x >> 3) & (KS - 1);
     }
 
-    // `on_arrival` runs once this stream's fragments are there (kWhole) — the place to begin() the
-    // next stream —, `per_step(ks)` behind the MFMAs of every contraction step — the place for the
-    // next stream's request_share(ks, KS).  For a stream deeper than its prefetch window both run
-    // up front, which is start() of the next stream ahead of this product.
+    // `before` runs ahead of the product — the place to begin() a later stream —, `per_step(ks)`
+    // behind the MFMAs of every contraction step — the place for that stream's
+    // request_share(ks, KS); the fragment registers of step ks are free by then, so the later
+    // stream may be this very object (the matrix two ahead goes where the current one was).  For a
+    // stream deeper than its prefetch window both run up front, which is start() of the later
+    // stream ahead of this product.
     template <typename Hook = NoHook, typename StepHook = NoHook>
     __device__ __forceinline__ void run(acc_t (&acc)[NB], const T *a_lds, int ld, int c, int hb,
                                         Hook on_arrival = Hook{}, StepHook per_step = StepHook{}) {
-        if (kWhole) {
-            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // this stream is all that is in flight: it has arrived
-            __builtin_amdgcn_sched_barrier(0);
-        }
         on_arrival();
         if (!kWhole) {
 #pragma unroll
@@ -604,10 +602,11 @@ __device__ __forceinline__ void stage_pre_vectors(const FusedPreParams &P, T *ve
 template <typename T, int TR>
 constexpr int fused_blocks(int N, int NW) { return (N / Tile<T, TR>::kBlock + NW - 1) / NW; }
 
-template <typename T, int D, int TR, bool X_IN_LDS>
+template <typename T, int D, int TR, bool X_IN_LDS, bool Q_REQUESTED = false>
 __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T *a1, float *red_a, float *red_b,
                                                long row0, int valid,
                                                WeightStream<T, D, fused_blocks<T, TR>(D, fused_waves(D)), TR> &w_a,
+                                               WeightStream<T, D, fused_blocks<T, TR>(D, fused_waves(D)), TR> &w_b,
                                                T *vecs, int vec_ld) {
     typedef Tile<T, TR> TL;
     constexpr int NW = fused_waves(D), NT = NW * 64;
@@ -621,16 +620,23 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
 #pragma unroll
     for (int b = 0; b < NB; ++b) nblk[b] = wave + NW * b;
 
-    WeightStream<T, D, NB, TR> w_b;
-    if (!X_IN_LDS) {  // else requested by the caller already
+    // Weight order: W_fo (w_a), q (w_b), k (w_a again), v (w_b again).  With X_IN_LDS the caller has
+    // requested W_fo and, with Q_REQUESTED, the q weights already.
+    constexpr bool kWhole = WeightStream<T, D, NB, TR>::kWhole;
+    if (!X_IN_LDS) {
         w_a.start(static_cast<const T *>(P.w_fo), nblk, lane);
         dma_tile<T, D, NT, TR>(a0, LD, static_cast<const T *>(P.x) + row0 * P.ldx, P.ldx, valid, tid);
         stage_pre_vectors<T, D, NT>(P, vecs, vec_ld, tid);
         wait_all_loads();
         __syncthreads();
     }
-    constexpr bool kWhole = WeightStream<T, D, NB, TR>::kWhole;
-    if (!kWhole) w_b.start(static_cast<const T *>(P.w_qkv), nblk, lane);  // q columns
+    if (!Q_REQUESTED) w_b.start(static_cast<const T *>(P.w_qkv), nblk, lane);  // q columns
+    int nb_k[NB], nb_v[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        nb_k[b] = (D / TL::kBlock) + nblk[b];
+        nb_v[b] = 2 * (D / TL::kBlock) + nblk[b];
+    }
     float gam[NB][VB], bet[NB][VB];
     load_cols<T, NB, TR>(vecs + kVecG1 * vec_ld, nblk, hb, gam);
     load_cols<T, NB, TR>(vecs + kVecB1 * vec_ld, nblk, hb, bet);
@@ -638,9 +644,9 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
     // ---- y = LN1(x + x W_fo^T)
     {
         typename TL::acc_t acc[NB];
-        w_a.run(acc, a0, LD, c, hb,
-                [&]() { if (kWhole) w_b.begin(static_cast<const T *>(P.w_qkv), nblk, lane); },  // q columns
-                [&](int ks) { if (kWhole) w_b.request_share(ks, WeightStream<T, D, NB, TR>::KS); });
+        // whole-matrix streams: the k weights go where W_fo's fragments were, step by step
+        w_a.run(acc, a0, LD, c, hb, [&]() { if (kWhole) w_a.begin(static_cast<const T *>(P.w_qkv), nb_k, lane); },
+                [&](int ks) { if (kWhole) w_a.request_share(ks, WeightStream<T, D, NB, TR>::KS); });
         float v[NB][VB];
 #pragma unroll
         for (int b = 0; b < NB; ++b)
@@ -662,17 +668,22 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
     for (int part = 0; part < 3; ++part) {
         WeightStream<T, D, NB, TR> &cur = (part & 1) ? w_a : w_b, &nxt = (part & 1) ? w_b : w_a;
         typename TL::acc_t acc[NB];
+        // whole-matrix streams: the v weights follow the q weights through w_b during the q pass (k
+        // is on its way already); deeper ones: the next pass's weights ahead of this pass
         cur.run(acc, a1, LD, c, hb,
                 [&]() {
-                    if (part < 2) {
-                        int nb2[NB];
-#pragma unroll
-                        for (int b = 0; b < NB; ++b) nb2[b] = (part + 1) * (D / TL::kBlock) + nblk[b];
-                        nxt.begin(static_cast<const T *>(P.w_qkv), nb2, lane);
+                    if (kWhole) {
+                        if (part == 0) w_b.begin(static_cast<const T *>(P.w_qkv), nb_v, lane);
+                    } else if (part < 2) {
+                        nxt.begin(static_cast<const T *>(P.w_qkv), part == 0 ? nb_k : nb_v, lane);
                     }
                 },
                 [&](int ks) {
-                    if (part < 2) nxt.request_share(ks, WeightStream<T, D, NB, TR>::KS);
+                    if (kWhole) {
+                        if (part == 0) w_b.request_share(ks, WeightStream<T, D, NB, TR>::KS);
+                    } else if (part < 2) {
+                        nxt.request_share(ks, WeightStream<T, D, NB, TR>::KS);
+                    }
                 });
         if (part) __syncthreads();  // the previous pass has been copied out of a0
 #pragma unroll
@@ -695,21 +706,23 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_pre_kernel(FusedPre
     const long row0 = static_cast<long>(blockIdx.x) * TR;
     const int valid = static_cast<int>(min(static_cast<long>(TR), P.rows - row0));
     __shared__ __attribute__((aligned(16))) T vecs[kVecSlots * D];
-    WeightStream<T, D, fused_blocks<T, TR>(D, NW), TR> w_a;
-    fused_pre_body<T, D, TR, false>(P, a0, a1, red_a, red_b, row0, valid, w_a, vecs, D);
+    WeightStream<T, D, fused_blocks<T, TR>(D, NW), TR> w_a, w_b;
+    fused_pre_body<T, D, TR, false>(P, a0, a1, red_a, red_b, row0, valid, w_a, w_b, vecs, D);
 }
 
 // Body of the post kernel on one TR-row tile.  a0 (row stride max(D, F) + 8): attn tile, gelu
 // output, finally the finished tile (row stride D + 8); a1: y tile, then x1 = LN2(...).  With
 // WRITE_OUT the tile is stored to P.out; otherwise it is left in a0, synchronised, for the
 // caller (the next layer's pre body).
-// `before_last` runs when the last product's weights have arrived (two of the three weight
-// streams are dead by then): the fused layer boundary uses it to request the next layer's first
-// weights.
-template <typename T, int D, int F, int TR, bool WRITE_OUT, typename Hook, typename StepHook>
+// The caller's requests for what follows this body ride on its last two products:
+// `mid_begin()` / `mid_steps(ks)` around the feed-forward product's contraction steps,
+// `last_begin()` / `last_steps(ks)` around the last product's (see WeightStream::run).  The fused
+// layer boundary requests the next layer's first two matrices there.
+template <typename T, int D, int F, int TR, bool WRITE_OUT, typename MidBegin, typename MidSteps, typename LastBegin,
+          typename LastSteps>
 __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0, T *a1, float *red_a, float *red_b,
-                                                long row0, int valid, Hook before_last, StepHook last_steps, T *vecs,
-                                                int vec_ld) {
+                                                long row0, int valid, MidBegin mid_begin, MidSteps mid_steps,
+                                                LastBegin last_begin, LastSteps last_steps, T *vecs, int vec_ld) {
     typedef Tile<T, TR> TL;
     constexpr int NW = fused_waves(D), NT = NW * 64;
     constexpr int LDD = D + 8, LDF = F + 8;
@@ -777,7 +790,11 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
             for (int b = 0; b < NBD; ++b)
 #pragma unroll
                 for (int q = 0; q < TL::kVals; ++q) acc[b][q] = 0.f;
-            w.multiply(acc, a0, LDD, c, hb);
+            // W_2 goes where W_o's fragments were, step by step: two matrices (W_1, W_2) are then
+            // on their way while this product's epilogue runs, and the memory pipeline never idles
+            if (kWhole) w_2.begin(static_cast<const T *>(P.w_2), nbd, lane);
+            w.multiply(acc, a0, LDD, c, hb,
+                       [&](int ks) { if (kWhole) w_2.request_share(ks, WeightStream<T, D, NBD, TR>::KS); });
         }
         if (!kWhole) w_2.start(static_cast<const T *>(P.w_2), nbd, lane);
         float v[NBD][VB];
@@ -799,9 +816,7 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
         float bias[NBF][VB];
         load_cols<T, NBF, TR>(vecs + kVecBias1 * vec_ld, nbf, hb, bias);
         typename TL::acc_t acc[NBF];
-        w_1.run(acc, a1, LDD, c, hb,
-                [&]() { if (kWhole) w_2.begin(static_cast<const T *>(P.w_2), nbd, lane); },
-                [&](int ks) { if (kWhole) w_2.request_share(ks, WeightStream<T, D, NBF, TR>::KS); });
+        w_1.run(acc, a1, LDD, c, hb, mid_begin, mid_steps);
 #pragma unroll
         for (int b = 0; b < NBF; ++b)
 #pragma unroll
@@ -814,8 +829,10 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
                 }
                 store4f<T>(a0 + c * LDF + TL::col(nbf[b], g, hb), o[0], o[1], o[2], o[3]);
             }
-    } else if (kWhole) {
-        w_2.start(static_cast<const T *>(P.w_2), nbd, lane);
+    } else {  // a wavefront that sits the feed-forward product out still makes the caller's requests
+        mid_begin();
+#pragma unroll
+        for (int ks = 0; ks < WeightStream<T, D, NBF, TR>::KS; ++ks) mid_steps(ks);
     }
     float gam[NBD][VB], bet[NBD][VB], bias[NBD][VB];
     load_cols<T, NBD, TR>(vecs + kVecG3 * vec_ld, nbd, hb, gam);
@@ -826,7 +843,7 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
     // ---- out = LN3(x1 + h W_2^T + b_2), staged through a0 for row-contiguous stores
     {
         typename TL::acc_t acc[NBD];
-        w_2.run(acc, a0, LDF, c, hb, before_last, last_steps);
+        w_2.run(acc, a0, LDF, c, hb, last_begin, last_steps);
         float v[NBD][VB];
 #pragma unroll
         for (int b = 0; b < NBD; ++b)
@@ -855,7 +872,8 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_kernel(FusedPo
     const int valid = static_cast<int>(min(static_cast<long>(TR), P.rows - row0));
     constexpr int VW = D > F ? D : F;
     __shared__ __attribute__((aligned(16))) T vecs[kVecSlots * VW];
-    fused_post_body<T, D, F, TR, true>(P, a0, a1, red_a, red_b, row0, valid, NoHook{}, NoHook{}, vecs, VW);
+    fused_post_body<T, D, F, TR, true>(P, a0, a1, red_a, red_b, row0, valid, NoHook{}, NoHook{}, NoHook{}, NoHook{},
+                                       vecs, VW);
 }
 
 // The post part of layer L and the pre part of layer L+1 on the same rows: the layer output
@@ -873,14 +891,35 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_pre_kernel(Fus
     int nblk[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b) nblk[b] = wave + NW * b;
-    WeightStream<T, D, NB, TR> next_fo;
+    WeightStream<T, D, NB, TR> next_fo, next_q;
     constexpr int VW = D > F ? D : F;
     __shared__ __attribute__((aligned(16))) T vecs[kVecSlots * VW];
     stage_pre_vectors<T, D, NW * 64>(N, vecs, VW, threadIdx.x);  // visible after the first barrier below
+    // Whole-matrix streams: the next layer's W_fo is requested during the feed-forward product and
+    // its q weights during the last product.  Deeper ones: W_fo ahead of the last product, the q
+    // weights by the pre body (the order that measured best for them).
+    constexpr int NBF = fused_blocks<T, TR>(F, NW);
+    constexpr bool kWhole = WeightStream<T, D, NB, TR>::kWhole && WeightStream<T, D, NBF, TR>::kWhole &&
+                            WeightStream<T, F, NB, TR>::kWhole;
+    const T *w_fo = static_cast<const T *>(N.w_fo), *w_q = static_cast<const T *>(N.w_qkv);
     fused_post_body<T, D, F, TR, false>(
-        P, a0, a1, red_a, red_b, row0, valid, [&]() { next_fo.begin(static_cast<const T *>(N.w_fo), nblk, lane); },
-        [&](int ks) { next_fo.request_share(ks, WeightStream<T, F, NB, TR>::KS); }, vecs, VW);
-    fused_pre_body<T, D, TR, true>(N, a0, a1, red_a, red_b, row0, valid, next_fo, vecs, VW);
+        P, a0, a1, red_a, red_b, row0, valid,
+        [&]() { if (kWhole) next_fo.begin(w_fo, nblk, lane); },
+        [&](int ks) { if (kWhole) next_fo.request_share(ks, WeightStream<T, D, NBF, TR>::KS); },
+        [&]() {
+            if (kWhole)
+                next_q.begin(w_q, nblk, lane);
+            else
+                next_fo.begin(w_fo, nblk, lane);
+        },
+        [&](int ks) {
+            if (kWhole)
+                next_q.request_share(ks, WeightStream<T, F, NB, TR>::KS);
+            else
+                next_fo.request_share(ks, WeightStream<T, F, NB, TR>::KS);
+        },
+        vecs, VW);
+    fused_pre_body<T, D, TR, true, kWhole>(N, a0, a1, red_a, red_b, row0, valid, next_fo, next_q, vecs, VW);
 }
 
 // ---- end of a decode step: final norm + mixture head + one sample per trajectory + the
