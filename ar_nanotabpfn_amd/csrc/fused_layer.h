@@ -327,10 +327,12 @@ struct PartialIndex {
 constexpr int kMergeBatch = 9;  // partials fetched per round (8 context slices + the buffer pass)
 
 // `on_arrival` runs once every load issued so far (the caller's and the partials') has come back
-// and before the merge arithmetic: the place to request the next weight stream.
-template <typename T, int D, int NT, int TR, typename Hook>
+// and before the merge arithmetic — the place to begin() the next weight stream —, `per_slot(u)`,
+// u = 0 .. kMergeBatch-1, between the slots of the merge arithmetic of the last item: the place for
+// that stream's request_share(u, kMergeBatch), so that its requests queue while the merge computes.
+template <typename T, int D, int NT, int TR, typename Hook, typename SlotHook>
 __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const FusedPostParams &P, long row0,
-                                                       int valid, int tid, Hook on_arrival) {
+                                                       int valid, int tid, Hook on_arrival, SlotHook per_slot) {
     const int dh = D / P.H;          // head dim, a multiple of 8
     const PartialIndex where(P.Lq, P.H, dh);
     const unsigned tok0 = static_cast<unsigned>(row0);  // the launcher keeps rows below 2^31
@@ -387,6 +389,10 @@ __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const
                             acc[2 * e + 1] = fmaf(w, unpack_hi<T>(ov[g][u][e]), acc[2 * e + 1]);
                         }
                     }
+                    if (g == G - 1 && it0 + G >= ITEMS) {
+                        per_slot(u);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
                 const float inv = 1.f / wsum;
                 u32x4 packed = {0u, 0u, 0u, 0u};
@@ -401,6 +407,8 @@ __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const
     }
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     on_arrival();
+#pragma unroll
+    for (int u = 0; u < kMergeBatch; ++u) per_slot(u);
     for (int idx = tid; idx < TR * CPR; idx += NT) {
         const int r = idx / CPR, ch = idx % CPR;
         u32x4 packed = {0u, 0u, 0u, 0u};
@@ -763,9 +771,10 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
             if (tid == 0) order_wait_device(P.order_wait, 0, P.order_limit);
             __syncthreads();
         }
-        stage_merged_attention<T, D, NT, TR>(a0, LDD, P, row0, valid, tid, [&]() {
-            if (kWhole && ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane);
-        });
+        stage_merged_attention<T, D, NT, TR>(
+            a0, LDD, P, row0, valid, tid,
+            [&]() { if (kWhole && ff_active) w_1.begin(static_cast<const T *>(P.w_1), nbf, lane); },
+            [&](int u) { if (kWhole && ff_active) w_1.request_share(u, kMergeBatch); });
         if (!kWhole) {
             w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
             wait_all_loads();
