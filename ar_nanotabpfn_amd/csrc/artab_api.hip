@@ -297,7 +297,7 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineParams P) {
     for (int s = 0; s < P.n_split; ++s) mx = fmaxf(mx, P.part_lse[s * P.rows + row]);
     float wsum = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
     for (int s = 0; s < P.n_split; ++s) {
-        float w = expf(P.part_lse[s * P.rows + row] - mx);
+        float w = merge_weight(P.part_lse[s * P.rows + row], mx);
         const T *o = static_cast<const T *>(P.part_o) + (s * P.rows + row) * P.Dh + d0;
         wsum += w;
 #pragma unroll

@@ -85,6 +85,10 @@ __device__ __forceinline__ float unpack_hi<f16_t>(unsigned u) {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+// Weight of a partial attention result in a log-sum-exp merge, exp(lse - max): one hardware exp2.
+// Every merge of partials (the stand-alone launch and the one inside the layer kernels) uses this
+// one expression, so that they agree bit for bit.
+__device__ __forceinline__ float merge_weight(float lse, float mx) { return fast_exp2((lse - mx) * kLog2e); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
 // Sum / max across the 64 lanes of a wavefront.

@@ -381,7 +381,7 @@ __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const
 #pragma unroll
                 for (int u = 0; u < kMergeBatch; ++u) {
                     if (u < P.n_slots) {
-                        const float w = expf(lv[g][u] - mx);
+                        const float w = merge_weight(lv[g][u], mx);
                         wsum += w;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
@@ -442,7 +442,7 @@ __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const
 #pragma unroll
                 for (int u = 0; u < kMergeBatch; ++u) {
                     if (s0 + u < P.n_slots) {
-                        const float w = expf(lv[u] - mx);
+                        const float w = merge_weight(lv[u], mx);
                         wsum += w;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
