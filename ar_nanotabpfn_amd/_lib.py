@@ -16,6 +16,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libartab_attention.so")
 
+ABI_VERSION = 3  # ARTAB_VERSION of include/artab_attention.h
 ARTAB_BF16, ARTAB_F16, ARTAB_F32 = 0, 1, 2
 IMPL_AUTO, IMPL_PORTABLE, IMPL_MFMA = 0, 1, 2
 
@@ -146,8 +147,8 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes
-    if lib.artab_version() != 3:
-        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.artab_version()} != 3; rebuild the extension")
+    if lib.artab_version() != ABI_VERSION:
+        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.artab_version()} != {ABI_VERSION}; rebuild the extension")
     _lib = lib
     return lib
 

@@ -732,7 +732,7 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
             memset(&D, 0, sizeof(D));
             D.q = dv(q); D.kb = dv(k_ctx); D.vb = dv(v_ctx); D.knew = dv(k_new); D.vnew = dv(v_new); D.out = dv(out);
             D.B = B; D.H = H; D.n_split = 0; D.n_buf = n_buf; D.n_buf_dev = n_buf_device; D.n_base = Nc;
-            D.has_new = has_new;
+            D.has_new = has_new; D.capacity = buf_capacity;
             D.qscale = scale * kLog2e;
             return launch_status(launch_decode(D, dtype, Dh, Lq, st), "decode over a per-trajectory cache");
         }
@@ -747,6 +747,7 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
         P.new_row = has_new ? n_buf : -1;
         P.append = has_new;
         P.nbuf_dev = n_buf_device;
+        P.capacity = buf_capacity;
         P.mode = kModePlain; P.Dh = Dh; P.scale = scale;
         P.vec_ok = aligned ? 1 : 0;
         return launch_status(launch_portable_dtype(P, dtype, st), "decode attention (portable)");
@@ -770,6 +771,7 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
     D.q = dv(q); D.kb = dv(k_buf); D.vb = dv(v_buf); D.knew = dv(k_new); D.vnew = dv(v_new); D.out = dv(out);
     D.part_o = F.part_o; D.part_lse = F.part_lse; D.lse = nullptr;
     D.B = B; D.H = H; D.n_split = pl.n_split; D.n_buf = n_buf; D.n_buf_dev = n_buf_device; D.has_new = has_new;
+    D.capacity = buf_capacity;
     D.qscale = scale * kLog2e;
 
     if (!stream_buf) {

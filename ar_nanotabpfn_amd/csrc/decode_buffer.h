@@ -30,8 +30,23 @@ struct DecodeParams {
     int n_base;   // rows of kb/vb that precede the counted ones (a per-trajectory context stored in
                   // front of the buffer rows); 0 for a shared context
     int has_new;  // 1: row n_buf comes from knew/vnew, is attended and appended
+    int capacity; // counted rows the cache holds (behind n_base); a length read from n_buf_dev is
+                  // clamped to it, and a new row that would land behind it is not appended
     float qscale; // scale * log2(e)
 };
+
+// Committed length of a decode call.  A host value has been validated by the caller of the
+// kernel; a value read from device memory (a recorded launch replayed more often than the
+// cache has slots, a cell that was never reset) is clamped so that every access stays inside
+// the cache.  `fits` tells whether slot n of the cache exists for the new row.
+__device__ __forceinline__ int committed_rows(const DecodeParams &P, bool &fits) {
+    fits = true;
+    if (!P.n_buf_dev) return P.n_buf;
+    const int raw = *P.n_buf_dev;
+    const int hi = P.capacity - (P.has_new ? 1 : 0);
+    fits = raw >= 0 && raw <= hi;
+    return raw < 0 ? 0 : (raw > hi ? (hi > 0 ? hi : 0) : raw);
+}
 
 constexpr int kDecodeWaves = 4;
 constexpr int kDecodeUnroll = 4;
@@ -96,7 +111,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
             for (int i = 0; i < LQ; ++i) M[i] = fmaxf(M[i], v[u][i] * kLog2e);
     }
 
-    const int n_buf = P.n_base + (P.n_buf_dev ? *P.n_buf_dev : P.n_buf);
+    bool slot_fits;
+    const int n_buf = P.n_base + committed_rows(P, slot_fits);
     const int n_total = n_buf + (P.has_new ? 1 : 0);
     const T *knew_row = P.has_new ? view_row<T>(P.knew, b, h, 0) : nullptr;
     const T *vnew_row = P.has_new ? view_row<T>(P.vnew, b, h, 0) : nullptr;
@@ -221,7 +237,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
         view_row<T>(P.out, b, h, i)[d] = from_f32<T>(den > 0.f ? num / den : 0.f);
         if (P.lse && d == 0) P.lse[pair * LQ + i] = den > 0.f ? (Mi + fast_log2(den)) * kLn2 : -INFINITY;
     }
-    if (grp == 1 && P.has_new) {
+    if (grp == 1 && P.has_new && slot_fits) {
         // In-place append: slot n_buf of the cache receives the new row.
         *reinterpret_cast<u32x4 *>(view_row<T>(P.kb, b, h, n_buf) + 8 * sub) =
             *reinterpret_cast<const u32x4 *>(knew_row + 8 * sub);

@@ -112,7 +112,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
     T *const part_o = static_cast<T *>(P.buf_part_o);
     float *const part_lse = P.buf_part_lse;
     const int n_pairs = P.B * H;
-    const int n_buf = P.n_buf_dev ? *P.n_buf_dev : P.n_buf;
+    bool slot_fits;
+    const int n_buf = committed_rows(P, slot_fits);
     const int n_total = n_buf + (has_new ? 1 : 0);
 
     const int lane = threadIdx.x;
@@ -214,7 +215,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
 #pragma unroll
     for (int u = 0; u < 8; ++u) o[u] = f32x4{0.f, 0.f, 0.f, 0.f};
     int task = blockIdx.x, g = 0, slot = 0, qsel = 0;
-    const int new_group = has_new ? n_buf >> 2 : -1;  // the chunk that holds the row to append
+    const int new_group = has_new && slot_fits ? n_buf >> 2 : -1;  // the chunk that holds the row to append
     for (int c = 0; c < total_chunks; ++c) {
         // chunk c must have landed; only the chunks requested after it (8 loads each) may be pending
         switch (issued - c - 1) {

@@ -138,8 +138,10 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
     __shared__ __attribute__((aligned(16))) T v_lds[3][BN * VPAD];
     __shared__ int redo_flag;
 
+    // (release: whatever this queue's earlier launches wrote is visible to the watcher that sees
+    // the new count)
     if (P.started && blockIdx.x == 0 && threadIdx.x == 0)
-        __hip_atomic_fetch_add(P.started, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_fetch_add(P.started, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 
     // ---- workgroup -> (kv-sharing group, q tile, context split); XCD-aware: the
     // hardware deals consecutive workgroup ids round-robin over the 8 XCDs, so all

@@ -24,6 +24,7 @@ struct PortableParams {
     int B, H, Lq, Nc, Nb;
     int new_row;  // buffer row index served from knew/vnew, or -1
     const int *nbuf_dev;  // decode: committed buffer length read at run time (overrides Nb / new_row)
+    int capacity;         // rows the buffer cache holds (bound for a length read from nbuf_dev)
     int append;   // copy knew/vnew to kb/vb[new_row]
     int mode;
     int Nt;
@@ -138,7 +139,12 @@ __global__ __launch_bounds__(kPortableWaves * 64) void portable_attention_kernel
 
     // Buffer segment: keys [0, limit) with the mode's visibility rule.
     if (P.nbuf_dev) {
-        const int n = *P.nbuf_dev;
+        // a length read from device memory is clamped to the cache; a new row that would land
+        // behind the last slot is attended but not stored
+        const int hi = P.capacity - (P.new_row >= 0 ? 1 : 0);
+        const int raw = *P.nbuf_dev;
+        const int n = raw < 0 ? 0 : (raw > hi ? (hi > 0 ? hi : 0) : raw);
+        if (raw != n) P.append = 0;
         P.Nb = n + (P.new_row >= 0 ? 1 : 0);
         if (P.new_row >= 0) P.new_row = n;
     }

@@ -86,6 +86,7 @@ class ARTabPFNPredictor:
         self.target_only_last_layer = True
         self._side_streams = {}
         self._graph_state = None
+        self.graph_recordings = 0    # HIP graphs recorded so far (a run that only replays leaves it unchanged)
 
     @classmethod
     def from_trained_model(cls, model, backend: str = "flex_attention") -> "ARTabPFNPredictor":
@@ -418,7 +419,10 @@ class ARTabPFNPredictor:
         params = list(self.backbone.parameters()) + list(self.embedder.parameters()) + list(self.head.parameters())
         params.append(self.ar_tokens)
         chain_rows = self._chain_rows(B)
-        key = (B, Nt, F_, self.context_len, dtype, str(device), layer0.k_ctx_cache.data_ptr(),
+        # The recorded step depends on the capacity of the buffer cache, not on how many steps are
+        # replayed: loop state is sized for the capacity, so runs of any length share one recording.
+        cap = self.max_buffer_len
+        key = (B, cap, F_, self.context_len, dtype, str(device), layer0.k_ctx_cache.data_ptr(),
                layer0.k_buf_cache.data_ptr(), self.fuse_step_tail, self.overlap_buffer_pass, self.merge_in_layer,
                len(chain_rows), int(self.steps_per_graph), bool(self.counter_ordering),
                bool(self.target_only_last_layer), tuple((p.data_ptr(), p._version) for p in params))
@@ -426,7 +430,7 @@ class ARTabPFNPredictor:
         if gs is None or gs.key != key:
             gs = _GraphState()
             gs.key = key
-            gs.x_target = torch.empty((B, Nt, F_), device=device, dtype=dtype)
+            gs.x_target = torch.zeros((B, cap, F_), device=device, dtype=dtype)
             gs.chains = []
             fused_tail = self.fuse_step_tail and SampleEmbedStep.supported(self.embedder, self.backbone, self.head,
                                                                            x_target)
@@ -438,7 +442,7 @@ class ARTabPFNPredictor:
                 st.stream = torch.cuda.Stream(device=device) if len(chain_rows) > 1 else None  # default priority
                 st.x_target = gs.x_target[rows]
                 st.y_prev = torch.zeros((Bc, 1), device=device, dtype=dtype)
-                st.preds = torch.zeros((Bc, Nt), device=device, dtype=dtype)
+                st.preds = torch.zeros((Bc, cap), device=device, dtype=dtype)
                 st.counters = torch.zeros(2, device=device, dtype=torch.int32)  # (step index t, buffer length)
                 st.t, st.nbuf = st.counters[0:1], st.counters[1:2]
                 st.graph = None
@@ -453,15 +457,15 @@ class ARTabPFNPredictor:
                 if fused_tail:
                     D = self.backbone.d_model
                     st.emb = torch.zeros((Bc, 2, D), device=device, dtype=dtype)
-                    st.x_mean = torch.zeros((Bc, Nt), device=device, dtype=dtype)
-                    st.rand_u = torch.zeros((Nt, Bc), device=device, dtype=torch.float32)
-                    st.rand_n = torch.zeros((Nt, Bc), device=device, dtype=torch.float32)
+                    st.x_mean = torch.zeros((Bc, cap), device=device, dtype=dtype)
+                    st.rand_u = torch.zeros((cap, Bc), device=device, dtype=torch.float32)
+                    st.rand_n = torch.zeros((cap, Bc), device=device, dtype=torch.float32)
                     st.tail = SampleEmbedStep(self.embedder, self.backbone, self.head, self.ar_tokens, st.x_mean,
                                               st.rand_u, st.rand_n, st.t, st.preds, st.emb, advance=st.counters)
                 gs.chains.append(st)
             gs.tail = gs.chains[0].tail
             self._graph_state = gs
-        gs.x_target.copy_(x_target)
+        gs.x_target[:, :Nt].copy_(x_target)
 
         # first target: no buffer row yet (N = 1), launched directly for all trajectories
         y0 = self.autoregressive_decode(gs.x_target[:, 0:1, :], None, None, 0)
@@ -470,10 +474,10 @@ class ARTabPFNPredictor:
             bs = self.ar_tokens.shape[0]
             emb1 = torch.cat([self.embedder.embed_buffer(gs.x_target[:, 0:1], y0) + self.ar_tokens[1 % bs],
                               self.embedder.embed_target(gs.x_target[:, 1:2])], dim=1)
-            x_mean = gs.x_target.mean(dim=-1)
+            x_mean = gs.x_target[:, :Nt].mean(dim=-1)
             for st in gs.chains:
                 rows = st.rows if st.rows is not None else slice(0, B)
-                st.x_mean.copy_(x_mean[rows])
+                st.x_mean[:, :Nt].copy_(x_mean[rows])
                 self._draw_step_variates(st.rand_u, st.rand_n)
 
         def reset(st):
@@ -501,7 +505,7 @@ class ARTabPFNPredictor:
                 current.wait_stream(warm)
                 reset(st)
                 st.graph = self._record_steps(st, 1)
-                if self.steps_per_graph > 1 and Nt - 1 >= self.steps_per_graph:
+                if self.steps_per_graph > 1 and cap - 1 >= self.steps_per_graph:
                     reset(st)
                     st.graph_many = self._record_steps(st, self.steps_per_graph)
         gs.graph = gs.chains[0].graph
@@ -536,8 +540,8 @@ class ARTabPFNPredictor:
         self.buffer_len = Nt - 1
         self.seq_len = self.context_len + self.buffer_len
         if len(gs.chains) == 1:
-            return gs.chains[0].preds.clone()
-        return torch.cat([st.preds for st in gs.chains], dim=0)
+            return gs.chains[0].preds[:, :Nt].clone()
+        return torch.cat([st.preds[:, :Nt] for st in gs.chains], dim=0)
 
     def _counter_ordering_applies(self, x: Tensor) -> bool:
         """Whether every layer's decode call takes the schedule that the counters can order: the
@@ -551,6 +555,7 @@ class ARTabPFNPredictor:
         ordering the side stream joins the recording once and rejoins at the end; the per-layer
         dependencies between the two streams are the counters' waits."""
         graph = torch.cuda.CUDAGraph()
+        self.graph_recordings += 1
         with torch.cuda.graph(graph):
             if st.order is None:
                 for _ in range(n_steps):

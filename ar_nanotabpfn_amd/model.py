@@ -267,7 +267,13 @@ class MixtureGaussianHead(nn.Module):
         mean, std, weight, _ = self._parameterize(z)
         B, T, K, Dy = mean.shape
         flat = lambda t: t.permute(0, 1, 3, 2).reshape(B * T * Dy, K)  # noqa: E731
-        idx = torch.multinomial(flat(weight), num_samples, replacement=True)
+        # Component = first k whose cumulative weight exceeds a uniform variate times the total
+        # (the law of a multinomial draw, and the rule of the fused step tail).  The index is
+        # clamped, so non-finite weights give non-finite samples instead of a device-side
+        # index assertion.
+        cdf = flat(weight).float().cumsum(dim=1)
+        u = torch.rand((cdf.shape[0], num_samples), device=cdf.device, dtype=cdf.dtype) * cdf[:, -1:]
+        idx = (u.unsqueeze(-1) >= cdf.unsqueeze(1)).sum(dim=-1).clamp_(max=K - 1)
         mu = torch.gather(flat(mean), 1, idx).view(B, T, Dy, num_samples)
         sd = torch.gather(flat(std), 1, idx).view(B, T, Dy, num_samples)
         return (mu + sd * torch.randn_like(mu)).permute(0, 1, 3, 2)
