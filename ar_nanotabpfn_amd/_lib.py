@@ -16,7 +16,8 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libartab_attention.so")
 
-ABI_VERSION = 3  # ARTAB_VERSION of include/artab_attention.h
+ABI_VERSION = 4  # ARTAB_VERSION of include/artab_attention.h
+STATIC_SCRATCH_BYTES = 32 << 20  # ARTAB_STATIC_SCRATCH_BYTES
 ARTAB_BF16, ARTAB_F16, ARTAB_F32 = 0, 1, 2
 IMPL_AUTO, IMPL_PORTABLE, IMPL_MFMA = 0, 1, 2
 
@@ -84,6 +85,10 @@ SIGNATURES = {
     "artab_decode_attention": (
         _i,
         [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _p, _i, _i, _f, _i, _p, _sz, _i, _p],
+    ),
+    "artab_decode_attention_static": (
+        _i,
+        [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _p, _i, _i, _f, _i, _i, _p],
     ),
     "artab_decode_attention_overlapped": (
         _i,

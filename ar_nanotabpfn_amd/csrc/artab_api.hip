@@ -893,6 +893,54 @@ int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const a
                        buf_capacity, Dh, scale, dtype, workspace, workspace_bytes, impl, stream, nullptr);
 }
 
+// ---------------------------------------------------------------------------------------------
+// The entry point that allocates nothing: the split-context workspace of artab_decode_attention
+// in a file-scope device array instead of caller memory.
+// ---------------------------------------------------------------------------------------------
+
+static __device__ __align__(256) unsigned char scratch[ARTAB_STATIC_SCRATCH_BYTES];
+
+// Device address of `scratch` on the current device.  In host code the array's name is only a
+// stand-in for the symbol, and every device holds its own copy at its own address: the address
+// is looked up once per device, with that device current, and kept.
+static int static_scratch(void **ptr) {
+    constexpr int kDevices = 16;
+    static void *addr[kDevices];
+    static std::mutex mu;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kDevices)
+        return fail(ARTAB_ERR_UNSUPPORTED, "no current HIP device (or index above %d)", kDevices - 1);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!addr[dev]) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fail(ARTAB_ERR_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        addr[dev] = p;
+    }
+    *ptr = addr[dev];
+    return ARTAB_OK;
+}
+
+int artab_decode_attention_static(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                                  const artab_view *k_buf, const artab_view *v_buf, const artab_view *k_new,
+                                  const artab_view *v_new, const artab_view *out, int B, int H, int Lq, int Nc,
+                                  int n_buf, const int32_t *n_buf_device, int buf_capacity, int Dh, float scale,
+                                  int dtype, int impl, void *stream) {
+    // the bound that artab_workspace_bytes gives callers of artab_decode_attention
+    const size_t need = artab_workspace_bytes(B, H, Lq, Nc, Dh, dtype);
+    if (need > static_cast<size_t>(ARTAB_STATIC_SCRATCH_BYTES))
+        return fail(ARTAB_ERR_WORKSPACE,
+                    "artab_decode_attention_static: this problem needs %zu bytes of scratch, the built-in array holds "
+                    "%zu; use artab_decode_attention with a workspace of your own",
+                    need, static_cast<size_t>(ARTAB_STATIC_SCRATCH_BYTES));
+    void *ws = nullptr;
+    ARTAB_TRY(static_scratch(&ws));
+    return decode_impl(q, k_ctx, v_ctx, k_buf, v_buf, k_new, v_new, out, B, H, Lq, Nc, n_buf, n_buf_device,
+                       buf_capacity, Dh, scale, dtype, ws, static_cast<size_t>(ARTAB_STATIC_SCRATCH_BYTES), impl, stream,
+                       nullptr);
+}
+
 int artab_decode_attention_partials(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
                                     const artab_view *k_buf, const artab_view *v_buf, const artab_view *k_new,
                                     const artab_view *v_new, const artab_view *out, int B, int H, int Lq, int Nc,

@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define ARTAB_VERSION 3
+#define ARTAB_VERSION 4
 
 typedef enum artab_dtype {
     ARTAB_BF16 = 0,
@@ -136,6 +136,30 @@ int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const a
                            int B, int H, int Lq, int Nc, int n_buf, const int32_t *n_buf_device,
                            int buf_capacity, int Dh, float scale, int dtype,
                            void *workspace, size_t workspace_bytes, int impl, void *stream);
+
+/*
+ * artab_decode_attention for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the same kernels and results,
+ * with the split-context workspace taken from a device array built into the library instead of
+ * from the caller.  No counterpart in the reference.  It calls no hipMalloc, hipFree or other
+ * allocating routine; inputs and outputs are still the caller's.
+ *   - The array is ARTAB_STATIC_SCRATCH_BYTES per device and is held by every device the library
+ *     is loaded on until the process ends.  A problem whose artab_workspace_bytes() exceeds it is
+ *     rejected with ARTAB_ERR_WORKSPACE before anything is launched.
+ *   - Every call on a device uses that device's one array, whose contents a call overwrites
+ *     before it reads them (nothing has to be cleared): two calls that overlap in time on one
+ *     device (different streams, no ordering between them) race on it.  Calls on one stream, or
+ *     ordered by events, are fine.
+ *   - The first call on a device looks up the array's device address (hipGetSymbolAddress, no
+ *     allocation); make that first call outside a stream capture.
+ */
+#define ARTAB_STATIC_SCRATCH_BYTES (32u << 20)
+int artab_decode_attention_static(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
+                                  const artab_view *k_buf, const artab_view *v_buf,
+                                  const artab_view *k_new, const artab_view *v_new,
+                                  const artab_view *out,
+                                  int B, int H, int Lq, int Nc, int n_buf, const int32_t *n_buf_device,
+                                  int buf_capacity, int Dh, float scale, int dtype, int impl, void *stream);
 
 /*
  * artab_decode_attention with the two passes side by side.  The context pass (bound by the
