@@ -19,6 +19,7 @@
 #include "mfma_flash.h"
 #include "portable_kernels.h"
 #include "queue_order.h"
+#include "launchers.h"
 
 namespace artab {
 
@@ -125,11 +126,6 @@ struct FlashPlan {
     int G;
 };
 
-static int env_int(const char *name, int fallback) {
-    const char *v = getenv(name);
-    return (v && *v) ? atoi(v) : fallback;
-}
-
 // Tile planning.  Query tiles of 256 rows (two 32-row blocks per wavefront) give the
 // best MFMA-per-LDS-byte ratio; smaller tiles are used only when a group has fewer
 // rows (no wavefronts of pure padding) or, for the unsplittable phases, when the
@@ -171,57 +167,6 @@ static FlashPlan plan_flash(int B, int H, int Lq, int Nc, int Dh, bool stacked, 
     pl.n_split = (Nc + per - 1) / per;
     if (pl.n_split < 1) pl.n_split = 1;
     return pl;
-}
-
-// Keys per LDS tile: 64, or 128 for head_dim 32 when ARTAB_BN=128 (tuning aid).
-static int flash_bn(int Dh) { return (Dh == 32 && env_int("ARTAB_BN", 64) == 128) ? 128 : 64; }
-
-template <typename T, int DH>
-static hipError_t launch_flash_bm(const FlashParams &P, int BM, hipStream_t stream) {
-    const int W = P.tiles_per_group * P.n_split;
-    const int n_kvg = P.H * P.n_groups;
-    const unsigned grid = static_cast<unsigned>(((n_kvg + 7) / 8) * W * 8);
-    if (grid == 0) return hipSuccess;
-    if constexpr (DH == 32) {
-        if (flash_bn(DH) == 128) {
-            if (BM == 256)
-                hipLaunchKernelGGL((flash_kernel<T, DH, 2, 4, 128>), dim3(grid), dim3(256), 0, stream, P);
-            else if (BM == 128)
-                hipLaunchKernelGGL((flash_kernel<T, DH, 1, 4, 128>), dim3(grid), dim3(256), 0, stream, P);
-            else
-                hipLaunchKernelGGL((flash_kernel<T, DH, 1, 2, 128>), dim3(grid), dim3(128), 0, stream, P);
-            return hipGetLastError();
-        }
-    }
-    if constexpr (DH <= 64) {
-        if (BM == 256) {
-            hipLaunchKernelGGL((flash_kernel<T, DH, 2, 4, kFlashBN>), dim3(grid), dim3(256), 0, stream, P);
-            return hipGetLastError();
-        }
-        if (BM == 128 && env_int("ARTAB_NW", 4) == 2) {  // two wavefronts of two query blocks each
-            hipLaunchKernelGGL((flash_kernel<T, DH, 2, 2, kFlashBN>), dim3(grid), dim3(128), 0, stream, P);
-            return hipGetLastError();
-        }
-    }
-    if (BM == 128) {
-        hipLaunchKernelGGL((flash_kernel<T, DH, 1, 4, kFlashBN>), dim3(grid), dim3(256), 0, stream, P);
-    } else {
-        hipLaunchKernelGGL((flash_kernel<T, DH, 1, 2, kFlashBN>), dim3(grid), dim3(128), 0, stream, P);
-    }
-    return hipGetLastError();
-}
-
-template <typename T>
-static hipError_t launch_flash(const FlashParams &P, int Dh, int BM, hipStream_t stream) {
-    switch (Dh) {
-        case 32: return launch_flash_bm<T, 32>(P, BM, stream);
-        case 64: return launch_flash_bm<T, 64>(P, BM, stream);
-        default: return launch_flash_bm<T, 128>(P, BM, stream);
-    }
-}
-
-static hipError_t launch_flash_dtype(const FlashParams &P, int dtype, int Dh, int BM, hipStream_t stream) {
-    return dtype == ARTAB_BF16 ? launch_flash<bf16_t>(P, Dh, BM, stream) : launch_flash<f16_t>(P, Dh, BM, stream);
 }
 
 template <typename T, int LQ>
@@ -368,108 +313,6 @@ static int fork_join_events(hipEvent_t *fork, hipEvent_t *join) {
 
 namespace {
 
-// Token rows per workgroup of the layer kernels: 16 while that still leaves the launch within a
-// few workgroups per CU (everything a workgroup does per row is bound by its one CU), else 32
-// (half the weight traffic per row).
-inline int fused_tile_rows(long rows) {
-    if (const char *e = getenv("ARTAB_TILE_ROWS")) {  // tuning / test hook
-        const int v = atoi(e);
-        if (v == kFusedRows || v == kFusedRowsSmall) return v;
-    }
-    return rows <= kFusedSmallMaxRows ? kFusedRowsSmall : kFusedRows;
-}
-
-template <typename T, int TR>
-hipError_t launch_pre_r(const FusedPreParams &P, int D, hipStream_t st) {
-    dim3 grid(static_cast<unsigned>((P.rows + TR - 1) / TR)), block(fused_waves(D) * 64);
-    switch (D) {
-        case 128: hipLaunchKernelGGL((fused_pre_kernel<T, 128, TR>), grid, block, 0, st, P); break;
-        case 256: hipLaunchKernelGGL((fused_pre_kernel<T, 256, TR>), grid, block, 0, st, P); break;
-        default: hipLaunchKernelGGL((fused_pre_kernel<T, 512, TR>), grid, block, 0, st, P); break;
-    }
-    return hipGetLastError();
-}
-template <typename T>
-hipError_t launch_pre(const FusedPreParams &P, int D, hipStream_t st) {
-    return fused_tile_rows(P.rows) == kFusedRowsSmall ? launch_pre_r<T, kFusedRowsSmall>(P, D, st)
-                                                      : launch_pre_r<T, kFusedRows>(P, D, st);
-}
-
-template <typename T, int D, int TR>
-hipError_t launch_post_d(const FusedPostParams &P, int F, hipStream_t st) {
-    dim3 grid(static_cast<unsigned>((P.rows + TR - 1) / TR)), block(fused_waves(D) * 64);
-    switch (F) {
-        case 128: hipLaunchKernelGGL((fused_post_kernel<T, D, 128, TR>), grid, block, 0, st, P); break;
-        case 256: hipLaunchKernelGGL((fused_post_kernel<T, D, 256, TR>), grid, block, 0, st, P); break;
-        default: hipLaunchKernelGGL((fused_post_kernel<T, D, 512, TR>), grid, block, 0, st, P); break;
-    }
-    return hipGetLastError();
-}
-
-template <typename T, int D, int TR>
-hipError_t launch_post_pre_d(const FusedPostParams &P, const FusedPreParams &N, int F, hipStream_t st) {
-    dim3 grid(static_cast<unsigned>((P.rows + TR - 1) / TR)), block(fused_waves(D) * 64);
-    switch (F) {
-        case 128: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 128, TR>), grid, block, 0, st, P, N); break;
-        case 256: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 256, TR>), grid, block, 0, st, P, N); break;
-        default: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 512, TR>), grid, block, 0, st, P, N); break;
-    }
-    return hipGetLastError();
-}
-
-template <typename T, int TR>
-hipError_t launch_post_pre_r(const FusedPostParams &P, const FusedPreParams &N, int D, int F, hipStream_t st) {
-    switch (D) {
-        case 128: return launch_post_pre_d<T, 128, TR>(P, N, F, st);
-        case 256: return launch_post_pre_d<T, 256, TR>(P, N, F, st);
-        default: return launch_post_pre_d<T, 512, TR>(P, N, F, st);
-    }
-}
-template <typename T>
-hipError_t launch_post_pre(const FusedPostParams &P, const FusedPreParams &N, int D, int F, hipStream_t st) {
-    return fused_tile_rows(P.rows) == kFusedRowsSmall ? launch_post_pre_r<T, kFusedRowsSmall>(P, N, D, F, st)
-                                                      : launch_post_pre_r<T, kFusedRows>(P, N, D, F, st);
-}
-
-template <typename T, int TR>
-hipError_t launch_post_r(const FusedPostParams &P, int D, int F, hipStream_t st) {
-    switch (D) {
-        case 128: return launch_post_d<T, 128, TR>(P, F, st);
-        case 256: return launch_post_d<T, 256, TR>(P, F, st);
-        default: return launch_post_d<T, 512, TR>(P, F, st);
-    }
-}
-template <typename T>
-hipError_t launch_post(const FusedPostParams &P, int D, int F, hipStream_t st) {
-    return fused_tile_rows(P.rows) == kFusedRowsSmall ? launch_post_r<T, kFusedRowsSmall>(P, D, F, st)
-                                                      : launch_post_r<T, kFusedRows>(P, D, F, st);
-}
-
-template <typename T, int D, int TR>
-hipError_t launch_sample_d(const SampleEmbedParams &P, int F, hipStream_t st) {
-    dim3 grid(static_cast<unsigned>((P.B + TR - 1) / TR)), block(fused_waves(D) * 64);
-    switch (F) {
-        case 128: hipLaunchKernelGGL((sample_embed_kernel<T, D, 128, TR>), grid, block, 0, st, P); break;
-        case 256: hipLaunchKernelGGL((sample_embed_kernel<T, D, 256, TR>), grid, block, 0, st, P); break;
-        default: hipLaunchKernelGGL((sample_embed_kernel<T, D, 512, TR>), grid, block, 0, st, P); break;
-    }
-    return hipGetLastError();
-}
-
-template <typename T, int TR>
-hipError_t launch_sample_r(const SampleEmbedParams &P, int D, int F, hipStream_t st) {
-    switch (D) {
-        case 128: return launch_sample_d<T, 128, TR>(P, F, st);
-        case 256: return launch_sample_d<T, 256, TR>(P, F, st);
-        default: return launch_sample_d<T, 512, TR>(P, F, st);
-    }
-}
-template <typename T>
-hipError_t launch_sample(const SampleEmbedParams &P, int D, int F, hipStream_t st) {
-    return fused_tile_rows(P.B) == kFusedRowsSmall ? launch_sample_r<T, kFusedRowsSmall>(P, D, F, st)
-                                                   : launch_sample_r<T, kFusedRows>(P, D, F, st);
-}
-
 bool fused_width_ok(int n) { return n == 128 || n == 256 || n == 512; }
 bool misaligned16(const void *p) { return p && reinterpret_cast<uintptr_t>(p) % 16 != 0; }
 
@@ -603,7 +446,7 @@ int artab_context_attention(const artab_view *q, const artab_view *k_ctx, const 
     }
     {
         ProfileScope prof(st);
-        ARTAB_TRY(launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "context attention (mfma)"));
+        ARTAB_TRY(launch_status(launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st), "context attention (mfma)"));
     }
     if (pl.n_split > 1) {
         CombineParams C;
@@ -777,7 +620,7 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
     if (!stream_buf) {
         {
             ProfileScope prof(st);
-            ARTAB_TRY(launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "decode context pass"));
+            ARTAB_TRY(launch_status(launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st), "decode context pass"));
         }
         if (!need_ws) return ARTAB_OK;
         return launch_status(launch_decode(D, dtype, Dh, Lq, st), "decode buffer pass");
@@ -805,7 +648,7 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
         hipError_t e_ctx, e_buf;
         {
             ProfileScope prof(st);
-            e_ctx = launch_flash_dtype(F, dtype, Dh, pl.BM, st);
+            e_ctx = launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st);
         }
         e_buf = launch_stream(D, dtype, Lq, side);
         ARTAB_TRY(launch_status(e_ctx, "decode context pass"));
@@ -832,7 +675,7 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
     hipError_t e_ctx, e_buf, e_join = hipSuccess;
     {
         ProfileScope prof(st);
-        e_ctx = launch_flash_dtype(F, dtype, Dh, pl.BM, st);
+        e_ctx = launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st);
     }
     e_buf = launch_stream(D, dtype, Lq, side);
     if (side != st) {
@@ -1022,7 +865,7 @@ int artab_teacher_forcing_attention(const artab_view *q, const artab_view *k_ctx
     F.qscale = scale * kLog2e;
     F.mode = kFlashTeacher;
     ProfileScope prof(st);
-    return launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "teacher forcing (mfma)");
+    return launch_status(launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st), "teacher forcing (mfma)");
 }
 
 int artab_prefill_attention(const artab_view *q, const artab_view *k, const artab_view *v, const artab_view *out,
@@ -1071,7 +914,7 @@ int artab_prefill_attention(const artab_view *q, const artab_view *k, const arta
     F.qscale = scale * kLog2e;
     F.mode = kFlashPrefill;
     ProfileScope prof(st);
-    return launch_status(launch_flash_dtype(F, dtype, Dh, pl.BM, st), "prefill (mfma)");
+    return launch_status(launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st), "prefill (mfma)");
 }
 
 int artab_buffer_attention(const artab_view *q, const artab_view *k_buf, const artab_view *v_buf,
@@ -1285,7 +1128,7 @@ int artab_layer_pre(const void *x, int64_t ldx, const void *w_fo, const void *ln
     ARTAB_TRY(fill_pre(P, x, ldx, w_fo, ln1_gamma, ln1_beta, eps1, w_qkv, y, qkv, rows, D, true));
     if (rows == 0) return ARTAB_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipError_t e = dtype == ARTAB_BF16 ? launch_pre<bf16_t>(P, D, st) : launch_pre<f16_t>(P, D, st);
+    hipError_t e = launch_layer_pre(P, D, dtype == ARTAB_BF16, st);
     return launch_status(e, "layer_pre");
 }
 
@@ -1299,7 +1142,7 @@ int artab_layer_post(const void *attn, int64_t lda, const void *y, int64_t ldy, 
                         ln3_beta, eps3, out, rows, D, F, true));
     if (rows == 0) return ARTAB_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipError_t e = dtype == ARTAB_BF16 ? launch_post<bf16_t>(P, D, F, st) : launch_post<f16_t>(P, D, F, st);
+    hipError_t e = launch_layer_post(P, D, F, dtype == ARTAB_BF16, st);
     return launch_status(e, "layer_post");
 }
 
@@ -1320,7 +1163,7 @@ static int layer_post_pre_impl(const artab_attention_partials *parts, const void
     hipStream_t st = static_cast<hipStream_t>(stream);
     ARTAB_TRY(apply_partials_order(parts, P, rows, st));
     if (rows == 0) return ARTAB_OK;
-    hipError_t e = dtype == ARTAB_BF16 ? launch_post_pre<bf16_t>(P, N, D, F, st) : launch_post_pre<f16_t>(P, N, D, F, st);
+    hipError_t e = launch_layer_post_pre(P, N, D, F, dtype == ARTAB_BF16, st);
     return launch_status(e, "layer_post_pre");
 }
 
@@ -1362,7 +1205,7 @@ int artab_layer_post_from_partials(const artab_attention_partials *parts, const 
     hipStream_t st = static_cast<hipStream_t>(stream);
     ARTAB_TRY(apply_partials_order(parts, P, rows, st));
     if (rows == 0) return ARTAB_OK;
-    hipError_t e = dtype == ARTAB_BF16 ? launch_post<bf16_t>(P, D, F, st) : launch_post<f16_t>(P, D, F, st);
+    hipError_t e = launch_layer_post(P, D, F, dtype == ARTAB_BF16, st);
     return launch_status(e, "layer_post");
 }
 
@@ -1398,7 +1241,7 @@ int artab_decode_sample_embed(const artab_sample_embed_args *a, int dtype, void 
         return fail(ARTAB_ERR_BAD_SHAPE, "advance needs 1..8 counters and a ticket word");
     P.advance = a->advance; P.n_advance = a->advance ? a->n_advance : 0; P.ticket = a->ticket;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipError_t e = dtype == ARTAB_BF16 ? launch_sample<bf16_t>(P, a->D, a->F, st) : launch_sample<f16_t>(P, a->D, a->F, st);
+    hipError_t e = launch_sample_embed(P, a->D, a->F, dtype == ARTAB_BF16, st);
     return launch_status(e, "decode_sample_embed");
 }
 

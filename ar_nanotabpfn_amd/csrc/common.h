@@ -84,6 +84,16 @@ __device__ __forceinline__ float unpack_hi<f16_t>(unsigned u) {
     return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(u >> 16)));
 }
 
+// Eight packed 16-bit values -> float32.
+template <typename T>
+__device__ __forceinline__ void unpack8(const u32x4 &raw, float (&f)[8]) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        f[2 * e] = unpack_lo<T>(raw[e]);
+        f[2 * e + 1] = unpack_hi<T>(raw[e]);
+    }
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 // Weight of a partial attention result in a log-sum-exp merge, exp(lse - max): one hardware exp2.
 // Every merge of partials (the stand-alone launch and the one inside the layer kernels) uses this

@@ -52,15 +52,6 @@ constexpr int kDecodeWaves = 4;
 constexpr int kDecodeUnroll = 4;
 constexpr int kSplitBatch = 8;  // context partials fetched per round of the merge
 
-template <typename T>
-__device__ __forceinline__ void unpack8(const u32x4 &raw, float (&f)[8]) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        f[2 * e] = unpack_lo<T>(raw[e]);
-        f[2 * e + 1] = unpack_hi<T>(raw[e]);
-    }
-}
-
 template <typename T, int DH, int LQ>
 __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(DecodeParams P) {
     constexpr int LPR = DH / 8;    // lanes per key row

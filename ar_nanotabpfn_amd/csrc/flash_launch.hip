@@ -1,0 +1,69 @@
+// Launches of the matrix-core attention kernel (mfma_flash.h): template selection by element
+// type, head_dim and query-tile size.
+#include "launchers.h"
+
+namespace artab {
+
+constexpr int kFlashBN = 64;
+
+// Keys per LDS tile: 64, or 128 for head_dim 32 when ARTAB_BN=128 (tuning aid).
+static int flash_bn(int Dh) { return (Dh == 32 && env_int("ARTAB_BN", 64) == 128) ? 128 : 64; }
+
+template <typename T, int DH>
+static hipError_t launch_flash_bm(const FlashParams &P, int BM, hipStream_t stream) {
+    const int W = P.tiles_per_group * P.n_split;
+    const int n_kvg = P.H * P.n_groups;
+    const unsigned grid = static_cast<unsigned>(((n_kvg + 7) / 8) * W * 8);
+    if (grid == 0) return hipSuccess;
+    if constexpr (DH == 32) {
+        if (flash_bn(DH) == 128) {
+            if (BM == 256)
+                hipLaunchKernelGGL((flash_kernel<T, DH, 2, 4, 128>), dim3(grid), dim3(256), 0, stream, P);
+            else if (BM == 128)
+                hipLaunchKernelGGL((flash_kernel<T, DH, 1, 4, 128>), dim3(grid), dim3(256), 0, stream, P);
+            else
+                hipLaunchKernelGGL((flash_kernel<T, DH, 1, 2, 128>), dim3(grid), dim3(128), 0, stream, P);
+            return hipGetLastError();
+        }
+    }
+    if constexpr (DH == 32) {
+        // the lean pass: 256 query rows as eight wavefronts of one 32-row block each, four
+        // wavefronts per SIMD (ARTAB_LEAN=0 selects the software-pipelined form; tuning aid)
+        if (BM == 256 && env_int("ARTAB_LEAN", 1) != 0) {
+            hipLaunchKernelGGL((flash_kernel<T, DH, 1, 8, kFlashBN, true>), dim3(grid), dim3(512), 0, stream, P);
+            return hipGetLastError();
+        }
+    }
+    if constexpr (DH <= 64) {
+        if (BM == 256) {
+            hipLaunchKernelGGL((flash_kernel<T, DH, 2, 4, kFlashBN>), dim3(grid), dim3(256), 0, stream, P);
+            return hipGetLastError();
+        }
+        if (BM == 128 && env_int("ARTAB_NW", 4) == 2) {  // two wavefronts of two query blocks each
+            hipLaunchKernelGGL((flash_kernel<T, DH, 2, 2, kFlashBN>), dim3(grid), dim3(128), 0, stream, P);
+            return hipGetLastError();
+        }
+    }
+    if (BM == 128) {
+        hipLaunchKernelGGL((flash_kernel<T, DH, 1, 4, kFlashBN>), dim3(grid), dim3(256), 0, stream, P);
+    } else {
+        hipLaunchKernelGGL((flash_kernel<T, DH, 1, 2, kFlashBN>), dim3(grid), dim3(128), 0, stream, P);
+    }
+    return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_flash(const FlashParams &P, int Dh, int BM, hipStream_t stream) {
+    switch (Dh) {
+        case 32: return launch_flash_bm<T, 32>(P, BM, stream);
+        case 64: return launch_flash_bm<T, 64>(P, BM, stream);
+        default: return launch_flash_bm<T, 128>(P, BM, stream);
+    }
+}
+
+hipError_t launch_flash_dtype(const FlashParams &P, bool is_bf16, int Dh, int BM, hipStream_t stream) {
+    return is_bf16 ? launch_flash<bf16_t>(P, Dh, BM, stream) : launch_flash<f16_t>(P, Dh, BM, stream);
+}
+
+
+}  // namespace artab

@@ -1,0 +1,157 @@
+// Launches of the fused layer kernels (fused_layer.h).  Compiled once per element type and kernel
+// group: -DARTAB_LAYER_BF16=0|1 and -DARTAB_LAYER_GROUP=0 (pre, post) | 1 (post+pre) | 2 (step tail);
+// the type-dispatching entry points live in the bf16 object of each group.
+#include "launchers.h"
+
+#ifndef ARTAB_LAYER_BF16
+#error "define ARTAB_LAYER_BF16 (0 or 1) and ARTAB_LAYER_GROUP (0, 1 or 2)"
+#endif
+
+namespace artab {
+
+#if ARTAB_LAYER_BF16
+typedef bf16_t LayerT;
+#else
+typedef f16_t LayerT;
+#endif
+
+namespace {
+
+template <typename T, int TR>
+hipError_t launch_pre_r(const FusedPreParams &P, int D, hipStream_t st) {
+    dim3 grid(static_cast<unsigned>((P.rows + TR - 1) / TR)), block(fused_waves(D) * 64);
+    switch (D) {
+        case 128: hipLaunchKernelGGL((fused_pre_kernel<T, 128, TR>), grid, block, 0, st, P); break;
+        case 256: hipLaunchKernelGGL((fused_pre_kernel<T, 256, TR>), grid, block, 0, st, P); break;
+        default: hipLaunchKernelGGL((fused_pre_kernel<T, 512, TR>), grid, block, 0, st, P); break;
+    }
+    return hipGetLastError();
+}
+template <typename T>
+hipError_t launch_pre(const FusedPreParams &P, int D, hipStream_t st) {
+    return fused_tile_rows(P.rows) == kFusedRowsSmall ? launch_pre_r<T, kFusedRowsSmall>(P, D, st)
+                                                      : launch_pre_r<T, kFusedRows>(P, D, st);
+}
+
+template <typename T, int D, int TR>
+hipError_t launch_post_d(const FusedPostParams &P, int F, hipStream_t st) {
+    dim3 grid(static_cast<unsigned>((P.rows + TR - 1) / TR)), block(fused_waves(D) * 64);
+    switch (F) {
+        case 128: hipLaunchKernelGGL((fused_post_kernel<T, D, 128, TR>), grid, block, 0, st, P); break;
+        case 256: hipLaunchKernelGGL((fused_post_kernel<T, D, 256, TR>), grid, block, 0, st, P); break;
+        default: hipLaunchKernelGGL((fused_post_kernel<T, D, 512, TR>), grid, block, 0, st, P); break;
+    }
+    return hipGetLastError();
+}
+
+template <typename T, int D, int TR>
+hipError_t launch_post_pre_d(const FusedPostParams &P, const FusedPreParams &N, int F, hipStream_t st) {
+    dim3 grid(static_cast<unsigned>((P.rows + TR - 1) / TR)), block(fused_waves(D) * 64);
+    switch (F) {
+        case 128: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 128, TR>), grid, block, 0, st, P, N); break;
+        case 256: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 256, TR>), grid, block, 0, st, P, N); break;
+        default: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 512, TR>), grid, block, 0, st, P, N); break;
+    }
+    return hipGetLastError();
+}
+
+template <typename T, int TR>
+hipError_t launch_post_pre_r(const FusedPostParams &P, const FusedPreParams &N, int D, int F, hipStream_t st) {
+    switch (D) {
+        case 128: return launch_post_pre_d<T, 128, TR>(P, N, F, st);
+        case 256: return launch_post_pre_d<T, 256, TR>(P, N, F, st);
+        default: return launch_post_pre_d<T, 512, TR>(P, N, F, st);
+    }
+}
+template <typename T>
+hipError_t launch_post_pre(const FusedPostParams &P, const FusedPreParams &N, int D, int F, hipStream_t st) {
+    return fused_tile_rows(P.rows) == kFusedRowsSmall ? launch_post_pre_r<T, kFusedRowsSmall>(P, N, D, F, st)
+                                                      : launch_post_pre_r<T, kFusedRows>(P, N, D, F, st);
+}
+
+template <typename T, int TR>
+hipError_t launch_post_r(const FusedPostParams &P, int D, int F, hipStream_t st) {
+    switch (D) {
+        case 128: return launch_post_d<T, 128, TR>(P, F, st);
+        case 256: return launch_post_d<T, 256, TR>(P, F, st);
+        default: return launch_post_d<T, 512, TR>(P, F, st);
+    }
+}
+template <typename T>
+hipError_t launch_post(const FusedPostParams &P, int D, int F, hipStream_t st) {
+    return fused_tile_rows(P.rows) == kFusedRowsSmall ? launch_post_r<T, kFusedRowsSmall>(P, D, F, st)
+                                                      : launch_post_r<T, kFusedRows>(P, D, F, st);
+}
+
+template <typename T, int D, int TR>
+hipError_t launch_sample_d(const SampleEmbedParams &P, int F, hipStream_t st) {
+    dim3 grid(static_cast<unsigned>((P.B + TR - 1) / TR)), block(fused_waves(D) * 64);
+    switch (F) {
+        case 128: hipLaunchKernelGGL((sample_embed_kernel<T, D, 128, TR>), grid, block, 0, st, P); break;
+        case 256: hipLaunchKernelGGL((sample_embed_kernel<T, D, 256, TR>), grid, block, 0, st, P); break;
+        default: hipLaunchKernelGGL((sample_embed_kernel<T, D, 512, TR>), grid, block, 0, st, P); break;
+    }
+    return hipGetLastError();
+}
+
+template <typename T, int TR>
+hipError_t launch_sample_r(const SampleEmbedParams &P, int D, int F, hipStream_t st) {
+    switch (D) {
+        case 128: return launch_sample_d<T, 128, TR>(P, F, st);
+        case 256: return launch_sample_d<T, 256, TR>(P, F, st);
+        default: return launch_sample_d<T, 512, TR>(P, F, st);
+    }
+}
+template <typename T>
+hipError_t launch_sample(const SampleEmbedParams &P, int D, int F, hipStream_t st) {
+    return fused_tile_rows(P.B) == kFusedRowsSmall ? launch_sample_r<T, kFusedRowsSmall>(P, D, F, st)
+                                                   : launch_sample_r<T, kFusedRows>(P, D, F, st);
+}
+
+
+}  // namespace
+
+// fp16 forms, defined in the fp16 objects
+hipError_t launch_layer_pre_f16(const FusedPreParams &P, int D, hipStream_t st);
+hipError_t launch_layer_post_f16(const FusedPostParams &P, int D, int F, hipStream_t st);
+hipError_t launch_layer_post_pre_f16(const FusedPostParams &P, const FusedPreParams &N, int D, int F, hipStream_t st);
+hipError_t launch_sample_embed_f16(const SampleEmbedParams &P, int D, int F, hipStream_t st);
+
+#if ARTAB_LAYER_GROUP == 0
+#if ARTAB_LAYER_BF16
+hipError_t launch_layer_pre(const FusedPreParams &P, int D, bool is_bf16, hipStream_t st) {
+    return is_bf16 ? launch_pre<LayerT>(P, D, st) : launch_layer_pre_f16(P, D, st);
+}
+hipError_t launch_layer_post(const FusedPostParams &P, int D, int F, bool is_bf16, hipStream_t st) {
+    return is_bf16 ? launch_post<LayerT>(P, D, F, st) : launch_layer_post_f16(P, D, F, st);
+}
+#else
+hipError_t launch_layer_pre_f16(const FusedPreParams &P, int D, hipStream_t st) { return launch_pre<LayerT>(P, D, st); }
+hipError_t launch_layer_post_f16(const FusedPostParams &P, int D, int F, hipStream_t st) {
+    return launch_post<LayerT>(P, D, F, st);
+}
+#endif
+#elif ARTAB_LAYER_GROUP == 1
+#if ARTAB_LAYER_BF16
+hipError_t launch_layer_post_pre(const FusedPostParams &P, const FusedPreParams &N, int D, int F, bool is_bf16,
+                                 hipStream_t st) {
+    return is_bf16 ? launch_post_pre<LayerT>(P, N, D, F, st) : launch_layer_post_pre_f16(P, N, D, F, st);
+}
+#else
+hipError_t launch_layer_post_pre_f16(const FusedPostParams &P, const FusedPreParams &N, int D, int F, hipStream_t st) {
+    return launch_post_pre<LayerT>(P, N, D, F, st);
+}
+#endif
+#else
+#if ARTAB_LAYER_BF16
+hipError_t launch_sample_embed(const SampleEmbedParams &P, int D, int F, bool is_bf16, hipStream_t st) {
+    return is_bf16 ? launch_sample<LayerT>(P, D, F, st) : launch_sample_embed_f16(P, D, F, st);
+}
+#else
+hipError_t launch_sample_embed_f16(const SampleEmbedParams &P, int D, int F, hipStream_t st) {
+    return launch_sample<LayerT>(P, D, F, st);
+}
+#endif
+#endif
+
+}  // namespace artab

@@ -31,6 +31,8 @@
 // exponent range is too small for the fast path, always takes that robust path.
 #pragma once
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace artab {
@@ -44,8 +46,12 @@ template <>
 struct MfmaOps<bf16_t> {
     typedef bf16x8 vec;
     static constexpr bool kWideExponent = true;
+    static constexpr unsigned kOnes2 = 0x3f803f80u;  // (1, 1) packed
     static __device__ __forceinline__ f32x16 mma(vec a, vec b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4 mma16(vec a, vec b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
     }
     static __device__ __forceinline__ float dot2(unsigned packed, float acc) {
         typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -58,8 +64,12 @@ template <>
 struct MfmaOps<f16_t> {
     typedef f16x8 vec;
     static constexpr bool kWideExponent = false;
+    static constexpr unsigned kOnes2 = 0x3c003c00u;  // (1, 1) packed
     static __device__ __forceinline__ f32x16 mma(vec a, vec b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4 mma16(vec a, vec b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
     }
     static __device__ __forceinline__ float dot2(unsigned packed, float acc) {
         typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
@@ -118,8 +128,11 @@ struct BoolTag {
     static constexpr bool value = V;
 };
 
-template <typename T, int DH, int QB, int NW, int BN>
-__global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
+// LEAN selects the fast pass: false = the software-pipelined loop (two wavefronts per SIMD, 216
+// registers), true = the plain loop built for four wavefronts per SIMD (see lean_pass).
+template <typename T, int DH, int QB, int NW, int BN, bool LEAN = false>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(LEAN ? 4 : 1)))
+void flash_kernel(FlashParams P) {
     typedef MfmaOps<T> Ops;
     typedef typename Ops::vec vec;
     constexpr int KS = DH / 16;
@@ -134,8 +147,12 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
     constexpr int NCH = (CHUNKS + NT - 1) / NT;
     constexpr int CPR = DH / 8;  // chunks per row
 
-    __shared__ __attribute__((aligned(16))) T k_lds[3][BN * KPAD];
-    __shared__ __attribute__((aligned(16))) T v_lds[3][BN * VPAD];
+    // three stages; a stage is the K tile followed by the V tile, so that both have the same
+    // stage stride and a stage index folds into the immediate offset of every LDS access
+    constexpr int STAGE = BN * KPAD + BN * VPAD;
+    __shared__ __attribute__((aligned(16))) T kv_lds[3 * STAGE];
+    auto k_stage = [&](int st_) -> T * { return kv_lds + st_ * STAGE; };
+    auto v_stage = [&](int st_) -> T * { return kv_lds + st_ * STAGE + BN * KPAD; };
     __shared__ int redo_flag;
 
     // (release: whatever this queue's earlier launches wrote is visible to the watcher that sees
@@ -160,7 +177,9 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
     const long kvb = P.n_groups == 1 ? 0 : g;  // batch entry whose K/V this group reads
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
+    // wavefront index as a scalar: everything derived from it (the wavefront's rows, its
+    // teacher-forcing key limits) then steers scalar branches instead of exec-mask ones
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int c = lane & 31, hb = lane >> 5;
     const int row0_wg = tile * BM;
     const int row0_w = row0_wg + wave * ROWS_W;
@@ -324,8 +343,8 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
 #pragma unroll
         for (int x = 0; x < NCH; ++x) {
             if (NCH * NT == CHUNKS || tid + x * NT < CHUNKS) {
-                *reinterpret_cast<u32x4 *>(&k_lds[buf][st_row[x] * KPAD + st_col[x]]) = kst[x];
-                *reinterpret_cast<u32x4 *>(&v_lds[buf][st_row[x] * VPAD + st_col[x]]) = vst[x];
+                *reinterpret_cast<u32x4 *>(k_stage(buf) + st_row[x] * KPAD + st_col[x]) = kst[x];
+                *reinterpret_cast<u32x4 *>(v_stage(buf) + st_row[x] * VPAD + st_col[x]) = vst[x];
             }
         }
     };
@@ -374,8 +393,8 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
             const int seg_end = is_ctx ? ctx_end : P.Nb;
             const int w_min = is_ctx ? seg_end : wave_lim_min;
             const int w_max = is_ctx ? seg_end : wave_lim_max;
-            const T *kt = &k_lds[cur][k_rd];
-            const T *vt = &v_lds[cur][v_rd];
+            const T *kt = k_stage(cur) + k_rd;
+            const T *vt = v_stage(cur) + v_rd;
 
             auto block = [&](int sb, auto mask_tag) {
                 constexpr bool MASK = decltype(mask_tag)::value;
@@ -534,7 +553,7 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
         f32x16 s_cur[QB];
         {
             vec ak0[KS];
-            load_k(ak0, &k_lds[0][k_rd]);
+            load_k(ak0, k_stage(0) + k_rd);
             scores(s_cur, ak0);
         }
 
@@ -547,11 +566,11 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
             const int kv0 = is_ctx ? ctx_begin + it * BN : (it - ctx_tiles) * BN;
             const int seg_end = is_ctx ? ctx_end : P.Nb;
             const int w_min = is_ctx ? seg_end : wave_lim_min;
-            const T *kt = &k_lds[stage][k_rd];
-            const T *vt = &v_lds[stage][v_rd];
+            const T *kt = k_stage(stage) + k_rd;
+            const T *vt = v_stage(stage) + v_rd;
             // the block after this tile's last one is block 0 of the next tile (on the very
             // last tile any valid address will do: those scores are never used)
-            const T *kt_next = (it + 1 < n_tiles) ? &k_lds[stage_next][k_rd] : kt;
+            const T *kt_next = (it + 1 < n_tiles) ? k_stage(stage_next) + k_rd : kt;
 
             auto tile_body = [&](auto mask_tag) {
                 constexpr bool MASK = decltype(mask_tag)::value;
@@ -633,9 +652,248 @@ __global__ __launch_bounds__(NW * 64) void flash_kernel(FlashParams P) {
         __syncthreads();
     };
 
+
+    // Lean fast pass.  On this part a matrix instruction holds the SIMD's vector issue port for
+    // its whole duration: MFMA and ordinary VALU work of the same SIMD do not overlap, whichever
+    // wavefronts they come from (only the tail of a transcendental does).  The time of a 32x32
+    // score block is therefore the SUM of its instructions' issue cycles, and software pipelining
+    // inside a wavefront buys nothing that more resident wavefronts do not give as well.  So this
+    // pass keeps the instruction count minimal and the register count low enough for four
+    // wavefronts per SIMD:
+    //  * a plain in-order block: K fragments, S = K Q^T, p = 2^s, P V; no second score buffer;
+    //  * the row sum of the rounded probabilities comes from the matrix pipe: with
+    //    v_mfma_f32_16x16x32 a lane's four packed registers are 8 contraction entries of column
+    //    lane%16, contraction group lane/16.  A lane here is (query c = lane%32, half hb), i.e.
+    //    column c%16 and group c/16 + 2 hb: an A operand that is all ones in row 0 for groups
+    //    {0, 2} and in row 1 for groups {1, 3} sums queries 0..15 into row 0 and 16..31 into
+    //    row 1 (lanes 0..15, registers 0 and 1).  Two such products per block replace eight
+    //    v_dot2c (which, issued between MFMAs, cost five times their nominal four cycles).
+    //  * K and V tiles of a stage are one list of 16-byte pieces dealt over the whole workgroup.
+    // Three LDS stages, one barrier per tile, tiles requested two ahead (as in fast_pass).
+    auto lean_pass = [&]() {
+        f32x4 lsum[QB][2];
+#pragma unroll
+        for (int j = 0; j < QB; ++j) {
+            m_run[j] = 0.f;
+            l_run[j] = 0.f;
+            lsum[j][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+            lsum[j][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) o_acc[j][db][v] = 0.f;
+        }
+        const unsigned one2 = (lane == 0 || lane == 32 || lane == 17 || lane == 49) ? Ops::kOnes2 : 0u;
+        const vec ones_sel = __builtin_bit_cast(vec, u32x4{one2, one2, one2, one2});
+
+        // ---- staging.  A stage's 2*CHUNKS 16-byte pieces (K pieces, then V pieces) are dealt over
+        // the workgroup, NP rounds of NT pieces.  CHUNKS is a multiple of 64, so whether a piece
+        // is K or V is uniform over a wavefront: sources are a scalar base plus a 32-bit lane
+        // offset, and the base moves on by one tile with scalar arithmetic.
+        constexpr int NP = (2 * CHUNKS + NT - 1) / NT;
+        static_assert(CHUNKS % 64 == 0, "K/V choice must be wavefront-uniform");
+        bool p_on[NP], p_v[NP];
+        int p_row[NP], p_col[NP];
+        int p_dst[NP];       // element offset inside a stage
+#pragma unroll
+        for (int x = 0; x < NP; ++x) {
+            const int idx0 = wave * 64 + x * NT;  // scalar: first piece of this wavefront in round x
+            p_on[x] = idx0 < 2 * CHUNKS;
+            p_v[x] = idx0 >= CHUNKS;
+            const int cidx = idx0 + lane - (p_v[x] ? CHUNKS : 0);
+            p_row[x] = cidx / CPR;
+            p_col[x] = (cidx % CPR) * 8;
+            p_dst[x] = p_v[x] ? BN * KPAD + p_row[x] * VPAD + p_col[x] : p_row[x] * KPAD + p_col[x];
+        }
+        u32x4 st_a[NP], st_b[NP];
+
+        // Full context tiles (every row present, nothing masked): the steady state.
+        const int n_main = (ctx_end - ctx_begin) / BN;
+        const char *m_src[NP];   // scalar: this round's source of the tile to be requested next
+        unsigned m_off[NP];      // lane: byte offset of this lane's piece inside a tile
+        long m_step[NP];
+#pragma unroll
+        for (int x = 0; x < NP; ++x) {
+            const View &src = p_v[x] ? P.vc : P.kc;
+            m_src[x] = reinterpret_cast<const char *>(view_row<T>(src, kvb, h, ctx_begin));
+            m_off[x] = static_cast<unsigned>((p_row[x] * src.sn + p_col[x]) * static_cast<long>(sizeof(T)));
+            m_step[x] = static_cast<long>(BN) * src.sn * static_cast<long>(sizeof(T));
+        }
+        auto main_fetch = [&](u32x4(&st)[NP]) {
+#pragma unroll
+            for (int x = 0; x < NP; ++x) {
+                if (p_on[x]) st[x] = *reinterpret_cast<const u32x4 *>(m_src[x] + m_off[x]);
+                m_src[x] += m_step[x];
+            }
+        };
+
+        // Every other tile (the partial last context tile, buffer tiles of teacher forcing) goes
+        // the general way: per-lane pointers, row guards, zero fill.
+        const T *g_src[NP];
+        long g_step[NP];
+        int rows_left = 0;
+        auto gseek = [&](int it) {
+            const bool is_ctx = it < ctx_tiles;
+            const View &ks_ = is_ctx ? P.kc : P.kb;
+            const View &vs_ = is_ctx ? P.vc : P.vb;
+            const long bb = is_ctx ? kvb : g;
+            const int kv0 = is_ctx ? ctx_begin + it * BN : (it - ctx_tiles) * BN;
+            rows_left = (is_ctx ? ctx_end : P.Nb) - kv0;
+#pragma unroll
+            for (int x = 0; x < NP; ++x) {
+                const View &src = p_v[x] ? vs_ : ks_;
+                g_src[x] = view_row<T>(src, bb, h, kv0) + p_row[x] * src.sn + p_col[x];
+                g_step[x] = static_cast<long>(BN) * src.sn;
+            }
+        };
+        auto gfetch = [&](int it, u32x4(&st)[NP]) {
+            if (it == n_main || it == ctx_tiles) gseek(it);
+#pragma unroll
+            for (int x = 0; x < NP; ++x) {
+                st[x] = u32x4{0u, 0u, 0u, 0u};
+                if (p_on[x] && (rows_left >= BN || p_row[x] < rows_left)) st[x] = *reinterpret_cast<const u32x4 *>(g_src[x]);
+                g_src[x] += g_step[x];
+            }
+            rows_left -= BN;
+        };
+        auto fetch_tile = [&](int it, u32x4(&st)[NP]) {
+            if (it < n_main)
+                main_fetch(st);
+            else
+                gfetch(it, st);
+        };
+        auto stash_tile = [&](auto stage_, const u32x4(&st)[NP]) {
+#pragma unroll
+            for (int x = 0; x < NP; ++x)
+                if (p_on[x]) *reinterpret_cast<u32x4 *>(kv_lds + stage_ * STAGE + p_dst[x]) = st[x];
+        };
+
+        // One 32-key block of the tile in `stage_` against this wavefront's queries.
+        auto block = [&](auto stage_, int sb, auto mask_tag, int blk0, bool is_ctx, int seg_end) {
+            constexpr bool MASK = decltype(mask_tag)::value;
+            const T *kt = kv_lds + stage_ * STAGE + k_rd;
+            const T *vt = kv_lds + stage_ * STAGE + BN * KPAD + v_rd;
+            vec ak[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) ak[ks] = *reinterpret_cast<const vec *>(kt + 32 * sb * KPAD + 16 * ks);
+            vec av[DB][2];
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const T *vp_ = vt + (32 * sb + 16 * t) * VPAD + 32 * db;
+                    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp_));
+                    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) s16x4 *)(vp_ + 8 * VPAD));
+                    typedef short s16x8 __attribute__((ext_vector_type(8)));
+                    s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    av[db][t] = __builtin_bit_cast(vec, both);
+                }
+#pragma unroll
+            for (int j = 0; j < QB; ++j) {
+                f32x16 s;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) s = Ops::mma(ak[ks], qreg[j][ks], s);
+                if constexpr (MASK) {
+                    const int lj = is_ctx ? seg_end : lim[j];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        int kv = blk0 + 8 * (v >> 2) + 4 * hb + (v & 3);
+                        if (kv >= lj) s[v] = -INFINITY;
+                    }
+                }
+                u32x4 pb[2];
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        pb[t][e] = pack2<T>(fast_exp2(s[8 * t + 2 * e]), fast_exp2(s[8 * t + 2 * e + 1]));
+#pragma unroll
+                for (int t = 0; t < 2; ++t) lsum[j][t] = Ops::mma16(ones_sel, __builtin_bit_cast(vec, pb[t]), lsum[j][t]);
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+                        o_acc[j][db] = Ops::mma(av[db][t], __builtin_bit_cast(vec, pb[t]), o_acc[j][db]);
+            }
+        };
+
+        // Tile `it` out of `stage_`: barrier, request tile it + 2, compute, store the requested
+        // tile into the stage that tile it - 1 has left.  STEADY: a full, unmasked context tile
+        // whose successor two ahead is one as well — no condition anywhere, one kind of request
+        // (a second kind of request in the same loop makes the compiler wait for the request
+        // before the tile's first LDS read).
+        auto tile = [&](int it, auto stage_, auto steady_tag) {
+            constexpr bool STEADY = decltype(steady_tag)::value;
+            __syncthreads();
+            if constexpr (STEADY) {
+                main_fetch(st_a);
+#pragma unroll
+                for (int sb = 0; sb < SB; ++sb) block(stage_, sb, BoolTag<false>{}, 0, true, 0);
+                stash_tile((stage_ + 2) % 3, st_a);
+            } else {
+                if (it + 2 < n_tiles) fetch_tile(it + 2, st_a);
+                const bool is_ctx = it < ctx_tiles;
+                const int kv0 = is_ctx ? ctx_begin + it * BN : (it - ctx_tiles) * BN;
+                const int seg_end = is_ctx ? ctx_end : P.Nb;
+                const int w_min = is_ctx ? seg_end : wave_lim_min;
+                const int w_max = is_ctx ? seg_end : wave_lim_max;
+#pragma unroll
+                for (int sb = 0; sb < SB; ++sb) {
+                    const int blk0 = kv0 + 32 * sb;
+                    if (blk0 >= w_max) continue;  // wave-uniform: nothing visible to this wavefront
+                    if (blk0 + 32 > w_min)
+                        block(stage_, sb, BoolTag<true>{}, blk0, is_ctx, seg_end);
+                    else
+                        block(stage_, sb, BoolTag<false>{}, blk0, is_ctx, seg_end);
+                }
+                if (it + 2 < n_tiles) stash_tile((stage_ + 2) % 3, st_a);
+            }
+        };
+
+        {
+            u32x4 qraw[QB][KS];
+            request_q(qraw);
+            if (n_tiles > 0) fetch_tile(0, st_a);
+            if (n_tiles > 1) fetch_tile(1, st_b);
+            scale_q(qraw);
+            if (n_tiles > 0) stash_tile(0, st_a);
+            if (n_tiles > 1) stash_tile(1, st_b);
+        }
+
+        int it = 0;
+        const int n_steady = n_main - 2;
+        while (it < n_steady) {  // stages as compile-time constants: every LDS offset is an immediate
+            tile(it, std::integral_constant<int, 0>{}, BoolTag<true>{});
+            if (++it >= n_steady) break;
+            tile(it, std::integral_constant<int, 1>{}, BoolTag<true>{});
+            if (++it >= n_steady) break;
+            tile(it, std::integral_constant<int, 2>{}, BoolTag<true>{});
+            ++it;
+        }
+        for (int stage = it % 3; it < n_tiles; ++it) {
+            tile(it, stage, BoolTag<false>{});
+            stage = stage == 2 ? 0 : stage + 1;
+        }
+        __syncthreads();
+        // row sums: query c of this lane's block sits in lane c % 16, register c / 16; the total
+        // already covers both halves, so only the hb = 0 lane carries it into the epilogue
+#pragma unroll
+        for (int j = 0; j < QB; ++j) {
+            const float r0 = lsum[j][0][0] + lsum[j][1][0], r1 = lsum[j][0][1] + lsum[j][1][1];
+            const float a0 = __shfl(r0, lane & 15, 64), a1 = __shfl(r1, lane & 15, 64);
+            l_run[j] = hb == 0 ? ((lane & 16) ? a1 : a0) : 0.f;
+        }
+    };
+
     bool robust = !Ops::kWideExponent || P.force_robust;
     if (!robust) {
-        fast_pass();
+        if constexpr (LEAN)
+            lean_pass();
+        else
+            fast_pass();
         bool bad = false;
 #pragma unroll
         for (int j = 0; j < QB; ++j) {

@@ -66,11 +66,11 @@ __device__ __forceinline__ void order_wait_device(unsigned *state, int side, uns
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 }
 
-__global__ __launch_bounds__(64) void order_signal_kernel(unsigned *counter) {
+static __global__ __launch_bounds__(64) void order_signal_kernel(unsigned *counter) {
     if (threadIdx.x == 0) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-__global__ __launch_bounds__(64) void order_gate_kernel(unsigned *state, int side, unsigned long long limit_ticks) {
+static __global__ __launch_bounds__(64) void order_gate_kernel(unsigned *state, int side, unsigned long long limit_ticks) {
     if (threadIdx.x == 0) order_wait_device(state, side, limit_ticks);
 }
 
