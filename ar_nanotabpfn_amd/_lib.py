@@ -80,6 +80,7 @@ SIGNATURES = {
     "artab_last_error": (ctypes.c_char_p, []),
     "artab_profile_begin": (_i, [_i]),
     "artab_profile_end": (_i, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_i)]),
+    "artab_bench_instruction_mix": (_i, [_i, _i, _i, _i, _sz, _p, _p, _p]),
     "artab_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
     "artab_context_attention": (_i, [_VP, _VP, _VP, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _p, _sz, _i, _p]),
     "artab_decode_attention": (
@@ -107,6 +108,7 @@ SIGNATURES = {
     "artab_order_signal": (_i, [_p, _i, _p]),
     "artab_order_wait": (_i, [_p, _i, ctypes.c_uint64, _p]),
     "artab_teacher_forcing_attention": (_i, [_VP, _VP, _VP, _VP, _VP, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
+    "artab_row_mask_attention": (_i, [_VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "artab_prefill_attention": (_i, [_VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "artab_buffer_attention": (_i, [_VP, _VP, _VP, _p, _i64, _i64, _i64, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _p]),
     "artab_merge_attention_outputs": (_i, [_VP, _p, _VP, _p, _VP, _i, _i, _i, _i, _i, _p]),
@@ -224,7 +226,6 @@ def check(status: int) -> None:
 
 
 _workspaces = {}
-_retired_workspaces = []  # outgrown scratch tensors: recorded graphs may still point at them
 _workspace_tag = 0
 
 
@@ -255,8 +256,18 @@ def workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
     key = (device.type, device.index if device.index is not None else torch.cuda.current_device(), _workspace_tag)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() * 4 < nbytes:
-        if ws is not None:
-            _retired_workspaces.append(ws)
+        # the outgrown tensor is dropped here; whoever recorded launches that point at it (a HIP
+        # graph) keeps it alive through ``held_workspace``
         ws = torch.empty((nbytes + 3) // 4, device=device, dtype=torch.float32)
         _workspaces[key] = ws
     return ws
+
+
+def held_workspace(device: torch.device, tag: Optional[int] = None) -> Optional[torch.Tensor]:
+    """The scratch tensor that calls on ``device`` under ``tag`` (default: the current tag) use at
+    the moment.  A caller that records such calls into a HIP graph keeps the returned tensor for as
+    long as the graph lives: the module itself lets go of a scratch tensor when a larger one is
+    needed."""
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device(),
+           _workspace_tag if tag is None else int(tag))
+    return _workspaces.get(key)

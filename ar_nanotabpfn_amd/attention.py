@@ -10,8 +10,8 @@ a tile schedule — with the same constructor names and the same caching:
 * ``DecodeMask`` (inference.py:500-523) and ``TeacherForcingMask``
   (inference.py:525-577) are built by the predictor.
 
-The training row mask (``create_row_mask``, attention.py:86-175) belongs to the
-training loop, which is outside this package.
+* ``create_row_mask`` (attention.py:86-175): the context / buffer / target mask of the
+  training forward, forward only (no backward pass exists in this package).
 """
 
 from __future__ import annotations
@@ -29,6 +29,7 @@ __all__ = [
     "DenseMask",
     "DecodeMask",
     "TeacherForcingMask",
+    "RowMask",
     "create_dense_mask",
     "create_context_self_attention_mask",
     "create_row_mask",
@@ -60,6 +61,31 @@ class TeacherForcingMask:
     num_targets: int
 
 
+@dataclass(frozen=True)
+class RowMask:
+    """Rows ``[context | buffer | target]`` of the training forward (attention.py:86-175):
+    everyone sees the context; buffer row j also sees buffers ``<= j``; target row with offset
+    ``o`` sees buffers ``<= o % buffer_len`` while ``o < attending_chunks * buffer_len``; target
+    keys are seen by nobody."""
+
+    num_rows: int
+    context_len: int
+    buffer_len: int
+    attending_chunks: int
+
+    def dense(self, device="cpu") -> Tensor:
+        """The mask as a ``[R, R]`` boolean tensor (True = attend), for inspection and tests."""
+        q = torch.arange(self.num_rows, device=device)[:, None]
+        kv = torch.arange(self.num_rows, device=device)[None, :]
+        Nc, Nb, A = self.context_len, self.buffer_len, self.attending_chunks
+        tstart = Nc + Nb
+        prefix = kv < Nc
+        ctx_buf = (q < tstart) & (kv < tstart) & (q >= kv)
+        off = q - tstart
+        tgt_buf = (q >= tstart) & (kv >= Nc) & (kv < tstart) & (off < A * Nb) & ((kv - Nc) <= off % max(Nb, 1))
+        return prefix | ctx_buf | tgt_buf
+
+
 _mask_cache = {}
 
 
@@ -77,11 +103,17 @@ def create_context_self_attention_mask(context_len: int, device="cuda") -> Dense
     return _mask_cache[key]
 
 
-def create_row_mask(*args, **kwargs):
-    raise NotImplementedError(
-        "create_row_mask builds the training-time context/buffer/target mask; training is not part of "
-        "this inference package."
-    )
+def create_row_mask(num_rows: int, context_len: int, buffer_len: int, attending_chunks=None,
+                    device="cuda") -> RowMask:
+    """Row mask with context / buffer / target sections (attention.py:86-175).  By default half
+    of the target chunks attend to the buffer: ``target_len // (2 * buffer_len)`` (:111-112)."""
+    target_len = num_rows - context_len - buffer_len
+    if attending_chunks is None:
+        attending_chunks = target_len // (2 * buffer_len)
+    key = ("row", num_rows, context_len, buffer_len, attending_chunks, str(device))
+    if key not in _mask_cache:
+        _mask_cache[key] = RowMask(num_rows, context_len, buffer_len, attending_chunks)
+    return _mask_cache[key]
 
 
 def clear_mask_cache() -> None:
@@ -109,13 +141,20 @@ class MultiheadAttention(nn.Module):
         B, S, _ = x.shape
         return x.view(B, S, self.n_heads, self.head_dim).transpose(1, 2)
 
-    def forward(self, q: Tensor, k: Tensor, v: Tensor, block_mask: DenseMask) -> Tuple[Tensor, Tuple[Tensor, Tensor]]:
-        if not isinstance(block_mask, DenseMask):
-            raise NotImplementedError("MultiheadAttention.forward runs dense self-attention; other masks go through the predictor")
+    def forward(self, q: Tensor, k: Tensor, v: Tensor, block_mask) -> Tuple[Tensor, Tuple[Tensor, Tensor]]:
+        if not isinstance(block_mask, (DenseMask, RowMask)):
+            raise NotImplementedError("MultiheadAttention.forward takes a DenseMask or a RowMask; decode and "
+                                      "teacher-forcing masks go through the predictor")
         B, Sq, D = q.shape
         qh = self.split_heads(self.q_proj(q))
         kh = self.split_heads(self.k_proj(k))
         vh = self.split_heads(self.v_proj(v))
+        if isinstance(block_mask, RowMask):
+            if kh.shape[2] != Sq or block_mask.num_rows != Sq:
+                raise ValueError("row mask expects num_rows queries and keys")
+            out = ak.row_mask_attention(qh, kh, vh, block_mask.context_len, block_mask.buffer_len,
+                                        block_mask.attending_chunks)
+            return self.out_proj(out.transpose(1, 2).reshape(B, Sq, D)), (kh, vh)
         if kh.shape[2] != Sq or block_mask.seq_len != Sq:
             raise ValueError("dense mask expects equally many queries and keys")
         out = ak.prefill_attention(qh, kh, vh)

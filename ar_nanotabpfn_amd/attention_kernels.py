@@ -42,6 +42,7 @@ __all__ = [
     "decode_attention",
     "teacher_forcing_attention",
     "prefill_attention",
+    "row_mask_attention",
 ]
 
 
@@ -444,6 +445,27 @@ def prefill_attention(
         lib.artab_prefill_attention(
             _lib.ref(qv), _lib.ref(kv), _lib.ref(vv), _lib.ref(ov), _lib.ref(kcv), _lib.ref(vcv), cache_batches,
             B, H, Nc, Dh, 0.0, _lib.dtype_code(q.dtype), _impl(use_triton), _lib.current_stream(dev),
+        )
+    )
+    return out
+
+
+def row_mask_attention(q: Tensor, k: Tensor, v: Tensor, context_len: int, buffer_len: int, attending_chunks: int,
+                       use_triton: bool = True) -> Tensor:
+    """Row attention of the training forward: ``q, k, v [B,H,R,D]`` with rows
+    ``[context | buffer | target]`` under the mask of ``create_row_mask``
+    (attention.py:86-175), carried as a tile schedule.  Forward only."""
+    dev = _lib.require_device(q, k, v)
+    lib = _lib.load()
+    B, H, R, Dh = q.shape
+    if k.shape != q.shape or v.shape != q.shape:
+        raise ValueError("row-mask attention expects q, k, v of one shape [B,H,R,D]")
+    out = _alloc_out(q)
+    qv, kv, vv, ov = _lib.view4(q), _lib.view4(k), _lib.view4(v), _lib.view4(out)
+    _lib.check(
+        lib.artab_row_mask_attention(
+            _lib.ref(qv), _lib.ref(kv), _lib.ref(vv), _lib.ref(ov), B, H, R, int(context_len), int(buffer_len),
+            int(attending_chunks), Dh, 0.0, _lib.dtype_code(q.dtype), _impl(use_triton), _lib.current_stream(dev),
         )
     )
     return out

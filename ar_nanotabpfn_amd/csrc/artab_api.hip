@@ -201,8 +201,15 @@ static hipError_t launch_stream_t(const DecodeParams &P, int Lq, hipStream_t str
     long per_cu = 2;  // what fits beside two workgroups of the context pass
     if (const char *e = getenv("ARTAB_STREAM_PER_CU")) per_cu = atol(e) >= 1 && atol(e) <= 4 ? atol(e) : per_cu;  // tuning hook
     dim3 grid(static_cast<unsigned>(tasks < per_cu * cus ? tasks : per_cu * cus)), block(64);
+    const int prio = env_int("ARTAB_STREAM_PRIO", 3);  // tuning aid
     if (Lq == 1)
         hipLaunchKernelGGL((decode_stream_kernel<T, 1>), grid, block, kStreamLdsBytes, stream, P);
+    else if (prio == 0)
+        hipLaunchKernelGGL((decode_stream_kernel<T, 2, 0>), grid, block, kStreamLdsBytes, stream, P);
+    else if (prio == 1)
+        hipLaunchKernelGGL((decode_stream_kernel<T, 2, 1>), grid, block, kStreamLdsBytes, stream, P);
+    else if (prio == 2)
+        hipLaunchKernelGGL((decode_stream_kernel<T, 2, 2>), grid, block, kStreamLdsBytes, stream, P);
     else
         hipLaunchKernelGGL((decode_stream_kernel<T, 2>), grid, block, kStreamLdsBytes, stream, P);
     return hipGetLastError();
@@ -866,6 +873,53 @@ int artab_teacher_forcing_attention(const artab_view *q, const artab_view *k_ctx
     F.mode = kFlashTeacher;
     ProfileScope prof(st);
     return launch_status(launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st), "teacher forcing (mfma)");
+}
+
+int artab_row_mask_attention(const artab_view *q, const artab_view *k, const artab_view *v, const artab_view *out,
+                             int B, int H, int R, int Nc, int Nb, int attending_chunks, int Dh, float scale,
+                             int dtype, int impl, void *stream) {
+    ARTAB_TRY(check_common(B, H, R, Dh, dtype));
+    if (Nc < 1 || Nb < 0 || Nc + Nb > R || attending_chunks < 0)
+        return fail(ARTAB_ERR_BAD_SHAPE, "row mask needs 1 <= Nc, 0 <= Nb, Nc + Nb <= R, attending_chunks >= 0 (got Nc=%d Nb=%d R=%d A=%d)",
+                    Nc, Nb, R, attending_chunks);
+    if (B == 0 || R == 0) return ARTAB_OK;
+    ARTAB_TRY(check_view(q, "q", dtype, true));
+    ARTAB_TRY(check_view(k, "k", dtype, true));
+    ARTAB_TRY(check_view(v, "v", dtype, true));
+    ARTAB_TRY(check_view(out, "out", dtype, true));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    scale = resolve_scale(scale, Dh);
+    const bool aligned = vec_aligned(q, dtype, Dh) && vec_aligned(k, dtype, Dh) && vec_aligned(v, dtype, Dh) &&
+                         vec_aligned(out, dtype, Dh);
+    const bool use_mfma = impl != ARTAB_IMPL_PORTABLE && mfma_shape_ok(dtype, Dh) && aligned;
+    if (impl == ARTAB_IMPL_MFMA && !use_mfma)
+        return fail(ARTAB_ERR_UNSUPPORTED, "MFMA path needs bf16/f16, head_dim in {32,64,128}, 16-byte aligned rows");
+    // buffer keys: rows [Nc, Nc + Nb) of the same tensors
+    View kb = dv(k), vb = dv(v);
+    kb.p += static_cast<size_t>(Nc) * k->stride_n * elem_size(dtype);
+    vb.p += static_cast<size_t>(Nc) * v->stride_n * elem_size(dtype);
+    if (!use_mfma) {
+        PortableParams P;
+        memset(&P, 0, sizeof(P));
+        P.q = dv(q); P.kc = dv(k); P.vc = dv(v); P.kb = kb; P.vb = vb; P.out = dv(out);
+        P.B = B; P.H = H; P.Lq = R; P.Nc = Nc; P.Nb = Nb;
+        P.rm_nc = Nc; P.rm_attend = attending_chunks;
+        P.new_row = -1; P.mode = kModeRowMask; P.Dh = Dh; P.scale = scale;
+        P.vec_ok = aligned ? 1 : 0;
+        return launch_status(launch_portable_dtype(P, dtype, st), "row-mask attention (portable)");
+    }
+    FlashPlan pl = plan_flash(B, H, R, Nc, Dh, /*stacked=*/false, /*allow_split=*/false);
+    FlashParams F;
+    memset(&F, 0, sizeof(F));
+    F.q = dv(q); F.kc = dv(k); F.vc = dv(v); F.kb = kb; F.vb = vb; F.out = dv(out);
+    F.B = B; F.H = H; F.Lq = R; F.Nc = Nc; F.Nb = Nb;
+    F.rm_nc = Nc; F.rm_attend = attending_chunks;
+    F.G = pl.G; F.tiles_per_group = pl.tiles_per_group; F.n_groups = pl.n_groups;
+    F.n_split = 1; F.kv_per_split = pl.kv_per_split;
+    F.qscale = scale * kLog2e;
+    F.mode = kFlashRowMask;
+    ProfileScope prof(st);
+    return launch_status(launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st), "row-mask attention (mfma)");
 }
 
 int artab_prefill_attention(const artab_view *q, const artab_view *k, const artab_view *v, const artab_view *out,

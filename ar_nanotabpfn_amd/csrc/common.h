@@ -144,4 +144,16 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
 // query i (< Nt) sees keys [0, i]; target query i (>= Nt) sees keys [0, i - Nt).
 __host__ __device__ __forceinline__ int tf_limit(int i, int Nt) { return i < Nt ? i + 1 : i - Nt; }
 
+// Visible-key limit among the Nb buffer keys of row i under the training row mask (rows are
+// [context Nc | buffer Nb | target ...], ar_tabpfn/model/attention.py:86-175): a context row sees
+// no buffer key, buffer row j sees keys [0, j], target row with offset o sees keys [0, o mod Nb]
+// while o < attend * Nb and none after that.  Every row sees the whole context; nobody sees a
+// target key.
+__host__ __device__ __forceinline__ int row_mask_limit(int i, int Nc, int Nb, int attend) {
+    if (i < Nc || Nb <= 0) return 0;
+    if (i < Nc + Nb) return i - Nc + 1;
+    const int o = i - Nc - Nb;
+    return o < attend * Nb ? o % Nb + 1 : 0;
+}
+
 }  // namespace artab

@@ -98,7 +98,7 @@ struct Mfma4<f16_t> {
 
 // One wavefront per workgroup; a task = 16 consecutive (trajectory, head) pairs; tasks are dealt
 // round-robin over the grid.  Dynamic LDS: kStreamLdsBytes.
-template <typename T, int LQ>
+template <typename T, int LQ, int PRIO = 3>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void decode_stream_kernel(DecodeParams P) {
     constexpr int DH = 32;
     constexpr int S = kStreamChunks;
@@ -142,7 +142,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
 
     // This wavefront shares its SIMD with two older, compute-bound ones; without a raised
     // priority it is only issued in their gaps.  It issues little: the priority costs them little.
-    __builtin_amdgcn_s_setprio(3);
+    __builtin_amdgcn_s_setprio(PRIO);
 
     // ---- producer: chunk `issue_g` of task `issue_task` into ring slot issue_slot.  Row pointers
     // are kept per task and advanced by four rows per chunk; only a task's last chunk (clamped

@@ -30,7 +30,12 @@ static hipError_t launch_flash_bm(const FlashParams &P, int BM, hipStream_t stre
         // the lean pass: 256 query rows as eight wavefronts of one 32-row block each, four
         // wavefronts per SIMD (ARTAB_LEAN=0 selects the software-pipelined form; tuning aid)
         if (BM == 256 && env_int("ARTAB_LEAN", 1) != 0) {
-            hipLaunchKernelGGL((flash_kernel<T, DH, 1, 8, kFlashBN, true>), dim3(grid), dim3(512), 0, stream, P);
+            // 96 registers (five per SIMD by the register file) leave room for the streaming
+            // buffer pass beside four of these wavefronts; ARTAB_LEAN_OCC=4 takes 128 (tuning aid)
+            if (env_int("ARTAB_LEAN_OCC", 5) == 4)
+                hipLaunchKernelGGL((flash_kernel<T, DH, 1, 8, kFlashBN, true, 4>), dim3(grid), dim3(512), 0, stream, P);
+            else
+                hipLaunchKernelGGL((flash_kernel<T, DH, 1, 8, kFlashBN, true, 5>), dim3(grid), dim3(512), 0, stream, P);
             return hipGetLastError();
         }
     }

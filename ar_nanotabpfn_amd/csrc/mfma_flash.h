@@ -78,7 +78,7 @@ struct MfmaOps<f16_t> {
     }
 };
 
-enum FlashMode : int { kFlashContext = 0, kFlashTeacher = 1, kFlashPrefill = 2 };
+enum FlashMode : int { kFlashContext = 0, kFlashTeacher = 1, kFlashPrefill = 2, kFlashRowMask = 3 };
 
 struct FlashParams {
     View q, kc, vc, kb, vb, out;
@@ -96,6 +96,7 @@ struct FlashParams {
     int n_split, kv_per_split;
     float qscale;  // softmax scale * log2(e), folded into Q
     int mode;
+    int rm_nc, rm_attend;  // row-mask mode: context rows in front of the Nb buffer rows, attending chunks
     int force_robust;  // 1: skip the fast path (testing the online-softmax path)
     unsigned *started;  // optional counter that the first thread of the grid advances at once: "the
                         // launches ahead of this one on its queue are complete" for a watcher on
@@ -130,8 +131,9 @@ struct BoolTag {
 
 // LEAN selects the fast pass: false = the software-pipelined loop (two wavefronts per SIMD, 216
 // registers), true = the plain loop built for four wavefronts per SIMD (see lean_pass).
-template <typename T, int DH, int QB, int NW, int BN, bool LEAN = false>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(LEAN ? 4 : 1)))
+// OCC: wavefronts per SIMD the register allocation is held to (1 = no constraint).
+template <typename T, int DH, int QB, int NW, int BN, bool LEAN = false, int OCC = 1>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 void flash_kernel(FlashParams P) {
     typedef MfmaOps<T> Ops;
     typedef typename Ops::vec vec;
@@ -154,6 +156,7 @@ void flash_kernel(FlashParams P) {
     auto k_stage = [&](int st_) -> T * { return kv_lds + st_ * STAGE; };
     auto v_stage = [&](int st_) -> T * { return kv_lds + st_ * STAGE + BN * KPAD; };
     __shared__ int redo_flag;
+    __shared__ int wg_lims[NW];
 
     // (release: whatever this queue's earlier launches wrote is visible to the watcher that sees
     // the new count)
@@ -270,6 +273,29 @@ void flash_kernel(FlashParams P) {
         }
 #pragma unroll
         for (int j = 0; j < QB; ++j) lim[j] = qi[j] >= 0 ? min(P.Nb, tf_limit(qi[j], P.Nt)) : 0;
+    } else if (P.mode == kFlashRowMask) {
+        // the limit is not monotone in the row here (targets count modulo Nb): the wavefront's and
+        // the workgroup's bounds come from reductions over the rows' own limits
+        int lo = P.Nb, hi = 0;
+#pragma unroll
+        for (int j = 0; j < QB; ++j) {
+            lim[j] = qi[j] >= 0 ? min(P.Nb, row_mask_limit(qi[j], P.rm_nc, P.Nb, P.rm_attend)) : 0;
+            lo = min(lo, lim[j]);
+            hi = max(hi, lim[j]);
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            lo = min(lo, __shfl_xor(lo, o, 64));
+            hi = max(hi, __shfl_xor(hi, o, 64));
+        }
+        wave_lim_min = __builtin_amdgcn_readfirstlane(lo);
+        wave_lim_max = __builtin_amdgcn_readfirstlane(hi);
+        if (lane == 0) wg_lims[wave] = wave_lim_max;
+        __syncthreads();
+        int wg_max = 0;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) wg_max = max(wg_max, wg_lims[w]);
+        buf_tiles = (wg_max + BN - 1) / BN;
     }
     const int n_tiles = ctx_tiles + buf_tiles;
 
@@ -727,6 +753,58 @@ void flash_kernel(FlashParams P) {
             }
         };
 
+        // In the steady state the tiles do not pass through registers at all: a stage is a whole
+        // number of KiB (K region and V region each), so it is filled by NI direct global->LDS
+        // loads of one KiB (lane l lands at base + 16 l), dealt over the wavefronts, each wholly
+        // inside K or inside V.  A lane whose 16 bytes fall into a row's padding re-reads the
+        // row's first piece (never used).  The loads are inline assembly: the compiler does not
+        // know of them and therefore does not drain them in front of every LDS read; they are
+        // waited for by hand (vmcnt) in front of the barrier that publishes their stage.
+        constexpr int STAGE_BYTES = STAGE * static_cast<int>(sizeof(T));
+        constexpr int NI = STAGE_BYTES / 1024, NKI = BN * KPAD * static_cast<int>(sizeof(T)) / 1024;
+        static_assert(STAGE_BYTES % 1024 == 0 && (BN * KPAD * sizeof(T)) % 1024 == 0, "stage must be whole KiB");
+        constexpr int NR = (NI + NW - 1) / NW;
+        static_assert(!LEAN || NR <= 2, "at most two direct loads per wavefront and tile");
+        const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(kv_lds));
+        unsigned d_off[NR];
+        const char *d_src[NR];
+        long d_step[NR];
+        int n_dma = 0;  // direct loads this wavefront issues per tile
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int i = wave + NW * r;  // scalar
+            const bool is_v = i >= NKI;
+            const View &src = is_v ? P.vc : P.kc;
+            const int byte = (i - (is_v ? NKI : 0)) * 1024 + lane * 16;
+            const int row_bytes = (is_v ? VPAD : KPAD) * static_cast<int>(sizeof(T));
+            const int row = byte / row_bytes;
+            int piece = (byte % row_bytes) / 16;
+            piece = piece < CPR ? piece : 0;
+            d_off[r] = static_cast<unsigned>(row * src.sn * static_cast<long>(sizeof(T)) + piece * 16);
+            d_step[r] = static_cast<long>(BN) * src.sn * static_cast<long>(sizeof(T));
+            // tiles 0 and 1 are requested by the prologue through registers
+            d_src[r] = reinterpret_cast<const char *>(view_row<T>(src, kvb, h, ctx_begin)) + 2 * d_step[r];
+            if (i < NI) ++n_dma;
+        }
+        auto dma_tile = [&](auto stage_) {
+#pragma unroll
+            for (int r = 0; r < NR; ++r) {
+                const int i = wave + NW * r;
+                if (i < NI) {
+                    const unsigned m0v = lds_base + stage_ * STAGE_BYTES + i * 1024;
+                    unsigned m0_saved;  // M0 (the LDS base of a direct load) is left as it was found
+                    asm volatile(
+                        "s_mov_b32 %0, m0\n\t"
+                        "s_mov_b32 m0, %1\n\t"
+                        "global_load_lds_dwordx4 %2, %3\n\t"
+                        "s_mov_b32 m0, %0"
+                        : "=&s"(m0_saved)
+                        : "s"(m0v), "v"(d_off[r]), "s"(d_src[r]));
+                }
+                d_src[r] += d_step[r];
+            }
+        };
+
         // Every other tile (the partial last context tile, buffer tiles of teacher forcing) goes
         // the general way: per-lane pointers, row guards, zero fill.
         const T *g_src[NP];
@@ -820,20 +898,28 @@ void flash_kernel(FlashParams P) {
             }
         };
 
-        // Tile `it` out of `stage_`: barrier, request tile it + 2, compute, store the requested
-        // tile into the stage that tile it - 1 has left.  STEADY: a full, unmasked context tile
-        // whose successor two ahead is one as well — no condition anywhere, one kind of request
-        // (a second kind of request in the same loop makes the compiler wait for the request
-        // before the tile's first LDS read).
+        // Tile `it` out of `stage_`: barrier, request tile it + 2 (into the stage that tile it - 1
+        // has left), compute.  STEADY: a full, unmasked context tile whose successor two ahead is
+        // one as well — no condition anywhere, the request is a direct global->LDS load.
+        // Otherwise the requested tile passes through registers and is stored after the compute.
         auto tile = [&](int it, auto stage_, auto steady_tag) {
             constexpr bool STEADY = decltype(steady_tag)::value;
-            __syncthreads();
             if constexpr (STEADY) {
-                main_fetch(st_a);
+                // this tile's direct loads (issued two tiles ago) must have landed; those of the
+                // next tile (issued one tile ago) may still be on their way
+                if (n_dma == 2)
+                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(2));
+                else if (n_dma == 1)
+                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(1));
+                else
+                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+                __syncthreads();
+                dma_tile((stage_ + 2) % 3);
 #pragma unroll
                 for (int sb = 0; sb < SB; ++sb) block(stage_, sb, BoolTag<false>{}, 0, true, 0);
-                stash_tile((stage_ + 2) % 3, st_a);
             } else {
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // direct loads of the steady state
+                __syncthreads();
                 if (it + 2 < n_tiles) fetch_tile(it + 2, st_a);
                 const bool is_ctx = it < ctx_tiles;
                 const int kv0 = is_ctx ? ctx_begin + it * BN : (it - ctx_tiles) * BN;

@@ -11,6 +11,7 @@ namespace artab {
 enum PortableMode : int {
     kModePlain = 0,    // every query row sees buffer keys [0, Nb)
     kModeTeacher = 1,  // per-row limit tf_limit(i, Nt)
+    kModeRowMask = 3,  // per-row limit row_mask_limit(i, rm_nc, Nb, rm_attend)
     kModeMasked = 2    // explicit uint8 mask over the buffer keys
 };
 
@@ -25,6 +26,7 @@ struct PortableParams {
     int new_row;  // buffer row index served from knew/vnew, or -1
     const int *nbuf_dev;  // decode: committed buffer length read at run time (overrides Nb / new_row)
     int capacity;         // rows the buffer cache holds (bound for a length read from nbuf_dev)
+    int rm_nc, rm_attend; // kModeRowMask: context rows in front of the buffer rows, attending chunks
     int append;   // copy knew/vnew to kb/vb[new_row]
     int mode;
     int Nt;
@@ -150,6 +152,7 @@ __global__ __launch_bounds__(kPortableWaves * 64) void portable_attention_kernel
     }
     int limit = P.Nb;
     if (P.mode == kModeTeacher) limit = min(P.Nb, tf_limit(i, P.Nt));
+    if (P.mode == kModeRowMask) limit = min(P.Nb, row_mask_limit(i, P.rm_nc, P.Nb, P.rm_attend));
     const T *knew_row = P.new_row >= 0 ? view_row<T>(P.knew, b, h, 0) : nullptr;
     const T *vnew_row = P.new_row >= 0 ? view_row<T>(P.vnew, b, h, 0) : nullptr;
     const uint8_t *mrow = P.mask ? P.mask + b * P.m_sb + h * P.m_sh + static_cast<long>(i) * P.m_sq : nullptr;

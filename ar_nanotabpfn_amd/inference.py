@@ -508,6 +508,8 @@ class ARTabPFNPredictor:
                 if self.steps_per_graph > 1 and cap - 1 >= self.steps_per_graph:
                     reset(st)
                     st.graph_many = self._record_steps(st, self.steps_per_graph)
+                # the recorded launches point into this scratch tensor: it lives as long as they do
+                st.workspace = _lib.held_workspace(device)
         gs.graph = gs.chains[0].graph
         for st in gs.chains:
             reset(st)

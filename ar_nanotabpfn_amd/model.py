@@ -298,11 +298,24 @@ class ARTabPFN(nn.Module):
         self.head = MixtureGaussianHead(d_model, d_ff, dim_y=1, num_components=num_components)
         self.ar_tokens = nn.Parameter(torch.randn(buffer_size, d_model) * 0.02)
 
-    def forward(self, *args, **kwargs):
-        raise NotImplementedError(
-            "the training forward (context/buffer/target row mask with a backward pass) is not part of this "
-            "inference package; use ARTabPFNPredictor.from_trained_model(model)"
-        )
+    @torch.no_grad()
+    def forward(self, x_context: Tensor, y_context: Tensor, x_buffer: Tensor, y_buffer: Tensor, x_target: Tensor,
+                mask_features, mask_rows, y_target: Optional[Tensor] = None):
+        """The training objective, forward only (model.py:317-369): context, buffer and target rows
+        in one pass under the row mask of ``create_row_mask``; returns the mean negative
+        log-likelihood of ``y_target`` (None without it).  The attention runs on the device kernels,
+        which have no backward pass: the call is always under ``no_grad``."""
+        ctx_emb = self.embedder.embed_context(x_context, y_context)
+        buf_emb = self.embedder.embed_buffer(x_buffer, y_buffer) + self.ar_tokens[: x_buffer.size(1)]
+        tgt_emb = self.embedder.embed_target(x_target)
+        Nc, Nb = ctx_emb.size(1), buf_emb.size(1)
+        embeddings = torch.cat([ctx_emb, buf_emb, tgt_emb], dim=1).unsqueeze(2)
+        z, _ = self.backbone(embeddings, mask_features, mask_rows)
+        z_target = z[:, Nc + Nb:, 0, :]
+        if y_target is not None and y_target.dim() == 2:
+            y_target = y_target.unsqueeze(-1)
+        loss, _, _, _ = self.head(z_target, y_target)
+        return loss
 
     # ---- checkpoints written by the reference's training loop (train.py:336-343): a dict
     # {"step": int, "model": state_dict}.  With `compile_model` the embedder and the head were

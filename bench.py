@@ -25,6 +25,8 @@ Prints one JSON line:
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
        python bench.py --kernel-shapes   (instead: one decode layer-step at the shapes of
                                           configs[1], [3] and [4], timings on stderr)
+       python bench.py --mix-ceiling     (instead: the instruction mix of one 32x32 score block from
+                                          registers: what the SIMD's issue port allows)
 """
 
 from __future__ import annotations
@@ -100,10 +102,38 @@ def run_decode(pred, x_context, y_context, x_target, steps, device, dtype):
     return ev[0].elapsed_time(ev[1]), ev[2].elapsed_time(ev[3]), wall_ms
 
 
-def cpu_decode_baseline(model, x_context, y_context, x_target, sample_steps=(1, 128)):
-    """The numpy oracle on the host: prefill is skipped (random K/V of the right shape
-    stand in for the context cache: attention cost does not depend on values), then one
-    decode step at each buffer length in `sample_steps` with B=1024."""
+def host_info():
+    """Cores, thread counts and CPU model of the host the CPU legs run on."""
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    blas = None
+    try:
+        from threadpoolctl import threadpool_info
+
+        blas = max((int(d.get("num_threads", 0)) for d in threadpool_info()), default=None)
+    except Exception:
+        pass
+    return {"cpu_model": model, "os_cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads(),
+            "blas_threads": blas}
+
+
+CPU_DECODE_B = 256            # trajectories of the CPU sample (a quarter of the batch; a step is linear in B)
+CPU_DECODE_NBUF = (1, 128, 255)
+
+
+def cpu_decode_baseline(model, x_context, y_context, x_target, n_bufs=CPU_DECODE_NBUF, b_sample=CPU_DECODE_B):
+    """The numpy oracle (float32) on the host: one full 12-layer decode step of `b_sample`
+    trajectories at each buffer length in `n_bufs`, one warm-up and the median of three timed runs
+    each; the context K/V are random tensors of the right shape (the prefill is not part of the
+    timed GPU region either, and attention cost does not depend on values).  Returns seconds per
+    step of the FULL batch (the sample's median scaled by B / b_sample) averaged over `n_bufs`."""
     from oracle import model_oracle as mo
 
     sd = {k: v.detach().float().cpu().numpy() for k, v in model.state_dict().items()}
@@ -111,25 +141,30 @@ def cpu_decode_baseline(model, x_context, y_context, x_target, sample_steps=(1, 
     op = mo.OraclePredictor(om, "shared")
     H, Dh, L = CFG3["n_heads"], CFG3["d_model"] // CFG3["n_heads"], CFG3["n_layers"]
     rng = np.random.default_rng(0)
-    xt = x_target[:, :2].float().cpu().numpy()
-    times = []
-    for n in sample_steps:
-        op.init_kv_cache(B3, NT3)
-        op.context_len = NC3
-        op.k_ctx = [rng.standard_normal((H, NC3, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
-        op.v_ctx = [rng.standard_normal((H, NC3, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
-        op.k_buf = [rng.standard_normal((B3, H, n - 1, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
-        op.v_buf = [rng.standard_normal((B3, H, n - 1, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
-        op.buffer_len = n - 1
+    xt = x_target[:b_sample, :2].float().cpu().numpy()
+    k_ctx = [rng.standard_normal((H, NC3, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
+    v_ctx = [rng.standard_normal((H, NC3, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
+    per_n = []
+    for n in n_bufs:
+        k_buf = [rng.standard_normal((b_sample, H, n - 1, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
+        v_buf = [rng.standard_normal((b_sample, H, n - 1, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
         emb = np.concatenate(
-            [om.embed_buffer(xt[:, 0:1], np.zeros((B3, 1), np.float32)) + om.ar_tokens[n % om.ar_tokens.shape[0]],
+            [om.embed_buffer(xt[:, 0:1], np.zeros((b_sample, 1), np.float32)) + om.ar_tokens[n % om.ar_tokens.shape[0]],
              om.embed_target(xt[:, 1:2])], axis=1)
-        t0 = time.perf_counter()
-        z = op.transformer_decode(emb, commit=1)
-        om.head_parameterize(z[:, -1:])
-        times.append(time.perf_counter() - t0)
-        log(f"[cpu] decode step at n_buf={n}: {times[-1]:.2f} s")
-    return float(np.mean(times)), list(sample_steps)
+        times = []
+        for rep in range(4):  # the first run is the warm-up
+            op.init_kv_cache(b_sample, NT3)
+            op.context_len, op.k_ctx, op.v_ctx = NC3, k_ctx, v_ctx
+            op.k_buf, op.v_buf, op.buffer_len = list(k_buf), list(v_buf), n - 1
+            t0 = time.perf_counter()
+            z = op.transformer_decode(emb, commit=1)
+            om.head_parameterize(z[:, -1:])
+            if rep:
+                times.append(time.perf_counter() - t0)
+        per_n.append(float(np.median(times)) * (B3 / b_sample))
+        log(f"[cpu] decode step at n_buf={n}: median {np.median(times):.2f} s for {b_sample} trajectories "
+            f"-> {per_n[-1]:.2f} s for {B3}")
+    return float(np.mean(per_n)), per_n
 
 
 def log_density_bench(device, dtype, model, with_cpu):
@@ -163,16 +198,25 @@ def log_density_bench(device, dtype, model, with_cpu):
     if with_cpu:
         from oracle import model_oracle as mo
 
+        # host leg: the numpy oracle in float32 on a bounded sample (the first 16 of the 64
+        # datasets; datasets are independent, so the evaluation is linear in their number), one
+        # warm-up and the median of three timed runs, scaled to the 64 datasets
         sd = {k: v.detach().float().cpu().numpy() for k, v in model.state_dict().items()}
         om = mo.OracleModel(sd, CFG3["n_heads"], compute=np.float32)
-        a32 = [t.float().cpu().numpy() for t in args]
-        t0 = time.perf_counter()
-        ll_cpu = mo.OraclePredictor(om, "per_dataset").evaluate_joint_density(*a32)
-        cpu_s = time.perf_counter() - t0
-        d = np.abs(ll.float().cpu().numpy() - ll_cpu)
+        n_cpu = 16
+        a32 = [t[:n_cpu].float().cpu().numpy() for t in args]
+        times = []
+        for rep in range(4):
+            t0 = time.perf_counter()
+            ll_cpu = mo.OraclePredictor(om, "per_dataset").evaluate_joint_density(*a32)
+            if rep:
+                times.append(time.perf_counter() - t0)
+        cpu_s = float(np.median(times)) * (B2 / n_cpu)
+        d = np.abs(ll[:n_cpu].float().cpu().numpy() - ll_cpu)
         res.update(cpu_s=round(cpu_s, 3), speedup=round(cpu_s * 1e3 / gpu_ms, 1),
-                   mean_abs_dlogp_vs_cpu_f32=float(d.mean()))
-        log(f"[cpu] configs[2] log-density: {cpu_s:.2f} s  (GPU {gpu_ms:.2f} ms)")
+                   cpu_sample=f"numpy float32 oracle on {n_cpu} of the {B2} datasets, 1 warm-up + median of 3, x{B2 // n_cpu}",
+                   mean_abs_dlogp_vs_cpu_f32=float(d.mean()), max_abs_dlogp_vs_cpu_f32=float(d.max()))
+        log(f"[cpu] configs[2] log-density: {cpu_s:.2f} s for {B2} datasets (from {n_cpu})  (GPU {gpu_ms:.2f} ms)")
     return res
 
 
@@ -237,6 +281,50 @@ def kernel_shapes(device):
     print(json.dumps({"kernel_shapes": out}))
 
 
+def mix_ceiling(device):
+    """The instruction mix of one 32x32 score block of the head_dim-32 kernel, issued from registers
+    with no memory traffic (``artab_bench_instruction_mix``): the rate the SIMD's issue port allows,
+    for the software-pipelined pass (row sum on v_dot2c) and the lean pass (row sum on the matrix
+    pipe), on constant and on random operands, with two and four wavefronts per SIMD."""
+    import ctypes
+
+    from ar_nanotabpfn_amd import _lib
+
+    lib = _lib.load()
+    iters = 20000
+    names = {0: "pipelined pass: 4 mfma32 + 16 exp + 8 cvt + 8 dot2c", 1: "lean pass: 4 mfma32 + 2 mfma16 + 16 exp + 8 cvt",
+             2: "matrix instructions of the lean pass alone", 3: "vector instructions of the lean pass alone"}
+    rows = []
+    for waves, lds in ((2, 64 * 1024), (4, 36 * 1024)):  # LDS per workgroup fixes how many share a CU
+        wgs = 256 * waves
+        out = torch.empty(wgs * 256, device=device, dtype=torch.float32)
+        stamps = torch.zeros(wgs * 4 * 2, device=device, dtype=torch.int64)
+        for rnd in (0, 1):
+            for variant in (0, 1, 2, 3):
+                def launch():
+                    _lib.check(lib.artab_bench_instruction_mix(variant, rnd, wgs, iters, lds, ctypes.c_void_p(out.data_ptr()),
+                                                               ctypes.c_void_p(stamps.data_ptr()), _lib.current_stream(device)))
+                launch()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                launch()
+                e1.record()
+                torch.cuda.synchronize()
+                ms = e0.elapsed_time(e1)
+                st = stamps.view(-1, 2).double()
+                ghz = float((st[:, 0] / st[:, 1]).mean()) * 0.1  # shader cycles per 10 ns tick
+                ns_block = ms * 1e6 / (iters * waves)            # per SIMD and block
+                tflops = 4 * 32768.0 * 1024 / ns_block / 1e3 if variant != 3 else None
+                rows.append(dict(variant=names[variant], data="random" if rnd else "constant", waves_per_simd=waves,
+                                 ns_per_block=round(ns_block, 1), cycles_per_block=round(ns_block * ghz, 1),
+                                 clock_ghz=round(ghz, 2), tflops_equivalent=round(tflops, 1) if tflops else None,
+                                 frac_of_peak=round(tflops / MFMA_BF16_PEAK_TFLOPS, 3) if tflops else None))
+                log(f"[mix] {names[variant]:58s} {'random' if rnd else 'const ':6s} data, {waves} waves/SIMD: {ns_block:6.1f} ns/block "
+                    f"= {ns_block * ghz:5.0f} cycles at {ghz:.2f} GHz" + (f", {tflops:6.0f} TFLOP/s-equivalent" if tflops else ""))
+    print(json.dumps({"mix_ceiling": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -249,6 +337,8 @@ def main():
                     help="order the two streams of the recorded step with events instead of device-side counters")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only copy a 256 MiB buffer five times (reference kernel for scaling HBM counters)")
+    ap.add_argument("--mix-ceiling", action="store_true",
+                    help="only run the instruction mix of one score block from registers (issue-port ceiling of the kernel)")
     ap.add_argument("--kernel-shapes", action="store_true",
                     help="only time one decode layer-step at the attention shapes of configs[1], [3], [4]")
     args = ap.parse_args()
@@ -275,6 +365,9 @@ def main():
     lib = _lib.load()  # fails loudly when the extension is not built
     if args.kernel_shapes:
         kernel_shapes(torch.device("cuda:0"))
+        return
+    if args.mix_ceiling:
+        mix_ceiling(torch.device("cuda:0"))
         return
     device, dtype = torch.device("cuda:0"), torch.bfloat16
     model = build_model(device, dtype)
@@ -385,14 +478,20 @@ def main():
     }
 
     if not args.no_cpu:
-        cpu_s, sample = cpu_decode_baseline(model, x_context, y_context, x_target)
+        cpu_s, per_n = cpu_decode_baseline(model, x_context, y_context, x_target)
+        host = host_info()
         out["cpu_baseline"] = {
             "value": round(1.0 / cpu_s, 4),
             "unit": "target-steps/s",
-            "cores": os.cpu_count() if not os.environ.get("OMP_NUM_THREADS") else int(os.environ["OMP_NUM_THREADS"]),
+            "cores": host["blas_threads"] or host["torch_threads"],
             "kind": "port",
-            "sample": f"numpy float32 oracle, one full 12-layer decode step (B=1024, N_ctx=16384) at each of "
-                      f"N_buf={sample}, mean; context K/V random (prefill skipped)",
+            "dtype": "f32",
+            "sample": f"numpy float32 oracle (a port of the reference's arithmetic), one full 12-layer decode step "
+                      f"(N_ctx=16384) of {CPU_DECODE_B} of the {B3} trajectories at each of N_buf={list(CPU_DECODE_NBUF)}: "
+                      f"1 warm-up + median of 3, scaled x{B3 // CPU_DECODE_B} to the batch, mean over N_buf; "
+                      f"context K/V random (the prefill is outside the timed GPU region as well)",
+            "seconds_per_step_by_n_buf": [round(t, 3) for t in per_n],
+            "host": host,
         }
     else:
         out["cpu_baseline"] = None

@@ -86,6 +86,23 @@ const char *artab_last_error(void);
 int artab_profile_begin(int max_records);
 int artab_profile_end(double *total_ms, int *records);
 
+/*
+ * Benchmark aid without a counterpart in the reference: the instruction mix of one 32x32 score
+ * block of the head_dim-32 attention kernel (ar_tabpfn/model/triton_kernels.py:131-162 is the
+ * loop it stands for), issued from registers with no memory traffic, to measure what the SIMD's
+ * issue port alone allows.  `workgroups` workgroups of four wavefronts run `iters` (even)
+ * iterations; `lds_bytes` of dynamic LDS per workgroup fixes how many share a compute unit.
+ *   variant 0: 4 MFMA 32x32x16 + 16 exp2 + 8 cvt_pk + 8 dot2c    (software-pipelined pass)
+ *   variant 1: 4 MFMA 32x32x16 + 2 MFMA 16x16x32 + 16 exp2 + 8 cvt_pk   (lean pass)
+ *   variant 2: the matrix instructions of variant 1 alone; 3: its vector instructions alone
+ * random_data != 0 fills the operands with pseudo-random bf16 values instead of constants.
+ *   out     float32 [workgroups * 256] (written, contents meaningless)
+ *   stamps  uint64 [workgroups * 4][2] or NULL: per wavefront, shader cycles and 100 MHz ticks spent
+ * The call only launches on `stream`; the caller times it.
+ */
+int artab_bench_instruction_mix(int variant, int random_data, int workgroups, int iters, size_t lds_bytes,
+                                float *out, unsigned long long *stamps, void *stream);
+
 /* Bytes of workspace the split-context paths need for the given problem
  * (artab_context_attention, artab_decode_attention).  0 means no workspace is
  * needed.  Pure host arithmetic, no device access. */
@@ -312,6 +329,20 @@ int artab_prefill_attention(const artab_view *q, const artab_view *k, const arta
                             const artab_view *k_cache, const artab_view *v_cache, int cache_batches,
                             int B, int H, int Nc, int Dh, float scale, int dtype,
                             int impl, void *stream);
+
+/*
+ * Row attention of the training forward under the context / buffer / target mask.
+ * Replaces flex_attention under create_row_mask (ar_tabpfn/model/attention.py:86-175), as called
+ * by the training forward (ar_tabpfn/model/model.py:317-369 through :95-126).  Rows are
+ * [context Nc | buffer Nb | target R - Nc - Nb]; q, k, v, out are [B,H,R,Dh].  The mask is a tile
+ * schedule, not a tensor: every row sees the Nc context keys; buffer row j also sees buffer keys
+ * [0, j]; target row with offset o sees buffer keys [0, o mod Nb] while o < attending_chunks * Nb
+ * and no buffer key after that; target keys are never visited (no self-attention of targets).
+ * Forward only.  Nc >= 1.
+ */
+int artab_row_mask_attention(const artab_view *q, const artab_view *k, const artab_view *v, const artab_view *out,
+                             int B, int H, int R, int Nc, int Nb, int attending_chunks, int Dh, float scale,
+                             int dtype, int impl, void *stream);
 
 /*
  * Buffer attention with log-sum-exp and an optional boolean mask.

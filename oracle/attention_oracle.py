@@ -30,6 +30,10 @@ live in ``tests/test_oracle.py``):
 * ``hybrid_attention`` / ``hybrid_teacher_forcing_attention``: pinned by
   equality with masked full attention (tests/test_triton_kernel.py:157-198,
   :288-339).
+* ``row_mask`` (training forward): pinned against the second, region-wise statement of
+  the same mask that the reference holds (tests/visualize_masks.py:57-85), by the
+  closed-form pair count, by a hand-written tiny case, and through the training loss
+  the reference itself computed for the fixture (tests/golden/tiny_model.npz).
 """
 
 from __future__ import annotations
@@ -49,6 +53,8 @@ __all__ = [
     "hybrid_teacher_forcing_attention",
     "decode_mask",
     "teacher_forcing_mask",
+    "row_mask",
+    "row_mask_attention",
     "masked_full_attention",
     "dense_self_attention",
     "decode_step_attention",
@@ -252,6 +258,46 @@ def teacher_forcing_mask(num_cached: int, num_targets: int) -> np.ndarray:
     target_idx = q_idx - Nt
     target_to_buffer = kv_is_buffer & (buffer_kv_idx < target_idx)
     return attends_context | (is_buffer_query & buffer_causal) | (is_target_query & target_to_buffer)
+
+
+def row_mask(num_rows: int, context_len: int, buffer_len: int, attending_chunks: Optional[int] = None) -> np.ndarray:
+    """Dense ``[R, R]`` form of the training row mask over ``[context | buffer | target]`` rows.
+
+    attention.py:86-175, the three mask_mods that are or-ed (:165-169): ``prefix_mask``
+    (kv < context_len, :127-129), ``localized_causal_ctx_buf`` (q and kv below
+    context_len + buffer_len and q >= kv, :131-136) and ``chunked_target_buffer`` (q a target,
+    kv a buffer, target offset below attending_chunks * buffer_len, buffer offset <=
+    target offset mod buffer_len, :138-160).  attending_chunks defaults to
+    target_len // (2 * buffer_len) (:111-112).
+    """
+    target_len = num_rows - context_len - buffer_len
+    if attending_chunks is None:
+        attending_chunks = target_len // (2 * buffer_len)
+    target_start = context_len + buffer_len
+    q_idx = np.arange(num_rows)[:, None]
+    kv_idx = np.arange(num_rows)[None, :]
+    prefix = kv_idx < context_len
+    ctx_buf_end = context_len + buffer_len
+    localized = (q_idx < ctx_buf_end) & (kv_idx < ctx_buf_end) & (q_idx >= kv_idx)
+    q_in_target = q_idx >= target_start
+    kv_in_buffer = (kv_idx >= context_len) & (kv_idx < target_start)
+    target_offset = q_idx - target_start
+    buffer_offset = kv_idx - context_len
+    in_attending_region = target_offset < attending_chunks * buffer_len
+    chunk_position = target_offset % max(buffer_len, 1)
+    chunked = q_in_target & kv_in_buffer & in_attending_region & (buffer_offset <= chunk_position)
+    return prefix | localized | chunked
+
+
+def row_mask_attention(q, k, v, context_len: int, buffer_len: int, attending_chunks: Optional[int] = None,
+                       compute=np.float64):
+    """Row attention of the training forward: one masked softmax over all rows under
+    ``row_mask`` (flex_attention with the BlockMask of attention.py:86-175, as called at
+    attention.py:57-59).  ``q, k, v [B,H,R,D]``; returns ``out``."""
+    R = q.shape[2]
+    mask = row_mask(R, context_len, buffer_len, attending_chunks)[None, None]
+    out, _ = buffer_attention(q, k, v, mask=mask, compute=compute)
+    return out
 
 
 def masked_full_attention(q, k_full, v_full, mask=None, scale=None, compute=np.float64):

@@ -153,6 +153,27 @@ class OracleModel:
         return ll.sum(axis=-1)
 
 
+def training_forward(m: "OracleModel", x_context, y_context, x_buffer, y_buffer, x_target, y_target,
+                     attending_chunks: Optional[int] = None):
+    """The training forward of model.py:317-369: context, buffer (+ ar_tokens[:Nb], :347-350)
+    and target rows concatenated (:355), the stack under the row mask, the target rows of the
+    normed output (:362) into the head; returns ``(loss, z_target)`` with the loss the mean
+    negative log-likelihood over all targets (model.py:251-261 without a loss mask)."""
+    ctx = m.embed_context(x_context, y_context)
+    buf = m.embed_buffer(x_buffer, y_buffer) + m.ar_tokens[: x_buffer.shape[1]]
+    tgt = m.embed_target(x_target)
+    Nc, Nb = ctx.shape[1], buf.shape[1]
+    x = np.concatenate([ctx, buf, tgt], axis=1)
+    for i in range(m.n_layers):
+        x_row = m.feature_stage(i, x)
+        q, k, v = m.qkv(i, x_row)
+        attn = ao.row_mask_attention(q, k, v, Nc, Nb, attending_chunks, compute=m.compute)
+        x = m.post_attention(i, x_row, attn)
+    z_target = m.final_norm(x)[:, Nc + Nb:]
+    ll = m.head_log_likelihood(z_target, y_target)
+    return float(-ll.mean()), z_target
+
+
 class OraclePredictor:
     """State machine of inference.py:32-453 with both cache layouts.
 

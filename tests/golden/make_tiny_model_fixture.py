@@ -11,7 +11,8 @@ container only (the reference checkout is not available elsewhere):
 Contents: weights (float32), x/y context and targets, teacher-forced log-density for
 the per-dataset ("flex_attention") and shared ("triton_shared_context") backends, and
 the per-step target representation of a decode with prescribed buffer values under
-the reference's sampling rule for AR tokens.
+the reference's sampling rule for AR tokens, and the training forward (context, buffer and
+target rows in one pass under ``create_row_mask``): its loss and the target rows' output.
 """
 
 import os
@@ -84,6 +85,23 @@ def main(ref_root: str) -> None:
                 zs.append(p.transformer_decode(emb, commit=commit)[:, -1:])
             out[f"z_decode_{name}"] = torch.cat(zs, dim=1).numpy()
             clear(model)
+
+        # training forward under the row mask (model.py:317-369, attention.py:86-175): buffer_size
+        # buffer rows, 4 * buffer_size target rows (two of the four chunks attend to the buffer)
+        from ar_tabpfn.model.attention import create_dense_mask, create_row_mask  # noqa: E402
+
+        Nb, Ntr = cfg["buffer_size"], 4 * cfg["buffer_size"]
+        g = torch.Generator().manual_seed(3)
+        x_buf, y_buf = torch.randn(B, Nb, F, generator=g), torch.randn(B, Nb, generator=g)
+        x_trn, y_trn = torch.randn(B, Ntr, F, generator=g), torch.randn(B, Ntr, generator=g)
+        mask_rows = create_row_mask(Nc + Nb + Ntr, Nc, Nb, device="cpu")
+        mask_feat = create_dense_mask(1, device="cpu")
+        loss = model(x_ctx, y_ctx, x_buf, y_buf, x_trn, mask_feat, mask_rows, y_target=y_trn)
+        out.update(train_x_buf=x_buf.numpy(), train_y_buf=y_buf.numpy(), train_x_tgt=x_trn.numpy(),
+                   train_y_tgt=y_trn.numpy(), train_loss=np.array(float(loss)))
+        # the same pass with three attending chunks
+        mask3 = create_row_mask(Nc + Nb + Ntr, Nc, Nb, attending_chunks=3, device="cpu")
+        out["train_loss_attend3"] = np.array(float(model(x_ctx, y_ctx, x_buf, y_buf, x_trn, mask_feat, mask3, y_target=y_trn)))
 
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tiny_model.npz")
     np.savez_compressed(path, **out)

@@ -63,3 +63,20 @@ def test_oracle_fixed_buffer_decode_matches_reference(fx, backend):
         xc, yc = np.repeat(xc[0:1], B, axis=0), np.repeat(yc[0:1], B, axis=0)
     z = mo.OraclePredictor(m, backend).fixed_buffer_decode(xc, yc, data["x_tgt"], data["y_tgt"], ar_rule="sampling")
     np.testing.assert_allclose(z, data[f"z_decode_{backend}"], atol=2e-5, rtol=0)
+
+
+def test_training_forward_matches_reference_fixture():
+    """The training forward under the row mask (model.py:317-369, attention.py:86-175): the loss
+    the reference computed for the fixture, with the default and with three attending chunks."""
+    from oracle import model_oracle as mo
+
+    data = np.load(FIXTURE, allow_pickle=False)
+    sd = {k[3:]: data[k] for k in data.files if k.startswith("w::")}
+    om = mo.OracleModel(sd, int(data["cfg"][1]))
+    args = (data["x_ctx"], data["y_ctx"], data["train_x_buf"], data["train_y_buf"], data["train_x_tgt"], data["train_y_tgt"])
+    loss, z = mo.training_forward(om, *args)
+    assert z.shape == (3, 16, 32)
+    assert abs(loss - float(data["train_loss"])) <= 2e-5
+    loss3, _ = mo.training_forward(om, *args, attending_chunks=3)
+    assert abs(loss3 - float(data["train_loss_attend3"])) <= 2e-5
+    assert abs(loss - loss3) > 1e-4  # the attending region matters

@@ -116,8 +116,15 @@ def test_model_tree_and_state_dict_keys():
     assert m.ar_tokens.shape == (4, 32) and m.head.head[2].out_features == 9
     a = m.backbone.layers[0].attn_rows
     assert (a.n_heads, a.head_dim, a.scale) == (2, 16, 16 ** -0.5)
-    with pytest.raises(NotImplementedError):
-        m()
+    # the training forward exists (forward only) and runs on the device kernels: CPU tensors raise
+    from ar_nanotabpfn_amd.attention import create_dense_mask, create_row_mask
+
+    rm = create_row_mask(2 + 4 + 16, 2, 4, device="cpu")
+    assert (rm.num_rows, rm.context_len, rm.buffer_len, rm.attending_chunks) == (22, 2, 4, 2)  # 16 // (2 * 4)
+    assert create_row_mask(22, 2, 4, device="cpu") is rm  # cached, as in attention.py:113-121
+    z = torch.zeros
+    with pytest.raises(RuntimeError):
+        m(z(1, 2, 3), z(1, 2), z(1, 4, 3), z(1, 4), z(1, 16, 3), create_dense_mask(1, "cpu"), rm, y_target=z(1, 16))
 
 
 def test_reference_checkpoint_format_loads(tmp_path):
@@ -221,5 +228,8 @@ def test_mask_descriptors_are_cached():
     assert att.create_context_self_attention_mask(9, "cpu").seq_len == 9
     att.clear_mask_cache()
     assert att.create_dense_mask(5, "cpu") is not a
-    with pytest.raises(NotImplementedError):
-        att.create_row_mask(10, 4, 2)
+    r = att.create_row_mask(10, 4, 2)  # target_len 4 -> 4 // (2 * 2) = 1 attending chunk
+    assert r.attending_chunks == 1 and r is att.create_row_mask(10, 4, 2)
+    dense = r.dense()
+    assert dense.shape == (10, 10) and bool(dense[:, :4].all()) and not bool(dense[:, 6:].any())
+    assert dense[6].tolist() == [True] * 5 + [False] * 5 and dense[8].tolist() == [True] * 4 + [False] * 6

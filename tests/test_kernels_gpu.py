@@ -1163,3 +1163,42 @@ def test_layer_kernels_wait_for_the_side_queue_themselves(device, monkeypatch, t
         assert torch.equal(got_out[s], ref_out[s]), f"step {s}"
     for (k0, v0), (k1, v1) in zip(ref_caches, got_caches):
         assert torch.equal(k0, k1) and torch.equal(v0, v1)
+
+
+# ----- a buffer length read from device memory never takes an access outside the cache ---------------
+
+
+@pytest.mark.parametrize("dtype,schedule", [(torch.float32, "portable"), (torch.bfloat16, "sequential"),
+                                            (torch.bfloat16, "two streams")])
+@pytest.mark.parametrize("cell", [8, 9, 100, -3])
+def test_decode_device_length_beyond_capacity_stays_inside_the_cache(device, dtype, schedule, cell):
+    """A recorded launch replayed once more than the cache has slots (or a cell that was never
+    reset) hands the kernels a length the host never validated.  They clamp it to the capacity:
+    rows behind the cache keep their contents, a new row that has no slot is not stored, and the
+    call completes.  capacity = 8 rows; the cache is a view into a larger tensor whose remaining
+    rows are the guard."""
+    ak = _ak()
+    B, H, D, Nc, cap, guard = 33, 8, 32, 700, 8, 4
+    q = randn((B, H, 2, D), 1, dtype, 0.5).to(device)
+    kc, vc = randn((H, Nc, D), 2, dtype, 0.5).to(device), randn((H, Nc, D), 3, dtype, 0.5).to(device)
+    kbig = randn((B, H, cap + guard, D), 4, dtype, 0.5).to(device)
+    vbig = randn((B, H, cap + guard, D), 5, dtype, 0.5).to(device)
+    kb, vb = kbig[:, :, :cap], vbig[:, :, :cap]
+    k0, v0 = kbig.clone(), vbig.clone()
+    kn, vn = randn((B, H, 1, D), 6, dtype, 0.5).to(device), randn((B, H, 1, D), 7, dtype, 0.5).to(device)
+    nbuf = torch.full((1,), cell, device=device, dtype=torch.int32)
+    side = torch.cuda.Stream(device=device) if schedule == "two streams" else None
+    out = ak.decode_attention(q, kc, vc, kb, vb, cap - 1, kn, vn, n_buf_device=nbuf, side_stream=side)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    assert torch.equal(kbig[:, :, cap:], k0[:, :, cap:]) and torch.equal(vbig[:, :, cap:], v0[:, :, cap:])
+    # nothing inside the cache changed either: no slot exists for the new row at these lengths
+    assert torch.equal(kbig, k0) and torch.equal(vbig, v0)
+    # with the largest valid length the same call does append, in the last slot
+    nbuf.fill_(cap - 1)
+    out = ak.decode_attention(q, kc, vc, kb, vb, cap - 1, kn, vn, n_buf_device=nbuf, side_stream=side)
+    torch.cuda.synchronize()
+    assert torch.equal(kbig[:, :, cap - 1], kn[:, :, 0]) and torch.equal(kbig[:, :, cap:], k0[:, :, cap:])
+    ref, _, _ = ao.decode_step_attention(to_np(q), to_np(kc), to_np(vc), to_np(k0[:, :, : cap - 1]),
+                                         to_np(v0[:, :, : cap - 1]), to_np(kn), to_np(vn))
+    assert max_abs(to_np(out), ref) <= out_tol(dtype)

@@ -389,3 +389,68 @@ def test_feature_stage_equals_single_key_attention():
     att = att.transpose(0, 2, 1, 3).reshape(6, 1, 16) @ sd["backbone.layers.0.attn_features.out_proj.weight"].T
     ref = mo._layer_norm(att + xf, sd["backbone.layers.0.norm1.weight"], sd["backbone.layers.0.norm1.bias"])
     np.testing.assert_allclose(m.feature_stage(0, x).reshape(6, 1, 16), ref, atol=1e-12)
+
+
+# ----- training row mask (attention.py:86-175) ---------------------------------------------------------
+
+
+def _row_mask_by_regions(C, B, T, attending_chunks=None):
+    """The second statement of the mask that the reference holds: region by region, as
+    tests/visualize_masks.py:57-85 composes it for its figure."""
+    total = C + B + T
+    if attending_chunks is None:
+        attending_chunks = T // (2 * B)
+    M, N = np.meshgrid(np.arange(total), np.arange(total), indexing="ij")
+    q_ctx, k_ctx = M < C, N < C
+    q_buf, k_buf = (M >= C) & (M < C + B), (N >= C) & (N < C + B)
+    q_tgt = M >= C + B
+    causal = M >= N
+    tgt_buf = q_tgt & k_buf & ((M - C - B) < attending_chunks * B) & ((N - C) <= (M - C - B) % max(B, 1))
+    return (q_ctx & k_ctx) | (q_buf & k_buf & causal) | (q_tgt & k_ctx) | (q_buf & k_ctx) | tgt_buf
+
+
+@pytest.mark.parametrize("C,B,T,A", [(7, 4, 16, None), (1, 1, 2, None), (5, 3, 12, 0), (5, 3, 12, 4), (64, 8, 32, 1), (3, 8, 16, None)])
+def test_row_mask_two_statements_agree(C, B, T, A):
+    m = ao.row_mask(C + B + T, C, B, A)
+    assert m.shape == (C + B + T, C + B + T)
+    assert np.array_equal(m, _row_mask_by_regions(C, B, T, A))
+    a = T // (2 * B) if A is None else A
+    # closed-form pair count: everyone sees the context; buffers are causal among themselves;
+    # each of the first min(a*B, T) target rows sees (offset mod B) + 1 buffers
+    n_att = min(a * B, T)
+    full, rest = divmod(n_att, B)
+    expect = (C + B + T) * C + B * (B + 1) // 2 + full * B * (B + 1) // 2 + rest * (rest + 1) // 2
+    assert int(m.sum()) == expect
+    assert not m[:, C + B:].any()          # nobody sees a target key, not even itself
+    assert not m[:C, C:].any()             # the context sees the context only
+
+
+def test_row_mask_tiny_case_by_hand():
+    # rows: c0 c1 | b0 b1 | t0 t1 t2 t3, one attending chunk (targets t0, t1)
+    X, o = True, False
+    expect = np.array([
+        [X, X, o, o, o, o, o, o],
+        [X, X, o, o, o, o, o, o],
+        [X, X, X, o, o, o, o, o],
+        [X, X, X, X, o, o, o, o],
+        [X, X, X, o, o, o, o, o],   # t0: buffers <= 0
+        [X, X, X, X, o, o, o, o],   # t1: buffers <= 1
+        [X, X, o, o, o, o, o, o],   # t2: outside the attending region
+        [X, X, o, o, o, o, o, o],
+    ])
+    assert np.array_equal(ao.row_mask(8, 2, 2, 1), expect)
+    assert np.array_equal(ao.row_mask(8, 2, 2), expect)  # default: 4 // (2 * 2) = 1
+
+
+def test_row_mask_attention_equals_per_row_softmax():
+    rng = np.random.default_rng(0)
+    C, B, T, D = 5, 3, 6, 8
+    R = C + B + T
+    q, k, v = (rng.standard_normal((2, 2, R, D)) for _ in range(3))
+    out = ao.row_mask_attention(q, k, v, C, B)
+    m = ao.row_mask(R, C, B)
+    for r in (0, C, C + B - 1, C + B, C + B + 2, R - 1):
+        keys = np.nonzero(m[r])[0]
+        s = np.einsum("bhd,bhkd->bhk", q[:, :, r], k[:, :, keys]) / np.sqrt(D)
+        p = scipy.special.softmax(s, axis=-1)
+        assert np.abs(out[:, :, r] - np.einsum("bhk,bhkd->bhd", p, v[:, :, keys])).max() <= 1e-12
