@@ -160,6 +160,7 @@ void flash_kernel(FlashParams P) {
 
     // (release: whatever this queue's earlier launches wrote is visible to the watcher that sees
     // the new count)
+    if (LEAN && threadIdx.x == 0) redo_flag = 0;  // raised after the pass, at least one barrier later
     if (P.started && blockIdx.x == 0 && threadIdx.x == 0)
         __hip_atomic_fetch_add(P.started, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 
@@ -905,16 +906,28 @@ void flash_kernel(FlashParams P) {
         auto tile = [&](int it, auto stage_, auto steady_tag) {
             constexpr bool STEADY = decltype(steady_tag)::value;
             if constexpr (STEADY) {
+                // Two workgroups share a compute unit and the hardware serves the older wavefront
+                // first: left alone, one workgroup runs ahead and the other finishes the slice with
+                // the SIMDs half empty.  The priority falls with progress, so whoever is behind is
+                // served first (measured: the slower workgroup of a pair ends 2.5 us earlier).
+                if (it == n_main / 4)
+                    __builtin_amdgcn_s_setprio(2);
+                else if (it == n_main / 2)
+                    __builtin_amdgcn_s_setprio(1);
+                else if (it == 3 * n_main / 4)
+                    __builtin_amdgcn_s_setprio(0);
                 // this tile's direct loads (issued two tiles ago) must have landed; those of the
                 // next tile (issued one tile ago) may still be on their way
-                if (n_dma == 2)
-                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(2));
-                else if (n_dma == 1)
-                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(1));
-                else
+                // (the slice's last tile has no successor in flight)
+                const bool more = it + 2 < n_main;
+                if (it + 1 == n_main || n_dma == 0)
                     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+                else if (n_dma == 2)
+                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(2));
+                else
+                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(1));
                 __syncthreads();
-                dma_tile((stage_ + 2) % 3);
+                if (more) dma_tile((stage_ + 2) % 3);
 #pragma unroll
                 for (int sb = 0; sb < SB; ++sb) block(stage_, sb, BoolTag<false>{}, 0, true, 0);
             } else {
@@ -939,6 +952,7 @@ void flash_kernel(FlashParams P) {
             }
         };
 
+        __builtin_amdgcn_s_setprio(3);
         {
             u32x4 qraw[QB][KS];
             request_q(qraw);
@@ -950,7 +964,9 @@ void flash_kernel(FlashParams P) {
         }
 
         int it = 0;
-        const int n_steady = n_main - 2;
+        // with nothing but full context tiles the whole slice is steady state; otherwise its last
+        // two full tiles already request tiles of the other kind and take the general route
+        const int n_steady = n_tiles == n_main ? n_main : n_main - 2;
         while (it < n_steady) {  // stages as compile-time constants: every LDS offset is an immediate
             tile(it, std::integral_constant<int, 0>{}, BoolTag<true>{});
             if (++it >= n_steady) break;
@@ -963,7 +979,6 @@ void flash_kernel(FlashParams P) {
             tile(it, stage, BoolTag<false>{});
             stage = stage == 2 ? 0 : stage + 1;
         }
-        __syncthreads();
         // row sums: query c of this lane's block sits in lane c % 16, register c / 16; the total
         // already covers both halves, so only the hb = 0 lane carries it into the epilogue
 #pragma unroll
@@ -986,10 +1001,17 @@ void flash_kernel(FlashParams P) {
             const float l_tot = l_run[j] + __shfl_xor(l_run[j], 32, 64);
             bad = bad || !(l_tot > kFastMassMin && l_tot < kFastMassMax);
         }
-        if (tid == 0) redo_flag = 0;
-        __syncthreads();
-        if (bad) redo_flag = 1;
-        __syncthreads();
+        if constexpr (LEAN) {
+            // the pass ends without a barrier of its own: this one also separates its last LDS
+            // reads from the stores of a second, robust pass
+            if (bad) redo_flag = 1;
+            __syncthreads();
+        } else {
+            if (tid == 0) redo_flag = 0;
+            __syncthreads();
+            if (bad) redo_flag = 1;
+            __syncthreads();
+        }
         robust = redo_flag != 0;
     }
     if (robust) run_pass(BoolTag<true>{});
