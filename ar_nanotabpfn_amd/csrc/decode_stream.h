@@ -2,8 +2,9 @@
 //
 // The context pass of a decode step is bound by the vector and matrix units and leaves HBM idle;
 // the buffer pass streams B*H*n_buf*128 bytes and needs almost no arithmetic.  To run the two side
-// by side the buffer pass has to fit in what two resident context-pass wavefronts leave on a SIMD
-// (80 registers, one wavefront) and must not compete for vector-ALU issue slots.  Hence:
+// by side the buffer pass has to fit in what the resident context-pass wavefronts leave on a SIMD
+// (four of them at 96 registers leave 128: one wavefront) and must not compete for vector-ALU
+// issue slots.  Hence:
 //
 //  * dot products on the matrix pipe with v_mfma_f32_4x4x4 (16 independent 4x4x4 products per
 //    instruction): one block = one (trajectory, head) pair, lane 4p+i of a wavefront is
@@ -17,19 +18,22 @@
 //    (8 cycles each) and 16 LDS reads per 4 keys x 16 pairs.
 //  * loads land in LDS, not in registers: every wavefront keeps a ring of 8 KiB chunks (4 keys x
 //    16 pairs x K and V) filled by direct global->LDS loads (16 bytes per lane, lane l lands at
-//    chunk + 16 l), three chunks in flight while one is consumed, and reads a chunk back
-//    lane-locally (K) or transposed (V).
+//    chunk + 16 l), three chunks in flight while two are being read, and reads a chunk back
+//    lane-locally (K) or transposed (V).  The wavefront is alone with its latencies, so the LDS
+//    reads run one chunk ahead of the arithmetic that uses them.
 //
 // Output per (pair, query): normalised partial result in the input type + float32 LSE, i.e. one
 // more "context slice" for the combine step; the new row is appended to the cache on the way.
 #pragma once
+
+#include <type_traits>
 
 #include "common.h"
 #include "decode_buffer.h"
 
 namespace artab {
 
-constexpr int kStreamChunks = 4;           // ring depth per wavefront
+constexpr int kStreamChunks = 3;           // ring depth per wavefront
 constexpr int kStreamDeepRows = 224;       // buffers longer than this use the whole ring
 constexpr int kStreamChunkBytes = 8192;    // 4 keys x 16 pairs x (64 B of K + 64 B of V)
 constexpr int kStreamQBytes = 4096;        // one task's queries: 4 x (64 lanes x 16 B)
@@ -37,45 +41,64 @@ constexpr size_t kStreamLdsBytes = kStreamChunks * kStreamChunkBytes + 2 * kStre
 
 // LDS reads of the ring go through inline assembly: the compiler must not see an LDS read that
 // could alias the asynchronous fills, or it would drain every load before each read.
-// Two 16-byte pieces of this lane's K row (addr_k, +1024) and of its query row (addr_q, +1024):
-// one LDS round trip.
-__device__ __forceinline__ void lds_read_kq(u32x4 &k0, u32x4 &k1, u32x4 &q0, u32x4 &q1, unsigned addr_k,
-                                            unsigned addr_q) {
+// A read is issued by one statement and waited for by another, with arithmetic in between: the
+// wait names the registers as in/out operands, so every use of them is ordered behind it.
+// Four 16-byte pieces of this lane's row (a K row of a chunk, a query row): pieces 1 KiB apart.
+__device__ __forceinline__ void lds_issue_k(u32x4 (&k)[4], unsigned addr) {
     asm volatile(
         "ds_read_b128 %0, %4\n\t"
-        "ds_read_b128 %2, %5\n\t"
         "ds_read_b128 %1, %4 offset:1024\n\t"
-        "ds_read_b128 %3, %5 offset:1024\n\t"
-        "s_waitcnt lgkmcnt(0)"
-        : "=&v"(k0), "=&v"(k1), "=&v"(q0), "=&v"(q1)
-        : "v"(addr_k), "v"(addr_q)
+        "ds_read_b128 %2, %4 offset:2048\n\t"
+        "ds_read_b128 %3, %4 offset:3072"
+        : "=&v"(k[0]), "=&v"(k[1]), "=&v"(k[2]), "=&v"(k[3])
+        : "v"(addr)
         : "memory");
 }
-__device__ __forceinline__ void lds_read2x128(u32x4 &a, u32x4 &b, unsigned addr) {
+__device__ __forceinline__ void lds_read4x128(u32x4 (&k)[4], unsigned addr) {
     asm volatile(
-        "ds_read_b128 %0, %2\n\t"
-        "ds_read_b128 %1, %2 offset:1024\n\t"
+        "ds_read_b128 %0, %4\n\t"
+        "ds_read_b128 %1, %4 offset:1024\n\t"
+        "ds_read_b128 %2, %4 offset:2048\n\t"
+        "ds_read_b128 %3, %4 offset:3072\n\t"
         "s_waitcnt lgkmcnt(0)"
-        : "=&v"(a), "=&v"(b)
+        : "=&v"(k[0]), "=&v"(k[1]), "=&v"(k[2]), "=&v"(k[3])
         : "v"(addr)
         : "memory");
 }
 __device__ __forceinline__ void lds_write128(unsigned addr, u32x4 v) {
     asm volatile("ds_write_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : : "v"(addr), "v"(v) : "memory");
 }
-// Four transposing reads: the V operands of four 4-dim groups of one 4-key chunk.
+// Eight transposing reads: the V operands of the eight 4-dim groups of one 4-key chunk.
 // Address layout of a V chunk: sub-slot t (1 KiB) holds dims 8t..8t+7, so group u = 2t + half
-// sits at t * 1024 + 8 * half; one call covers sub-slots t and t + 1.
-__device__ __forceinline__ void lds_read4_tr(u32x2 (&v)[4], unsigned addr) {
+// sits at t * 1024 + 8 * half.
+__device__ __forceinline__ void lds_issue_v(u32x2 (&v)[8], unsigned addr) {
     asm volatile(
-        "ds_read_b64_tr_b16 %0, %4\n\t"
-        "ds_read_b64_tr_b16 %1, %4 offset:8\n\t"
-        "ds_read_b64_tr_b16 %2, %4 offset:1024\n\t"
-        "ds_read_b64_tr_b16 %3, %4 offset:1032\n\t"
-        "s_waitcnt lgkmcnt(0)"
-        : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3])
+        "ds_read_b64_tr_b16 %0, %8\n\t"
+        "ds_read_b64_tr_b16 %1, %8 offset:8\n\t"
+        "ds_read_b64_tr_b16 %2, %8 offset:1024\n\t"
+        "ds_read_b64_tr_b16 %3, %8 offset:1032\n\t"
+        "ds_read_b64_tr_b16 %4, %8 offset:2048\n\t"
+        "ds_read_b64_tr_b16 %5, %8 offset:2056\n\t"
+        "ds_read_b64_tr_b16 %6, %8 offset:3072\n\t"
+        "ds_read_b64_tr_b16 %7, %8 offset:3080"
+        : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
         : "v"(addr)
         : "memory");
+}
+__device__ __forceinline__ void lds_wait(u32x4 (&k)[4], u32x2 (&v)[8]) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(k[0]), "+v"(k[1]), "+v"(k[2]), "+v"(k[3]), "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]),
+                   "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])
+                 :
+                 : "memory");
+}
+
+// The lane index again, as a value the compiler cannot trace: what the rare steps of the loop
+// derive from it (pair, row, base addresses) is then computed where it is used instead of being
+// kept in registers across the steps that are not rare.
+__device__ __forceinline__ int opaque(int v) {
+    asm volatile("" : "+v"(v));
+    return v;
 }
 
 template <typename T>
@@ -99,7 +122,7 @@ struct Mfma4<f16_t> {
 // One wavefront per workgroup; a task = 16 consecutive (trajectory, head) pairs; tasks are dealt
 // round-robin over the grid.  Dynamic LDS: kStreamLdsBytes.
 template <typename T, int LQ, int PRIO = 3>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void decode_stream_kernel(DecodeParams P) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void decode_stream_kernel(DecodeParams P) {
     constexpr int DH = 32;
     constexpr int S = kStreamChunks;
     extern __shared__ __attribute__((aligned(16))) unsigned char stream_lds[];
@@ -155,8 +178,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
     const T *p_k = nullptr, *p_v = nullptr;  // this lane's row of the chunk to be requested next
     auto issue_one = [&]() {
         const bool first = issue_g == 0, last = issue_g + 1 == n_groups;  // wavefront-uniform
-        int p_b = 0, p_h = 0;
+        int p_b = 0, p_h = 0, pl = 0, sub = 0;
         if (first || last) {  // the (trajectory, head) of this lane's pair: twice per task at most
+            const int ln = opaque(lane);
+            pl = ln >> 2;
+            sub = ln & 3;
             int pair = 16 * issue_task + pl;
             pair = pair < n_pairs ? pair : n_pairs - 1;  // a ragged last task re-reads the last pair; never stored
             p_b = pair / H;
@@ -205,64 +231,56 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
     // next door needs for its own tiles; a buffer that is finished before that pass anyway uses
     // half the ring and disturbs it less (measured at B=1024, H=8: 950 -> 974 steps/s; a quarter of
     // the ring is too little: 933).  A long one is on the critical path itself.
-    const int depth = n_total > P.deep_rows ? S : S / 2;
+    const int depth = S;
     for (int i = 0; i < depth; ++i)
         if (may_issue()) issue_one();
 
-    // ---- consumer
+    // ---- consumer.  The LDS reads of a chunk are split in time so that no read is waited for right
+    // after it is issued (the wavefront has nobody to hide a round trip behind but itself): the K
+    // rows of chunk c + 1 and the V rows of chunk c are requested early in step c and arrive while
+    // the softmax of chunk c (whose K rows came in during step c - 1) is computed; the queries sit
+    // in registers for the whole task.
     float m = -INFINITY, mq = 0.f, l = 0.f;  // running maximum of the raw scores, and times qscale
     f32x4 o[8];  // output dims 4u..4u+3 of this lane's query
 #pragma unroll
     for (int u = 0; u < 8; ++u) o[u] = f32x4{0.f, 0.f, 0.f, 0.f};
     int task = blockIdx.x, g = 0, slot = 0, qsel = 0;
     const int new_group = has_new && slot_fits ? n_buf >> 2 : -1;  // the chunk that holds the row to append
-    for (int c = 0; c < total_chunks; ++c) {
-        // chunk c must have landed; only the chunks requested after it (8 loads each) may be pending
+    u32x4 qr[4];  // this lane's query row (zero for lanes that stand for no query)
+    u32x4 kr[4];  // the K rows of the chunk whose scores come next
+
+    // chunk `c` must have landed; only the chunks requested after it (8 loads each: 4 for the K
+    // rows, then 4 for the V rows) may be pending
+    auto wait_chunk = [&](int c) {
         switch (issued - c - 1) {
             case 3: __builtin_amdgcn_s_waitcnt(vmcnt_imm(24)); break;
             case 2: __builtin_amdgcn_s_waitcnt(vmcnt_imm(16)); break;
             case 1: __builtin_amdgcn_s_waitcnt(vmcnt_imm(8)); break;
             default: __builtin_amdgcn_s_waitcnt(vmcnt_imm(0)); break;
         }
-        const unsigned chunk = lds0 + static_cast<unsigned>(slot) * kStreamChunkBytes;
-        const unsigned qaddr = q_lds0 + static_cast<unsigned>(qsel) * kStreamQBytes + lane * 16u;
-
-        // ---- scores of 4 keys for this lane's query, head dims in two halves (register budget)
+    };
+    // the same for the K rows of chunk `c` alone: its V rows may be pending as well
+    auto wait_chunk_k = [&](int c) {
+        switch (issued - c - 1) {
+            case 3: __builtin_amdgcn_s_waitcnt(vmcnt_imm(28)); break;
+            case 2: __builtin_amdgcn_s_waitcnt(vmcnt_imm(20)); break;
+            case 1: __builtin_amdgcn_s_waitcnt(vmcnt_imm(12)); break;
+            default: __builtin_amdgcn_s_waitcnt(vmcnt_imm(4)); break;
+        }
+    };
+    // ---- the arithmetic of one chunk, shared by the two kinds of step below
+    auto scores = [&]() {
         f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            u32x4 k0, k1, q0, q1;
-            lds_read_kq(k0, k1, q0, q1, chunk + 2048u * half + lane * 16u, qaddr + 2048u * half);
-            s = Mfma4<T>::mma(u32x2{k0[0], k0[1]}, u32x2{q0[0], q0[1]}, s);
-            s = Mfma4<T>::mma(u32x2{k0[2], k0[3]}, u32x2{q0[2], q0[3]}, s);
-            s = Mfma4<T>::mma(u32x2{k1[0], k1[1]}, u32x2{q1[0], q1[1]}, s);
-            s = Mfma4<T>::mma(u32x2{k1[2], k1[3]}, u32x2{q1[2], q1[3]}, s);
+        for (int e = 0; e < 4; ++e) {
+            s = Mfma4<T>::mma(u32x2{kr[e][0], kr[e][1]}, u32x2{qr[e][0], qr[e][1]}, s);
+            s = Mfma4<T>::mma(u32x2{kr[e][2], kr[e][3]}, u32x2{qr[e][2], qr[e][3]}, s);
         }
-        if (g == new_group) {
-            // in-place append (once per task): the lane that holds the new row copies it from the
-            // chunk, lane-locally, into slot n_buf of the cache
-            const int pair = 16 * task + pl;
-            if (4 * g + sub == n_buf && pair < n_pairs) {
-                const int b = pair / H, h = pair % H;
-                T *kd = view_row<T>(vkb, b, h, n_buf), *vd = view_row<T>(vvb, b, h, n_buf);
-#pragma unroll
-                for (int half = 0; half < 2; ++half) {
-                    u32x4 k0, k1, v0, v1;
-                    lds_read2x128(k0, k1, chunk + 2048u * half + lane * 16u);
-                    lds_read2x128(v0, v1, chunk + 4096u + 2048u * half + lane * 16u);
-                    *reinterpret_cast<u32x4 *>(kd + 16 * half) = k0;
-                    *reinterpret_cast<u32x4 *>(kd + 16 * half + 8) = k1;
-                    *reinterpret_cast<u32x4 *>(vd + 16 * half) = v0;
-                    *reinterpret_cast<u32x4 *>(vd + 16 * half + 8) = v1;
-                }
-            }
-        }
-        float sc[4] = {s[0], s[1], s[2], s[3]};  // raw dot products; qscale (> 0) enters with the exponent
-        if (g + 1 == n_groups) {  // only a task's last chunk can hold keys past the end
-#pragma unroll
-            for (int r = 0; r < 4; ++r) sc[r] = 4 * g + r < n_total ? sc[r] : -INFINITY;
-        }
-        // online softmax; the rescale is skipped (wavefront-uniformly) while no maximum moves
+        return s;
+    };
+    // online softmax of four raw dot products (qscale > 0 enters with the exponent); the rescale is
+    // skipped (wavefront-uniformly) while no maximum moves.  Returns the packed probabilities.
+    auto softmax = [&](const float (&sc)[4]) {
         const float m_new = max3(max3(m, sc[0], sc[1]), sc[2], sc[3]);
         if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
             const float alpha = m == -INFINITY ? 0.f : fast_exp2((m - m_new) * qscale);
@@ -276,13 +294,93 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
 #pragma unroll
         for (int r = 0; r < 4; ++r) p[r] = fast_exp2(fmaf(sc[r], qscale, -mq));  // m is finite here: key 4g is always valid
         l += (p[0] + p[1]) + (p[2] + p[3]);
-        const u32x2 pop = {pack2<T>(p[0], p[1]), pack2<T>(p[2], p[3])};
+        return u32x2{pack2<T>(p[0], p[1]), pack2<T>(p[2], p[3])};
+    };
+
+    // ---- a step in the middle of a task, for consumer and producer alike (no query fetch, no
+    // ragged or new row, nothing to store, ring full): nothing is decided at run time, the waits
+    // are constants.  D chunks are live at its start: c .. c + D - 1.
+    auto steady_step = [&](auto depth_tag) {
+        constexpr int D = decltype(depth_tag)::value;
+        const unsigned chunk = lds0 + static_cast<unsigned>(slot) * kStreamChunkBytes;
+        u32x2 vop[8];
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(8 * (D - 1)));  // chunk c has landed
+        lds_issue_v(vop, chunk + 4096u + tr_off);
+        const f32x4 s = scores();
+        slot = slot + 1 == S ? 0 : slot + 1;
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(8 * (D - 2) + 4));  // and the K rows of chunk c + 1
+        lds_issue_k(kr, lds0 + static_cast<unsigned>(slot) * kStreamChunkBytes + lane * 16u);
+        const float sc[4] = {s[0], s[1], s[2], s[3]};
+        const u32x2 pop = softmax(sc);
+        lds_wait(kr, vop);
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            u32x2 vop[4];
-            lds_read4_tr(vop, chunk + 4096u + 2048u * half + tr_off);
+        for (int u = 0; u < 8; ++u) o[u] = Mfma4<T>::mma(vop[u], pop, o[u]);
+        unsigned char *cd = stream_lds + issue_slot * kStreamChunkBytes;
+        load_row64_to_lds(p_k, cd);
+        load_row64_to_lds(p_v, cd + 4096);
+        p_k += chunk_step;
+        p_v += chunk_step_v;
+        issue_slot = issue_slot + 1 == S ? 0 : issue_slot + 1;
+    };
+
+    if (total_chunks == 0) return;
+    wait_chunk_k(0);
+    lds_read4x128(kr, lds0 + lane * 16u);
+    int c = 0;
+    while (c < total_chunks) {
+        // how many steady steps lie ahead: consumer and producer both strictly inside a task
+        if (g >= 1 && issue_g >= 1 && issued - c == depth && issue_seq <= seq + 1) {
+            int run = n_groups - 1 - (g > issue_g ? g : issue_g);
+            if (new_group >= g && new_group - g < run) run = new_group - g;
+            if (run > 0) {
+                for (int r = 0; r < run; ++r) steady_step(std::integral_constant<int, S>{});
+                c += run;
+                g += run;
+                issue_g += run;
+                issued += run;
+                continue;
+            }
+        }
+        const unsigned chunk = lds0 + static_cast<unsigned>(slot) * kStreamChunkBytes;
+        const bool more = c + 1 < total_chunks;
+        if (g == 0) lds_read4x128(qr, q_lds0 + static_cast<unsigned>(qsel) * kStreamQBytes + lane * 16u);
+        u32x2 vop[8];
+        wait_chunk(c);
+        lds_issue_v(vop, chunk + 4096u + tr_off);
+        const f32x4 s = scores();
+        // the products have taken their operands: the same registers receive the next chunk's rows
+        if (more) {
+            wait_chunk_k(c + 1);
+            const int nslot = slot + 1 == S ? 0 : slot + 1;
+            lds_issue_k(kr, lds0 + static_cast<unsigned>(nslot) * kStreamChunkBytes + lane * 16u);
+        }
+        float sc[4] = {s[0], s[1], s[2], s[3]};
+        if (g + 1 == n_groups) {  // only a task's last chunk can hold keys past the end
 #pragma unroll
-            for (int u = 0; u < 4; ++u) o[4 * half + u] = Mfma4<T>::mma(vop[u], pop, o[4 * half + u]);
+            for (int r = 0; r < 4; ++r) sc[r] = 4 * g + r < n_total ? sc[r] : -INFINITY;
+        }
+        const u32x2 pop = softmax(sc);
+        lds_wait(kr, vop);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) o[u] = Mfma4<T>::mma(vop[u], pop, o[u]);
+
+        if (g == new_group) {
+            // in-place append (once per task): the lane that holds the new row copies it from the
+            // chunk, lane-locally, into slot n_buf of the cache
+            const int ln = opaque(lane), pl = ln >> 2, sub = ln & 3;
+            const int pair = 16 * task + pl;
+            if (4 * g + sub == n_buf && pair < n_pairs) {
+                const int b = pair / H, h = pair % H;
+                T *kd = view_row<T>(vkb, b, h, n_buf), *vd = view_row<T>(vvb, b, h, n_buf);
+                u32x4 kk[4], vv[4];
+                lds_read4x128(kk, chunk + lane * 16u);
+                lds_read4x128(vv, chunk + 4096u + lane * 16u);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    *reinterpret_cast<u32x4 *>(kd + 8 * e) = kk[e];
+                    *reinterpret_cast<u32x4 *>(vd + 8 * e) = vv[e];
+                }
+            }
         }
         // the chunk has been read: refill its slot (and any the producer had to leave empty)
         if (g + 1 == n_groups) ++seq;
@@ -291,6 +389,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
         slot = slot + 1 == S ? 0 : slot + 1;
         if (++g == n_groups) {
             // ---- task done: write this lane's partial (lanes of real queries of real pairs)
+            const int ln = opaque(lane), pl = ln >> 2, sub = ln & 3;
             const int pair = 16 * task + pl;
             if (pair < n_pairs && sub < LQ) {
                 const float inv = l > 0.f ? 1.f / l : 0.f;
@@ -313,6 +412,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(6))) void de
             task += gridDim.x;
             qsel ^= 1;
         }
+        ++c;
     }
 }
 

@@ -152,7 +152,8 @@ void flash_kernel(FlashParams P) {
     // three stages; a stage is the K tile followed by the V tile, so that both have the same
     // stage stride and a stage index folds into the immediate offset of every LDS access
     constexpr int STAGE = BN * KPAD + BN * VPAD;
-    __shared__ __attribute__((aligned(16))) T kv_lds[3 * STAGE];
+    constexpr int NST = LEAN ? 4 : 3;  // stages: tiles are requested NST - 1 ahead at most
+    __shared__ __attribute__((aligned(16))) T kv_lds[NST * STAGE];
     auto k_stage = [&](int st_) -> T * { return kv_lds + st_ * STAGE; };
     auto v_stage = [&](int st_) -> T * { return kv_lds + st_ * STAGE + BN * KPAD; };
     __shared__ int redo_flag;
@@ -696,7 +697,7 @@ void flash_kernel(FlashParams P) {
     //    row 1 (lanes 0..15, registers 0 and 1).  Two such products per block replace eight
     //    v_dot2c (which, issued between MFMAs, cost five times their nominal four cycles).
     //  * K and V tiles of a stage are one list of 16-byte pieces dealt over the whole workgroup.
-    // Three LDS stages, one barrier per tile, tiles requested two ahead (as in fast_pass).
+    // Four LDS stages, one barrier per tile, full tiles requested three ahead.
     auto lean_pass = [&]() {
         f32x4 lsum[QB][2];
 #pragma unroll
@@ -899,10 +900,13 @@ void flash_kernel(FlashParams P) {
             }
         };
 
-        // Tile `it` out of `stage_`: barrier, request tile it + 2 (into the stage that tile it - 1
-        // has left), compute.  STEADY: a full, unmasked context tile whose successor two ahead is
-        // one as well — no condition anywhere, the request is a direct global->LDS load.
-        // Otherwise the requested tile passes through registers and is stored after the compute.
+        // Tile `it` out of stage it % 4: barrier, request a later tile into a stage that is free,
+        // compute.  STEADY: a full, unmasked context tile; it requests the full tile three ahead (if
+        // there is one) by direct global->LDS loads, into the stage that tile it - 1 has just left.
+        // Otherwise: any tile; it requests the tile two ahead through registers and stores it after
+        // the compute, unless that tile is a full one (then a direct load is or was under way).
+        // So full tiles 2 .. n_main - 1 arrive by direct loads (tile 2 from the prologue), all
+        // others through registers, and the tile in front of the first non-full one is never STEADY.
         auto tile = [&](int it, auto stage_, auto steady_tag) {
             constexpr bool STEADY = decltype(steady_tag)::value;
             if constexpr (STEADY) {
@@ -916,24 +920,24 @@ void flash_kernel(FlashParams P) {
                     __builtin_amdgcn_s_setprio(1);
                 else if (it == 3 * n_main / 4)
                     __builtin_amdgcn_s_setprio(0);
-                // this tile's direct loads (issued two tiles ago) must have landed; those of the
-                // next tile (issued one tile ago) may still be on their way
-                // (the slice's last tile has no successor in flight)
-                const bool more = it + 2 < n_main;
-                if (it + 1 == n_main || n_dma == 0)
-                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-                else if (n_dma == 2)
-                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(2));
-                else
-                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(1));
+                // this tile's direct loads must have landed; those of the next two full tiles may
+                // still be on their way
+                const int behind = n_main - 1 - it;
+                switch ((behind >= 2 ? 2 : behind) * n_dma) {
+                    case 0: __builtin_amdgcn_s_waitcnt(vmcnt_imm(0)); break;
+                    case 1: __builtin_amdgcn_s_waitcnt(vmcnt_imm(1)); break;
+                    case 2: __builtin_amdgcn_s_waitcnt(vmcnt_imm(2)); break;
+                    default: __builtin_amdgcn_s_waitcnt(vmcnt_imm(4)); break;
+                }
                 __syncthreads();
-                if (more) dma_tile((stage_ + 2) % 3);
+                if (behind >= 3) dma_tile((stage_ + 3) % 4);
 #pragma unroll
                 for (int sb = 0; sb < SB; ++sb) block(stage_, sb, BoolTag<false>{}, 0, true, 0);
             } else {
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // direct loads of the steady state
                 __syncthreads();
-                if (it + 2 < n_tiles) fetch_tile(it + 2, st_a);
+                const bool fetch = it + 2 < n_tiles && it + 2 >= n_main;
+                if (fetch) fetch_tile(it + 2, st_a);
                 const bool is_ctx = it < ctx_tiles;
                 const int kv0 = is_ctx ? ctx_begin + it * BN : (it - ctx_tiles) * BN;
                 const int seg_end = is_ctx ? ctx_end : P.Nb;
@@ -948,7 +952,7 @@ void flash_kernel(FlashParams P) {
                     else
                         block(stage_, sb, BoolTag<false>{}, blk0, is_ctx, seg_end);
                 }
-                if (it + 2 < n_tiles) stash_tile((stage_ + 2) % 3, st_a);
+                if (fetch) stash_tile((stage_ + 2) % 4, st_a);
             }
         };
 
@@ -961,11 +965,12 @@ void flash_kernel(FlashParams P) {
             scale_q(qraw);
             if (n_tiles > 0) stash_tile(0, st_a);
             if (n_tiles > 1) stash_tile(1, st_b);
+            if (n_main > 2) dma_tile(std::integral_constant<int, 2>{});
         }
 
         int it = 0;
-        // with nothing but full context tiles the whole slice is steady state; otherwise its last
-        // two full tiles already request tiles of the other kind and take the general route
+        // with nothing but full context tiles the whole slice is steady state; otherwise the last
+        // two full tiles have to request tiles of the other kind and take the general route
         const int n_steady = n_tiles == n_main ? n_main : n_main - 2;
         while (it < n_steady) {  // stages as compile-time constants: every LDS offset is an immediate
             tile(it, std::integral_constant<int, 0>{}, BoolTag<true>{});
@@ -973,11 +978,13 @@ void flash_kernel(FlashParams P) {
             tile(it, std::integral_constant<int, 1>{}, BoolTag<true>{});
             if (++it >= n_steady) break;
             tile(it, std::integral_constant<int, 2>{}, BoolTag<true>{});
+            if (++it >= n_steady) break;
+            tile(it, std::integral_constant<int, 3>{}, BoolTag<true>{});
             ++it;
         }
-        for (int stage = it % 3; it < n_tiles; ++it) {
+        for (int stage = it % 4; it < n_tiles; ++it) {
             tile(it, stage, BoolTag<false>{});
-            stage = stage == 2 ? 0 : stage + 1;
+            stage = stage == 3 ? 0 : stage + 1;
         }
         // row sums: query c of this lane's block sits in lane c % 16, register c / 16; the total
         // already covers both halves, so only the hb = 0 lane carries it into the epilogue
