@@ -13,6 +13,7 @@
 #include "../../include/artab_attention.h"
 #include "common.h"
 #include "decode_buffer.h"
+#include "decode_small.h"
 #include "decode_stream.h"
 #include "fused_layer.h"
 #include "glue_kernels.h"
@@ -188,7 +189,41 @@ static hipError_t launch_decode(const DecodeParams &P, int dtype, int Dh, int Lq
     return Lq == 1 ? launch_decode_lq<f16_t, 1>(P, Dh, stream) : launch_decode_lq<f16_t, 2>(P, Dh, stream);
 }
 
-// The streaming buffer pass: one wavefront per workgroup, two per CU.
+// The whole decode call in one launch (decode_small.h).  Worth it while the three launches of the
+// general route are mostly launch latency: few enough workgroups to be on the chip at once or
+// twice, and a context that a CU streams from L2 in a few microseconds (every workgroup reads its
+// head's whole context: 2.6 us for 1024 rows of 64 at the ~100 GB/s a CU draws from L2).
+static bool small_decode_applies(int B, int H, int Lq, int Nc, int Dh) {
+    if (env_int("ARTAB_SMALL", 1) == 0 || (Dh != 32 && Dh != 64) || Lq < 1 || Lq > 2) return false;
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        cus = 256;
+    const long groups = static_cast<long>((B + kSmallTraj - 1) / kSmallTraj) * H;
+    return groups <= 2L * cus && static_cast<long>(Nc) * Dh <= 2048L * 64;
+}
+
+template <typename T>
+static hipError_t launch_small_t(const DecodeParams &P, const View &kc, const View &vc, int Nc, int Dh, int Lq,
+                                 hipStream_t stream) {
+    dim3 grid(static_cast<unsigned>((P.B + kSmallTraj - 1) / kSmallTraj) * P.H), block(kSmallWaves * 64);
+    if (Dh == 32) {
+        if (Lq == 1)
+            hipLaunchKernelGGL((decode_small_kernel<T, 32, 1>), grid, block, 0, stream, P, kc, vc, Nc);
+        else
+            hipLaunchKernelGGL((decode_small_kernel<T, 32, 2>), grid, block, 0, stream, P, kc, vc, Nc);
+    } else {
+        if (Lq == 1)
+            hipLaunchKernelGGL((decode_small_kernel<T, 64, 1>), grid, block, 0, stream, P, kc, vc, Nc);
+        else
+            hipLaunchKernelGGL((decode_small_kernel<T, 64, 2>), grid, block, 0, stream, P, kc, vc, Nc);
+    }
+    return hipGetLastError();
+}
+
+// The streaming buffer pass: one wavefront per workgroup.  Two of them fit on a CU beside the context
+// pass; the grid holds up to four per CU, so that with more tasks than that (B*H above 8192) the
+// rest moves in as the context pass leaves (measured at B*H = 32768, 255 rows: 276 -> 257 us).
 template <typename T>
 static hipError_t launch_stream_t(const DecodeParams &P, int Lq, hipStream_t stream) {
     const long pairs = static_cast<long>(P.B) * P.H;
@@ -198,7 +233,7 @@ static hipError_t launch_stream_t(const DecodeParams &P, int Lq, hipStream_t str
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
         cus = 256;
     const long tasks = (pairs + 15) / 16;
-    long per_cu = 2;  // what fits beside two workgroups of the context pass
+    long per_cu = 4;
     if (const char *e = getenv("ARTAB_STREAM_PER_CU")) per_cu = atol(e) >= 1 && atol(e) <= 4 ? atol(e) : per_cu;  // tuning hook
     dim3 grid(static_cast<unsigned>(tasks < per_cu * cus ? tasks : per_cu * cus)), block(64);
     const int prio = env_int("ARTAB_STREAM_PRIO", 3);  // tuning aid
@@ -539,6 +574,20 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
     const bool shared_ctx = (k_ctx->stride_b == 0 && v_ctx->stride_b == 0) || B == 1;
     bool use_mfma = impl != ARTAB_IMPL_PORTABLE && mfma_shape_ok(dtype, Dh) && aligned && shared_ctx;
     const long rows = static_cast<long>(B) * H * Lq;
+    if (use_mfma && !leave_partials && !order_state && env_int("ARTAB_STREAM", 0) == 0 &&
+        small_decode_applies(B, H, Lq, Nc, Dh)) {
+        DecodeParams D;
+        memset(&D, 0, sizeof(D));
+        D.q = dv(q); D.kb = dv(k_buf); D.vb = dv(v_buf); D.knew = dv(k_new); D.vnew = dv(v_new); D.out = dv(out);
+        D.B = B; D.H = H; D.n_buf = n_buf; D.n_buf_dev = n_buf_device; D.has_new = has_new;
+        D.capacity = buf_capacity;
+        D.qscale = scale * kLog2e;
+        const View kc = dv(k_ctx), vc = dv(v_ctx);
+        ProfileScope prof(st);
+        const hipError_t e = dtype == ARTAB_BF16 ? launch_small_t<bf16_t>(D, kc, vc, Nc, Dh, Lq, st)
+                                                 : launch_small_t<f16_t>(D, kc, vc, Nc, Dh, Lq, st);
+        return launch_status(e, "decode attention (one launch)");
+    }
     FlashPlan pl;
     size_t need_ws = 0;
     bool stream_buf = false;

@@ -52,18 +52,42 @@ constexpr int kDecodeWaves = 4;
 constexpr int kDecodeUnroll = 4;
 constexpr int kSplitBatch = 8;  // context partials fetched per round of the merge
 
+// Where the buffer pass finds the context pass's partial results of its (trajectory, head) pair:
+// in the split workspace in global memory (normalised outputs in the input type, natural-log LSE) ...
 template <typename T, int DH, int LQ>
-__global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(DecodeParams P) {
+struct WorkspacePartials {
+    const T *part_o;
+    const float *part_lse;
+    long total_rows, row0;  // rows per slot; the pair's first row (pair * LQ)
+    int n;
+    __device__ __forceinline__ int count() const { return n; }
+    __device__ __forceinline__ float lse2(int sp, int i) const { return part_lse[sp * total_rows + row0 + i] * kLog2e; }
+    __device__ __forceinline__ float o(int sp, int i, int d) const {
+        return to_f32(part_o[(sp * total_rows + row0 + i) * DH + d]);
+    }
+};
+// ... or in LDS, left there by the wavefronts of the same workgroup (float32, base-2 LSE).
+template <int DH, int LQ>
+struct LdsPartials {
+    const float *part_o;     // [n][ld_cols][DH]
+    const float *part_lse2;  // [n][ld_cols]
+    int ld_cols, col0, n;    // columns per slot; the pair's first column
+    __device__ __forceinline__ int count() const { return n; }
+    __device__ __forceinline__ float lse2(int sp, int i) const { return part_lse2[sp * ld_cols + col0 + i]; }
+    __device__ __forceinline__ float o(int sp, int i, int d) const { return part_o[(sp * ld_cols + col0 + i) * DH + d]; }
+};
+
+// The buffer pass of one (trajectory, head) pair by one wavefront: streams the committed buffer
+// rows, appends the new one, merges with the context partials `parts` and writes the final output.
+// `wave` (0 .. NWAVES-1) selects the wavefront's private LDS region.
+template <typename T, int DH, int LQ, int NWAVES, typename Parts>
+__device__ __forceinline__ void decode_buffer_pair(const DecodeParams &P, long b, int h, int wave, int lane,
+                                                   const Parts &parts) {
     constexpr int LPR = DH / 8;    // lanes per key row
     constexpr int RPW = 64 / LPR;  // key rows per wavefront load
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const long pair = static_cast<long>(blockIdx.x) * kDecodeWaves + wave;  // b*H + h
-    if (pair >= static_cast<long>(P.B) * P.H) return;
-    const long b = pair / P.H;
-    const int h = static_cast<int>(pair % P.H);
+    const long pair = b * P.H + h;
     const int grp = lane / LPR;  // which row of a load this lane works on
     const int sub = lane % LPR;  // which 8-element slice of the head dimension
-    const long total_rows = static_cast<long>(P.B) * P.H * LQ;
 
     float qf[LQ][8];
 #pragma unroll
@@ -88,18 +112,19 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
     float M[LQ];
 #pragma unroll
     for (int i = 0; i < LQ; ++i) M[i] = -INFINITY;
-    for (int sp0 = 0; sp0 < P.n_split; sp0 += kSplitBatch) {
+    const int n_parts = parts.count();
+    for (int sp0 = 0; sp0 < n_parts; sp0 += kSplitBatch) {
         float v[kSplitBatch][LQ];  // a batch of loads in flight, then the maxima
 #pragma unroll
         for (int u = 0; u < kSplitBatch; ++u) {
-            const int sp = sp0 + u < P.n_split ? sp0 + u : P.n_split - 1;
+            const int sp = sp0 + u < n_parts ? sp0 + u : n_parts - 1;
 #pragma unroll
-            for (int i = 0; i < LQ; ++i) v[u][i] = P.part_lse[static_cast<long>(sp) * total_rows + pair * LQ + i];
+            for (int i = 0; i < LQ; ++i) v[u][i] = parts.lse2(sp, i);
         }
 #pragma unroll
         for (int u = 0; u < kSplitBatch; ++u)
 #pragma unroll
-            for (int i = 0; i < LQ; ++i) M[i] = fmaxf(M[i], v[u][i] * kLog2e);
+            for (int i = 0; i < LQ; ++i) M[i] = fmaxf(M[i], v[u][i]);
     }
 
     bool slot_fits;
@@ -172,9 +197,9 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
     // version is two short phases of independent accesses.)  Every wavefront has its own region;
     // its LDS operations execute in issue order, wave_barrier keeps the compiler from moving
     // them across the phases.
-    __shared__ float lds_m[kDecodeWaves][RPW][LQ];
-    __shared__ float lds_l[kDecodeWaves][RPW][LQ];
-    __shared__ __attribute__((aligned(16))) float lds_acc[kDecodeWaves][RPW][LQ][DH];
+    __shared__ float lds_m[NWAVES][RPW][LQ];
+    __shared__ float lds_l[NWAVES][RPW][LQ];
+    __shared__ __attribute__((aligned(16))) float lds_acc[NWAVES][RPW][LQ][DH];
     if (sub == 0) {
 #pragma unroll
         for (int i = 0; i < LQ; ++i) lds_m[wave][grp][i] = m[i];
@@ -208,19 +233,18 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
             num += lds_acc[wave][g][i][d];
             den += lds_l[wave][g][i];
         }
-        for (int sp0 = 0; sp0 < P.n_split; sp0 += kSplitBatch) {
+        for (int sp0 = 0; sp0 < n_parts; sp0 += kSplitBatch) {
             float lv[kSplitBatch], ov[kSplitBatch];
 #pragma unroll
             for (int u = 0; u < kSplitBatch; ++u) {
-                const int sp = sp0 + u < P.n_split ? sp0 + u : P.n_split - 1;
-                const long row = static_cast<long>(sp) * total_rows + pair * LQ + i;
-                lv[u] = P.part_lse[row];
-                ov[u] = to_f32(static_cast<const T *>(P.part_o)[row * DH + d]);
+                const int sp = sp0 + u < n_parts ? sp0 + u : n_parts - 1;
+                lv[u] = parts.lse2(sp, i);
+                ov[u] = parts.o(sp, i, d);
             }
 #pragma unroll
             for (int u = 0; u < kSplitBatch; ++u) {
-                const float lse2 = lv[u] * kLog2e;
-                const float w = (sp0 + u < P.n_split && lse2 != -INFINITY) ? fast_exp2(lse2 - Mi) : 0.f;
+                const float lse2 = lv[u];
+                const float w = (sp0 + u < n_parts && lse2 != -INFINITY) ? fast_exp2(lse2 - Mi) : 0.f;
                 num = fmaf(w, ov[u], num);
                 den += w;
             }
@@ -235,6 +259,16 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
         *reinterpret_cast<u32x4 *>(view_row<T>(P.vb, b, h, n_buf) + 8 * sub) =
             *reinterpret_cast<const u32x4 *>(vnew_row + 8 * sub);
     }
+}
+
+template <typename T, int DH, int LQ>
+__global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(DecodeParams P) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const long pair = static_cast<long>(blockIdx.x) * kDecodeWaves + wave;  // b*H + h
+    if (pair >= static_cast<long>(P.B) * P.H) return;
+    const WorkspacePartials<T, DH, LQ> parts{static_cast<const T *>(P.part_o), P.part_lse,
+                                             static_cast<long>(P.B) * P.H * LQ, pair * LQ, P.n_split};
+    decode_buffer_pair<T, DH, LQ, kDecodeWaves>(P, pair / P.H, static_cast<int>(pair % P.H), wave, lane, parts);
 }
 
 }  // namespace artab

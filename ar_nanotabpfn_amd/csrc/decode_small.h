@@ -1,0 +1,205 @@
+// A whole decode attention call in one launch, for problems too small to be worth three
+// (gfx950; bf16/f16; head_dim 32/64/128; shared context).
+//
+// At B*H*Lq of a few thousand query rows and a context of a thousand rows the split-context pass,
+// the buffer pass and their merge are each a launch of a few microseconds of work: the call is
+// bound by launch latency (23 us for 0.5 GFLOP at B=256, H=8, head_dim 64, N_ctx=1024).  Here one
+// workgroup owns 8 trajectories of one head and does everything for them:
+//
+//   phase 1  the 8*Lq queries are columns of one 32-column MFMA tile (S^T = K Q^T, O^T = V^T P^T
+//            as in mfma_flash.h); the 8 wavefronts deal the context's 32-key blocks among
+//            themselves, each with its own online softmax, K operands straight from global
+//            memory, V through a wavefront-private LDS tile for the transposing read; every
+//            wavefront leaves a normalised partial (float32) and its base-2 LSE in LDS;
+//   phase 2  wavefront w runs the buffer pass of trajectory w (decode_buffer_pair: streams the
+//            committed rows, appends the new one) and merges with the 8 partials from LDS.
+//
+// No workspace, no second launch.  Every workgroup reads its head's whole context (N_ctx * Dh * 4
+// bytes from L2), which is what limits the shapes it is used for (see small_decode_applies()).
+#pragma once
+
+#include "common.h"
+#include "decode_buffer.h"
+#include "mfma_flash.h"
+
+namespace artab {
+
+constexpr int kSmallWaves = 8;
+constexpr int kSmallTraj = 8;  // trajectories per workgroup: one per wavefront in phase 2
+
+template <typename T, int DH, int LQ>
+__global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodeParams P, View kc, View vc, int Nc) {
+    typedef MfmaOps<T> Ops;
+    typedef typename Ops::vec vec;
+    constexpr int KS = DH / 16, DB = DH / 32, NW = kSmallWaves, NCOL = kSmallTraj * LQ;
+    constexpr int VPAD = DH + 16;  // row stride = 32 or 96 bytes mod 128 for the transposing reads
+    constexpr int CPR = DH / 8;    // 16-byte pieces per row
+    constexpr int VP = 32 * CPR / 64;  // V pieces per lane and block
+    static_assert(NCOL <= 32, "the queries of a workgroup are one MFMA tile");
+
+    __shared__ __attribute__((aligned(16))) T v_lds[NW][32 * VPAD];
+    __shared__ float part_lse2[NW][NCOL];
+    __shared__ __attribute__((aligned(16))) float part_o[NW][NCOL][DH];
+
+    const int h = blockIdx.x % P.H;
+    const long b0 = static_cast<long>(blockIdx.x / P.H) * kSmallTraj;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int c = lane & 31, hb = lane >> 5;
+
+    // ---- phase 1: context.  Column c = (trajectory c / LQ, query c % LQ); columns past the end
+    // carry zero queries (their results are never read).
+    vec qreg[KS];
+    {
+        const long b = b0 + c / LQ;
+        const bool live = c < NCOL && b < P.B;
+        const T *qrow = view_row<T>(P.q, live ? b : 0, h, live ? c % LQ : 0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            u32x4 raw = {0u, 0u, 0u, 0u};
+            if (live) raw = *reinterpret_cast<const u32x4 *>(qrow + 16 * ks + 8 * hb);
+            u32x4 sc;  // scale * log2(e) folded in and rounded to the input type (triton_kernels.py:120-121)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sc[e] = pack2<T>(unpack_lo<T>(raw[e]) * P.qscale, unpack_hi<T>(raw[e]) * P.qscale);
+            qreg[ks] = __builtin_bit_cast(vec, sc);
+        }
+    }
+
+    const int n_blocks = (Nc + 31) / 32;
+    const int my_blocks = wave < n_blocks ? (n_blocks - wave + NW - 1) / NW : 0;
+    // operands of a block as they come from global memory: K in MFMA order (row c, 8 elements at
+    // 16 ks + 8 hb), V as 16-byte pieces of a row-major tile (piece lane + 64 x)
+    struct Raw {
+        u32x4 k[KS];
+        u32x4 v[VP];
+    };
+    auto fetch = [&](int blk, Raw &r) {
+        const int row = 32 * blk + c;
+        const bool ok = row < Nc;
+        const T *kr = view_row<T>(kc, 0, h, ok ? row : 0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            r.k[ks] = u32x4{0u, 0u, 0u, 0u};
+            if (ok) r.k[ks] = *reinterpret_cast<const u32x4 *>(kr + 16 * ks + 8 * hb);
+        }
+#pragma unroll
+        for (int x = 0; x < VP; ++x) {
+            const int idx = lane + 64 * x, vrow = 32 * blk + idx / CPR;
+            r.v[x] = u32x4{0u, 0u, 0u, 0u};
+            if (vrow < Nc) r.v[x] = *reinterpret_cast<const u32x4 *>(view_row<T>(vc, 0, h, vrow) + 8 * (idx % CPR));
+        }
+    };
+
+    f32x16 o_acc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o_acc[db][v] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;  // per column: both lanes of a column hold the same maximum
+    T *vt = v_lds[wave];
+    const int v_rd = (4 * hb + ((lane & 15) >> 2)) * VPAD + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+    auto compute = [&](int blk, const Raw &r) {
+        // V tile of this block into the wavefront's LDS region (its previous reads were issued
+        // earlier by the same wavefront: LDS operations of a wavefront execute in order)
+#pragma unroll
+        for (int x = 0; x < VP; ++x) {
+            const int idx = lane + 64 * x;
+            *reinterpret_cast<u32x4 *>(vt + (idx / CPR) * VPAD + 8 * (idx % CPR)) = r.v[x];
+        }
+        f32x16 s;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) s = Ops::mma(__builtin_bit_cast(vec, r.k[ks]), qreg[ks], s);
+        const int key0 = 32 * blk;
+        if (key0 + 32 > Nc) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                if (key0 + 8 * (v >> 2) + 4 * hb + (v & 3) >= Nc) s[v] = -INFINITY;
+        }
+        float tmax = s[0];
+#pragma unroll
+        for (int v = 1; v < 16; ++v) tmax = fmaxf(tmax, s[v]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m_run, tmax);  // finite: the first key of a block always exists
+        const float alpha = fast_exp2(m_run - m_new);  // 2^(-inf) = 0 on the first block
+        if (__any(alpha != 1.f)) {
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) o_acc[db][v] *= alpha;
+        }
+        m_run = m_new;
+        u32x4 pb[2];
+        float lsum = 0.f;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float p0 = fast_exp2(s[8 * t + 2 * e] - m_new), p1 = fast_exp2(s[8 * t + 2 * e + 1] - m_new);
+                lsum += p0 + p1;
+                pb[t][e] = pack2<T>(p0, p1);
+            }
+        l_run += lsum;
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const T *vp_ = vt + (16 * t) * VPAD + 32 * db + v_rd;
+                s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp_));
+                s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) s16x4 *)(vp_ + 8 * VPAD));
+                typedef short s16x8 __attribute__((ext_vector_type(8)));
+                s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                o_acc[db] = Ops::mma(__builtin_bit_cast(vec, both), __builtin_bit_cast(vec, pb[t]), o_acc[db]);
+            }
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    // blocks wave, wave + NW, ...: two requested ahead of the one being multiplied
+    {
+        Raw r0, r1, r2;
+        if (my_blocks > 0) fetch(wave, r0);
+        if (my_blocks > 1) fetch(wave + NW, r1);
+        int i = 0;
+        while (i < my_blocks) {
+            if (i + 2 < my_blocks) fetch(wave + NW * (i + 2), r2);
+            compute(wave + NW * i, r0);
+            if (++i >= my_blocks) break;
+            if (i + 2 < my_blocks) fetch(wave + NW * (i + 2), r0);
+            compute(wave + NW * i, r1);
+            if (++i >= my_blocks) break;
+            if (i + 2 < my_blocks) fetch(wave + NW * (i + 2), r1);
+            compute(wave + NW * i, r2);
+            ++i;
+        }
+    }
+
+    // this wavefront's partial: normalised, with its base-2 LSE (-inf: it had no block)
+    {
+        const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        if (c < NCOL) {
+            if (hb == 0) part_lse2[wave][c] = l_tot > 0.f ? m_run + fast_log2(l_tot) : -INFINITY;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    const f32x4 val = {o_acc[db][4 * q4] * inv, o_acc[db][4 * q4 + 1] * inv, o_acc[db][4 * q4 + 2] * inv,
+                                       o_acc[db][4 * q4 + 3] * inv};
+                    *reinterpret_cast<f32x4 *>(&part_o[wave][c][32 * db + 8 * q4 + 4 * hb]) = val;
+                }
+        }
+    }
+    __syncthreads();
+
+    // ---- phase 2: buffer rows of trajectory b0 + wave, merged with the eight partials
+    const long b = b0 + wave;
+    if (b >= P.B) return;
+    const LdsPartials<DH, LQ> parts{&part_o[0][0][0], &part_lse2[0][0], NCOL, wave * LQ, NW};
+    decode_buffer_pair<T, DH, LQ, NW>(P, b, h, wave, lane, parts);
+}
+
+}  // namespace artab

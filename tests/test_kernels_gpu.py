@@ -141,6 +141,14 @@ def _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, use_mfma,
     assert torch.equal(kc_d.cpu(), exp_k) and torch.equal(vc_d.cpu(), exp_v)
 
 
+@pytest.fixture(params=[1, 0], ids=["one-launch", "general-route"])
+def small_route(request, monkeypatch):
+    """Small decode problems take a single-launch kernel (ARTAB_SMALL, on by default); with it
+    switched off the same call goes through the context pass, the buffer pass and their merge."""
+    monkeypatch.setenv("ARTAB_SMALL", str(request.param))
+    return request.param
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("use_mfma", [True, False])
 @pytest.mark.parametrize(
@@ -155,9 +163,13 @@ def _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, use_mfma,
         (33, 8, 2, 100, 64, 19, 64, True),
         (5, 2, 2, 300, 128, 70, 80, True),
         (4, 3, 2, 50, 16, 9, 12, True),  # portable-only head_dim
+        (9, 2, 1, 31, 32, 0, 4, False),  # context shorter than one key block
+        (37, 3, 2, 1000, 64, 33, 48, True),  # ragged trajectory group, ragged last key block
+        (64, 8, 2, 2048, 64, 63, 64, True),  # the largest context the one-launch kernel takes at head_dim 64
+        (11, 5, 1, 257, 32, 40, 41, True),  # one key block more than the wavefronts share evenly
     ],
 )
-def test_decode_attention_matches_oracle(device, dtype, use_mfma, B, H, Lq, Nc, D, n_buf, cap, with_new):
+def test_decode_attention_matches_oracle(device, small_route, dtype, use_mfma, B, H, Lq, Nc, D, n_buf, cap, with_new):
     _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, use_mfma)
 
 
@@ -180,8 +192,9 @@ def test_decode_attention_matches_oracle(device, dtype, use_mfma, B, H, Lq, Nc, 
         (4, 3, 2, 50, 16, 9, 12, True),  # portable-only head_dim: side stream is ignored
     ],
 )
-def test_decode_attention_overlapped_matches_oracle(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new):
-    """Buffer pass on a side stream next to the context pass, then the combine launch."""
+def test_decode_attention_overlapped_matches_oracle(device, small_route, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new):
+    """Buffer pass on a side stream next to the context pass, then the combine launch (small
+    problems take the one-launch kernel instead unless it is switched off)."""
     _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, True, scale=0.6, overlapped=True)
 
 
@@ -329,7 +342,7 @@ def test_decode_attention_per_trajectory_cache(device, dtype, B, H, Lq, Nc, D, n
 
 
 @pytest.mark.parametrize("n_buf", [1, 2, 17, 33, 64])
-def test_decode_attention_config1_shape(device, n_buf):
+def test_decode_attention_config1_shape(device, small_route, n_buf):
     """BASELINE configs[1]: H=8, Dh=64, Nc=1024, B=256, entries ~N(0,1)/8, N_buf swept."""
     _decode_case(device, torch.bfloat16, 256, 8, 1, 1024, 64, n_buf, 64, False, True, scale=0.125, seed=0)
 
@@ -983,12 +996,15 @@ def test_layer_post_pre_falls_back_when_not_covered(device):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,H,Lq,Nc,n_buf,cap", [(64, 4, 2, 4096, 9, 16), (33, 8, 2, 2048, 0, 8), (40, 8, 1, 4096, 5, 8)])
-def test_decode_partials_merged_in_layer_kernel(device, tile_rows, dtype, B, H, Lq, Nc, n_buf, cap):
+def test_decode_partials_merged_in_layer_kernel(device, monkeypatch, tile_rows, dtype, B, H, Lq, Nc, n_buf, cap):
     """decode_attention(leave_partials=True) + the layer kernels that merge the partials while
     loading, against the merged attention output fed to the same kernels: the merge is the same
-    arithmetic rounded at the same point, so the results must agree bit for bit."""
+    arithmetic rounded at the same point, so the results must agree bit for bit.  (Both legs on the
+    general route: the one-launch kernel merges float32 partials and differs in the last bit.)"""
     from ar_nanotabpfn_amd import attention_kernels as ak
     from ar_nanotabpfn_amd import model as m
+
+    monkeypatch.setenv("ARTAB_SMALL", "0")
 
     D, Dh, F = 32 * H, 32, 256
     torch.manual_seed(2)
@@ -1070,11 +1086,12 @@ def test_queue_order_argument_checks(device):
 
 @pytest.mark.parametrize("absorb", [False, True])
 @pytest.mark.parametrize("B,H,Nc,cap", [(64, 8, 2048, 8), (600, 8, 1024, 12)])
-def test_decode_attention_ordered_by_counters_equals_event_ordered(device, B, H, Nc, cap, absorb):
+def test_decode_attention_ordered_by_counters_equals_event_ordered(device, monkeypatch, B, H, Nc, cap, absorb):
     """A run of decode steps whose two streams are ordered by device-side counters (one fork
     before the first call, one join after the last) against the same steps ordered by two events
     per call: same partials (bit for bit after the merge), same cache, no wait timed out."""
     ak = _ak()
+    monkeypatch.setenv("ARTAB_SMALL", "0")  # the event-ordered leg on the two-stream route as well
     dtype, D = torch.bfloat16, 32
     q0, k_ctx, v_ctx = (t.to(device) for t in _ctx_inputs(B, H, 2, Nc, D, dtype, seed=1, scale=0.6))
     k_ref, v_ref = torch.zeros((B, H, cap, D), device=device, dtype=dtype), torch.zeros((B, H, cap, D), device=device, dtype=dtype)
