@@ -134,6 +134,20 @@ __device__ __forceinline__ void load_row64_to_lds(const void *global_src, unsign
     __builtin_amdgcn_global_load_lds(global_src, lds_dst + 3024, 16, 48, 0);
 }
 
+// acc + a.lo * b.lo + a.hi * b.hi of two packed 16-bit pairs, accumulated in float32
+template <typename T>
+__device__ __forceinline__ float dot2_acc(unsigned a, unsigned b, float acc);
+template <>
+__device__ __forceinline__ float dot2_acc<bf16_t>(unsigned a, unsigned b, float acc) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), acc, false);
+}
+template <>
+__device__ __forceinline__ float dot2_acc<f16_t>(unsigned a, unsigned b, float acc) {
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), acc, false);
+}
+
 __device__ __forceinline__ float max3(float a, float b, float c) {
     float r;
     asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));

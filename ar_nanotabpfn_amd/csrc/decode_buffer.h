@@ -77,26 +77,70 @@ struct LdsPartials {
     __device__ __forceinline__ float o(int sp, int i, int d) const { return part_o[(sp * ld_cols + col0 + i) * DH + d]; }
 };
 
+// What a wavefront asks for before it can start on a pair: its slice of the queries, the committed
+// length and the first batch of buffer rows.  Requested by decode_buffer_request() — as early as
+// the caller likes: the one-launch kernel does it in front of its context phase — and consumed by
+// decode_buffer_pair().
+template <typename T, int DH, int LQ>
+struct BufferHead {
+    u32x4 qraw[LQ];
+    u32x4 kraw[kDecodeUnroll], vraw[kDecodeUnroll];
+    int n_buf, n_total;
+    bool slot_fits;
+};
+
+template <typename T, int DH, int LQ>
+__device__ __forceinline__ void decode_buffer_rows(const DecodeParams &P, long b, int h, int lane, int kv0, int n_buf,
+                                                   int n_total, u32x4 (&kraw)[kDecodeUnroll],
+                                                   u32x4 (&vraw)[kDecodeUnroll]) {
+    constexpr int LPR = DH / 8, RPW = 64 / LPR;
+    const int grp = lane / LPR, sub = lane % LPR;
+#pragma unroll
+    for (int u = 0; u < kDecodeUnroll; ++u) {
+        const int kv = kv0 + u * RPW + grp;
+        kraw[u] = u32x4{0u, 0u, 0u, 0u};
+        vraw[u] = u32x4{0u, 0u, 0u, 0u};
+        if (kv < n_total) {
+            const bool is_new = P.has_new && kv == n_buf;
+            const T *kr = is_new ? view_row<T>(P.knew, b, h, 0) : view_row<T>(P.kb, b, h, kv);
+            const T *vr = is_new ? view_row<T>(P.vnew, b, h, 0) : view_row<T>(P.vb, b, h, kv);
+            kraw[u] = *reinterpret_cast<const u32x4 *>(kr + 8 * sub);
+            vraw[u] = *reinterpret_cast<const u32x4 *>(vr + 8 * sub);
+        }
+    }
+}
+
+template <typename T, int DH, int LQ>
+__device__ __forceinline__ void decode_buffer_request(const DecodeParams &P, long b, int h, int lane,
+                                                      BufferHead<T, DH, LQ> &hd) {
+    const int sub = lane % (DH / 8);
+#pragma unroll
+    for (int i = 0; i < LQ; ++i) hd.qraw[i] = *reinterpret_cast<const u32x4 *>(view_row<T>(P.q, b, h, i) + 8 * sub);
+    hd.n_buf = P.n_base + committed_rows(P, hd.slot_fits);
+    hd.n_total = hd.n_buf + (P.has_new ? 1 : 0);
+    decode_buffer_rows<T, DH, LQ>(P, b, h, lane, 0, hd.n_buf, hd.n_total, hd.kraw, hd.vraw);
+}
+
 // The buffer pass of one (trajectory, head) pair by one wavefront: streams the committed buffer
 // rows, appends the new one, merges with the context partials `parts` and writes the final output.
 // `wave` (0 .. NWAVES-1) selects the wavefront's private LDS region.
 template <typename T, int DH, int LQ, int NWAVES, typename Parts>
 __device__ __forceinline__ void decode_buffer_pair(const DecodeParams &P, long b, int h, int wave, int lane,
-                                                   const Parts &parts) {
+                                                   const Parts &parts, const BufferHead<T, DH, LQ> &hd) {
     constexpr int LPR = DH / 8;    // lanes per key row
     constexpr int RPW = 64 / LPR;  // key rows per wavefront load
     const long pair = b * P.H + h;
     const int grp = lane / LPR;  // which row of a load this lane works on
     const int sub = lane % LPR;  // which 8-element slice of the head dimension
 
-    float qf[LQ][8];
+    // the lane's query slice, scale * log2(e) folded in and rounded to the input type (the matrix
+    // kernels round it at the same point, triton_kernels.py:120-121): packed pairs for v_dot2
+    unsigned qp[LQ][4];
 #pragma unroll
-    for (int i = 0; i < LQ; ++i) {
-        u32x4 raw = *reinterpret_cast<const u32x4 *>(view_row<T>(P.q, b, h, i) + 8 * sub);
-        unpack8<T>(raw, qf[i]);
+    for (int i = 0; i < LQ; ++i)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) qf[i][e] *= P.qscale;
-    }
+        for (int e = 0; e < 4; ++e)
+            qp[i][e] = pack2<T>(unpack_lo<T>(hd.qraw[i][e]) * P.qscale, unpack_hi<T>(hd.qraw[i][e]) * P.qscale);
 
     float m[LQ], l[LQ], acc[LQ][8];
 #pragma unroll
@@ -127,39 +171,42 @@ __device__ __forceinline__ void decode_buffer_pair(const DecodeParams &P, long b
             for (int i = 0; i < LQ; ++i) M[i] = fmaxf(M[i], v[u][i]);
     }
 
-    bool slot_fits;
-    const int n_buf = P.n_base + committed_rows(P, slot_fits);
-    const int n_total = n_buf + (P.has_new ? 1 : 0);
+    const bool slot_fits = hd.slot_fits;
+    const int n_buf = hd.n_buf, n_total = hd.n_total;
     const T *knew_row = P.has_new ? view_row<T>(P.knew, b, h, 0) : nullptr;
     const T *vnew_row = P.has_new ? view_row<T>(P.vnew, b, h, 0) : nullptr;
 
+    // the batch after the one being worked on is always on its way
+    u32x4 knext[kDecodeUnroll], vnext[kDecodeUnroll];
+#pragma unroll
+    for (int u = 0; u < kDecodeUnroll; ++u) {
+        knext[u] = hd.kraw[u];
+        vnext[u] = hd.vraw[u];
+    }
     for (int kv0 = 0; kv0 < n_total; kv0 += RPW * kDecodeUnroll) {
         u32x4 kraw[kDecodeUnroll], vraw[kDecodeUnroll];
         bool ok[kDecodeUnroll];
 #pragma unroll
         for (int u = 0; u < kDecodeUnroll; ++u) {
-            int kv = kv0 + u * RPW + grp;
-            ok[u] = kv < n_total;
-            kraw[u] = u32x4{0u, 0u, 0u, 0u};
-            vraw[u] = u32x4{0u, 0u, 0u, 0u};
-            if (ok[u]) {
-                const bool is_new = P.has_new && kv == n_buf;
-                const T *kr = is_new ? knew_row : view_row<T>(P.kb, b, h, kv);
-                const T *vr = is_new ? vnew_row : view_row<T>(P.vb, b, h, kv);
-                kraw[u] = *reinterpret_cast<const u32x4 *>(kr + 8 * sub);
-                vraw[u] = *reinterpret_cast<const u32x4 *>(vr + 8 * sub);
-            }
+            ok[u] = kv0 + u * RPW + grp < n_total;
+            kraw[u] = knext[u];
+            vraw[u] = vnext[u];
         }
+        if (kv0 + RPW * kDecodeUnroll < n_total)
+            decode_buffer_rows<T, DH, LQ>(P, b, h, lane, kv0 + RPW * kDecodeUnroll, n_buf, n_total, knext, vnext);
         float s[LQ][kDecodeUnroll];
 #pragma unroll
         for (int u = 0; u < kDecodeUnroll; ++u) {
-            float kf[8];
-            unpack8<T>(kraw[u], kf);
+            if (kv0 + u * RPW >= n_total) {  // wavefront-uniform: no lane group has a row in this sub-step
+#pragma unroll
+                for (int i = 0; i < LQ; ++i) s[i][u] = -INFINITY;
+                continue;
+            }
 #pragma unroll
             for (int i = 0; i < LQ; ++i) {
                 float d = 0.f;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) d = fmaf(qf[i][e], kf[e], d);
+                for (int e = 0; e < 4; ++e) d = dot2_acc<T>(qp[i][e], kraw[u][e], d);
 #pragma unroll
                 for (int o = 1; o < LPR; o <<= 1) d += __shfl_xor(d, o, 64);
                 s[i][u] = ok[u] ? d : -INFINITY;
@@ -180,6 +227,7 @@ __device__ __forceinline__ void decode_buffer_pair(const DecodeParams &P, long b
         }
 #pragma unroll
         for (int u = 0; u < kDecodeUnroll; ++u) {
+            if (kv0 + u * RPW >= n_total) continue;
             float vf[8];
             unpack8<T>(vraw[u], vf);
 #pragma unroll
@@ -268,7 +316,11 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
     if (pair >= static_cast<long>(P.B) * P.H) return;
     const WorkspacePartials<T, DH, LQ> parts{static_cast<const T *>(P.part_o), P.part_lse,
                                              static_cast<long>(P.B) * P.H * LQ, pair * LQ, P.n_split};
-    decode_buffer_pair<T, DH, LQ, kDecodeWaves>(P, pair / P.H, static_cast<int>(pair % P.H), wave, lane, parts);
+    const long b = pair / P.H;
+    const int h = static_cast<int>(pair % P.H);
+    BufferHead<T, DH, LQ> hd;
+    decode_buffer_request<T, DH, LQ>(P, b, h, lane, hd);
+    decode_buffer_pair<T, DH, LQ, kDecodeWaves>(P, b, h, wave, lane, parts, hd);
 }
 
 }  // namespace artab

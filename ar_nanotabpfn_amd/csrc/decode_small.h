@@ -46,6 +46,12 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodePa
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int c = lane & 31, hb = lane >> 5;
 
+    // what phase 2 needs from global memory is requested first: its round trips (the buffer rows
+    // come from HBM) run under phase 1
+    const long b2 = b0 + wave;
+    BufferHead<T, DH, LQ> head2;
+    if (b2 < P.B) decode_buffer_request<T, DH, LQ>(P, b2, h, lane, head2);
+
     // ---- phase 1: context.  Column c = (trajectory c / LQ, query c % LQ); columns past the end
     // carry zero queries (their results are never read).
     vec qreg[KS];
@@ -72,21 +78,36 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodePa
         u32x4 k[KS];
         u32x4 v[VP];
     };
+    // Row pointers of the block to be requested next (blocks wave, wave + NW, ... in order): full
+    // blocks advance them by NW * 32 rows; the context's ragged last block computes clamped rows the
+    // long way (rows past the end re-read the last one: their scores are masked and their
+    // probabilities are zero, only finite values are needed).
+    const long k_step = static_cast<long>(NW) * 32 * kc.sn, v_step = static_cast<long>(NW) * 32 * vc.sn;
+    const T *k_ptr = view_row<T>(kc, 0, h, min(32 * wave + c, Nc - 1)) + 8 * hb;
+    const T *v_ptr[VP];
+#pragma unroll
+    for (int x = 0; x < VP; ++x)
+        v_ptr[x] = view_row<T>(vc, 0, h, min(32 * wave + (lane + 64 * x) / CPR, Nc - 1)) + 8 * ((lane + 64 * x) % CPR);
     auto fetch = [&](int blk, Raw &r) {
-        const int row = 32 * blk + c;
-        const bool ok = row < Nc;
-        const T *kr = view_row<T>(kc, 0, h, ok ? row : 0);
+        if (32 * blk + 32 <= Nc) {
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            r.k[ks] = u32x4{0u, 0u, 0u, 0u};
-            if (ok) r.k[ks] = *reinterpret_cast<const u32x4 *>(kr + 16 * ks + 8 * hb);
-        }
+            for (int ks = 0; ks < KS; ++ks) r.k[ks] = *reinterpret_cast<const u32x4 *>(k_ptr + 16 * ks);
 #pragma unroll
-        for (int x = 0; x < VP; ++x) {
-            const int idx = lane + 64 * x, vrow = 32 * blk + idx / CPR;
-            r.v[x] = u32x4{0u, 0u, 0u, 0u};
-            if (vrow < Nc) r.v[x] = *reinterpret_cast<const u32x4 *>(view_row<T>(vc, 0, h, vrow) + 8 * (idx % CPR));
+            for (int x = 0; x < VP; ++x) r.v[x] = *reinterpret_cast<const u32x4 *>(v_ptr[x]);
+        } else {
+            const T *kr = view_row<T>(kc, 0, h, min(32 * blk + c, Nc - 1)) + 8 * hb;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) r.k[ks] = *reinterpret_cast<const u32x4 *>(kr + 16 * ks);
+#pragma unroll
+            for (int x = 0; x < VP; ++x) {
+                const int idx = lane + 64 * x;
+                r.v[x] = *reinterpret_cast<const u32x4 *>(view_row<T>(vc, 0, h, min(32 * blk + idx / CPR, Nc - 1)) +
+                                                          8 * (idx % CPR));
+            }
         }
+        k_ptr += k_step;
+#pragma unroll
+        for (int x = 0; x < VP; ++x) v_ptr[x] += v_step;
     };
 
     f32x16 o_acc[DB];
@@ -96,16 +117,14 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodePa
         for (int v = 0; v < 16; ++v) o_acc[db][v] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;  // per column: both lanes of a column hold the same maximum
     T *vt = v_lds[wave];
+    T *v_wr = vt + (lane / CPR) * VPAD + 8 * (lane % CPR);  // piece lane + 64 x sits 64 / CPR rows further down
     const int v_rd = (4 * hb + ((lane & 15) >> 2)) * VPAD + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
     auto compute = [&](int blk, const Raw &r) {
         // V tile of this block into the wavefront's LDS region (its previous reads were issued
         // earlier by the same wavefront: LDS operations of a wavefront execute in order)
 #pragma unroll
-        for (int x = 0; x < VP; ++x) {
-            const int idx = lane + 64 * x;
-            *reinterpret_cast<u32x4 *>(vt + (idx / CPR) * VPAD + 8 * (idx % CPR)) = r.v[x];
-        }
+        for (int x = 0; x < VP; ++x) *reinterpret_cast<u32x4 *>(v_wr + x * (64 / CPR) * VPAD) = r.v[x];
         f32x16 s;
 #pragma unroll
         for (int v = 0; v < 16; ++v) s[v] = 0.f;
@@ -196,10 +215,9 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodePa
     __syncthreads();
 
     // ---- phase 2: buffer rows of trajectory b0 + wave, merged with the eight partials
-    const long b = b0 + wave;
-    if (b >= P.B) return;
+    if (b2 >= P.B) return;
     const LdsPartials<DH, LQ> parts{&part_o[0][0][0], &part_lse2[0][0], NCOL, wave * LQ, NW};
-    decode_buffer_pair<T, DH, LQ, NW>(P, b, h, wave, lane, parts);
+    decode_buffer_pair<T, DH, LQ, NW>(P, b2, h, wave, lane, parts, head2);
 }
 
 }  // namespace artab
