@@ -400,6 +400,16 @@ class ARTabPFNPredictor:
         st.y_prev.copy_(y)
         st.counters.add_(1)
 
+    def _first_step(self, st) -> None:
+        """The step of the first target (``[target]`` alone, empty buffer) in the form that can be
+        recorded: embedding from the device-side copy of the targets, the layer stack against the
+        context, then the one-launch tail with the step counter at 0."""
+        emb0 = self.embedder.embed_target(st.x_target[:, 0:1])
+        x_row = self._run_layers(emb0, lambda layer, q, k, v: self._attend_decode_shared(layer, q, k, v,
+                                                                                        rows=st.rows, chain=st.chain))
+        st.tail(x_row)    # norm, head, draw, preds[:, 0], embedding of step 1, (t, nbuf) += 1
+        st.nbuf.zero_()   # the first target commits no buffer row
+
     def _last_layer_rows(self) -> Optional[slice]:
         """Rows of a ``[buffer, target]`` step that the last layer has to finish: the target."""
         return slice(1, 2) if self.target_only_last_layer else None
@@ -447,6 +457,7 @@ class ARTabPFNPredictor:
                 st.t, st.nbuf = st.counters[0:1], st.counters[1:2]
                 st.graph = None
                 st.graph_many = None   # steps_per_graph steps in one graph
+                st.graph_first = None  # the first target's step (no buffer row yet)
                 st.tail = None
                 st.order = st.order_active = None
                 if self._counter_ordering_applies(x_target):
@@ -467,18 +478,44 @@ class ARTabPFNPredictor:
             self._graph_state = gs
         gs.x_target[:, :Nt].copy_(x_target)
 
-        # first target: no buffer row yet (N = 1), launched directly for all trajectories
-        y0 = self.autoregressive_decode(gs.x_target[:, 0:1, :], None, None, 0)
-        emb1 = None
+        current = torch.cuda.current_stream(device)
+        # First target: no buffer row yet (N = 1).  With the one-launch tail and one trajectory
+        # group it is a recorded graph of its own (the tail draws y_0, writes it, leaves the
+        # embedding of step 1 and moves the step counter on); otherwise it is launched directly.
+        recorded_first = gs.tail is not None and len(gs.chains) == 1 and cap >= 2
         if gs.tail is not None:
-            bs = self.ar_tokens.shape[0]
-            emb1 = torch.cat([self.embedder.embed_buffer(gs.x_target[:, 0:1], y0) + self.ar_tokens[1 % bs],
-                              self.embedder.embed_target(gs.x_target[:, 1:2])], dim=1)
             x_mean = gs.x_target[:, :Nt].mean(dim=-1)
             for st in gs.chains:
                 rows = st.rows if st.rows is not None else slice(0, B)
                 st.x_mean[:, :Nt].copy_(x_mean[rows])
                 self._draw_step_variates(st.rand_u, st.rand_n)
+        if recorded_first:
+            st = gs.chains[0]
+            if st.graph_first is None:
+                with _lib.workspace_tag(1 + st.chain):
+                    warm = torch.cuda.Stream(device=device)
+                    warm.wait_stream(current)
+                    with torch.cuda.stream(warm):
+                        st.counters.zero_()
+                        self._first_step(st)
+                    current.wait_stream(warm)
+                    st.graph_first = torch.cuda.CUDAGraph()
+                    self.graph_recordings += 1
+                    with torch.cuda.graph(st.graph_first):
+                        self._first_step(st)
+                    st.workspace_first = _lib.held_workspace(device)
+            st.counters.zero_()
+            st.graph_first.replay()
+            y0 = emb1 = None
+            if st.graph is None:  # the step graphs are still to be recorded: their warm-up starts from here
+                y0, emb1 = st.preds[:, 0:1].clone(), st.emb.clone()
+        else:
+            y0 = self.autoregressive_decode(gs.x_target[:, 0:1, :], None, None, 0)
+            emb1 = None
+            if gs.tail is not None:
+                bs = self.ar_tokens.shape[0]
+                emb1 = torch.cat([self.embedder.embed_buffer(gs.x_target[:, 0:1], y0) + self.ar_tokens[1 % bs],
+                                  self.embedder.embed_target(gs.x_target[:, 1:2])], dim=1)
 
         def reset(st):
             rows = st.rows if st.rows is not None else slice(0, B)
@@ -489,7 +526,6 @@ class ARTabPFNPredictor:
             if st.tail is not None:
                 st.emb.copy_(emb1[rows])
 
-        current = torch.cuda.current_stream(device)
         for st in gs.chains:
             if st.graph is not None:
                 continue
@@ -511,8 +547,9 @@ class ARTabPFNPredictor:
                 # the recorded launches point into this scratch tensor: it lives as long as they do
                 st.workspace = _lib.held_workspace(device)
         gs.graph = gs.chains[0].graph
-        for st in gs.chains:
-            reset(st)
+        if y0 is not None:  # (a recorded first step has left exactly this state behind)
+            for st in gs.chains:
+                reset(st)
         k = self.steps_per_graph if gs.chains[0].graph_many is not None else 1
         n_many, n_single = (Nt - 1) // k if k > 1 else 0, (Nt - 1) % k if k > 1 else Nt - 1
         if len(gs.chains) == 1:
