@@ -86,6 +86,7 @@ class ARTabPFNPredictor:
         self.target_only_last_layer = True
         self._side_streams = {}
         self._graph_state = None
+        self._graph_params = None    # the tensors a recorded step points at (collected at first use)
         self.graph_recordings = 0    # HIP graphs recorded so far (a run that only replays leaves it unchanged)
 
     @classmethod
@@ -426,8 +427,12 @@ class ARTabPFNPredictor:
         B, Nt, F_ = x_target.shape
         device, dtype = x_target.device, x_target.dtype
         layer0 = self.backbone.layers[0]
-        params = list(self.backbone.parameters()) + list(self.embedder.parameters()) + list(self.head.parameters())
-        params.append(self.ar_tokens)
+        # (walking the module tree costs a millisecond of host time with the GPU idle: done once; a
+        # weight that is updated or moved changes its version or address and is seen through the key)
+        if self._graph_params is None:
+            self._graph_params = (list(self.backbone.parameters()) + list(self.embedder.parameters()) +
+                                  list(self.head.parameters()) + [self.ar_tokens])
+        params = self._graph_params
         chain_rows = self._chain_rows(B)
         # The recorded step depends on the capacity of the buffer cache, not on how many steps are
         # replayed: loop state is sized for the capacity, so runs of any length share one recording.
@@ -567,6 +572,10 @@ class ARTabPFNPredictor:
                         (st.graph_many if i < n_many else st.graph).replay()
             for st in gs.chains:
                 current.wait_stream(st.stream)
+        # the result is copied before the host waits for the failure flag of the counters, so that
+        # the device does not sit idle between the last step and the copy
+        result = (gs.chains[0].preds[:, :Nt].clone() if len(gs.chains) == 1
+                  else torch.cat([st.preds[:, :Nt] for st in gs.chains], dim=0))
         if any(st.order is not None and st.order.failed() for st in gs.chains):
             # a wait on the counters timed out: the recorded streams did not run side by side.
             # The step's results are void; record it again with events and sample afresh.
@@ -578,9 +587,7 @@ class ARTabPFNPredictor:
             return self._sample_sequence_graph(x_target)
         self.buffer_len = Nt - 1
         self.seq_len = self.context_len + self.buffer_len
-        if len(gs.chains) == 1:
-            return gs.chains[0].preds[:, :Nt].clone()
-        return torch.cat([st.preds[:, :Nt] for st in gs.chains], dim=0)
+        return result
 
     def _counter_ordering_applies(self, x: Tensor) -> bool:
         """Whether every layer's decode call takes the schedule that the counters can order: the
