@@ -45,6 +45,8 @@ import numpy as np
 
 __all__ = [
     "context_attention",
+    "round_bf16",
+    "context_attention_same_dtype",
     "buffer_attention",
     "merge_attention_outputs",
     "teacher_forcing_buffer_mask",
@@ -122,6 +124,35 @@ def context_attention(
     scores = np.matmul(q, k.transpose(0, 1, 3, 2)) * scale
     lse = _logsumexp(scores)
     out = np.matmul(_softmax(scores), v)
+    return out, lse
+
+
+def round_bf16(x) -> np.ndarray:
+    """Round float32 values to the nearest bfloat16 (ties to even), returned as float32: what
+    ``tensor.to(torch.bfloat16)`` does to finite values."""
+    a = np.ascontiguousarray(np.asarray(x, dtype=np.float32))
+    u = a.view(np.uint32)
+    bias = np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))
+    r = ((u + bias) & np.uint32(0xFFFF0000)).astype(np.uint32)
+    return r.view(np.float32).reshape(a.shape)
+
+
+def context_attention_same_dtype(q, k_ctx, v_ctx, scale: Optional[float] = None) -> Tuple[np.ndarray, np.ndarray]:
+    """``pytorch_context_attention`` (triton_kernels.py:532-567) as it evaluates on bfloat16
+    tensors: every tensor-valued intermediate is rounded to bfloat16 where torch materialises one —
+    the score matrix (:558, product accumulated in float32, rounded, scaled, rounded), the softmax
+    (:564, computed in float32 from the rounded scores, rounded) and the output (:565) — while the
+    LSE is the float32 logsumexp of the rounded scores (:561).  Secondary reference: looser than
+    the float64 one by construction.  Shared ``[H,Nc,D]`` context only."""
+    q32, k32, v32 = (round_bf16(a) for a in (q, k_ctx, v_ctx))
+    D = q32.shape[-1]
+    if scale is None:
+        scale = D ** -0.5
+    scores = round_bf16(np.einsum("bhqd,hnd->bhqn", q32, k32, dtype=np.float32))
+    scores = round_bf16(scores * np.float32(scale))
+    lse = _logsumexp(scores.astype(np.float32))
+    attn = round_bf16(_softmax(scores.astype(np.float32)))
+    out = round_bf16(np.einsum("bhqn,hnd->bhqd", attn, v32, dtype=np.float32))
     return out, lse
 
 

@@ -454,3 +454,31 @@ def test_row_mask_attention_equals_per_row_softmax():
         s = np.einsum("bhd,bhkd->bhk", q[:, :, r], k[:, :, keys]) / np.sqrt(D)
         p = scipy.special.softmax(s, axis=-1)
         assert np.abs(out[:, :, r] - np.einsum("bhk,bhkd->bhd", p, v[:, :, keys])).max() <= 1e-12
+
+
+def test_round_bf16_matches_torch_cast():
+    """The oracle's bfloat16 rounding against torch's cast: random values over many exponents,
+    exact ties (both parities of the kept mantissa bit), signed zeros, subnormals of bfloat16."""
+    import torch
+
+    rng = np.random.default_rng(0)
+    x = (rng.standard_normal(20000) * np.exp2(rng.integers(-30, 30, 20000))).astype(np.float32)
+    ties = np.array([0x3F808000, 0x3F818000, 0xBF808000, 0x3F80FFFF, 0x00008000, 0x00018000, 0x00000000, 0x80000000],
+                    dtype=np.uint32).view(np.float32)
+    x = np.concatenate([x, ties])
+    want = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
+    got = ao.round_bf16(x)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_same_dtype_context_attention_is_near_the_exact_one():
+    """The bfloat16-arithmetic evaluation of pytorch_context_attention stays within the tolerances
+    stated for 16-bit outputs at the scale the targets are stated for (entries ~N(0,1)/8), and is
+    an evaluation of the same function (not of something else) at unit scale."""
+    rng = np.random.default_rng(1)
+    B, H, Lq, Nc, D = 3, 2, 2, 300, 32
+    for s, tol_o, tol_l in ((0.125, 2e-2, 1e-3), (1.0, 6e-2, 5e-2)):
+        q, k, v = (ao.round_bf16(rng.standard_normal(sh) * s) for sh in ((B, H, Lq, D), (H, Nc, D), (H, Nc, D)))
+        o1, l1 = ao.context_attention_same_dtype(q, k, v)
+        o0, l0 = ao.context_attention(q, k, v)
+        assert np.abs(o1 - o0).max() <= tol_o and np.abs(l1 - l0).max() <= tol_l
