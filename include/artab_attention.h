@@ -145,6 +145,11 @@ int artab_context_attention(const artab_view *q, const artab_view *k_ctx, const 
  *                replayed while the length advances.  `n_buf` must then be an upper
  *                bound of every value the cell will hold (it is what is validated
  *                against buf_capacity).
+ * Route: a shared context with B*H small enough for every workgroup (8 trajectories of one
+ * head) to be on the chip at once or twice, head_dim 32 or 64 and Nc*Dh <= 2048*64 runs as ONE
+ * launch and touches no workspace; everything else as context pass (split over the workspace)
+ * + buffer pass with the merge.  Both routes give the same result up to the rounding of the
+ * partial results (16-bit in the workspace, float32 in the one-launch kernel).
  */
 int artab_decode_attention(const artab_view *q, const artab_view *k_ctx, const artab_view *v_ctx,
                            const artab_view *k_buf, const artab_view *v_buf,
