@@ -34,7 +34,7 @@
 namespace artab {
 
 constexpr int kStreamChunks = 3;           // ring depth per wavefront
-constexpr int kStreamDeepRows = 224;       // buffers longer than this use the whole ring
+constexpr int kStreamShortRows = 32;       // buffers longer than this are read 16 rows x 4 pairs at a time
 constexpr int kStreamChunkBytes = 8192;    // 4 keys x 16 pairs x (64 B of K + 64 B of V)
 constexpr int kStreamQBytes = 4096;        // one task's queries: 4 x (64 lanes x 16 B)
 constexpr size_t kStreamLdsBytes = kStreamChunks * kStreamChunkBytes + 2 * kStreamQBytes;
@@ -101,6 +101,13 @@ __device__ __forceinline__ int opaque(int v) {
     return v;
 }
 
+// The value held by another lane of this lane's row of 16: the row rotated by N places.
+template <int N>
+__device__ __forceinline__ float row_ror(float v) {
+    const int x = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(x, x, 0x120 + N, 0xf, 0xf, false));
+}
+
 template <typename T>
 struct Mfma4;
 template <>
@@ -119,13 +126,31 @@ struct Mfma4<f16_t> {
     }
 };
 
-// One wavefront per workgroup; a task = 16 consecutive (trajectory, head) pairs; tasks are dealt
-// round-robin over the grid.  Dynamic LDS: kStreamLdsBytes.
-template <typename T, int LQ, int PRIO = 3>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void decode_stream_kernel(DecodeParams P) {
+// One wavefront per workgroup, KEYS rows of 64 / KEYS consecutive (trajectory, head) pairs per
+// chunk; a task = those pairs over the whole buffer; tasks are dealt round-robin over the grid.
+//
+// KEYS = 4: 16 pairs per task, lane 4p + i loads row 4g + i of pair p.  Every lane group of four
+//   is one pair: softmax state and output of (pair, query) live in one lane for the whole task.
+//   A request touches 256 contiguous bytes per pair.
+// KEYS = 16: 4 pairs per task, lane 16p + r loads row 16g + r of pair p: 1 KiB contiguous per pair
+//   and request, which the memory system serves faster once the buffers outgrow the last-level
+//   cache and, above all, with less delay for the loads of a kernel running next door.  The four
+//   lane groups of a pair hold the keys 4k..4k+3 (k = 0..3) of a chunk and keep separate softmax
+//   states; they are merged (rotations within the row of 16 lanes) when the task ends.  More
+//   work per task: worth it only for buffers of some length.
+// The LDS side is the same for both: lane l's row at chunk + 1024 t + 16 l, a 4x4x4 block = four
+// consecutive lanes.  Only what a lane's row *is* differs.
+template <typename T, int LQ, int KEYS>
+__device__ __forceinline__ void decode_stream_body(const DecodeParams &P, unsigned char *stream_lds, int n_buf,
+                                                   bool slot_fits) {
     constexpr int DH = 32;
     constexpr int S = kStreamChunks;
-    extern __shared__ __attribute__((aligned(16))) unsigned char stream_lds[];
+    constexpr int PP = 64 / KEYS;             // pairs per task
+    constexpr int NKG = KEYS / 4;             // lane groups (of four keys each) per pair
+    constexpr int QREG = KEYS == 16 ? 1 : 2;  // 4 KiB query regions in use
+    constexpr int QS = QREG * NKG;            // query slots: lane group k of a region holds one task's queries
+    static_assert(KEYS == 4 || KEYS == 16, "chunk shapes: 16 pairs x 4 rows or 4 pairs x 16 rows");
+    static_assert(QS == 2 || QS == 4, "slot index is taken modulo a power of two");
 
     // Every argument the loop needs, as plain values: the inline assembly clobbers memory, and
     // anything still read through the argument block would be re-read after every such statement.
@@ -135,24 +160,22 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void de
     T *const part_o = static_cast<T *>(P.buf_part_o);
     float *const part_lse = P.buf_part_lse;
     const int n_pairs = P.B * H;
-    bool slot_fits;
-    const int n_buf = committed_rows(P, slot_fits);
     const int n_total = n_buf + (has_new ? 1 : 0);
 
     const int lane = threadIdx.x;
-    const int pl = lane >> 2, sub = lane & 3;  // pair within the task, row / query index
-    const int n_tasks = (n_pairs + 15) / 16;
-    const int n_groups = (n_total + 3) / 4;    // 4-key chunks per task
+    const int n_tasks = (n_pairs + PP - 1) / PP;
+    const int n_groups = (n_total + KEYS - 1) / KEYS;  // chunks per task
 
     const unsigned lds0 = static_cast<unsigned>(reinterpret_cast<uintptr_t>(stream_lds));
     const unsigned q_lds0 = lds0 + S * kStreamChunkBytes;
-    // transposing read: within a 16-lane group lane L supplies the row of (pair L%4, key L/4)
+    // transposing read: within a 16-lane group lane L supplies LDS row 4 (L % 4) + L / 4 of the group
     const unsigned tr_off = 16u * (4u * (4u * (lane >> 4) + (lane & 3)) + ((lane & 15) >> 2));
 
     if (n_total == 0) {  // nothing to attend to: empty partials (weight 0 in the combine)
         for (int task = blockIdx.x; task < n_tasks; task += gridDim.x) {
-            const int pair = 16 * task + pl;
-            if (pair < n_pairs && sub < LQ) {
+            const int pair = PP * task + lane / KEYS;
+            if (pair < n_pairs && lane % KEYS < LQ) {
+                const int sub = lane % KEYS;
                 part_lse[static_cast<long>(pair) * LQ + sub] = -INFINITY;
                 u32x4 z = {0u, 0u, 0u, 0u};
                 T *po = part_o + (static_cast<long>(pair) * LQ + sub) * DH;
@@ -163,42 +186,39 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void de
         return;
     }
 
-    // This wavefront shares its SIMD with two older, compute-bound ones; without a raised
-    // priority it is only issued in their gaps.  It issues little: the priority costs them little.
-    __builtin_amdgcn_s_setprio(PRIO);
-
     // ---- producer: chunk `issue_g` of task `issue_task` into ring slot issue_slot.  Row pointers
-    // are kept per task and advanced by four rows per chunk; only a task's last chunk (clamped
+    // are kept per task and advanced by KEYS rows per chunk; only a task's last chunk (clamped
     // rows, the new row) computes addresses the long way.
     const int my_tasks = blockIdx.x < n_tasks ? (n_tasks - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
     const int total_chunks = my_tasks * n_groups;
-    const long chunk_step = 4 * vkb.sn, chunk_step_v = 4 * vvb.sn;  // elements between rows g*4 and (g+1)*4
-    int issued = 0, issue_task = blockIdx.x, issue_g = 0, issue_slot = 0, issue_q = 0;
+    const long chunk_step = KEYS * vkb.sn, chunk_step_v = KEYS * vvb.sn;  // elements from chunk g to g + 1
+    int issued = 0, issue_task = blockIdx.x, issue_g = 0, issue_slot = 0;
     int issue_seq = 0, seq = 0;  // how many of this wavefront's tasks the producer / consumer have finished
     const T *p_k = nullptr, *p_v = nullptr;  // this lane's row of the chunk to be requested next
     auto issue_one = [&]() {
         const bool first = issue_g == 0, last = issue_g + 1 == n_groups;  // wavefront-uniform
-        int p_b = 0, p_h = 0, pl = 0, sub = 0;
+        int p_b = 0, p_h = 0, kq = 0;
         if (first || last) {  // the (trajectory, head) of this lane's pair: twice per task at most
             const int ln = opaque(lane);
-            pl = ln >> 2;
-            sub = ln & 3;
-            int pair = 16 * issue_task + pl;
+            kq = ln % KEYS;
+            int pair = PP * issue_task + ln / KEYS;
             pair = pair < n_pairs ? pair : n_pairs - 1;  // a ragged last task re-reads the last pair; never stored
             p_b = pair / H;
             p_h = pair % H;
         }
         if (first) {
-            p_k = view_row<T>(vkb, p_b, p_h, sub);
-            p_v = view_row<T>(vvb, p_b, p_h, sub);
-            // the task's queries: lane (p, j < LQ) fetches its 64-byte row in four pieces; the
-            // pieces of the other lanes stay zero (cleared once, below)
-            unsigned char *qd = stream_lds + S * kStreamChunkBytes + issue_q * kStreamQBytes;
-            if (sub < LQ) load_row64_to_lds(view_row<T>(vq, p_b, p_h, sub), qd);
+            p_k = view_row<T>(vkb, p_b, p_h, kq);
+            p_v = view_row<T>(vvb, p_b, p_h, kq);
+            // the task's queries, fetched by the lanes of one lane group per pair (which group:
+            // the slot); the pieces of lanes that stand for no query stay zero (cleared once, below)
+            const int qslot = issue_seq & (QS - 1);
+            unsigned char *qd = stream_lds + S * kStreamChunkBytes + (qslot / NKG) * kStreamQBytes;
+            const int j = kq - 4 * (qslot % NKG);
+            if (j >= 0 && j < LQ) load_row64_to_lds(view_row<T>(vq, p_b, p_h, j), qd);
         }
         const T *kr = p_k, *vr = p_v;
         if (last) {
-            int row = 4 * issue_g + sub;
+            int row = KEYS * issue_g + kq;
             row = row < n_total ? row : n_total - 1;  // keys past the end re-read the last one and are masked
             const bool is_new = has_new && row == n_buf;
             kr = is_new ? view_row<T>(vkn, p_b, p_h, 0) : view_row<T>(vkb, p_b, p_h, row);
@@ -214,23 +234,18 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void de
         if (++issue_g == n_groups) {
             issue_g = 0;
             issue_task += gridDim.x;
-            issue_q ^= 1;
             ++issue_seq;
         }
     };
-    // Lanes that stand for no query (sub >= LQ) contribute zeros to the score product: their
-    // pieces of both query slots are cleared once and never written again.
-    if (sub >= LQ) {
+    // Lanes that stand for no query (index within the lane group >= LQ) contribute zeros to the
+    // score product: their pieces of every query region are cleared once and never written again.
+    if ((lane & 3) >= LQ) {
         const u32x4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
-        for (int t = 0; t < 8; ++t) lds_write128(q_lds0 + 1024u * t + lane * 16u, zero);
+        for (int t = 0; t < 4 * QREG; ++t) lds_write128(q_lds0 + 1024u * t + lane * 16u, zero);
     }
-    // two query slots: the producer may be at most one task ahead of the consumer
-    auto may_issue = [&]() { return issued < total_chunks && issue_seq <= seq + 1; };
-    // Chunks kept in flight.  The loads hold the CU's outstanding-miss slots that the context pass
-    // next door needs for its own tiles; a buffer that is finished before that pass anyway uses
-    // half the ring and disturbs it less (measured at B=1024, H=8: 950 -> 974 steps/s; a quarter of
-    // the ring is too little: 933).  A long one is on the critical path itself.
+    // QS query slots: the producer may be at most QS - 1 tasks ahead of the consumer
+    auto may_issue = [&]() { return issued < total_chunks && issue_seq <= seq + (QS - 1); };
     const int depth = S;
     for (int i = 0; i < depth; ++i)
         if (may_issue()) issue_one();
@@ -244,13 +259,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void de
     f32x4 o[8];  // output dims 4u..4u+3 of this lane's query
 #pragma unroll
     for (int u = 0; u < 8; ++u) o[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-    int task = blockIdx.x, g = 0, slot = 0, qsel = 0;
-    const int new_group = has_new && slot_fits ? n_buf >> 2 : -1;  // the chunk that holds the row to append
+    int task = blockIdx.x, g = 0, slot = 0;
+    const int new_group = has_new && slot_fits ? n_buf / KEYS : -1;  // the chunk that holds the row to append
     u32x4 qr[4];  // this lane's query row (zero for lanes that stand for no query)
     u32x4 kr[4];  // the K rows of the chunk whose scores come next
 
     // chunk `c` must have landed; only the chunks requested after it (8 loads each: 4 for the K
-    // rows, then 4 for the V rows) may be pending
+    // rows, then 4 for the V rows) may be pending.  (A task's query loads sit in front of its
+    // first chunk's: where they are in flight the wait is stricter than needed, never too lax.)
     auto wait_chunk = [&](int c) {
         switch (issued - c - 1) {
             case 3: __builtin_amdgcn_s_waitcnt(vmcnt_imm(24)); break;
@@ -280,6 +296,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void de
     };
     // online softmax of four raw dot products (qscale > 0 enters with the exponent); the rescale is
     // skipped (wavefront-uniformly) while no maximum moves.  Returns the packed probabilities.
+    // A lane group that has seen no valid key yet (KEYS = 16, short buffers) keeps m = -inf and
+    // mq = 0: its probabilities are exp2(-inf) = 0.
     auto softmax = [&](const float (&sc)[4]) {
         const float m_new = max3(max3(m, sc[0], sc[1]), sc[2], sc[3]);
         if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
@@ -288,11 +306,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void de
 #pragma unroll
             for (int u = 0; u < 8; ++u) o[u] *= alpha;
             m = m_new;
-            mq = m_new * qscale;
+            mq = KEYS > 4 && m_new == -INFINITY ? 0.f : m_new * qscale;
         }
         float p[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) p[r] = fast_exp2(fmaf(sc[r], qscale, -mq));  // m is finite here: key 4g is always valid
+        for (int r = 0; r < 4; ++r) p[r] = fast_exp2(fmaf(sc[r], qscale, -mq));
         l += (p[0] + p[1]) + (p[2] + p[3]);
         return u32x2{pack2<T>(p[0], p[1]), pack2<T>(p[2], p[3])};
     };
@@ -329,7 +347,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void de
     int c = 0;
     while (c < total_chunks) {
         // how many steady steps lie ahead: consumer and producer both strictly inside a task
-        if (g >= 1 && issue_g >= 1 && issued - c == depth && issue_seq <= seq + 1) {
+        if (g >= 1 && issue_g >= 1 && issued - c == depth && issue_seq <= seq + (QS - 1)) {
             int run = n_groups - 1 - (g > issue_g ? g : issue_g);
             if (new_group >= g && new_group - g < run) run = new_group - g;
             if (run > 0) {
@@ -343,7 +361,13 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void de
         }
         const unsigned chunk = lds0 + static_cast<unsigned>(slot) * kStreamChunkBytes;
         const bool more = c + 1 < total_chunks;
-        if (g == 0) lds_read4x128(qr, q_lds0 + static_cast<unsigned>(qsel) * kStreamQBytes + lane * 16u);
+        if (g == 0) {
+            // the task's queries: those of the lane's pair and query index, from the lane group
+            // that fetched them for this slot
+            const int ln = opaque(lane), qslot = seq & (QS - 1);
+            const int src = ln - 4 * ((ln % KEYS) >> 2) + 4 * (qslot % NKG);
+            lds_read4x128(qr, q_lds0 + static_cast<unsigned>(qslot / NKG) * kStreamQBytes + src * 16u);
+        }
         u32x2 vop[8];
         wait_chunk(c);
         lds_issue_v(vop, chunk + 4096u + tr_off);
@@ -356,8 +380,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void de
         }
         float sc[4] = {s[0], s[1], s[2], s[3]};
         if (g + 1 == n_groups) {  // only a task's last chunk can hold keys past the end
+            const int key0 = KEYS * g + ((opaque(lane) % KEYS) & ~3);  // first key of this lane group
 #pragma unroll
-            for (int r = 0; r < 4; ++r) sc[r] = 4 * g + r < n_total ? sc[r] : -INFINITY;
+            for (int r = 0; r < 4; ++r) sc[r] = key0 + r < n_total ? sc[r] : -INFINITY;
         }
         const u32x2 pop = softmax(sc);
         lds_wait(kr, vop);
@@ -367,9 +392,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void de
         if (g == new_group) {
             // in-place append (once per task): the lane that holds the new row copies it from the
             // chunk, lane-locally, into slot n_buf of the cache
-            const int ln = opaque(lane), pl = ln >> 2, sub = ln & 3;
-            const int pair = 16 * task + pl;
-            if (4 * g + sub == n_buf && pair < n_pairs) {
+            const int ln = opaque(lane);
+            const int pair = PP * task + ln / KEYS;
+            if (KEYS * g + ln % KEYS == n_buf && pair < n_pairs) {
                 const int b = pair / H, h = pair % H;
                 T *kd = view_row<T>(vkb, b, h, n_buf), *vd = view_row<T>(vvb, b, h, n_buf);
                 u32x4 kk[4], vv[4];
@@ -388,9 +413,31 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void de
 
         slot = slot + 1 == S ? 0 : slot + 1;
         if (++g == n_groups) {
-            // ---- task done: write this lane's partial (lanes of real queries of real pairs)
-            const int ln = opaque(lane), pl = ln >> 2, sub = ln & 3;
-            const int pair = 16 * task + pl;
+            // ---- task done
+            if (NKG > 1) {
+                // merge the lane groups of a pair: lanes l, l+4, l+8, l+12 of a row of 16 hold
+                // states of the same (pair, query) over disjoint keys; afterwards each holds the sum
+                float mt = fmaxf(m, row_ror<4>(m));
+                mt = fmaxf(mt, row_ror<8>(mt));
+                const float f = m == -INFINITY ? 0.f : fast_exp2((m - mt) * qscale);
+                l *= f;
+                l += row_ror<4>(l);
+                l += row_ror<8>(l);
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float x = o[u][e] * f;
+                        x += row_ror<4>(x);
+                        x += row_ror<8>(x);
+                        o[u][e] = x;
+                    }
+                mq = mt == -INFINITY ? 0.f : mt * qscale;
+            }
+            // write the partial of this lane's (pair, query): the first lane group of each pair,
+            // lanes of real queries of real pairs
+            const int ln = opaque(lane);
+            const int pair = PP * task + ln / KEYS, sub = ln % KEYS;
             if (pair < n_pairs && sub < LQ) {
                 const float inv = l > 0.f ? 1.f / l : 0.f;
                 T *po = part_o + (static_cast<long>(pair) * LQ + sub) * DH;
@@ -410,10 +457,26 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void de
             for (int u = 0; u < 8; ++u) o[u] = f32x4{0.f, 0.f, 0.f, 0.f};
             g = 0;
             task += gridDim.x;
-            qsel ^= 1;
         }
         ++c;
     }
+}
+
+// Buffers of at most `P.stream_short_rows` rows (committed + new) take the 16-pair chunks, longer
+// ones the 4-pair chunks: one kernel, so that a recorded launch serves every length.  KEYS != 0
+// pins the shape.  Dynamic LDS: kStreamLdsBytes.
+template <typename T, int LQ, int PRIO = 3, int KEYS = 0>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void decode_stream_kernel(DecodeParams P) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char stream_lds[];
+    bool slot_fits;
+    const int n_buf = committed_rows(P, slot_fits);
+    // This wavefront shares its SIMD with older, compute-bound ones; without a raised priority it
+    // is only issued in their gaps.  It issues little: the priority costs them little.
+    __builtin_amdgcn_s_setprio(PRIO);
+    if (KEYS == 4 || (KEYS == 0 && n_buf + (P.has_new ? 1 : 0) <= P.stream_short_rows))
+        decode_stream_body<T, LQ, 4>(P, stream_lds, n_buf, slot_fits);
+    else
+        decode_stream_body<T, LQ, 16>(P, stream_lds, n_buf, slot_fits);
 }
 
 }  // namespace artab

@@ -215,6 +215,44 @@ def test_decode_attention_overlapped_matches_oracle(device, small_route, dtype, 
     _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, True, scale=0.6, overlapped=True)
 
 
+@pytest.fixture(params=["0", "100000", None], ids=["16-row-chunks", "4-row-chunks", "by-length"])
+def stream_chunk_shape(request, monkeypatch):
+    """The streaming buffer pass reads 4 rows of 16 pairs or 16 rows of 4 pairs per request and
+    picks by buffer length (ARTAB_STREAM_SHORT: the longest buffer that takes the first shape)."""
+    monkeypatch.setenv("ARTAB_SMALL", "0")
+    if request.param is not None:
+        monkeypatch.setenv("ARTAB_STREAM_SHORT", request.param)
+    return request.param
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize(
+    "B,H,Lq,Nc,D,n_buf,cap,with_new",
+    [
+        (8, 4, 2, 64, 32, 0, 16, True),    # the new row alone: one lane group of a 16-row chunk has a key
+        (8, 4, 1, 64, 32, 1, 16, False),   # one committed row, one query
+        (8, 4, 2, 64, 32, 3, 16, True),    # 4 rows
+        (8, 4, 2, 64, 32, 4, 16, True),    # 5 rows: the second lane group holds the new row alone
+        (8, 4, 2, 64, 32, 15, 16, True),   # exactly one 16-row chunk, new row in its last lane
+        (8, 4, 2, 64, 32, 16, 32, True),   # 17 rows: the new row alone in a second chunk
+        (8, 4, 1, 64, 32, 16, 32, False),  # 16 committed rows, nothing to append
+        (7, 5, 2, 128, 32, 31, 48, True),  # 35 pairs (ragged for both shapes), two full chunks
+        (7, 5, 2, 128, 32, 32, 48, True),
+        (7, 5, 1, 128, 32, 47, 48, True),  # last slot of the cache, three chunks
+        (5, 3, 2, 200, 32, 22, 40, True),  # 15 pairs
+        (1, 1, 2, 64, 32, 20, 32, True),   # a single pair
+        (3, 2, 2, 64, 32, 77, 100, True),  # steady steps between a task's first and last chunk
+        (128, 8, 2, 2048, 32, 100, 128, True),
+        (600, 8, 2, 1024, 32, 37, 64, True),  # several tasks per wavefront with either shape
+        (600, 8, 1, 1024, 32, 9, 64, True),   # ... of one chunk each
+        (300, 8, 2, 512, 32, 255, 256, True),  # the longest buffer
+    ],
+)
+def test_decode_attention_stream_chunk_shapes(device, stream_chunk_shape, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new):
+    """The streaming buffer pass (beside the context pass) in both of its chunk shapes."""
+    _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, True, scale=0.6, overlapped=True)
+
+
 def test_decode_attention_overlapped_device_length_in_graph(device):
     """The overlapped call recorded into a graph (fork/join inside the capture) with the buffer
     length in device memory: every replay appends one row and must equal the eager plain call."""
