@@ -16,7 +16,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libartab_attention.so")
 
-ABI_VERSION = 4  # ARTAB_VERSION of include/artab_attention.h
+ABI_VERSION = 5  # ARTAB_VERSION of include/artab_attention.h
 STATIC_SCRATCH_BYTES = 32 << 20  # ARTAB_STATIC_SCRATCH_BYTES
 ARTAB_BF16, ARTAB_F16, ARTAB_F32 = 0, 1, 2
 IMPL_AUTO, IMPL_PORTABLE, IMPL_MFMA = 0, 1, 2
@@ -128,6 +128,11 @@ SIGNATURES = {
         [ctypes.POINTER(ArtabAttentionPartials), _p, _i64, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _f, _p, _p, _p, _f, _p, _p, _p, _i64, _i, _i, _i, _p],
     ),
     "artab_decode_sample_embed": (_i, [ctypes.POINTER(ArtabSampleEmbedArgs), _i, _p]),
+    "artab_decode_step_boundary": (
+        _i,
+        [ctypes.POINTER(ArtabAttentionPartials), _p, _i64, _p, _i64, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _f,
+         ctypes.POINTER(ArtabSampleEmbedArgs), _p, _p, _p, _f, _p, _p, _p, _i, _i, _p],
+    ),
     "artab_layer_post": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _f, _p, _i64, _i, _i, _i, _p]),
 }
 

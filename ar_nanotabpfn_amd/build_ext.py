@@ -35,7 +35,7 @@ HIPCC_FLAGS = [
 UNITS = [("artab_api.hip", [], "artab_api.o"), ("flash_launch.hip", [], "flash_launch.o"),
          ("mix_bench.hip", [], "mix_bench.o")]
 for _bf16 in (1, 0):
-    for _group in (0, 1, 2):
+    for _group in (0, 1, 2, 3):
         UNITS.append(("layer_launch.hip", [f"-DARTAB_LAYER_BF16={_bf16}", f"-DARTAB_LAYER_GROUP={_group}"],
                       f"layer_launch_{'bf16' if _bf16 else 'f16'}_{_group}.o"))
 

@@ -1206,7 +1206,7 @@ static int fill_post(FusedPostParams &P, const void *attn, int64_t lda, const vo
 // free — a waiting workgroup must not keep the buffer pass it waits for off the chip — and into a
 // launch of its own otherwise.
 static int apply_partials_order(const artab_attention_partials *parts, FusedPostParams &P, int64_t rows,
-                                hipStream_t st) {
+                                hipStream_t st, int64_t grid_of_launch = -1) {
     if (!parts || !(parts->order_flags & ARTAB_ORDER_WAIT)) return ARTAB_OK;
     ARTAB_TRY(check_order_args(parts->order_state, ARTAB_ORDER_MAIN));
     if (rows == 0) return fail(ARTAB_ERR_BAD_SHAPE, "ordered partials with no rows");
@@ -1215,7 +1215,8 @@ static int apply_partials_order(const artab_attention_partials *parts, FusedPost
         if (hipGetDevice(&dev) != hipSuccess ||
             hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
             cus = 0;
-        const int64_t grid = (rows + fused_tile_rows(rows) - 1) / fused_tile_rows(rows);
+        const int64_t grid =
+            grid_of_launch >= 0 ? grid_of_launch : (rows + fused_tile_rows(rows) - 1) / fused_tile_rows(rows);
         const uint64_t us = parts->order_timeout_us ? parts->order_timeout_us : 2000000;
         if (grid * 2 <= cus && env_int("ARTAB_ORDER_GATE_LAUNCH", 0) == 0) {
             P.order_wait = parts->order_state;
@@ -1323,7 +1324,7 @@ int artab_layer_post_from_partials(const artab_attention_partials *parts, const 
     return launch_status(e, "layer_post");
 }
 
-int artab_decode_sample_embed(const artab_sample_embed_args *a, int dtype, void *stream) {
+static int fill_sample(SampleEmbedParams &P, const artab_sample_embed_args *a, int dtype, bool x_required) {
     if (!a) return fail(ARTAB_ERR_NULL_POINTER, "args is NULL");
     if (dtype != ARTAB_BF16 && dtype != ARTAB_F16)
         return fail(ARTAB_ERR_UNSUPPORTED, "decode_sample_embed supports bf16 and fp16 only (dtype code %d)", dtype);
@@ -1333,16 +1334,15 @@ int artab_decode_sample_embed(const artab_sample_embed_args *a, int dtype, void 
         return fail(ARTAB_ERR_UNSUPPORTED, "decode_sample_embed needs D, F in {128, 256, 512} and K <= %d (got %d, %d, %d)",
                     kMaxMixture, a->D, a->F, a->K);
     if (a->B == 0) return ARTAB_OK;
-    if (!a->x_last || !a->norm_gamma || !a->norm_beta || !a->w_h1 || !a->w_h2 || !a->mean_bias || !a->std_bias ||
-        !a->weight_bias || !a->rand_u || !a->rand_n || !a->x_mean || !a->w_x || !a->b_x || !a->w_y || !a->b_y ||
-        !a->markers || !a->ar_tokens || !a->step || !a->preds || !a->emb_next)
+    if ((x_required && !a->x_last) || !a->norm_gamma || !a->norm_beta || !a->w_h1 || !a->w_h2 || !a->mean_bias ||
+        !a->std_bias || !a->weight_bias || !a->rand_u || !a->rand_n || !a->x_mean || !a->w_x || !a->b_x || !a->w_y ||
+        !a->b_y || !a->markers || !a->ar_tokens || !a->step || !a->preds || !a->emb_next)
         return fail(ARTAB_ERR_NULL_POINTER, "decode_sample_embed: only b_h1 and b_h2 may be NULL");
-    if (misaligned16(a->x_last) || misaligned16(a->w_h1) || misaligned16(a->w_h2) || misaligned16(a->b_h1) ||
-        misaligned16(a->b_h2) || misaligned16(a->norm_gamma) || misaligned16(a->norm_beta) || misaligned16(a->w_x) ||
-        misaligned16(a->b_x) || misaligned16(a->w_y) || misaligned16(a->b_y) || misaligned16(a->markers) ||
-        misaligned16(a->ar_tokens) || misaligned16(a->emb_next) || a->ld_row % 8 || a->ld_row < a->D)
+    if ((x_required && (misaligned16(a->x_last) || a->ld_row % 8 || a->ld_row < a->D)) || misaligned16(a->w_h1) ||
+        misaligned16(a->w_h2) || misaligned16(a->b_h1) || misaligned16(a->b_h2) || misaligned16(a->norm_gamma) ||
+        misaligned16(a->norm_beta) || misaligned16(a->w_x) || misaligned16(a->b_x) || misaligned16(a->w_y) ||
+        misaligned16(a->b_y) || misaligned16(a->markers) || misaligned16(a->ar_tokens) || misaligned16(a->emb_next))
         return fail(ARTAB_ERR_BAD_STRIDE, "decode_sample_embed: model vectors and rows must be 16-byte aligned");
-    SampleEmbedParams P;
     P.x_last = a->x_last; P.ld_row = a->ld_row; P.norm_g = a->norm_gamma; P.norm_b = a->norm_beta; P.eps = a->eps;
     P.w_h1 = a->w_h1; P.b_h1 = a->b_h1; P.w_h2 = a->w_h2; P.b_h2 = a->b_h2;
     P.mean_bias = a->mean_bias; P.std_bias = a->std_bias; P.weight_bias = a->weight_bias;
@@ -1354,9 +1354,47 @@ int artab_decode_sample_embed(const artab_sample_embed_args *a, int dtype, void 
     if (a->advance && (a->n_advance < 1 || a->n_advance > 8 || !a->ticket))
         return fail(ARTAB_ERR_BAD_SHAPE, "advance needs 1..8 counters and a ticket word");
     P.advance = a->advance; P.n_advance = a->advance ? a->n_advance : 0; P.ticket = a->ticket;
+    return ARTAB_OK;
+}
+
+int artab_decode_sample_embed(const artab_sample_embed_args *a, int dtype, void *stream) {
+    SampleEmbedParams P{};
+    ARTAB_TRY(fill_sample(P, a, dtype, true));
+    if (a->B == 0) return ARTAB_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipError_t e = launch_sample_embed(P, a->D, a->F, dtype == ARTAB_BF16, st);
     return launch_status(e, "decode_sample_embed");
+}
+
+int artab_decode_step_boundary(const artab_attention_partials *parts, const void *attn, int64_t lda, const void *y,
+                               int64_t ldy, const void *w_o, const void *ln2_gamma, const void *ln2_beta, float eps2,
+                               const void *w_1, const void *b_1, const void *w_2, const void *b_2,
+                               const void *ln3_gamma, const void *ln3_beta, float eps3,
+                               const artab_sample_embed_args *tail, const void *next_w_fo,
+                               const void *next_ln1_gamma, const void *next_ln1_beta, float next_eps1,
+                               const void *next_w_qkv, void *next_y, void *next_qkv, int F, int dtype, void *stream) {
+    SampleEmbedParams S{};
+    ARTAB_TRY(fill_sample(S, tail, dtype, false));
+    const int64_t B = tail->B;
+    const int D = tail->D;
+    if (F != tail->F)
+        return fail(ARTAB_ERR_UNSUPPORTED, "decode_step_boundary: head width %d differs from the layers' feed-forward width %d",
+                    tail->F, F);
+    if (fused_tile_rows(2 * B) != kFusedRowsSmall || fused_tile_rows(B) != kFusedRowsSmall)
+        return fail(ARTAB_ERR_UNSUPPORTED, "decode_step_boundary covers up to %ld trajectories on %d-row tiles",
+                    kFusedSmallMaxRows / 2, kFusedRowsSmall);
+    if (parts && parts->n_slots == 0) parts = nullptr;  // the call that made them wrote `attn` instead
+    FusedPostParams P{};
+    FusedPreParams N{};
+    ARTAB_TRY(fill_post(P, attn, lda, y, ldy, w_o, ln2_gamma, ln2_beta, eps2, w_1, b_1, w_2, b_2, ln3_gamma, ln3_beta,
+                        eps3, nullptr, B, D, F, false, parts));
+    ARTAB_TRY(fill_pre(N, nullptr, 0, next_w_fo, next_ln1_gamma, next_ln1_beta, next_eps1, next_w_qkv, next_y, next_qkv,
+                       2 * B, D, false));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    ARTAB_TRY(apply_partials_order(parts, P, B, st, (B + kFusedRowsSmall / 2 - 1) / (kFusedRowsSmall / 2)));
+    if (B == 0) return ARTAB_OK;
+    hipError_t e = launch_step_boundary(P, S, N, D, F, dtype == ARTAB_BF16, st);
+    return launch_status(e, "decode_step_boundary");
 }
 
 }  // extern "C"

@@ -185,8 +185,8 @@ struct WeightStream {
     // of the CU's address unit (64 B/clk: 1 us for a 128 KiB matrix over the eight wavefronts) and
     // the wavefront waits at each; run() can spread the requests of the NEXT stream over the steps
     // of its own product (`per_step`), so that its MFMAs execute while the requests queue.
-    __device__ __forceinline__ void start(const T *wp, const int (&nblk)[NB], int lane) {
-        begin(wp, nblk, lane);
+    __device__ __forceinline__ void start(const T *wp, const int (&nblk)[NB], int lane, int tile = -1) {
+        begin(wp, nblk, lane, tile);
 #pragma unroll
         for (int p = 0; p < PF; ++p) request(p);
         __builtin_amdgcn_sched_barrier(0);  // the prefetch stays where it was written
@@ -206,7 +206,10 @@ struct WeightStream {
             if (p * n_steps / PF == ks) request(p);
     }
 
-    __device__ __forceinline__ void begin(const T *wp, const int (&nblk)[NB], int lane) {
+    // `tile`: index of this workgroup's tile in the launch that would process the same rows on
+    // their own (default: the workgroup index).  A kernel that runs several bodies on differently
+    // sized tiles passes it, so that a row's sums are taken in the same order wherever it is computed.
+    __device__ __forceinline__ void begin(const T *wp, const int (&nblk)[NB], int lane, int tile = -1) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) wl[b] = wp + TL::weight_offset(nblk[b], K, lane);
         // Every workgroup streams the same matrix at about the same time, and the 16 of an XCD
@@ -214,7 +217,7 @@ struct WeightStream {
         // kernel).  Each starts its contraction at a different step instead; a sum does not care.
         // Workgroup ids are dealt round-robin over the 8 XCDs, so id / 8 counts within an XCD.
         static_assert((KS & (KS - 1)) == 0, "contraction steps must be a power of two");
-        rot = (blockIdx.x >> 3) & (KS - 1);
+        rot = ((tile < 0 ? static_cast<int>(blockIdx.x) : tile) >> 3) & (KS - 1);
     }
 
     // `before` runs ahead of the product — the place to begin() a later stream —, `per_step(ks)`
@@ -615,7 +618,7 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
                                                long row0, int valid,
                                                WeightStream<T, D, fused_blocks<T, TR>(D, fused_waves(D)), TR> &w_a,
                                                WeightStream<T, D, fused_blocks<T, TR>(D, fused_waves(D)), TR> &w_b,
-                                               T *vecs, int vec_ld) {
+                                               T *vecs, int vec_ld, int tile = -1) {
     typedef Tile<T, TR> TL;
     constexpr int NW = fused_waves(D), NT = NW * 64;
     constexpr int LD = D + 8;
@@ -632,13 +635,13 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
     // requested W_fo and, with Q_REQUESTED, the q weights already.
     constexpr bool kWhole = WeightStream<T, D, NB, TR>::kWhole;
     if (!X_IN_LDS) {
-        w_a.start(static_cast<const T *>(P.w_fo), nblk, lane);
+        w_a.start(static_cast<const T *>(P.w_fo), nblk, lane, tile);
         dma_tile<T, D, NT, TR>(a0, LD, static_cast<const T *>(P.x) + row0 * P.ldx, P.ldx, valid, tid);
         stage_pre_vectors<T, D, NT>(P, vecs, vec_ld, tid);
         wait_all_loads();
         __syncthreads();
     }
-    if (!Q_REQUESTED) w_b.start(static_cast<const T *>(P.w_qkv), nblk, lane);  // q columns
+    if (!Q_REQUESTED) w_b.start(static_cast<const T *>(P.w_qkv), nblk, lane, tile);  // q columns
     int nb_k[NB], nb_v[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
@@ -653,7 +656,7 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
     {
         typename TL::acc_t acc[NB];
         // whole-matrix streams: the k weights go where W_fo's fragments were, step by step
-        w_a.run(acc, a0, LD, c, hb, [&]() { if (kWhole) w_a.begin(static_cast<const T *>(P.w_qkv), nb_k, lane); },
+        w_a.run(acc, a0, LD, c, hb, [&]() { if (kWhole) w_a.begin(static_cast<const T *>(P.w_qkv), nb_k, lane, tile); },
                 [&](int ks) { if (kWhole) w_a.request_share(ks, WeightStream<T, D, NB, TR>::KS); });
         float v[NB][VB];
 #pragma unroll
@@ -681,9 +684,9 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
         cur.run(acc, a1, LD, c, hb,
                 [&]() {
                     if (kWhole) {
-                        if (part == 0) w_b.begin(static_cast<const T *>(P.w_qkv), nb_v, lane);
+                        if (part == 0) w_b.begin(static_cast<const T *>(P.w_qkv), nb_v, lane, tile);
                     } else if (part < 2) {
-                        nxt.begin(static_cast<const T *>(P.w_qkv), part == 0 ? nb_k : nb_v, lane);
+                        nxt.begin(static_cast<const T *>(P.w_qkv), part == 0 ? nb_k : nb_v, lane, tile);
                     }
                 },
                 [&](int ks) {
@@ -730,7 +733,8 @@ template <typename T, int D, int F, int TR, bool WRITE_OUT, typename MidBegin, t
           typename LastSteps>
 __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0, T *a1, float *red_a, float *red_b,
                                                 long row0, int valid, MidBegin mid_begin, MidSteps mid_steps,
-                                                LastBegin last_begin, LastSteps last_steps, T *vecs, int vec_ld) {
+                                                LastBegin last_begin, LastSteps last_steps, T *vecs, int vec_ld,
+                                                int tile = -1) {
     typedef Tile<T, TR> TL;
     constexpr int NW = fused_waves(D), NT = NW * 64;
     constexpr int LDD = D + 8, LDF = F + 8;
@@ -765,7 +769,7 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
     constexpr bool kWhole = WeightStream<T, D, NBD, TR>::kWhole && WeightStream<T, D, NBF, TR>::kWhole &&
                             WeightStream<T, F, NBD, TR>::kWhole;
     // the first weights travel while the partials are waited for, fetched and merged
-    if (kWhole) w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
+    if (kWhole) w_o.start(static_cast<const T *>(P.w_o), nbd, lane, tile);
     if (P.part_o) {
         if (P.order_wait) {  // the buffer pass's partial comes from the other queue
             if (tid == 0) order_wait_device(P.order_wait, 0, P.order_limit);
@@ -773,19 +777,19 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
         }
         stage_merged_attention<T, D, NT, TR>(
             a0, LDD, P, row0, valid, tid,
-            [&]() { if (kWhole && ff_active) w_1.begin(static_cast<const T *>(P.w_1), nbf, lane); },
+            [&]() { if (kWhole && ff_active) w_1.begin(static_cast<const T *>(P.w_1), nbf, lane, tile); },
             [&](int u) { if (kWhole && ff_active) w_1.request_share(u, kMergeBatch); });
         if (!kWhole) {
-            w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
+            w_o.start(static_cast<const T *>(P.w_o), nbd, lane, tile);
             wait_all_loads();
         }
     } else {
-        if (!kWhole) w_o.start(static_cast<const T *>(P.w_o), nbd, lane);
+        if (!kWhole) w_o.start(static_cast<const T *>(P.w_o), nbd, lane, tile);
         wait_all_loads();
-        if (kWhole && ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane);
+        if (kWhole && ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane, tile);
     }
     __syncthreads();
-    if (!kWhole && ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane);
+    if (!kWhole && ff_active) w_1.start(static_cast<const T *>(P.w_1), nbf, lane, tile);
 
     // ---- x1 = LN2(y + attn W_o^T); each lane replaces exactly the y entries it read
     {
@@ -801,11 +805,11 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
                 for (int q = 0; q < TL::kVals; ++q) acc[b][q] = 0.f;
             // W_2 goes where W_o's fragments were, step by step: two matrices (W_1, W_2) are then
             // on their way while this product's epilogue runs, and the memory pipeline never idles
-            if (kWhole) w_2.begin(static_cast<const T *>(P.w_2), nbd, lane);
+            if (kWhole) w_2.begin(static_cast<const T *>(P.w_2), nbd, lane, tile);
             w.multiply(acc, a0, LDD, c, hb,
                        [&](int ks) { if (kWhole) w_2.request_share(ks, WeightStream<T, D, NBD, TR>::KS); });
         }
-        if (!kWhole) w_2.start(static_cast<const T *>(P.w_2), nbd, lane);
+        if (!kWhole) w_2.start(static_cast<const T *>(P.w_2), nbd, lane, tile);
         float v[NBD][VB];
 #pragma unroll
         for (int b = 0; b < NBD; ++b)
@@ -962,8 +966,59 @@ struct SampleEmbedParams {
 
 constexpr int kMaxMixture = 10;  // 3 * K outputs must fit one 32-column block
 
-template <typename T, int D, int F, int TR>
-__global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(SampleEmbedParams P) {
+// What a thread of the step tail needs from memory for itself: its trajectory's variates (threads
+// 0 .. valid-1), the feature means of the rows its embedding items cover, and one of the 3 K
+// mixture biases (threads 0 .. 3K-1: mean, std, weight biases in turn).  Loaded as early as the
+// caller can afford the registers; used late.
+template <typename T, int N>
+struct StepTailRegs {
+    float u, n, xv[N];
+    T mix;
+};
+template <int D, int TR, bool FUSED>
+constexpr int step_tail_items() { return (FUSED ? TR / 2 : TR) * 2 * (D / 8) / (fused_waves(D) * 64); }
+
+template <typename T, int D, int TR, bool FUSED>
+__device__ __forceinline__ StepTailRegs<T, step_tail_items<D, TR, FUSED>()> load_step_tail_regs(
+    const SampleEmbedParams &P, int t, long row0, int valid) {
+    constexpr int NT = fused_waves(D) * 64, CPR_E = D / 8, N = step_tail_items<D, TR, FUSED>();
+    const int tid = threadIdx.x;
+    StepTailRegs<T, N> r;
+    r.u = r.n = 0.f;
+    if (tid < valid) {
+        r.u = P.rand_u[static_cast<long>(t) * P.B + row0 + tid];
+        r.n = P.rand_n[static_cast<long>(t) * P.B + row0 + tid];
+    }
+    const T *xm = static_cast<const T *>(P.x_mean);
+    const int tn = min(t + 1, P.Nt - 1);
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+        const int idx = tid + k * NT;
+        const int which = (idx / CPR_E) & 1, row = idx / (2 * CPR_E);
+        r.xv[k] = row < valid ? to_f32(xm[(row0 + row) * P.Nt + (which == 0 ? t : tn)]) : 0.f;
+    }
+    r.mix = from_f32<T>(0.f);
+    if (tid < 3 * P.K) {
+        const T *src = static_cast<const T *>(tid < P.K ? P.mean_bias : (tid < 2 * P.K ? P.std_bias : P.weight_bias));
+        r.mix = src[tid % P.K];
+    }
+    return r;
+}
+
+// Body of the step tail on the TR-row tile of trajectories row0 .. row0 + valid - 1.
+// Stand-alone (FUSED = false): the target rows are staged from P.x_last into a0 here and the
+// head's first matrix is requested here.  FUSED: a finished, synchronised tile is already in a0
+// (row stride D + 8), `w_1` has been requested by the caller when W1_REQUESTED, and the two
+// embedded rows of trajectory r are also left in `x_next` (an LDS tile, row stride D + 8, rows
+// 2 r and 2 r + 1; valid <= TR / 2 then) for the pre body that follows.  `before_draw` runs after
+// the first head product: the place to request what the caller needs next.
+// a0: z = norm(x_last) [TR, D + 8]; a1: gelu(head layer 1) [TR, F + 8].
+template <typename T, int D, int F, int TR, bool FUSED, bool W1_REQUESTED = false, typename Hook = NoHook>
+__device__ __forceinline__ void sample_embed_body(
+    const SampleEmbedParams &P, int t, T *a0, T *a1, float (*raw_s)[33], float *y_s, T *mix_s, long row0, int valid,
+    const StepTailRegs<T, step_tail_items<D, TR, FUSED>()> &regs,
+    WeightStream<T, D, fused_blocks<T, TR>(F, fused_waves(D)), TR> &w_1, T *x_next = nullptr, int tile = -1,
+    Hook before_draw = Hook{}, const T *mk_target = nullptr, const T *mk_buffer = nullptr, const T *token = nullptr) {
     typedef Tile<T, TR> TL;
     constexpr int NW = fused_waves(D), NT = NW * 64;
     constexpr int LDD = D + 8, LDF = F + 8;
@@ -971,16 +1026,9 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
     constexpr int NB2 = 32 / TL::kBlock;  // the second head layer is padded to 32 outputs: first wavefront
     constexpr int VB = TL::kVals, GB = TL::kGroups;
     constexpr int EPL = D / 64;  // elements per lane of one row in the row-wise norm
+    constexpr int ROWS = FUSED ? TR / 2 : TR;  // rows of the tile that can hold a trajectory
     static_assert(F / TL::kBlock >= NW ? (F / TL::kBlock) % NW == 0 : true, "unsupported widths");
-    __shared__ __attribute__((aligned(16))) T a0[TR * LDD];  // z = norm(x_last)
-    __shared__ __attribute__((aligned(16))) T a1[TR * LDF];  // gelu(head layer 1)
-    __shared__ float raw_s[TR][33];
-    __shared__ float y_s[TR];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = TL::token(lane), hb = TL::sub(lane);
-    const int t = *P.step;
-    if (t < 0 || t >= P.Nt) return;  // uniform over the grid
-    const long row0 = static_cast<long>(blockIdx.x) * TR;
-    const int valid = static_cast<int>(min(static_cast<long>(TR), P.B - row0));
 
     int nbf[NBF];
 #pragma unroll
@@ -989,10 +1037,9 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
 #pragma unroll
     for (int b = 0; b < NB2; ++b) nb0[b] = b;
     const bool ff_active = wave < F / TL::kBlock;
-    WeightStream<T, D, NBF, TR> w_1;
     WeightStream<T, F, NB2, TR> w_2;
-    if (ff_active) w_1.start(static_cast<const T *>(P.w_h1), nbf, lane);
-    if (wave == 0) w_2.start(static_cast<const T *>(P.w_h2), nb0, lane);
+    if (!W1_REQUESTED && ff_active) w_1.start(static_cast<const T *>(P.w_h1), nbf, lane, tile);
+    if (wave == 0) w_2.start(static_cast<const T *>(P.w_h2), nb0, lane, tile);
     // Everything small that a later phase reads from memory is requested here, in one round trip
     // with the weights and the input tile: fetched where it is used, each costs its phase (all far
     // shorter than a memory access) a round trip of its own.
@@ -1009,46 +1056,38 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
     if (wave == 0)
         load_cols<T, NB2, TR>(P.b_h2 ? static_cast<const T *>(P.b_h2) : reinterpret_cast<const T *>(kZeroVector), nb0,
                               hb, bias2);
-    float my_u = 0.f, my_n = 0.f;  // this trajectory's variates (threads 0 .. valid-1)
-    if (tid < valid) {
-        my_u = P.rand_u[static_cast<long>(t) * P.B + row0 + tid];
-        my_n = P.rand_n[static_cast<long>(t) * P.B + row0 + tid];
-    }
+    const float my_u = regs.u, my_n = regs.n;  // this trajectory's variates (threads 0 .. valid-1)
     // the model vectors of the embedding: a thread handles the same 8 columns in every item
     constexpr int CPR_E = D / 8;
     const int ch_e = tid % CPR_E;
     static_assert(NT % CPR_E == 0, "a thread's embedding items share their column chunk");
     u32x4 e_wx, e_bx, e_wy, e_by, e_mb, e_mt, e_tok;
     {
-        const T *tok = static_cast<const T *>(P.ar_tokens) + static_cast<long>((t + 1) % P.bs) * D;
-        const T *mk = static_cast<const T *>(P.markers);
+        // (copies the caller may have staged already: the markers "target" and "buffer", the token)
+        const T *tok = token ? token : static_cast<const T *>(P.ar_tokens) + static_cast<long>((t + 1) % P.bs) * D;
+        const T *mkt = mk_target ? mk_target : static_cast<const T *>(P.markers);
+        const T *mkb = mk_buffer ? mk_buffer : static_cast<const T *>(P.markers) + 2 * D;
         e_wx = *reinterpret_cast<const u32x4 *>(static_cast<const T *>(P.w_x) + 8 * ch_e);
         e_bx = *reinterpret_cast<const u32x4 *>(static_cast<const T *>(P.b_x) + 8 * ch_e);
         e_wy = *reinterpret_cast<const u32x4 *>(static_cast<const T *>(P.w_y) + 8 * ch_e);
         e_by = *reinterpret_cast<const u32x4 *>(static_cast<const T *>(P.b_y) + 8 * ch_e);
-        e_mb = *reinterpret_cast<const u32x4 *>(mk + 2 * D + 8 * ch_e);  // marker "buffer"
-        e_mt = *reinterpret_cast<const u32x4 *>(mk + 8 * ch_e);          // marker "target"
+        e_mb = *reinterpret_cast<const u32x4 *>(mkb + 8 * ch_e);
+        e_mt = *reinterpret_cast<const u32x4 *>(mkt + 8 * ch_e);
         e_tok = *reinterpret_cast<const u32x4 *>(tok + 8 * ch_e);
     }
-    constexpr int E_ITEMS = TR * 2 * CPR_E / NT;  // (trajectory, row, 8-column chunk) items per thread
-    static_assert(TR * 2 * CPR_E % NT == 0, "whole embedding items per thread");
-    float e_xv[E_ITEMS];  // feature mean of the row an item embeds: x_t for the buffer row, x_{t+1} for the target row
-    {
-        const T *xm = static_cast<const T *>(P.x_mean);
-        const int tn = min(t + 1, P.Nt - 1);
-#pragma unroll
-        for (int k = 0; k < E_ITEMS; ++k) {
-            const int idx = tid + k * NT;
-            const int which = (idx / CPR_E) & 1, r = idx / (2 * CPR_E);
-            e_xv[k] = r < valid ? to_f32(xm[(row0 + r) * P.Nt + (which == 0 ? t : tn)]) : 0.f;
-        }
+    constexpr int E_ITEMS = step_tail_items<D, TR, FUSED>();  // (trajectory, row, 8-column chunk) items per thread
+    static_assert(ROWS * 2 * CPR_E % NT == 0 && E_ITEMS >= 1, "whole embedding items per thread");
+    // the mixture biases go through LDS: read from memory where they are used, the pick of the
+    // component costs a round trip for the weight biases and another for the chosen mean and std
+    if (tid < 3 * P.K) mix_s[(tid / P.K) * kMaxMixture + tid % P.K] = regs.mix;  // published by the barriers below
+    if (!FUSED) {
+        stage_tile<T, D, NT, TR>(a0, LDD, static_cast<const T *>(P.x_last) + row0 * P.ld_row, P.ld_row, valid, tid);
+        __syncthreads();
     }
-    stage_tile<T, D, NT, TR>(a0, LDD, static_cast<const T *>(P.x_last) + row0 * P.ld_row, P.ld_row, valid, tid);
-    __syncthreads();
 
     // ---- z = LayerNorm(x_last), one wavefront per row, in place
     {
-        for (int r = wave; r < TR; r += NW) {
+        for (int r = wave; r < ROWS; r += NW) {
             T *row = a0 + r * LDD + lane * EPL;
             float x[EPL], sum = 0.f;
 #pragma unroll
@@ -1084,6 +1123,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
                 store4f<T>(a1 + c * LDF + TL::col(nbf[b], g, hb), o[0], o[1], o[2], o[3]);
             }
     }
+    before_draw();
     __syncthreads();
 
     // ---- raw = h W_h2^T + b_h2 (32 output columns, first wavefront), kept in float32
@@ -1105,8 +1145,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
         float y = 0.f;
         if (tid < valid) {
             const long row = row0 + tid;
-            const T *mb = static_cast<const T *>(P.mean_bias), *sb = static_cast<const T *>(P.std_bias),
-                    *wb = static_cast<const T *>(P.weight_bias);
+            const T *mb = mix_s, *sb = mix_s + kMaxMixture, *wb = mix_s + 2 * kMaxMixture;
             float logit[kMaxMixture], mx = -INFINITY;
 #pragma unroll
             for (int k = 0; k < kMaxMixture; ++k)
@@ -1157,7 +1196,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
             const int which = (idx / CPR_E) & 1, r = idx / (2 * CPR_E);
             if (r >= valid) continue;
             const long row = row0 + r;
-            const float xv = e_xv[k];
+            const float xv = regs.xv[k];
             float o[8];
             if (which == 0) {
                 const float yv = y_s[r];
@@ -1169,21 +1208,139 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(Sampl
             }
             u32x4 val = {pack2<T>(o[0], o[1]), pack2<T>(o[2], o[3]), pack2<T>(o[4], o[5]), pack2<T>(o[6], o[7])};
             *reinterpret_cast<u32x4 *>(static_cast<T *>(P.emb) + (row * 2 + which) * D + 8 * ch_e) = val;
+            if (FUSED) *reinterpret_cast<u32x4 *>(x_next + (2 * r + which) * LDD + 8 * ch_e) = val;
         }
     }
+}
 
-    // ---- the caller's loop counters: every workgroup read the step index when it started, so
-    // the one that takes the last ticket may move them on
+// The caller's loop counters: every workgroup read the step index when it started, so the one
+// that takes the last ticket may move them on.
+__device__ __forceinline__ void take_ticket(const SampleEmbedParams &P) {  // one thread of the workgroup
+    __threadfence();
+    if (atomicAdd(P.ticket, 1u) == gridDim.x - 1) {
+        for (int i = 0; i < P.n_advance; ++i) P.advance[i] += 1;
+        *P.ticket = 0u;
+    }
+}
+__device__ __forceinline__ void advance_loop_counters(const SampleEmbedParams &P) {
     if (P.advance) {
         __syncthreads();
-        if (tid == 0) {
-            __threadfence();
-            if (atomicAdd(P.ticket, 1u) == gridDim.x - 1) {
-                for (int i = 0; i < P.n_advance; ++i) P.advance[i] += 1;
-                *P.ticket = 0u;
-            }
-        }
+        if (threadIdx.x == 0) take_ticket(P);
     }
+}
+
+template <typename T, int D, int F, int TR>
+__global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(SampleEmbedParams P) {
+    constexpr int NW = fused_waves(D);
+    constexpr int LDD = D + 8, LDF = F + 8;
+    __shared__ __attribute__((aligned(16))) T a0[TR * LDD];  // z = norm(x_last)
+    __shared__ __attribute__((aligned(16))) T a1[TR * LDF];  // gelu(head layer 1)
+    __shared__ float raw_s[TR][33];
+    __shared__ float y_s[TR];
+    __shared__ T mix_s[3 * kMaxMixture];
+    const int t = *P.step;
+    if (t < 0 || t >= P.Nt) return;  // uniform over the grid
+    const long row0 = static_cast<long>(blockIdx.x) * TR;
+    const int valid = static_cast<int>(min(static_cast<long>(TR), P.B - row0));
+    WeightStream<T, D, fused_blocks<T, TR>(F, NW), TR> w_1;
+    const auto regs = load_step_tail_regs<T, D, TR, false>(P, t, row0, valid);
+    sample_embed_body<T, D, F, TR, false>(P, t, a0, a1, raw_s, y_s, mix_s, row0, valid, regs, w_1);
+    advance_loop_counters(P);
+}
+
+// ---- the whole boundary between two decode steps in one launch: the post part of the last
+// layer on the target rows, the step tail above, and the pre part of the first layer on the
+// rows it has just embedded.  A workgroup owns TR / 2 trajectories: their target rows fill half
+// a tile in the first two parts, their [buffer, target] rows of the next step the whole tile in
+// the third.  Row for row the arithmetic (and, through the `tile` argument of the weight
+// streams, its order) is that of fused_post_kernel, sample_embed_kernel and fused_pre_kernel
+// launched one after the other; what disappears is two launches, the store and reload of the
+// layer output and of the embedding, and two first round trips to memory.
+// P: rows = trajectories (their target rows), `out` unused.  S: x_last unused.  N: x unused,
+// rows = 2 * trajectories.  The head's hidden width equals the layers' feed-forward width F.
+template <typename T, int D, int F, int TR>
+__global__ __launch_bounds__(fused_waves(D) * 64) void decode_step_boundary_kernel(FusedPostParams P,
+                                                                                    SampleEmbedParams S,
+                                                                                    FusedPreParams N) {
+    constexpr int TJ = TR / 2;
+    constexpr int NW = fused_waves(D), LDD = D + 8, LDF = F + 8, LDM = LDD > LDF ? LDD : LDF;
+    __shared__ __attribute__((aligned(16))) T a0[TR * LDM];
+    __shared__ __attribute__((aligned(16))) T a1[TR * LDM];
+    __shared__ float red_a[NW * TR], red_b[NW * TR];
+    __shared__ float raw_s[TR][33];
+    __shared__ float y_s[TR];
+    constexpr int VW = D > F ? D : F;
+    __shared__ __attribute__((aligned(16))) T vecs[kVecSlots * VW];
+    const int t = *S.step;
+    if (t < 0 || t >= S.Nt) return;  // uniform over the grid
+    const long row0 = static_cast<long>(blockIdx.x) * TJ;
+    const int valid = static_cast<int>(min(static_cast<long>(TJ), static_cast<long>(S.B) - row0));
+    // tiles of the stand-alone launches that hold these rows
+    const int tile_t = static_cast<int>(row0 / TR), tile_n = static_cast<int>(blockIdx.x);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    constexpr int NB = fused_blocks<T, TR>(D, NW), NBF = fused_blocks<T, TR>(F, NW);
+    int nblk[NB], nbf[NBF];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) nblk[b] = wave + NW * b;
+#pragma unroll
+    for (int b = 0; b < NBF; ++b) nbf[b] = wave + NW * b;
+    const bool head_active = wave < F / Tile<T, TR>::kBlock;
+    WeightStream<T, D, NBF, TR> w_h1;
+    WeightStream<T, D, NB, TR> next_fo, next_q;
+    stage_pre_vectors<T, D, NW * 64>(N, vecs, VW, threadIdx.x);  // visible after the first barrier below
+    // whole-matrix streams: the head's first matrix is requested during the feed-forward product
+    constexpr bool kWhole = WeightStream<T, D, NB, TR>::kWhole && WeightStream<T, D, NBF, TR>::kWhole &&
+                            WeightStream<T, F, NB, TR>::kWhole;
+    // What the tail needs from memory is requested now, next to the post part's own prologue,
+    // and lands in LDS (vectors) or in a few registers (per-thread scalars): requested where the
+    // tail uses it, each item would cost a round trip between two phases that take far less.
+    __shared__ __attribute__((aligned(16))) T hvec[8 * D + F + 32];  // norm g, b; x/y embedding w, b; markers target, buffer; token; head biases
+    __shared__ T mix_s[3 * kMaxMixture];
+    T *const h_g = hvec, *const h_b = hvec + D, *const h_wx = hvec + 2 * D, *const h_bx = hvec + 3 * D,
+             *const h_wy = hvec + 4 * D, *const h_by = hvec + 5 * D, *const h_mk = hvec + 6 * D,
+             *const h_tok = hvec + 7 * D, *const h_b1 = hvec + 8 * D, *const h_b2 = hvec + 8 * D + F;
+    {
+        constexpr int NT = NW * 64;
+        const int tid = threadIdx.x;
+        const T *mk = static_cast<const T *>(S.markers);
+        dma_vector<T, D, NT>(h_g, S.norm_g, tid, 0);
+        dma_vector<T, D, NT>(h_b, S.norm_b, tid, 1);
+        dma_vector<T, D, NT>(h_wx, S.w_x, tid, 2);
+        dma_vector<T, D, NT>(h_bx, S.b_x, tid, 3);
+        dma_vector<T, D, NT>(h_wy, S.w_y, tid, 4);
+        dma_vector<T, D, NT>(h_by, S.b_y, tid, 5);
+        dma_vector<T, D, NT>(h_mk, mk, tid, 6);  // marker "target"
+        dma_vector<T, D, NT>(h_tok, static_cast<const T *>(S.ar_tokens) + static_cast<long>((t + 1) % S.bs) * D, tid, 7);
+        dma_vector<T, F, NT>(h_b1, S.b_h1, tid, 0);
+        dma_vector<T, 32, NT>(h_b2, S.b_h2, tid, 1);
+    }
+    __shared__ __attribute__((aligned(16))) T h_mkb[D];
+    dma_vector<T, D, NW * 64>(h_mkb, static_cast<const T *>(S.markers) + 2 * D, threadIdx.x, 2);
+    const auto regs = load_step_tail_regs<T, D, TR, true>(S, t, row0, valid);
+    const T *w_h1p = static_cast<const T *>(S.w_h1);
+    fused_post_body<T, D, F, TR, false>(
+        P, a0, a1, red_a, red_b, row0, valid,
+        [&]() { if (kWhole && head_active) w_h1.begin(w_h1p, nbf, lane, tile_t); },
+        [&](int ks) { if (kWhole && head_active) w_h1.request_share(ks, WeightStream<T, D, NBF, TR>::KS); },
+        NoHook{}, NoHook{}, vecs, VW, tile_t);
+    SampleEmbedParams S2 = S;  // the same tail, its small operands read from their LDS copies
+    S2.norm_g = h_g; S2.norm_b = h_b; S2.w_x = h_wx; S2.b_x = h_bx; S2.w_y = h_wy; S2.b_y = h_by;
+    S2.b_h1 = h_b1; S2.b_h2 = h_b2;
+    sample_embed_body<T, D, F, TR, true, kWhole>(
+        S2, t, a0, a1, raw_s, y_s, mix_s, row0, valid, regs, w_h1, a0, tile_t,
+        [&]() {
+            next_fo.start(static_cast<const T *>(N.w_fo), nblk, lane, tile_n);
+            if (kWhole) next_q.start(static_cast<const T *>(N.w_qkv), nblk, lane, tile_n);
+            // Every wavefront has read the step index (barriers of the post part lie behind it) and
+            // the buffer passes of this step, which read the buffer length, were waited for inside
+            // the post part: the loop counters may move on.  The last wavefront has nothing to do
+            // until the embedding: it takes the workgroup's ticket.
+            if (S.advance && threadIdx.x == NW * 64 - 1) take_ticket(S);
+        },
+        h_mk, h_mkb, h_tok);
+    __syncthreads();  // the embedded rows are complete in a0
+    fused_pre_body<T, D, TR, true, kWhole>(N, a0, a1, red_a, red_b, 2 * row0, 2 * valid, next_fo, next_q, vecs, VW,
+                                           tile_n);
 }
 
 }  // namespace artab

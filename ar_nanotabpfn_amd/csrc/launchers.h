@@ -37,5 +37,7 @@ hipError_t launch_layer_post(const FusedPostParams &P, int D, int F, bool is_bf1
 hipError_t launch_layer_post_pre(const FusedPostParams &P, const FusedPreParams &N, int D, int F, bool is_bf16,
                                  hipStream_t st);
 hipError_t launch_sample_embed(const SampleEmbedParams &P, int D, int F, bool is_bf16, hipStream_t st);
+hipError_t launch_step_boundary(const FusedPostParams &P, const SampleEmbedParams &S, const FusedPreParams &N, int D,
+                                int F, bool is_bf16, hipStream_t st);
 
 }  // namespace artab

@@ -1,10 +1,10 @@
 // Launches of the fused layer kernels (fused_layer.h).  Compiled once per element type and kernel
-// group: -DARTAB_LAYER_BF16=0|1 and -DARTAB_LAYER_GROUP=0 (pre, post) | 1 (post+pre) | 2 (step tail);
+// group: -DARTAB_LAYER_BF16=0|1 and -DARTAB_LAYER_GROUP=0 (pre, post) | 1 (post+pre) | 2 (step tail) | 3 (step boundary);
 // the type-dispatching entry points live in the bf16 object of each group.
 #include "launchers.h"
 
 #ifndef ARTAB_LAYER_BF16
-#error "define ARTAB_LAYER_BF16 (0 or 1) and ARTAB_LAYER_GROUP (0, 1 or 2)"
+#error "define ARTAB_LAYER_BF16 (0 or 1) and ARTAB_LAYER_GROUP (0 .. 3)"
 #endif
 
 namespace artab {
@@ -108,10 +108,33 @@ hipError_t launch_sample(const SampleEmbedParams &P, int D, int F, hipStream_t s
                                                    : launch_sample_r<T, kFusedRows>(P, D, F, st);
 }
 
+template <typename T, int D>
+hipError_t launch_boundary_d(const FusedPostParams &P, const SampleEmbedParams &S, const FusedPreParams &N, int F,
+                             hipStream_t st) {
+    constexpr int TR = kFusedRowsSmall;
+    dim3 grid(static_cast<unsigned>((S.B + TR / 2 - 1) / (TR / 2))), block(fused_waves(D) * 64);
+    switch (F) {
+        case 128: hipLaunchKernelGGL((decode_step_boundary_kernel<T, D, 128, TR>), grid, block, 0, st, P, S, N); break;
+        case 256: hipLaunchKernelGGL((decode_step_boundary_kernel<T, D, 256, TR>), grid, block, 0, st, P, S, N); break;
+        default: hipLaunchKernelGGL((decode_step_boundary_kernel<T, D, 512, TR>), grid, block, 0, st, P, S, N); break;
+    }
+    return hipGetLastError();
+}
+template <typename T>
+hipError_t launch_boundary(const FusedPostParams &P, const SampleEmbedParams &S, const FusedPreParams &N, int D, int F,
+                           hipStream_t st) {
+    switch (D) {
+        case 128: return launch_boundary_d<T, 128>(P, S, N, F, st);
+        case 256: return launch_boundary_d<T, 256>(P, S, N, F, st);
+        default: return launch_boundary_d<T, 512>(P, S, N, F, st);
+    }
+}
 
 }  // namespace
 
 // fp16 forms, defined in the fp16 objects
+hipError_t launch_step_boundary_f16(const FusedPostParams &P, const SampleEmbedParams &S, const FusedPreParams &N,
+                                    int D, int F, hipStream_t st);
 hipError_t launch_layer_pre_f16(const FusedPreParams &P, int D, hipStream_t st);
 hipError_t launch_layer_post_f16(const FusedPostParams &P, int D, int F, hipStream_t st);
 hipError_t launch_layer_post_pre_f16(const FusedPostParams &P, const FusedPreParams &N, int D, int F, hipStream_t st);
@@ -140,6 +163,18 @@ hipError_t launch_layer_post_pre(const FusedPostParams &P, const FusedPreParams 
 #else
 hipError_t launch_layer_post_pre_f16(const FusedPostParams &P, const FusedPreParams &N, int D, int F, hipStream_t st) {
     return launch_post_pre<LayerT>(P, N, D, F, st);
+}
+#endif
+#elif ARTAB_LAYER_GROUP == 3
+#if ARTAB_LAYER_BF16
+hipError_t launch_step_boundary(const FusedPostParams &P, const SampleEmbedParams &S, const FusedPreParams &N, int D,
+                                int F, bool is_bf16, hipStream_t st) {
+    return is_bf16 ? launch_boundary<LayerT>(P, S, N, D, F, st) : launch_step_boundary_f16(P, S, N, D, F, st);
+}
+#else
+hipError_t launch_step_boundary_f16(const FusedPostParams &P, const SampleEmbedParams &S, const FusedPreParams &N,
+                                    int D, int F, hipStream_t st) {
+    return launch_boundary<LayerT>(P, S, N, D, F, st);
 }
 #endif
 #else

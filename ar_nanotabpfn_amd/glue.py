@@ -19,7 +19,7 @@ from torch import Tensor, nn
 
 from . import _lib
 
-__all__ = ["add_layer_norm", "bias_gelu", "layer_fusable", "pack_weight", "layer_pre", "layer_post", "layer_post_pre", "SampleEmbedStep"]
+__all__ = ["add_layer_norm", "bias_gelu", "layer_fusable", "pack_weight", "layer_pre", "layer_post", "layer_post_pre", "SampleEmbedStep", "DecodeStepBoundary"]
 
 
 def _rows2d(t: Tensor) -> Tensor:
@@ -268,3 +268,70 @@ class SampleEmbedStep:
         self.args.x_last, self.args.ld_row = tgt.data_ptr(), tgt.stride(0)
         _lib.check(_lib.load().artab_decode_sample_embed(ctypes.byref(self.args), self.dtype_code,
                                                          _lib.current_stream(self.device)))
+
+
+class DecodeStepBoundary:
+    """Everything between the last attention call of one decode step and the first of the next
+    as one launch (``artab_decode_step_boundary``): the last layer's ``finish`` on the target
+    rows, the step tail (``SampleEmbedStep``) and the first layer's ``pre_attention`` on the rows
+    the tail has embedded.  Row for row the results are those of the three launches.
+
+    ``y_next [B,2,D]`` / ``qkv_next [B,2,3D]`` receive the first layer's normed feature stage and
+    projections of the next step; ``state`` is the ``(y, q, k, v)`` tuple over them in the form
+    ``TwoStageTransformerLayer.pre_attention`` returns.
+    """
+
+    MAX_TRAJECTORIES = 4096  # twice as many rows still take the 16-row tiles of the layer kernels
+
+    @staticmethod
+    def supported(tail: "SampleEmbedStep", first_layer, last_layer, x: Tensor) -> bool:
+        import os
+        F_ = last_layer.ff[0].out_features
+        return (tail is not None and tail.advances and tail.args.F == F_ and first_layer.ff[0].out_features == F_
+                and first_layer.attn_rows.n_heads == last_layer.attn_rows.n_heads
+                and last_layer.fused_for(x) and first_layer.fused_for(x)
+                and tail.args.B <= DecodeStepBoundary.MAX_TRAJECTORIES
+                and os.environ.get("ARTAB_TILE_ROWS", "16") == "16")
+
+    def __init__(self, tail: "SampleEmbedStep", first_layer, last_layer, y_next: Tensor, qkv_next: Tensor):
+        B, D = tail.args.B, tail.args.D
+        assert y_next.shape == (B, 2, D) and qkv_next.shape == (B, 2, 3 * D)
+        assert y_next.is_contiguous() and qkv_next.is_contiguous()
+        self.tail, self.first, self.last = tail, first_layer, last_layer
+        self.y_next, self.qkv_next = y_next, qkv_next
+        a = first_layer.attn_rows
+        qkv = qkv_next.view(B, 2, 3, a.n_heads, a.head_dim)
+        self.state = (y_next, qkv[:, :, 0].transpose(1, 2), qkv[:, :, 1].transpose(1, 2), qkv[:, :, 2].transpose(1, 2))
+
+    def load_state(self, emb: Tensor) -> None:
+        """The state a launch would have left for the embedded rows ``emb [B,2,D]``."""
+        p_fo, p_qkv = self.first.packed_weights()[:2]
+        y, qkv = layer_pre(emb, p_fo, self.first.norm1, p_qkv)
+        self.y_next.view(y.shape).copy_(y)
+        self.qkv_next.view(qkv.shape).copy_(qkv)
+
+    def __call__(self, y: Tensor, attn) -> None:
+        """``y [B,1,D]``: the last layer's normed feature stage of the target rows (any row
+        stride); ``attn``: their attention output ``[B,H,1,Dh]`` or its unmerged partials."""
+        last, first = self.last, self.first
+        B, D = self.tail.args.B, self.tail.args.D
+        y2 = y.reshape(B, D) if y.stride(-1) == 1 and y.stride(0) % 8 == 0 else y.reshape(B, D).contiguous()
+        if y2.data_ptr() % 16:
+            y2 = y2.contiguous()
+        p_o, p_1, p_2 = last.packed_weights()[2:]
+        n_fo, n_qkv = first.packed_weights()[:2]
+        if hasattr(attn, "desc"):
+            parts, a_ptr, lda = ctypes.byref(attn.desc), None, 0
+        else:
+            a2 = _rows16(attn.transpose(1, 2).reshape(B, D))
+            parts, a_ptr, lda = None, _ptr(a2), a2.stride(0)
+        _lib.check(
+            _lib.load().artab_decode_step_boundary(
+                parts, a_ptr, lda, _ptr(y2), y2.stride(0), _ptr(p_o), _ptr(last.norm2.weight), _ptr(last.norm2.bias),
+                float(last.norm2.eps), _ptr(p_1), _ptr(last.ff[0].bias), _ptr(p_2), _ptr(last.ff[2].bias),
+                _ptr(last.norm3.weight), _ptr(last.norm3.bias), float(last.norm3.eps), ctypes.byref(self.tail.args),
+                _ptr(n_fo), _ptr(first.norm1.weight), _ptr(first.norm1.bias), float(first.norm1.eps), _ptr(n_qkv),
+                _ptr(self.y_next), _ptr(self.qkv_next), last.ff[0].out_features, self.tail.dtype_code,
+                _lib.current_stream(self.tail.device),
+            )
+        )

@@ -26,7 +26,7 @@ from torch import Tensor
 from . import attention_kernels as ak
 from .attention import DecodeMask, TeacherForcingMask
 from . import _lib
-from .glue import SampleEmbedStep, add_layer_norm
+from .glue import SampleEmbedStep, DecodeStepBoundary, add_layer_norm
 
 __all__ = ["ARTabPFNPredictor"]
 
@@ -76,6 +76,7 @@ class ARTabPFNPredictor:
         # Decode steps recorded into one graph (a replay boundary costs about 5 us on the device); a
         # one-step graph covers the remainder.
         self.steps_per_graph = 4
+        self.fuse_step_boundary = True  # last layer's tail, step tail and first layer's head as one launch
         self.min_chain_batch = 256   # groups smaller than this are not worth their fixed costs
         # Order the two streams of the recorded step through counters in device memory instead of
         # two events per layer (``attention_kernels.QueueOrder``); used when the two streams are found
@@ -159,7 +160,8 @@ class ARTabPFNPredictor:
 
     # ------------------------------------------------------------------ the layer stack
 
-    def _run_layers(self, x_row: Tensor, attend, last_layer_rows: Optional[slice] = None) -> Tensor:
+    def _run_layers(self, x_row: Optional[Tensor], attend, last_layer_rows: Optional[slice] = None, state=None,
+                    finish=None) -> Tensor:
         """``x_row [B,N,D]`` through every layer; ``attend(layer, q, k, v) -> [B,H,N,Dh]`` is the
         row attention of the pass at hand (it also owns the cache writes).  Between two
         attention calls the tail of one layer and the head of the next run as one launch where
@@ -170,15 +172,22 @@ class ARTabPFNPredictor:
         projection in front of the attention call, which still sees every row), so the last layer
         runs its queries and everything behind them for those rows only; the result is then
         ``[B, len(rows), D]``.  A decode step reads the target row alone (inference.py:318-320):
-        half the queries of the last context pass."""
+        half the queries of the last context pass.
+
+        ``state``: the first layer's ``pre_attention`` result when somebody has computed it
+        already (``x_row`` is then not read); ``finish(y, attn)``: what to do with the last
+        layer's feature stage and attention output instead of ``layer.finish`` (the step
+        boundary launch of a recorded decode step, whose result this function then returns)."""
         layers = list(self.backbone.layers)
-        state = layers[0].pre_attention(x_row)
+        if state is None:
+            state = layers[0].pre_attention(x_row)
         for idx, layer in enumerate(layers):
             y, q, k, v = state
             if idx + 1 == len(layers):
                 if last_layer_rows is not None:
                     y, q = y[:, last_layer_rows], q[:, :, last_layer_rows]
-                return layer.finish(y, attend(layer, q, k, v))
+                attn = attend(layer, q, k, v)
+                return finish(y, attn) if finish is not None else layer.finish(y, attn)
             state = layer.finish_then_pre(y, attend(layer, q, k, v), layers[idx + 1])
 
     # ------------------------------------------------------------------ prefill
@@ -374,6 +383,15 @@ class ARTabPFNPredictor:
     def _graph_step(self, st) -> None:
         """One ``[buffer, target]`` decode step driven entirely by device-side state
         (the body that is recorded): step index ``st.t``, buffer length ``st.nbuf``."""
+        if st.boundary is not None:
+            # the previous step's boundary launch has left the first layer's feature stage and
+            # projections of this step's rows; this step's ends with the same launch
+            self._run_layers(
+                None, lambda layer, q, k, v: self._attend_decode_shared(layer, q, k, v, n_buf_device=st.nbuf,
+                                                                        rows=st.rows, chain=st.chain,
+                                                                        order=st.order_active),
+                last_layer_rows=self._last_layer_rows(), state=st.boundary.state, finish=st.boundary)
+            return
         if st.tail is not None:
             # embedding of this step was left in st.emb by the previous step's tail launch
             x_row = self._run_layers(
@@ -407,9 +425,11 @@ class ARTabPFNPredictor:
         context, then the one-launch tail with the step counter at 0."""
         emb0 = self.embedder.embed_target(st.x_target[:, 0:1])
         x_row = self._run_layers(emb0, lambda layer, q, k, v: self._attend_decode_shared(layer, q, k, v,
-                                                                                        rows=st.rows, chain=st.chain))
-        st.tail(x_row)    # norm, head, draw, preds[:, 0], embedding of step 1, (t, nbuf) += 1
-        st.nbuf.zero_()   # the first target commits no buffer row
+                                                                                        rows=st.rows, chain=st.chain),
+                                 finish=st.boundary)
+        if st.boundary is None:
+            st.tail(x_row)  # norm, head, draw, preds[:, 0], embedding of step 1, (t, nbuf) += 1
+        st.nbuf.zero_()     # the first target commits no buffer row
 
     def _last_layer_rows(self) -> Optional[slice]:
         """Rows of a ``[buffer, target]`` step that the last layer has to finish: the target."""
@@ -440,7 +460,7 @@ class ARTabPFNPredictor:
         key = (B, cap, F_, self.context_len, dtype, str(device), layer0.k_ctx_cache.data_ptr(),
                layer0.k_buf_cache.data_ptr(), self.fuse_step_tail, self.overlap_buffer_pass, self.merge_in_layer,
                len(chain_rows), int(self.steps_per_graph), bool(self.counter_ordering),
-               bool(self.target_only_last_layer), tuple((p.data_ptr(), p._version) for p in params))
+               bool(self.target_only_last_layer), bool(self.fuse_step_boundary), tuple((p.data_ptr(), p._version) for p in params))
         gs = self._graph_state
         if gs is None or gs.key != key:
             gs = _GraphState()
@@ -464,6 +484,7 @@ class ARTabPFNPredictor:
                 st.graph_many = None   # steps_per_graph steps in one graph
                 st.graph_first = None  # the first target's step (no buffer row yet)
                 st.tail = None
+                st.boundary = None  # last post + tail + first pre of the next step as one launch
                 st.order = st.order_active = None
                 if self._counter_ordering_applies(x_target):
                     order = ak.QueueOrder(device)
@@ -478,6 +499,12 @@ class ARTabPFNPredictor:
                     st.rand_n = torch.zeros((cap, Bc), device=device, dtype=torch.float32)
                     st.tail = SampleEmbedStep(self.embedder, self.backbone, self.head, self.ar_tokens, st.x_mean,
                                               st.rand_u, st.rand_n, st.t, st.preds, st.emb, advance=st.counters)
+                    layers = self.backbone.layers
+                    if (self.fuse_step_boundary and self.target_only_last_layer
+                            and DecodeStepBoundary.supported(st.tail, layers[0], layers[-1], x_target)):
+                        st.boundary = DecodeStepBoundary(
+                            st.tail, layers[0], layers[-1], torch.zeros((Bc, 2, D), device=device, dtype=dtype),
+                            torch.zeros((Bc, 2, 3 * D), device=device, dtype=dtype))
                 gs.chains.append(st)
             gs.tail = gs.chains[0].tail
             self._graph_state = gs
@@ -530,6 +557,8 @@ class ARTabPFNPredictor:
             st.nbuf.zero_()
             if st.tail is not None:
                 st.emb.copy_(emb1[rows])
+            if st.boundary is not None:
+                st.boundary.load_state(st.emb)
 
         for st in gs.chains:
             if st.graph is not None:

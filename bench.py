@@ -336,6 +336,8 @@ def main():
                     help="let the last layer of a decode step finish the buffer row too (its output is read by nobody)")
     ap.add_argument("--event-ordering", action="store_true",
                     help="order the two streams of the recorded step with events instead of device-side counters")
+    ap.add_argument("--separate-step-boundary", action="store_true",
+                    help="last layer's tail, step tail and first layer's head as three launches instead of one")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only copy a 256 MiB buffer five times (reference kernel for scaling HBM counters)")
     ap.add_argument("--mix-ceiling", action="store_true",
@@ -378,6 +380,8 @@ def main():
         pred.counter_ordering = False
     if args.full_last_layer:
         pred.target_only_last_layer = False
+    if args.separate_step_boundary:
+        pred.fuse_step_boundary = False
 
     torch.manual_seed(0)
     # Untimed warm-up: W decode steps (at least the three a recorded step needs).  The recorded
@@ -472,6 +476,9 @@ def main():
         # the last layer of a recorded step finishes the target row only (the buffer row's output of
         # that layer is read by nobody; --full-last-layer computes it as the reference does: -0.7 %)
         "target_only_last_layer": bool(pred.target_only_last_layer),
+        # last layer's tail + head/draw/embedding + first layer's head of the next step as one launch
+        "step_boundary_fused": bool(pred._graph_state is not None
+                                    and getattr(pred._graph_state.chains[0], "boundary", None) is not None),
         "stream_ordering": ("counters" if getattr(pred._graph_state.chains[0], "order", None) is not None else "events")
         if pred._graph_state is not None else None,
         "prefill_ms": round(prefill_ms, 3),

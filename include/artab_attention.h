@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define ARTAB_VERSION 4
+#define ARTAB_VERSION 5
 
 typedef enum artab_dtype {
     ARTAB_BF16 = 0,
@@ -481,6 +481,28 @@ typedef struct artab_sample_embed_args {
 } artab_sample_embed_args;
 
 int artab_decode_sample_embed(const artab_sample_embed_args *args, int dtype, void *stream);
+
+/*
+ * The boundary between two decode steps in one launch: artab_layer_post (or
+ * artab_layer_post_from_partials when `partials` is given and holds slots; `attn`, [B, D] with
+ * row stride lda, is read otherwise) of the last layer on the B target rows y (row stride ldy),
+ * artab_decode_sample_embed on its output (tail->x_last is not read), and artab_layer_pre of the
+ * first layer on the 2 B rows just embedded (next_y [2B, D], next_qkv [2B, 3D]; tail->emb_next is
+ * written as well).  Replaces inference.py:825-831 of the last layer, :318-320 and :355-362
+ * (head, draw, next embedding) and :770-783 of the first layer of the next step.  Row for row
+ * the results equal those of the three calls made one after the other, bit for bit.  The head's
+ * hidden width tail->F must equal the layers' feed-forward width F; up to 4096 trajectories
+ * (ARTAB_ERR_UNSUPPORTED otherwise: make the three calls).
+ */
+int artab_decode_step_boundary(const artab_attention_partials *partials, const void *attn, int64_t lda,
+                               const void *y, int64_t ldy, const void *w_o,
+                               const void *ln2_gamma, const void *ln2_beta, float eps2,
+                               const void *w_1, const void *b_1, const void *w_2, const void *b_2,
+                               const void *ln3_gamma, const void *ln3_beta, float eps3,
+                               const artab_sample_embed_args *tail,
+                               const void *next_w_fo, const void *next_ln1_gamma, const void *next_ln1_beta,
+                               float next_eps1, const void *next_w_qkv, void *next_y, void *next_qkv,
+                               int F, int dtype, void *stream);
 
 int artab_layer_post_pre(const void *attn, int64_t lda, const void *y, int64_t ldy, const void *w_o,
                          const void *ln2_gamma, const void *ln2_beta, float eps2,

@@ -1093,6 +1093,101 @@ def test_decode_partials_merged_in_layer_kernel(device, monkeypatch, tile_rows, 
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,D,F,H,Nc,n_buf,cap,partials", [
+    (64, 128, 128, 4, 256, 5, 16, True),     # whole workgroups
+    (200, 256, 256, 8, 4096, 9, 16, True),   # split context, the shape of configs[3]'s layers
+    (37, 256, 256, 8, 300, 0, 8, True),      # ragged last workgroup (5 of 8 trajectories), the new row alone
+    (1030, 128, 256, 4, 128, 3, 8, True),    # more than eight 16-row tiles: the contraction starts rotate
+    (21, 512, 256, 16, 200, 2, 8, True),     # matrices deeper than the prefetch window
+    (40, 128, 128, 4, 64, 0, 8, False),      # attention output given as a tensor (first target: context only)
+])
+def test_decode_step_boundary_equals_its_three_launches(device, monkeypatch, dtype, B, D, F, H, Nc, n_buf, cap, partials):
+    """artab_decode_step_boundary against artab_layer_post(_from_partials) on the target rows,
+    artab_decode_sample_embed and artab_layer_pre launched one after the other: predictions,
+    embedding, the next step's feature stage and projections, and the loop counters, bit for bit."""
+    from ar_nanotabpfn_amd import attention_kernels as ak
+    from ar_nanotabpfn_amd import model as m
+    from ar_nanotabpfn_amd.glue import DecodeStepBoundary, SampleEmbedStep
+
+    monkeypatch.setenv("ARTAB_SMALL", "0")
+    Dh, Nt, K = D // H, 6, 5
+    assert Dh == 32
+    torch.manual_seed(4)
+    net = m.ARTabPFN(d_model=D, n_heads=H, n_layers=2, d_ff=F, num_features=3, buffer_size=3, num_components=K)
+    with torch.no_grad():
+        for p in list(net.embedder.parameters()) + list(net.head.parameters()) + [net.ar_tokens]:
+            p.add_(0.3 * torch.randn_like(p))
+        for layer in net.backbone.layers:
+            for norm in (layer.norm1, layer.norm2, layer.norm3):
+                norm.weight.add_(0.2 * torch.randn(D))
+                norm.bias.add_(0.2 * torch.randn(D))
+    # the head's hidden width is the layers' feed-forward width in this model family
+    net = net.to(device=device, dtype=dtype)
+    first, last = net.backbone.layers[0], net.backbone.layers[1]
+    assert net.head.head[0].out_features == F
+
+    q, k_ctx, v_ctx = (t.to(device) for t in _ctx_inputs(B, H, 1, Nc, Dh, dtype, seed=5, scale=0.6))
+    k_cache, v_cache = randn((B, H, cap, Dh), 6, dtype, 0.6).to(device), randn((B, H, cap, Dh), 7, dtype, 0.6).to(device)
+    k_new, v_new = randn((B, H, 1, Dh), 8, dtype, 0.6).to(device), randn((B, H, 1, Dh), 9, dtype, 0.6).to(device)
+    y_rows = randn((B, 2, D), 10, dtype, 1.0).to(device)
+    y_tgt = y_rows[:, 1:2]  # the target rows: row stride 2 D
+    side = torch.cuda.Stream(device=device)
+    x_mean = randn((B, Nt), 11, dtype, 1.0).to(device)
+    u, n = torch.rand(Nt, B, device=device), torch.randn(Nt, B, device=device)
+
+    def attention():
+        if not partials:
+            return ak.context_attention(q, k_ctx, v_ctx)[0]
+        out = ak.decode_attention(q, k_ctx, v_ctx, k_cache.clone(), v_cache.clone(), n_buf, k_new, v_new,
+                                  side_stream=side, leave_partials=True)
+        assert isinstance(out, ak.AttentionPartials)
+        return out
+
+    def make_tail():
+        counters = torch.tensor([2, 1], dtype=torch.int32, device=device)
+        preds = torch.full((B, Nt), 7.0, device=device, dtype=dtype)
+        emb = torch.zeros((B, 2, D), device=device, dtype=dtype)
+        tail = SampleEmbedStep(net.embedder, net.backbone, net.head, net.ar_tokens, x_mean, u, n, counters[0:1],
+                               preds, emb, advance=counters)
+        return tail, counters, preds, emb
+
+    # three launches
+    tail, counters, preds, emb = make_tail()
+    x_last = last.finish(y_tgt, attention())
+    tail(x_last)
+    ref_state = first.pre_attention(emb)
+    torch.cuda.synchronize()
+
+    # one launch
+    tail2, counters2, preds2, emb2 = make_tail()
+    assert DecodeStepBoundary.supported(tail2, first, last, y_rows)
+    boundary = DecodeStepBoundary(tail2, first, last, torch.zeros((B, 2, D), device=device, dtype=dtype),
+                                  torch.zeros((B, 2, 3 * D), device=device, dtype=dtype))
+    boundary(y_tgt, attention())
+    torch.cuda.synchronize()
+    assert counters2.tolist() == counters.tolist() == [3, 2]
+    assert int(tail2._keep["ticket"].item()) == 0
+    assert torch.equal(preds2, preds) and torch.all(preds2[:, 3:] == 7.0) and not torch.all(preds2[:, 2] == 7.0)
+    assert torch.equal(emb2, emb)
+    for got, ref in zip(boundary.state, ref_state):
+        assert got.shape == ref.shape and torch.equal(got, ref)
+    # the state that reset() builds from an embedding is the same again
+    boundary.y_next.zero_()
+    boundary.qkv_next.zero_()
+    boundary.load_state(emb)
+    for got, ref in zip(boundary.state, ref_state):
+        assert torch.equal(got, ref)
+    # an out-of-range step index: nothing is written, nothing advances
+    counters2[0] = Nt
+    before = (preds2.clone(), emb2.clone(), boundary.y_next.clone(), boundary.qkv_next.clone())
+    boundary(y_tgt, attention())
+    torch.cuda.synchronize()
+    assert counters2.tolist() == [Nt, 2]
+    for a, b in zip(before, (preds2, emb2, boundary.y_next, boundary.qkv_next)):
+        assert torch.equal(a, b)
+
+
 def test_queue_order_wait_gives_up_after_its_time_limit(device):
     """A wait whose signal never comes (forced from the host: nothing is launched on the other
     stream) ends after its time limit, counts itself in `failed`, and every later wait falls

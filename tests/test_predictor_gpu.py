@@ -655,3 +655,39 @@ def test_graph_sampling_target_only_last_layer_changes_nothing_that_is_read(devi
     for (k0, v0), (k1, v1) in zip(c0, c1):
         assert max_abs(to_np(k0[:, :, :1]), to_np(k1[:, :, :1])) <= 2e-2  # the row appended by step 1
         assert max_abs(to_np(v0[:, :, :1]), to_np(v1[:, :, :1])) <= 2e-2
+
+
+@pytest.mark.parametrize("ordered", [True, False], ids=["counters", "events"])
+def test_graph_sampling_with_one_launch_step_boundary_equals_three_launches(device, ordered):
+    """The recorded decode step whose boundary (last layer's tail, head, draw, next embedding,
+    first layer's head of the next step) is one launch against the same step with the three
+    launches: same variates in, the same predictions and caches out, bit for bit (bf16, several
+    steps per graph and a remainder, both orderings of the two streams, graphs reused by a second
+    call)."""
+    from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
+
+    cfg = dict(d_model=128, n_heads=4, n_layers=3, d_ff=128, num_features=3, buffer_size=5, num_components=4)
+    model = _build(cfg, device, dtype=torch.bfloat16)
+    B, Nc, Nt = 70, 2100, 11
+    g = torch.Generator().manual_seed(6)
+    xc = torch.randn(1, Nc, 3, generator=g).expand(B, -1, -1).to(device, torch.bfloat16)
+    yc = torch.randn(1, Nc, generator=g).expand(B, -1).to(device, torch.bfloat16)
+    xt = torch.randn(B, Nt, 3, generator=g).to(device, torch.bfloat16)
+    results = {}
+    for fused in (False, True):
+        pred = ARTabPFNPredictor.from_trained_model(model, backend="triton_shared_context")
+        pred.counter_ordering = ordered
+        pred.fuse_step_boundary = fused
+        for n in (Nt, 4, Nt):  # a shorter run in between: the state of a run must not leak into the next
+            torch.manual_seed(13)
+            y = pred.sample_sequence(xc, yc, xt[:, :n])
+        st = pred._graph_state.chains[0]
+        assert (st.boundary is not None) == fused
+        if st.order is not None:
+            assert st.order.failed() == 0
+        results[fused] = (y, [(l.k_buf_cache.clone(), l.v_buf_cache.clone()) for l in model.backbone.layers])
+    (y0, c0), (y1, c1) = results[False], results[True]
+    assert y1.shape == (B, Nt) and torch.isfinite(y1).all()
+    assert torch.equal(y0, y1)
+    for (k0, v0), (k1, v1) in zip(c0, c1):
+        assert torch.equal(k0, k1) and torch.equal(v0, v1)
