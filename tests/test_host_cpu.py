@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     lib = L.load()
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.artab_version() == 4
+    assert lib.artab_version() == L.ABI_VERSION == 5
     assert lib.artab_status_string(0) == b"ok"
 
 
