@@ -7,8 +7,9 @@
 // issue slots.  Hence:
 //
 //  * dot products on the matrix pipe with v_mfma_f32_4x4x4 (16 independent 4x4x4 products per
-//    instruction): one block = one (trajectory, head) pair, lane 4p+i of a wavefront is
-//    (pair p, index i).  Scores S^T[key i][query j] = K[key i] . Q[query j]: A operand = 4
+//    instruction): one block = four keys of one (trajectory, head) pair, lane 4p+i of a
+//    wavefront is (block p, index i); described here for the chunk shape in which a block is a
+//    pair (the other shape, four blocks per pair, is described at decode_stream_body).  Scores S^T[key i][query j] = K[key i] . Q[query j]: A operand = 4
 //    head-dim elements of key row i (lane (p,i)), B operand = the same 4 elements of query j
 //    (lane (p,j); zero for j >= Lq), result: lane (p,j) holds the 4 keys' scores of query j.
 //    O^T[dim][query j] += V^T[dim][key] P^T[key][query j]: B operand = the lane's own four
@@ -16,10 +17,11 @@
 //    ds_read_b64_tr_b16; lane (p,j) accumulates all 32 output dims of query j.
 //    Softmax state (max, sum) is one scalar per lane.  About 35 vector instructions, 16 MFMAs
 //    (8 cycles each) and 16 LDS reads per 4 keys x 16 pairs.
-//  * loads land in LDS, not in registers: every wavefront keeps a ring of 8 KiB chunks (4 keys x
-//    16 pairs x K and V) filled by direct global->LDS loads (16 bytes per lane, lane l lands at
-//    chunk + 16 l), three chunks in flight while two are being read, and reads a chunk back
-//    lane-locally (K) or transposed (V).  The wavefront is alone with its latencies, so the LDS
+//  * loads land in LDS, not in registers: every wavefront keeps a ring of three 8 KiB chunks (64
+//    key rows, K and V: 4 keys x 16 pairs or 16 keys x 4 pairs) filled by direct global->LDS loads
+//    (16 bytes per lane, lane l lands at chunk + 16 l): the chunk being read and the two behind
+//    it, a slot being refilled as soon as its chunk has been read back lane-locally (K) or
+//    transposed (V).  The wavefront is alone with its latencies, so the LDS
 //    reads run one chunk ahead of the arithmetic that uses them.
 //
 // Output per (pair, query): normalised partial result in the input type + float32 LSE, i.e. one
@@ -35,8 +37,8 @@ namespace artab {
 
 constexpr int kStreamChunks = 3;           // ring depth per wavefront
 constexpr int kStreamShortRows = 32;       // buffers longer than this are read 16 rows x 4 pairs at a time
-constexpr int kStreamChunkBytes = 8192;    // 4 keys x 16 pairs x (64 B of K + 64 B of V)
-constexpr int kStreamQBytes = 4096;        // one task's queries: 4 x (64 lanes x 16 B)
+constexpr int kStreamChunkBytes = 8192;    // 64 key rows x (64 B of K + 64 B of V)
+constexpr int kStreamQBytes = 4096;        // a region of query slots: 4 x (64 lanes x 16 B)
 constexpr size_t kStreamLdsBytes = kStreamChunks * kStreamChunkBytes + 2 * kStreamQBytes;
 
 // LDS reads of the ring go through inline assembly: the compiler must not see an LDS read that
