@@ -282,6 +282,10 @@ class DecodeStepBoundary:
     """
 
     MAX_TRAJECTORIES = 4096  # twice as many rows still take the 16-row tiles of the layer kernels
+    # At d_model 512 a workgroup streams 3 MB of weights and is bound by that; eight trajectories
+    # per workgroup instead of sixteen rows then double the traffic of the first two parts for
+    # nothing (measured at B=2048, d_model 512: 457 against 462 target-steps/s with three launches).
+    MAX_WIDTH = 256
 
     @staticmethod
     def supported(tail: "SampleEmbedStep", first_layer, last_layer, x: Tensor) -> bool:
@@ -291,6 +295,7 @@ class DecodeStepBoundary:
                 and first_layer.attn_rows.n_heads == last_layer.attn_rows.n_heads
                 and last_layer.fused_for(x) and first_layer.fused_for(x)
                 and tail.args.B <= DecodeStepBoundary.MAX_TRAJECTORIES
+                and tail.args.D <= DecodeStepBoundary.MAX_WIDTH
                 and os.environ.get("ARTAB_TILE_ROWS", "16") == "16")
 
     def __init__(self, tail: "SampleEmbedStep", first_layer, last_layer, y_next: Tensor, qkv_next: Tensor):

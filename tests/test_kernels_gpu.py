@@ -1161,7 +1161,7 @@ def test_decode_step_boundary_equals_its_three_launches(device, monkeypatch, dty
 
     # one launch
     tail2, counters2, preds2, emb2 = make_tail()
-    assert DecodeStepBoundary.supported(tail2, first, last, y_rows)
+    assert DecodeStepBoundary.supported(tail2, first, last, y_rows) == (D <= DecodeStepBoundary.MAX_WIDTH)
     boundary = DecodeStepBoundary(tail2, first, last, torch.zeros((B, 2, D), device=device, dtype=dtype),
                                   torch.zeros((B, 2, 3 * D), device=device, dtype=dtype))
     boundary(y_tgt, attention())
