@@ -131,10 +131,23 @@ CFG3_Z_MAX = 8e-2
 CFG3_Z_MEAN = 1.2e-2
 
 
-def test_config3_full_size_decode_steps_vs_oracle(device, monkeypatch):
-    """Three decode steps (target alone, then two [buffer, target] steps) of the configs[3] model
-    at its full shape on the device; the oracle redoes the steps in float64 for eight of the 1024
-    trajectories, starting from the device's own context K/V (the 16384-row prefill in float64 on
+# configs[4]: d_model 512, 16 heads, B=2048 trajectories, N_ctx=4096.  Measured on MI355X: |dz| mean
+# 6.0e-3, max 4.0e-2 (float32 attention in the same model: 6.0e-3 / 4.6e-2); |dlogp| of a fixed y
+# mean 1.4e-2, max 2.0e-1 (the random-init head of this width has narrower components: the same
+# |dz| moves the density more; the float32-attention run is printed beside it).
+CFG4 = dict(d_model=512, n_heads=16, n_layers=12, d_ff=256, num_features=20, buffer_size=256, num_components=5)
+SAMPLE4 = [0, 1, 255, 256, 1023, 1024, 2046, 2047]
+
+
+@pytest.mark.parametrize("cfg,B,Nc,sample,z_max,z_mean,ll_mean,ll_max", [
+    (CFG3, 1024, 16384, SAMPLE, CFG3_Z_MAX, CFG3_Z_MEAN, 2e-2, 1.5e-1),
+    (CFG4, 2048, 4096, SAMPLE4, 8e-2, 1.2e-2, 3e-2, 4e-1),
+], ids=["configs3", "configs4"])
+def test_config3_full_size_decode_steps_vs_oracle(device, monkeypatch, cfg, B, Nc, sample, z_max, z_mean, ll_mean,
+                                                  ll_max):
+    """Three decode steps (target alone, then two [buffer, target] steps) of the configs[3] and
+    configs[4] models at their full shapes on the device; the oracle redoes the steps in float64
+    for eight of the trajectories, starting from the device's own context K/V (the 16384-row prefill in float64 on
     the host would need a 17 GB score matrix; the prefill kernel is checked against the oracle at
     full size in test_kernels_gpu.py).  Compared: the normed output of every step for the sampled
     trajectories, the appended buffer K/V rows of every layer, and the mixture log-density of a
@@ -142,13 +155,14 @@ def test_config3_full_size_decode_steps_vs_oracle(device, monkeypatch):
     import ar_nanotabpfn_amd.inference as inf
     from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
 
-    B, Nc, cap, dtype = 1024, 16384, 8, torch.bfloat16
-    model = _model(CFG3, device, dtype, seed=0)
+    cap, dtype, F_ = 8, torch.bfloat16, cfg["num_features"]
+    SAMPLE = sample
+    model = _model(cfg, device, dtype, seed=0)
     g = torch.Generator().manual_seed(7)
-    xc1 = torch.randn(1, Nc, 10, generator=g)
+    xc1 = torch.randn(1, Nc, F_, generator=g)
     yc1 = torch.sin(xc1.sum(-1)) + 0.05 * torch.randn(1, Nc, generator=g)
     xc, yc = xc1.expand(B, -1, -1).to(device, dtype), yc1.expand(B, -1).to(device, dtype)
-    xt = torch.randn(B, 3, 10, generator=g).to(device, dtype)
+    xt = torch.randn(B, 3, F_, generator=g).to(device, dtype)
     y_fixed = torch.randn(B, 3, generator=g).to(device, dtype)
 
     def steps(pred):
@@ -190,7 +204,7 @@ def test_config3_full_size_decode_steps_vs_oracle(device, monkeypatch):
     _, z_ref = steps(pred_ref)
 
     sd = {k: v.detach().float().cpu().numpy() for k, v in model.state_dict().items()}
-    om = mo.OracleModel(sd, CFG3["n_heads"])
+    om = mo.OracleModel(sd, cfg["n_heads"])
     op = mo.OraclePredictor(om, "shared")
     op.init_kv_cache(len(SAMPLE), cap)
     op.k_ctx, op.v_ctx, op.context_len = k_ctx, v_ctx, Nc
@@ -201,12 +215,16 @@ def test_config3_full_size_decode_steps_vs_oracle(device, monkeypatch):
     ll_true = om.head_log_likelihood(z_true, to_np(y_fixed[SAMPLE]))
     ll_hip = to_np(model.head.log_likelihood(z_hip[SAMPLE], y_fixed[SAMPLE].unsqueeze(-1)))
     dll = np.abs(ll_hip - ll_true)
-    print(f"\n[configs[3] full size] |dz| vs exact: hip mean {err_hip.mean():.3e} max {err_hip.max():.3e}; "
-          f"f32attn mean {err_ref.mean():.3e} max {err_ref.max():.3e}; |dlogp| mean {dll.mean():.3e} max {dll.max():.3e}")
+    dll_ref = np.abs(to_np(model.head.log_likelihood(z_ref[SAMPLE], y_fixed[SAMPLE].unsqueeze(-1))) - ll_true)
+    print(f"\n[{B} trajectories, d_model {cfg['d_model']}, full size] |dz| vs exact: hip mean {err_hip.mean():.3e} max {err_hip.max():.3e}; "
+          f"f32attn mean {err_ref.mean():.3e} max {err_ref.max():.3e}; |dlogp| mean {dll.mean():.3e} max {dll.max():.3e} "
+          f"median {np.median(dll):.3e} (f32attn {dll_ref.mean():.3e} / {dll_ref.max():.3e} / {np.median(dll_ref):.3e})")
     assert np.isfinite(to_np(z_hip)).all()
-    assert err_hip.max() <= CFG3_Z_MAX and err_hip.mean() <= CFG3_Z_MEAN
+    assert err_hip.max() <= z_max and err_hip.mean() <= z_mean
     assert err_hip.mean() <= 1.25 * err_ref.mean() + 1e-3
-    assert dll.mean() <= 2e-2 and dll.max() <= 1.5e-1
+    assert dll.mean() <= ll_mean and dll.max() <= ll_max
+    # (24 values, the density of a narrow component is steep: compared by their medians)
+    assert np.median(dll) <= 1.5 * np.median(dll_ref) + 2e-3
     for i in range(len(layers)):
         assert max_abs(kbuf_hip[i], to_np_f64(op.k_buf[i])) <= 6e-2 and max_abs(vbuf_hip[i], to_np_f64(op.v_buf[i])) <= 6e-2
     # trajectories differ (the sampled rows are not copies of one another)
