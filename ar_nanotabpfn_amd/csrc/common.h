@@ -134,6 +134,14 @@ __device__ __forceinline__ void load_row64_to_lds(const void *global_src, unsign
     __builtin_amdgcn_global_load_lds(global_src, lds_dst + 3024, 16, 48, 0);
 }
 
+// A value again, as one the compiler cannot trace (typically the lane index): what rarely
+// executed code derives from it (rows, base addresses) is then computed where it is used instead
+// of being kept in registers across a hot loop that does not need it.
+__device__ __forceinline__ int opaque(int v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
 // acc + a.lo * b.lo + a.hi * b.hi of two packed 16-bit pairs, accumulated in float32
 template <typename T>
 __device__ __forceinline__ float dot2_acc(unsigned a, unsigned b, float acc);

@@ -95,14 +95,6 @@ __device__ __forceinline__ void lds_wait(u32x4 (&k)[4], u32x2 (&v)[8]) {
                  : "memory");
 }
 
-// The lane index again, as a value the compiler cannot trace: what the rare steps of the loop
-// derive from it (pair, row, base addresses) is then computed where it is used instead of being
-// kept in registers across the steps that are not rare.
-__device__ __forceinline__ int opaque(int v) {
-    asm volatile("" : "+v"(v));
-    return v;
-}
-
 // The value held by another lane of this lane's row of 16: the row rotated by N places.
 template <int N>
 __device__ __forceinline__ float row_ror(float v) {

@@ -34,6 +34,8 @@ static hipError_t launch_flash_bm(const FlashParams &P, int BM, hipStream_t stre
             // buffer pass beside four of these wavefronts; ARTAB_LEAN_OCC=4 takes 128 (tuning aid)
             if (env_int("ARTAB_LEAN_OCC", 5) == 4)
                 hipLaunchKernelGGL((flash_kernel<T, DH, 1, 8, kFlashBN, true, 4>), dim3(grid), dim3(512), 0, stream, P);
+            else if (P.mode == kFlashContext)  // the decode launch: nothing but the context pass compiled in
+                hipLaunchKernelGGL((flash_kernel<T, DH, 1, 8, kFlashBN, true, 5, true>), dim3(grid), dim3(512), 0, stream, P);
             else
                 hipLaunchKernelGGL((flash_kernel<T, DH, 1, 8, kFlashBN, true, 5>), dim3(grid), dim3(512), 0, stream, P);
             return hipGetLastError();

@@ -132,7 +132,11 @@ struct BoolTag {
 // LEAN selects the fast pass: false = the software-pipelined loop (two wavefronts per SIMD, 216
 // registers), true = the plain loop built for four wavefronts per SIMD (see lean_pass).
 // OCC: wavefronts per SIMD the register allocation is held to (1 = no constraint).
-template <typename T, int DH, int QB, int NW, int BN, bool LEAN = false, int OCC = 1>
+// PLAIN: the launch is a context pass (P.mode == kFlashContext): no buffer keys, no masks, no
+// cache write — none of their state is computed or kept, which the 96-register form of the
+// decode launch would otherwise park in scratch memory (60 bytes per lane, written by every
+// wavefront whatever the mode).
+template <typename T, int DH, int QB, int NW, int BN, bool LEAN = false, int OCC = 1, bool PLAIN = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 void flash_kernel(FlashParams P) {
     typedef MfmaOps<T> Ops;
@@ -193,16 +197,15 @@ void flash_kernel(FlashParams P) {
     // The loads are only requested here; they are scaled into qreg once the first K/V tiles have
     // been requested too, so that the kernel's first memory round trips overlap.
     vec qreg[QB][KS];
-    long orow_idx[QB];  // (b*H + h)*Lq + i of this lane's query per block, or -1
-    int qi[QB];         // query index i within its batch entry
+    int qi[QB];  // query index i within its batch entry, or -1
     long qb[QB];
-#pragma unroll
-    for (int j = 0; j < QB; ++j) {
-        int r = row0_w + 32 * j + c;
-        bool valid = r < P.G;
-        long flat = static_cast<long>(g) * P.G + (valid ? r : 0);
-        long b;
-        int i;
+    // Batch entry b and index i of the query in column `col` (0..31) of block j of this wavefront;
+    // false beyond the last row.  The epilogue asks again (with a column the compiler cannot
+    // trace back to the lane index) instead of keeping addresses alive across the key loop.
+    auto query_of = [&](int j, int col, long &b, int &i) {
+        const int r = row0_w + 32 * j + col;
+        const bool valid = r < P.G;
+        const long flat = static_cast<long>(g) * P.G + (valid ? r : 0);
         if (P.Lq == 1) {  // decode: no 64-bit division on the way to the first load
             b = flat; i = 0;
         } else if (P.Lq == 2) {
@@ -210,9 +213,13 @@ void flash_kernel(FlashParams P) {
         } else {
             b = flat / P.Lq; i = static_cast<int>(flat % P.Lq);
         }
-        qb[j] = b;
+        return valid;
+    };
+#pragma unroll
+    for (int j = 0; j < QB; ++j) {
+        int i;
+        const bool valid = query_of(j, c, qb[j], i);
         qi[j] = valid ? i : -1;
-        orow_idx[j] = valid ? (b * P.H + h) * P.Lq + i : -1;
     }
     // Raw query fragments of this lane (addresses recomputed from qb/qi: nothing extra stays live
     // across the key loop), and their scaled, rounded form in qreg.
@@ -243,7 +250,7 @@ void flash_kernel(FlashParams P) {
     };
 
     // ---- prefill: this tile's own K/V rows go to the cache.
-    if (P.mode == kFlashPrefill && P.kcache.p && g < P.cache_batches) {
+    if (!PLAIN && P.mode == kFlashPrefill && P.kcache.p && g < P.cache_batches) {
         int nrows = min(BM, P.G - row0_wg);
         for (int idx = tid; idx < nrows * CPR; idx += NT) {
             int rr = row0_wg + idx / CPR, ch = idx % CPR;
@@ -263,7 +270,7 @@ void flash_kernel(FlashParams P) {
     int wave_lim_min = 0, wave_lim_max = 0;
 #pragma unroll
     for (int j = 0; j < QB; ++j) lim[j] = 0;
-    if (P.mode == kFlashTeacher) {
+    if (!PLAIN && P.mode == kFlashTeacher) {
         int last = min(row0_wg + BM, P.G) - 1;
         int wg_max = min(P.Nb, tf_range_max(row0_wg, last, P.Nt));
         buf_tiles = (wg_max + BN - 1) / BN;
@@ -275,7 +282,7 @@ void flash_kernel(FlashParams P) {
         }
 #pragma unroll
         for (int j = 0; j < QB; ++j) lim[j] = qi[j] >= 0 ? min(P.Nb, tf_limit(qi[j], P.Nt)) : 0;
-    } else if (P.mode == kFlashRowMask) {
+    } else if (!PLAIN && P.mode == kFlashRowMask) {
         // the limit is not monotone in the row here (targets count modulo Nb): the wavefront's and
         // the workgroup's bounds come from reductions over the rows' own limits
         int lo = P.Nb, hi = 0;
@@ -304,13 +311,11 @@ void flash_kernel(FlashParams P) {
     // ---- staging: global -> registers -> LDS.  Each thread owns NCH 16-byte chunks
     // (row st_row, column st_col) of the K tile and the same of V; their global
     // addresses are kept as running pointers that advance by one tile per fetch.
-    int st_row[NCH], st_col[NCH];
-#pragma unroll
-    for (int x = 0; x < NCH; ++x) {
-        int idx = tid + x * NT;
-        st_row[x] = idx / CPR;
-        st_col[x] = (idx % CPR) * 8;
-    }
+    // (In the lean form these tiles are the rare ones — a ragged last tile, buffer tiles under a
+    // mask —, so the chunk's place is worked out where it is needed, from a thread index the
+    // compiler cannot trace, instead of sitting in registers through the steady loop.)
+    auto st_row = [&](int x) { return ((LEAN ? opaque(tid) : tid) + x * NT) / CPR; };
+    auto st_col = [&](int x) { return (((LEAN ? opaque(tid) : tid) + x * NT) % CPR) * 8; };
     u32x4 kst[NCH], vst[NCH];
     const T *kp[NCH], *vp[NCH];
     long k_step = 0, v_step = 0;  // elements per tile
@@ -331,8 +336,8 @@ void flash_kernel(FlashParams P) {
         v_step = static_cast<long>(BN) * vs_.sn;
 #pragma unroll
         for (int x = 0; x < NCH; ++x) {
-            kp[x] = kbase + st_row[x] * ks_.sn + st_col[x];
-            vp[x] = vbase + st_row[x] * vs_.sn + st_col[x];
+            kp[x] = kbase + st_row(x) * ks_.sn + st_col(x);
+            vp[x] = vbase + st_row(x) * vs_.sn + st_col(x);
         }
     };
 
@@ -353,7 +358,7 @@ void flash_kernel(FlashParams P) {
             for (int x = 0; x < NCH; ++x) {
                 kst[x] = u32x4{0u, 0u, 0u, 0u};
                 vst[x] = u32x4{0u, 0u, 0u, 0u};
-                if ((NCH * NT == CHUNKS || tid + x * NT < CHUNKS) && st_row[x] < fetch_rows_left) {
+                if ((NCH * NT == CHUNKS || tid + x * NT < CHUNKS) && st_row(x) < fetch_rows_left) {
                     kst[x] = *reinterpret_cast<const u32x4 *>(kp[x]);
                     vst[x] = *reinterpret_cast<const u32x4 *>(vp[x]);
                 }
@@ -371,8 +376,8 @@ void flash_kernel(FlashParams P) {
 #pragma unroll
         for (int x = 0; x < NCH; ++x) {
             if (NCH * NT == CHUNKS || tid + x * NT < CHUNKS) {
-                *reinterpret_cast<u32x4 *>(k_stage(buf) + st_row[x] * KPAD + st_col[x]) = kst[x];
-                *reinterpret_cast<u32x4 *>(v_stage(buf) + st_row[x] * VPAD + st_col[x]) = vst[x];
+                *reinterpret_cast<u32x4 *>(k_stage(buf) + st_row(x) * KPAD + st_col(x)) = kst[x];
+                *reinterpret_cast<u32x4 *>(v_stage(buf) + st_row(x) * VPAD + st_col(x)) = vst[x];
             }
         }
     };
@@ -1028,12 +1033,15 @@ void flash_kernel(FlashParams P) {
 #pragma unroll
     for (int j = 0; j < QB; ++j) {
         float l_tot = l_run[j] + __shfl_xor(l_run[j], 32, 64);
-        if (orow_idx[j] < 0) continue;
+        long ob;
+        int oi;
+        if (!query_of(j, opaque(lane) & 31, ob, oi)) continue;
+        const long orow_idx = (ob * P.H + h) * P.Lq + oi;  // row of the [B, H, Lq] order
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
         const float m_fin = m_run[j] == -INFINITY ? 0.f : m_run[j];
         const float lse = l_tot > 0.f ? (m_fin + fast_log2(l_tot)) * kLn2 : -INFINITY;
         if (P.part_o) {
-            T *po = static_cast<T *>(P.part_o) + (static_cast<long>(split) * total_rows + orow_idx[j]) * DH;
+            T *po = static_cast<T *>(P.part_o) + (static_cast<long>(split) * total_rows + orow_idx) * DH;
 #pragma unroll
             for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -1042,9 +1050,9 @@ void flash_kernel(FlashParams P) {
                                  pack2<T>(o_acc[j][db][4 * gq + 2] * inv, o_acc[j][db][4 * gq + 3] * inv)};
                     *reinterpret_cast<u32x2 *>(po + 32 * db + 8 * gq + 4 * hb) = val;
                 }
-            if (hb == 0) P.part_lse[static_cast<long>(split) * total_rows + orow_idx[j]] = lse;
+            if (hb == 0) P.part_lse[static_cast<long>(split) * total_rows + orow_idx] = lse;
         } else {
-            T *orow = view_row<T>(P.out, qb[j], h, qi[j]);
+            T *orow = view_row<T>(P.out, ob, h, oi);
 #pragma unroll
             for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -1053,7 +1061,7 @@ void flash_kernel(FlashParams P) {
                                  pack2<T>(o_acc[j][db][4 * gq + 2] * inv, o_acc[j][db][4 * gq + 3] * inv)};
                     *reinterpret_cast<u32x2 *>(orow + 32 * db + 8 * gq + 4 * hb) = val;
                 }
-            if (P.lse && hb == 0) P.lse[orow_idx[j]] = lse;
+            if (P.lse && hb == 0) P.lse[orow_idx] = lse;
         }
     }
 }
