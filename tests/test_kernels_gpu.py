@@ -215,7 +215,7 @@ def test_decode_attention_overlapped_matches_oracle(device, small_route, dtype, 
     _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, True, scale=0.6, overlapped=True)
 
 
-@pytest.fixture(params=["0", "100000", None], ids=["16-row-chunks", "4-row-chunks", "by-length"])
+@pytest.fixture(params=["0", "100000", "20", None], ids=["16-row-chunks", "4-row-chunks", "switch-at-20-rows", "by-length"])
 def stream_chunk_shape(request, monkeypatch):
     """The streaming buffer pass reads 4 rows of 16 pairs or 16 rows of 4 pairs per request and
     picks by buffer length (ARTAB_STREAM_SHORT: the longest buffer that takes the first shape)."""
