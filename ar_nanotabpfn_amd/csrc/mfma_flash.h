@@ -742,23 +742,6 @@ void flash_kernel(FlashParams P) {
 
         // Full context tiles (every row present, nothing masked): the steady state.
         const int n_main = (ctx_end - ctx_begin) / BN;
-        const char *m_src[NP];   // scalar: this round's source of the tile to be requested next
-        unsigned m_off[NP];      // lane: byte offset of this lane's piece inside a tile
-        long m_step[NP];
-#pragma unroll
-        for (int x = 0; x < NP; ++x) {
-            const View &src = p_v[x] ? P.vc : P.kc;
-            m_src[x] = reinterpret_cast<const char *>(view_row<T>(src, kvb, h, ctx_begin));
-            m_off[x] = static_cast<unsigned>((p_row[x] * src.sn + p_col[x]) * static_cast<long>(sizeof(T)));
-            m_step[x] = static_cast<long>(BN) * src.sn * static_cast<long>(sizeof(T));
-        }
-        auto main_fetch = [&](u32x4(&st)[NP]) {
-#pragma unroll
-            for (int x = 0; x < NP; ++x) {
-                if (p_on[x]) st[x] = *reinterpret_cast<const u32x4 *>(m_src[x] + m_off[x]);
-                m_src[x] += m_step[x];
-            }
-        };
 
         // In the steady state the tiles do not pass through registers at all: a stage is a whole
         // number of KiB (K region and V region each), so it is filled by NI direct global->LDS
@@ -789,8 +772,7 @@ void flash_kernel(FlashParams P) {
             piece = piece < CPR ? piece : 0;
             d_off[r] = static_cast<unsigned>(row * src.sn * static_cast<long>(sizeof(T)) + piece * 16);
             d_step[r] = static_cast<long>(BN) * src.sn * static_cast<long>(sizeof(T));
-            // tiles 0 and 1 are requested by the prologue through registers
-            d_src[r] = reinterpret_cast<const char *>(view_row<T>(src, kvb, h, ctx_begin)) + 2 * d_step[r];
+            d_src[r] = reinterpret_cast<const char *>(view_row<T>(src, kvb, h, ctx_begin));
             if (i < NI) ++n_dma;
         }
         auto dma_tile = [&](auto stage_) {
@@ -840,12 +822,6 @@ void flash_kernel(FlashParams P) {
                 g_src[x] += g_step[x];
             }
             rows_left -= BN;
-        };
-        auto fetch_tile = [&](int it, u32x4(&st)[NP]) {
-            if (it < n_main)
-                main_fetch(st);
-            else
-                gfetch(it, st);
         };
         auto stash_tile = [&](auto stage_, const u32x4(&st)[NP]) {
 #pragma unroll
@@ -942,7 +918,7 @@ void flash_kernel(FlashParams P) {
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // direct loads of the steady state
                 __syncthreads();
                 const bool fetch = it + 2 < n_tiles && it + 2 >= n_main;
-                if (fetch) fetch_tile(it + 2, st_a);
+                if (fetch) gfetch(it + 2, st_a);
                 const bool is_ctx = it < ctx_tiles;
                 const int kv0 = is_ctx ? ctx_begin + it * BN : (it - ctx_tiles) * BN;
                 const int seg_end = is_ctx ? ctx_end : P.Nb;
@@ -963,14 +939,22 @@ void flash_kernel(FlashParams P) {
 
         __builtin_amdgcn_s_setprio(3);
         {
+            // the first three tiles are requested together with the queries: full tiles by direct
+            // loads into their stages, a ragged or buffer tile among the first two through registers
             u32x4 qraw[QB][KS];
             request_q(qraw);
-            if (n_tiles > 0) fetch_tile(0, st_a);
-            if (n_tiles > 1) fetch_tile(1, st_b);
-            scale_q(qraw);
-            if (n_tiles > 0) stash_tile(0, st_a);
-            if (n_tiles > 1) stash_tile(1, st_b);
+            if (n_main > 0)
+                dma_tile(std::integral_constant<int, 0>{});
+            else if (n_tiles > 0)
+                gfetch(0, st_a);
+            if (n_main > 1)
+                dma_tile(std::integral_constant<int, 1>{});
+            else if (n_tiles > 1)
+                gfetch(1, st_b);
             if (n_main > 2) dma_tile(std::integral_constant<int, 2>{});
+            scale_q(qraw);
+            if (n_main <= 0 && n_tiles > 0) stash_tile(std::integral_constant<int, 0>{}, st_a);
+            if (n_main <= 1 && n_tiles > 1) stash_tile(std::integral_constant<int, 1>{}, st_b);
         }
 
         int it = 0;
