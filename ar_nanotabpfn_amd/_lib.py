@@ -16,7 +16,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libartab_attention.so")
 
-ABI_VERSION = 5  # ARTAB_VERSION of include/artab_attention.h
+ABI_VERSION = 6  # ARTAB_VERSION of include/artab_attention.h
 STATIC_SCRATCH_BYTES = 32 << 20  # ARTAB_STATIC_SCRATCH_BYTES
 ARTAB_BF16, ARTAB_F16, ARTAB_F32 = 0, 1, 2
 IMPL_AUTO, IMPL_PORTABLE, IMPL_MFMA = 0, 1, 2
@@ -108,7 +108,9 @@ SIGNATURES = {
     "artab_order_signal": (_i, [_p, _i, _p]),
     "artab_order_wait": (_i, [_p, _i, ctypes.c_uint64, _p]),
     "artab_teacher_forcing_attention": (_i, [_VP, _VP, _VP, _VP, _VP, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
-    "artab_row_mask_attention": (_i, [_VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
+    "artab_row_mask_attention": (_i, [_VP, _VP, _VP, _VP, _p, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
+    "artab_row_mask_attention_backward": (
+        _i, [_VP, _VP, _VP, _VP, _VP, _p, _p, _VP, _VP, _VP, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "artab_prefill_attention": (_i, [_VP, _VP, _VP, _VP, _VP, _VP, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "artab_buffer_attention": (_i, [_VP, _VP, _VP, _p, _i64, _i64, _i64, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _p]),
     "artab_merge_attention_outputs": (_i, [_VP, _p, _VP, _p, _VP, _i, _i, _i, _i, _i, _p]),

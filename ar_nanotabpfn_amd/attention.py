@@ -11,7 +11,8 @@ a tile schedule — with the same constructor names and the same caching:
   (inference.py:525-577) are built by the predictor.
 
 * ``create_row_mask`` (attention.py:86-175): the context / buffer / target mask of the
-  training forward, forward only (no backward pass exists in this package).
+  training forward; the row attention under it has a device backward pass
+  (``attention_kernels.row_mask_attention``).
 """
 
 from __future__ import annotations
@@ -157,5 +158,8 @@ class MultiheadAttention(nn.Module):
             return self.out_proj(out.transpose(1, 2).reshape(B, Sq, D)), (kh, vh)
         if kh.shape[2] != Sq or block_mask.seq_len != Sq:
             raise ValueError("dense mask expects equally many queries and keys")
+        if torch.is_grad_enabled() and (qh.requires_grad or kh.requires_grad or vh.requires_grad):
+            raise NotImplementedError("dense attention has no backward pass (it serves the context prefill); "
+                                      "call it under torch.no_grad()")
         out = ak.prefill_attention(qh, kh, vh)
         return self.out_proj(out.transpose(1, 2).reshape(B, Sq, D)), (kh, vh)

@@ -43,6 +43,7 @@ __all__ = [
     "teacher_forcing_attention",
     "prefill_attention",
     "row_mask_attention",
+    "row_mask_attention_backward",
 ]
 
 
@@ -450,25 +451,86 @@ def prefill_attention(
     return out
 
 
-def row_mask_attention(q: Tensor, k: Tensor, v: Tensor, context_len: int, buffer_len: int, attending_chunks: int,
-                       use_triton: bool = True) -> Tensor:
-    """Row attention of the training forward: ``q, k, v [B,H,R,D]`` with rows
-    ``[context | buffer | target]`` under the mask of ``create_row_mask``
-    (attention.py:86-175), carried as a tile schedule.  Forward only."""
+def _row_mask_forward(q: Tensor, k: Tensor, v: Tensor, context_len: int, buffer_len: int, attending_chunks: int,
+                      use_triton: bool, want_lse: bool):
     dev = _lib.require_device(q, k, v)
     lib = _lib.load()
     B, H, R, Dh = q.shape
     if k.shape != q.shape or v.shape != q.shape:
         raise ValueError("row-mask attention expects q, k, v of one shape [B,H,R,D]")
     out = _alloc_out(q)
+    lse = torch.empty((B, H, R), device=q.device, dtype=torch.float32) if want_lse else None
     qv, kv, vv, ov = _lib.view4(q), _lib.view4(k), _lib.view4(v), _lib.view4(out)
     _lib.check(
         lib.artab_row_mask_attention(
-            _lib.ref(qv), _lib.ref(kv), _lib.ref(vv), _lib.ref(ov), B, H, R, int(context_len), int(buffer_len),
-            int(attending_chunks), Dh, 0.0, _lib.dtype_code(q.dtype), _impl(use_triton), _lib.current_stream(dev),
+            _lib.ref(qv), _lib.ref(kv), _lib.ref(vv), _lib.ref(ov), lse.data_ptr() if want_lse else None,
+            B, H, R, int(context_len), int(buffer_len), int(attending_chunks), Dh, 0.0, _lib.dtype_code(q.dtype),
+            _impl(use_triton), _lib.current_stream(dev),
         )
     )
-    return out
+    return out, lse
+
+
+def row_mask_attention_backward(q: Tensor, k: Tensor, v: Tensor, out: Tensor, dout: Tensor, lse: Tensor,
+                                context_len: int, buffer_len: int, attending_chunks: int,
+                                use_triton: bool = True) -> Tuple[Tensor, Tensor, Tensor]:
+    """Gradients of ``row_mask_attention`` for the output gradient ``dout``: ``(dq, dk, dv)``, each
+    ``[B,H,R,D]`` (views of one ``[B,R,3,H,D]`` tensor, the layout of a fused q/k/v projection).
+    ``out`` and ``lse`` are what the forward returned.  The gradients autograd derives for the
+    reference's flex_attention call under ``create_row_mask`` (attention.py:57-59, :86-175)."""
+    dev = _lib.require_device(q, k, v, out, dout)
+    lib = _lib.load()
+    B, H, R, Dh = q.shape
+    for name, t in (("k", k), ("v", v), ("out", out), ("dout", dout)):
+        if t.shape != q.shape or t.dtype != q.dtype:
+            raise ValueError(f"{name} must have q's shape {tuple(q.shape)} and dtype")
+    if lse.shape != (B, H, R) or lse.dtype != torch.float32 or not lse.is_contiguous():
+        raise ValueError("lse must be a contiguous float32 [B,H,R] tensor")
+    if dout.stride(-1) != 1 or any(st % (16 // dout.element_size()) for st in dout.stride()[:-1]):
+        dout = dout.contiguous()
+    grads = torch.empty((B, R, 3, H, Dh), device=q.device, dtype=q.dtype)
+    dq, dk, dv = (grads[:, :, i].transpose(1, 2) for i in range(3))
+    delta = torch.empty((B, H, R), device=q.device, dtype=torch.float32)
+    views = [_lib.view4(t) for t in (q, k, v, out, dout)]
+    gviews = [_lib.view4(t) for t in (dq, dk, dv)]
+    _lib.check(
+        lib.artab_row_mask_attention_backward(
+            *[_lib.ref(x) for x in views], lse.data_ptr(), delta.data_ptr(), *[_lib.ref(x) for x in gviews],
+            B, H, R, int(context_len), int(buffer_len), int(attending_chunks), Dh, 0.0, _lib.dtype_code(q.dtype),
+            _impl(use_triton), _lib.current_stream(dev),
+        )
+    )
+    return dq, dk, dv
+
+
+class _RowMaskAttention(torch.autograd.Function):
+    """``row_mask_attention`` with its device backward pass (two launches: dQ, then dK and dV)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, context_len, buffer_len, attending_chunks, use_triton):
+        out, lse = _row_mask_forward(q, k, v, context_len, buffer_len, attending_chunks, use_triton, want_lse=True)
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.mask = (context_len, buffer_len, attending_chunks, use_triton)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse = ctx.saved_tensors
+        context_len, buffer_len, attending_chunks, use_triton = ctx.mask
+        dq, dk, dv = row_mask_attention_backward(q, k, v, out, dout, lse, context_len, buffer_len, attending_chunks,
+                                                 use_triton)
+        return dq, dk, dv, None, None, None, None
+
+
+def row_mask_attention(q: Tensor, k: Tensor, v: Tensor, context_len: int, buffer_len: int, attending_chunks: int,
+                       use_triton: bool = True) -> Tensor:
+    """Row attention of the training forward: ``q, k, v [B,H,R,D]`` with rows
+    ``[context | buffer | target]`` under the mask of ``create_row_mask``
+    (attention.py:86-175), carried as a tile schedule.  Differentiable: when gradients are
+    being recorded for q, k or v the call goes through ``_RowMaskAttention``."""
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        return _RowMaskAttention.apply(q, k, v, int(context_len), int(buffer_len), int(attending_chunks), use_triton)
+    return _row_mask_forward(q, k, v, context_len, buffer_len, attending_chunks, use_triton, want_lse=False)[0]
 
 
 def hybrid_attention(

@@ -33,7 +33,7 @@ HIPCC_FLAGS = [
 
 # (source, extra defines, object name)
 UNITS = [("artab_api.hip", [], "artab_api.o"), ("flash_launch.hip", [], "flash_launch.o"),
-         ("mix_bench.hip", [], "mix_bench.o")]
+         ("mix_bench.hip", [], "mix_bench.o"), ("backward_launch.hip", [], "backward_launch.o")]
 for _bf16 in (1, 0):
     for _group in (0, 1, 2, 3):
         UNITS.append(("layer_launch.hip", [f"-DARTAB_LAYER_BF16={_bf16}", f"-DARTAB_LAYER_GROUP={_group}"],

@@ -936,7 +936,7 @@ int artab_teacher_forcing_attention(const artab_view *q, const artab_view *k_ctx
 }
 
 int artab_row_mask_attention(const artab_view *q, const artab_view *k, const artab_view *v, const artab_view *out,
-                             int B, int H, int R, int Nc, int Nb, int attending_chunks, int Dh, float scale,
+                             float *lse, int B, int H, int R, int Nc, int Nb, int attending_chunks, int Dh, float scale,
                              int dtype, int impl, void *stream) {
     ARTAB_TRY(check_common(B, H, R, Dh, dtype));
     if (Nc < 1 || Nb < 0 || Nc + Nb > R || attending_chunks < 0)
@@ -963,7 +963,7 @@ int artab_row_mask_attention(const artab_view *q, const artab_view *k, const art
         memset(&P, 0, sizeof(P));
         P.q = dv(q); P.kc = dv(k); P.vc = dv(v); P.kb = kb; P.vb = vb; P.out = dv(out);
         P.B = B; P.H = H; P.Lq = R; P.Nc = Nc; P.Nb = Nb;
-        P.rm_nc = Nc; P.rm_attend = attending_chunks;
+        P.rm_nc = Nc; P.rm_attend = attending_chunks; P.lse = lse;
         P.new_row = -1; P.mode = kModeRowMask; P.Dh = Dh; P.scale = scale;
         P.vec_ok = aligned ? 1 : 0;
         return launch_status(launch_portable_dtype(P, dtype, st), "row-mask attention (portable)");
@@ -973,13 +973,49 @@ int artab_row_mask_attention(const artab_view *q, const artab_view *k, const art
     memset(&F, 0, sizeof(F));
     F.q = dv(q); F.kc = dv(k); F.vc = dv(v); F.kb = kb; F.vb = vb; F.out = dv(out);
     F.B = B; F.H = H; F.Lq = R; F.Nc = Nc; F.Nb = Nb;
-    F.rm_nc = Nc; F.rm_attend = attending_chunks;
+    F.rm_nc = Nc; F.rm_attend = attending_chunks; F.lse = lse;
     F.G = pl.G; F.tiles_per_group = pl.tiles_per_group; F.n_groups = pl.n_groups;
     F.n_split = 1; F.kv_per_split = pl.kv_per_split;
     F.qscale = scale * kLog2e;
     F.mode = kFlashRowMask;
     ProfileScope prof(st);
     return launch_status(launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st), "row-mask attention (mfma)");
+}
+
+int artab_row_mask_attention_backward(const artab_view *q, const artab_view *k, const artab_view *v,
+                                      const artab_view *out, const artab_view *dout, const float *lse, float *delta,
+                                      const artab_view *grad_q, const artab_view *grad_k, const artab_view *grad_v,
+                                      int B, int H, int R, int Nc, int Nb, int attending_chunks, int Dh, float scale,
+                                      int dtype, int impl, void *stream) {
+    ARTAB_TRY(check_common(B, H, R, Dh, dtype));
+    if (Nc < 1 || Nb < 0 || Nc + Nb > R || attending_chunks < 0)
+        return fail(ARTAB_ERR_BAD_SHAPE, "row mask needs 1 <= Nc, 0 <= Nb, Nc + Nb <= R, attending_chunks >= 0 (got Nc=%d Nb=%d R=%d A=%d)",
+                    Nc, Nb, R, attending_chunks);
+    if (B == 0 || R == 0) return ARTAB_OK;
+    const artab_view *views[8] = {q, k, v, out, dout, grad_q, grad_k, grad_v};
+    const char *names[8] = {"q", "k", "v", "out", "dout", "grad_q", "grad_k", "grad_v"};
+    bool aligned = true;
+    for (int i = 0; i < 8; ++i) {
+        ARTAB_TRY(check_view(views[i], names[i], dtype, true));
+        aligned = aligned && vec_aligned(views[i], dtype, Dh);
+    }
+    if (!lse || !delta) return fail(ARTAB_ERR_NULL_POINTER, "lse and delta must be given");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool use_mfma = impl != ARTAB_IMPL_PORTABLE && (dtype == ARTAB_BF16 || dtype == ARTAB_F16) &&
+                          (Dh == 32 || Dh == 64) && aligned;
+    if (impl == ARTAB_IMPL_MFMA && !use_mfma)
+        return fail(ARTAB_ERR_UNSUPPORTED, "MFMA backward needs bf16/f16, head_dim in {32,64}, 16-byte aligned rows");
+    BackwardParams P;
+    memset(&P, 0, sizeof(P));
+    P.q = dv(q); P.k = dv(k); P.v = dv(v); P.out = dv(out); P.dout = dv(dout);
+    P.dq = dv(grad_q); P.dk = dv(grad_k); P.dv = dv(grad_v);
+    P.lse = lse; P.delta = delta;
+    P.B = B; P.H = H; P.R = R; P.Nc = Nc; P.Nb = Nb; P.attend = attending_chunks;
+    P.Dh = Dh; P.scale = resolve_scale(scale, Dh); P.vec_ok = aligned ? 1 : 0;
+    const int elem = dtype == ARTAB_BF16 ? kElemBf16 : dtype == ARTAB_F16 ? kElemF16 : kElemF32;
+    ProfileScope prof(st);
+    return launch_status(launch_row_mask_backward(P, elem, use_mfma, st),
+                         use_mfma ? "row-mask attention backward (mfma)" : "row-mask attention backward (portable)");
 }
 
 int artab_prefill_attention(const artab_view *q, const artab_view *k, const artab_view *v, const artab_view *out,

@@ -7,6 +7,7 @@
 
 #include <cstdlib>
 
+#include "attention_backward.h"
 #include "fused_layer.h"
 #include "mfma_flash.h"
 
@@ -30,6 +31,11 @@ inline int fused_tile_rows(long rows) {
 
 // flash_launch.hip: BM = query rows per workgroup (256, 128 or 64), as planned by the caller
 hipError_t launch_flash_dtype(const FlashParams &P, bool is_bf16, int Dh, int BM, hipStream_t stream);
+
+// backward_launch.hip: dQ launch, then dK/dV launch, of the training row attention.  `elem` is
+// the element type of every tensor; the matrix-core kernels take bf16 / f16 with head_dim 32 / 64.
+enum BackwardElem : int { kElemF32 = 0, kElemBf16 = 1, kElemF16 = 2 };
+hipError_t launch_row_mask_backward(const BackwardParams &P, int elem, bool use_mfma, hipStream_t stream);
 
 // layer_launch.hip (one object per element type and kernel group)
 hipError_t launch_layer_pre(const FusedPreParams &P, int D, bool is_bf16, hipStream_t st);

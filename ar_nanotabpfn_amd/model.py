@@ -8,8 +8,9 @@ follow the reference so checkpoints interchange: ``embedder.{x_embed,y_embed}``,
 ``backbone.norm``, ``head.head.{0,2}``, ``head.{mean_bias,std_bias,weight_bias}``,
 ``ar_tokens`` (model.py:33-37, :89-98, :138, :172-184, :315).
 
-The training forward (flex_attention with the context/buffer/target row mask,
-model.py:317-369) is not part of this package; inference goes through
+``ARTabPFN.forward`` is the training objective (model.py:317-369): with gradients being
+recorded the layers run as plain differentiable PyTorch around the device row attention and its
+device backward pass; without, through the fused inference kernels.  Inference goes through
 ``ARTabPFNPredictor``.
 """
 
@@ -192,11 +193,28 @@ class TwoStageTransformerLayer(nn.Module):
         h = bias_gelu(torch.mm(x2d, lin1.weight.t()), lin1.bias)
         return add_layer_norm(x_row, torch.mm(h, lin2.weight.t()).view_as(x_row), lin2.bias, self.norm3)
 
-    def forward(self, x: Tensor, mask_features: DenseMask, mask_rows: DenseMask) -> Tuple[Tensor, Tuple[Tensor, Tensor]]:
-        """``[B,R,C,D]`` with dense masks only (the bidirectional context pass)."""
+    def _forward_recording(self, x_row: Tensor, mask_rows) -> Tuple[Tensor, Tuple[Tensor, Tensor]]:
+        """The layer on ``[B,R,D]`` rows as differentiable PyTorch modules around the device row
+        attention (model.py:100-126 with C = 1): what a training step records."""
+        af = self.attn_features
+        # one key per query: the softmax weight is exactly 1 and the attention output is
+        # out_proj(v_proj(x)); q_proj and k_proj get the exact zero gradients autograd gives them
+        # in the reference (their parameters stay in the optimiser's bookkeeping)
+        feat = af.out_proj(af.v_proj(x_row)) + 0.0 * (af.q_proj.weight.sum() + af.k_proj.weight.sum())
+        x_row = self.norm1(feat + x_row)
+        attn, kv = self.attn_rows(x_row, x_row, x_row, mask_rows)
+        x_row = self.norm2(attn + x_row)
+        return self.norm3(x_row + self.ff(x_row)), kv
+
+    def forward(self, x: Tensor, mask_features, mask_rows) -> Tuple[Tensor, Tuple[Tensor, Tensor]]:
+        """``[B,R,C,D]`` under a dense mask (the bidirectional context pass) or the training row
+        mask.  While gradients are recorded the layer runs as differentiable modules."""
         B, R, C, D = x.shape
         if C != 1:
             raise NotImplementedError("only the single-column layout (C = 1) is used by this model")
+        if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
+            out, kv = self._forward_recording(x.squeeze(2), mask_rows)
+            return out.unsqueeze(2), kv
         x_row = self.feature_stage(x.squeeze(2))
         attn, kv = self.attn_rows(x_row, x_row, x_row, mask_rows)
         x_row = add_layer_norm(x_row, attn, None, self.norm2)
@@ -215,6 +233,8 @@ class TwoStageTransformer(nn.Module):
         for layer in self.layers:
             x, kv = layer(x, mask_features, mask_rows)
             kvs.append(kv)
+        if torch.is_grad_enabled() and x.requires_grad:
+            return self.norm(x), kvs
         return add_layer_norm(x, None, None, self.norm), kvs
 
 
@@ -298,13 +318,14 @@ class ARTabPFN(nn.Module):
         self.head = MixtureGaussianHead(d_model, d_ff, dim_y=1, num_components=num_components)
         self.ar_tokens = nn.Parameter(torch.randn(buffer_size, d_model) * 0.02)
 
-    @torch.no_grad()
     def forward(self, x_context: Tensor, y_context: Tensor, x_buffer: Tensor, y_buffer: Tensor, x_target: Tensor,
                 mask_features, mask_rows, y_target: Optional[Tensor] = None):
-        """The training objective, forward only (model.py:317-369): context, buffer and target rows
-        in one pass under the row mask of ``create_row_mask``; returns the mean negative
-        log-likelihood of ``y_target`` (None without it).  The attention runs on the device kernels,
-        which have no backward pass: the call is always under ``no_grad``."""
+        """The training objective (model.py:317-369): context, buffer and target rows in one pass
+        under the row mask of ``create_row_mask``; returns the mean negative log-likelihood of
+        ``y_target`` (None without it).  The row attention runs on the device kernels in both
+        directions: ``loss.backward()`` gives every parameter its gradient, as in the reference's
+        training step (train.py:289-300).  Under ``torch.no_grad()`` the layers take the fused
+        inference kernels instead."""
         ctx_emb = self.embedder.embed_context(x_context, y_context)
         buf_emb = self.embedder.embed_buffer(x_buffer, y_buffer) + self.ar_tokens[: x_buffer.size(1)]
         tgt_emb = self.embedder.embed_target(x_target)

@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define ARTAB_VERSION 5
+#define ARTAB_VERSION 6
 
 typedef enum artab_dtype {
     ARTAB_BF16 = 0,
@@ -343,11 +343,32 @@ int artab_prefill_attention(const artab_view *q, const artab_view *k, const arta
  * schedule, not a tensor: every row sees the Nc context keys; buffer row j also sees buffer keys
  * [0, j]; target row with offset o sees buffer keys [0, o mod Nb] while o < attending_chunks * Nb
  * and no buffer key after that; target keys are never visited (no self-attention of targets).
- * Forward only.  Nc >= 1.
+ * lse: float32 [B,H,R] natural-log log-sum-exp of every row's scores (what the backward pass
+ * needs), or NULL.  Nc >= 1.
  */
 int artab_row_mask_attention(const artab_view *q, const artab_view *k, const artab_view *v, const artab_view *out,
-                             int B, int H, int R, int Nc, int Nb, int attending_chunks, int Dh, float scale,
-                             int dtype, int impl, void *stream);
+                             float *lse, int B, int H, int R, int Nc, int Nb, int attending_chunks, int Dh,
+                             float scale, int dtype, int impl, void *stream);
+
+/*
+ * Backward pass of artab_row_mask_attention: the gradients that autograd derives for
+ * flex_attention under create_row_mask in the reference's training step
+ * (ar_tabpfn/model/attention.py:52-61 under the mask of :86-175; ar_tabpfn/train.py:289-300).
+ *   q, k, v, out, dout [B,H,R,Dh]: the forward's inputs, its output and the output's gradient;
+ *   lse float32 [B,H,R]: the forward's log-sum-exp;
+ *   delta float32 [B,H,R]: workspace (row sums of dout * out; written by the first launch, read by
+ *                          the second);
+ *   grad_q, grad_k, grad_v [B,H,R,Dh]: results, every element written (target keys get zeros).
+ * With P the masked softmax: grad_v = P^T dout, dS = P o (dout v^T - delta),
+ * grad_q = scale dS k, grad_k = scale dS^T q.  Two launches on `stream`, no atomics: the
+ * result does not depend on the schedule.  The matrix-core kernels take bf16 / f16 with head_dim
+ * 32 or 64; everything else runs the float32-arithmetic kernels.
+ */
+int artab_row_mask_attention_backward(const artab_view *q, const artab_view *k, const artab_view *v,
+                                      const artab_view *out, const artab_view *dout, const float *lse, float *delta,
+                                      const artab_view *grad_q, const artab_view *grad_k, const artab_view *grad_v,
+                                      int B, int H, int R, int Nc, int Nb, int attending_chunks, int Dh, float scale,
+                                      int dtype, int impl, void *stream);
 
 /*
  * Buffer attention with log-sum-exp and an optional boolean mask.

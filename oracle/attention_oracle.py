@@ -34,6 +34,13 @@ live in ``tests/test_oracle.py``):
   the same mask that the reference holds (tests/visualize_masks.py:57-85), by the
   closed-form pair count, by a hand-written tiny case, and through the training loss
   the reference itself computed for the fixture (tests/golden/tiny_model.npz).
+* ``row_mask_attention_backward``: pinned by central finite differences of
+  ``row_mask_attention`` (an independent function: the directional derivative of
+  sum(out * dout) along random directions in q, k and v), and by what the softmax fixes:
+  the key gradients sum to the zero vector (one vector added to every key shifts every
+  score of a row alike and leaves the output unchanged), the value gradients sum to the
+  sum of the output gradients (every row of P sums to one), and target keys, which no row
+  sees, get exact zeros.
 """
 
 from __future__ import annotations
@@ -57,6 +64,7 @@ __all__ = [
     "teacher_forcing_mask",
     "row_mask",
     "row_mask_attention",
+    "row_mask_attention_backward",
     "masked_full_attention",
     "dense_self_attention",
     "decode_step_attention",
@@ -329,6 +337,36 @@ def row_mask_attention(q, k, v, context_len: int, buffer_len: int, attending_chu
     mask = row_mask(R, context_len, buffer_len, attending_chunks)[None, None]
     out, _ = buffer_attention(q, k, v, mask=mask, compute=compute)
     return out
+
+
+def row_mask_attention_backward(q, k, v, dout, context_len: int, buffer_len: int,
+                                attending_chunks: Optional[int] = None, scale: Optional[float] = None,
+                                compute=np.float64):
+    """Gradients of ``row_mask_attention`` with respect to q, k and v for an output gradient
+    ``dout [B,H,R,D]``: what autograd derives for the reference's flex_attention call
+    (attention.py:57-59) inside its training step (train.py:289-300).  Written out from the
+    softmax Jacobian: with ``P`` the masked softmax of ``scale q k^T`` and ``O = P v``,
+
+        dv = P^T dout,  dP = dout v^T,  dS = P * (dP - rowsum(dout * O)),
+        dq = scale dS k,  dk = scale dS^T q.
+
+    Returns ``(dq, dk, dv)``."""
+    q, k, v, dout = _up(q, compute), _up(k, compute), _up(v, compute), _up(dout, compute)
+    R, D = q.shape[2], q.shape[3]
+    if scale is None:
+        scale = D ** -0.5
+    mask = row_mask(R, context_len, buffer_len, attending_chunks)[None, None]
+    s = np.einsum("bhqd,bhkd->bhqk", q, k) * compute(scale)
+    s = np.where(mask, s, -np.inf)
+    p = np.exp(s - s.max(axis=-1, keepdims=True))
+    p = p / p.sum(axis=-1, keepdims=True)
+    out = np.einsum("bhqk,bhkd->bhqd", p, v)
+    dv = np.einsum("bhqk,bhqd->bhkd", p, dout)
+    dp = np.einsum("bhqd,bhkd->bhqk", dout, v)
+    ds = p * (dp - (dout * out).sum(axis=-1, keepdims=True))
+    dq = np.einsum("bhqk,bhkd->bhqd", ds, k) * compute(scale)
+    dk = np.einsum("bhqk,bhqd->bhkd", ds, q) * compute(scale)
+    return dq, dk, dv
 
 
 def masked_full_attention(q, k_full, v_full, mask=None, scale=None, compute=np.float64):

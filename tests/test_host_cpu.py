@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     lib = L.load()
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.artab_version() == L.ABI_VERSION == 5
+    assert lib.artab_version() == L.ABI_VERSION == 6
     assert lib.artab_status_string(0) == b"ok"
 
 
@@ -66,6 +66,15 @@ def test_argument_validation_returns_before_launch():
     assert lib.artab_merge_attention_outputs(r(v), None, r(v), None, r(v), 1, 1, 1, 32, 0, None) == L.ARTAB_ERR_NULL_POINTER
     # empty problems are a no-op success
     assert lib.artab_context_attention(r(v), r(v), r(v), r(v), None, 0, 1, 1, 4, 32, 0.0, 0, None, 0, 0, None) == 0
+    # row-mask backward: no context, sections longer than the rows, missing statistics, MFMA for float32
+    bwd = lambda lse, delta, B, R, Nc, Nb, dtype, impl: lib.artab_row_mask_attention_backward(  # noqa: E731
+        r(v), r(v), r(v), r(v), r(v), lse, delta, r(v), r(v), r(v), B, 2, R, Nc, Nb, 1, 32, 0.0, dtype, impl, None)
+    assert bwd(0x1000, 0x1000, 1, 10, 0, 2, 0, 0) == L.ARTAB_ERR_BAD_SHAPE
+    assert bwd(0x1000, 0x1000, 1, 10, 8, 4, 0, 0) == L.ARTAB_ERR_BAD_SHAPE
+    assert bwd(None, 0x1000, 1, 10, 4, 2, 0, 0) == L.ARTAB_ERR_NULL_POINTER
+    assert bwd(0x1000, None, 1, 10, 4, 2, 0, 0) == L.ARTAB_ERR_NULL_POINTER
+    assert bwd(0x1000, 0x1000, 1, 10, 4, 2, 2, L.IMPL_MFMA) == L.ARTAB_ERR_UNSUPPORTED
+    assert bwd(0x1000, 0x1000, 0, 10, 4, 2, 0, 0) == 0
 
 
 def test_status_to_exception_mapping():

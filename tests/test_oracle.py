@@ -456,6 +456,48 @@ def test_row_mask_attention_equals_per_row_softmax():
         assert np.abs(out[:, :, r] - np.einsum("bhk,bhkd->bhd", p, v[:, :, keys])).max() <= 1e-12
 
 
+@pytest.mark.parametrize("C,B,T,A", [(5, 3, 6, None), (7, 4, 12, 1), (3, 2, 9, 3), (6, 0, 4, 0), (1, 5, 5, 1)])
+def test_row_mask_attention_backward_by_finite_differences(C, B, T, A):
+    """The analytic gradients against central differences of the forward oracle: for random
+    directions (eq, ek, ev) the derivative of sum(out * dout) along them must equal
+    <dq, eq> + <dk, ek> + <dv, ev>, direction by direction."""
+    rng = np.random.default_rng(10 * C + B)
+    D = 8
+    R = C + B + T
+    q, k, v, dout = (rng.standard_normal((2, 2, R, D)) for _ in range(4))
+    dq, dk, dv = ao.row_mask_attention_backward(q, k, v, dout, C, B, A)
+    f = lambda q_, k_, v_: (ao.row_mask_attention(q_, k_, v_, C, B, A) * dout).sum()  # noqa: E731
+    eps = 1e-5
+    for grad, which in ((dq, 0), (dk, 1), (dv, 2)):
+        for _ in range(3):
+            e = rng.standard_normal(q.shape)
+            args_p, args_m = [q, k, v], [q, k, v]
+            args_p[which] = args_p[which] + eps * e
+            args_m[which] = args_m[which] - eps * e
+            numeric = (f(*args_p) - f(*args_m)) / (2 * eps)
+            analytic = (grad * e).sum()
+            assert abs(numeric - analytic) <= 1e-7 * (1 + abs(analytic)), (which, numeric, analytic)
+
+
+def test_row_mask_attention_backward_invariants():
+    rng = np.random.default_rng(3)
+    C, B, T, D = 6, 4, 10, 8
+    R = C + B + T
+    q, k, v, dout = (rng.standard_normal((2, 3, R, D)) for _ in range(4))
+    dq, dk, dv = ao.row_mask_attention_backward(q, k, v, dout, C, B)
+    # one vector added to every key shifts all scores of a row alike: the output does not move
+    assert np.abs(dk.sum(axis=2)).max() <= 1e-12
+    # every row of P sums to one
+    assert np.abs(dv.sum(axis=2) - dout.sum(axis=2)).max() <= 1e-12
+    # nobody sees a target key
+    assert np.all(dk[:, :, C + B:] == 0) and np.all(dv[:, :, C + B:] == 0)
+    # an explicit scale is honoured: scale s on (q, k) equals scale 1 on (s q, k), with dq scaled back
+    dq1, dk1, dv1 = ao.row_mask_attention_backward(0.3 * q, k, v, dout, C, B, scale=1.0)
+    dq2, dk2, dv2 = ao.row_mask_attention_backward(q, k, v, dout, C, B, scale=0.3)
+    assert np.abs(0.3 * dq1 - dq2).max() <= 1e-12 and np.abs(dk1 - dk2).max() <= 1e-12
+    assert np.abs(dv1 - dv2).max() <= 1e-12
+
+
 def test_round_bf16_matches_torch_cast():
     """The oracle's bfloat16 rounding against torch's cast: random values over many exponents,
     exact ties (both parities of the kept mantissa bit), signed zeros, subnormals of bfloat16."""
