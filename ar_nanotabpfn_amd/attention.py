@@ -121,6 +121,20 @@ def clear_mask_cache() -> None:
     _mask_cache.clear()
 
 
+class _InferenceOnly(torch.autograd.Function):
+    """Marks the result of an attention call that has no backward pass: the forward value passes
+    through, a gradient arriving here raises instead of silently stopping."""
+
+    @staticmethod
+    def forward(ctx, out, *inputs):
+        return out.view_as(out)
+
+    @staticmethod
+    def backward(ctx, grad):
+        raise NotImplementedError("dense attention has no backward pass (it serves the context prefill); "
+                                  "only the row attention under a RowMask is differentiable")
+
+
 class MultiheadAttention(nn.Module):
     """Bias-free q/k/v/out projections around the device attention kernels; returns
     the per-head K and V for caching, like attention.py:31-61."""
@@ -158,8 +172,7 @@ class MultiheadAttention(nn.Module):
             return self.out_proj(out.transpose(1, 2).reshape(B, Sq, D)), (kh, vh)
         if kh.shape[2] != Sq or block_mask.seq_len != Sq:
             raise ValueError("dense mask expects equally many queries and keys")
-        if torch.is_grad_enabled() and (qh.requires_grad or kh.requires_grad or vh.requires_grad):
-            raise NotImplementedError("dense attention has no backward pass (it serves the context prefill); "
-                                      "call it under torch.no_grad()")
         out = ak.prefill_attention(qh, kh, vh)
+        if torch.is_grad_enabled() and (qh.requires_grad or kh.requires_grad or vh.requires_grad):
+            out = _InferenceOnly.apply(out, qh, kh, vh)
         return self.out_proj(out.transpose(1, 2).reshape(B, Sq, D)), (kh, vh)

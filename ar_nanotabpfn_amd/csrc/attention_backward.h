@@ -240,8 +240,8 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dq_mfma_kernel(B
     typedef typename Ops::vec vec;
     typedef BackwardTile<T, DH> Tile;
     constexpr int KS = DH / 16, DB = DH / 32;
-    __shared__ __attribute__((aligned(16))) T k_tile[32 * Tile::PAD];
-    __shared__ __attribute__((aligned(16))) T v_tile[32 * Tile::PAD];
+    __shared__ __attribute__((aligned(16))) T k_tiles[2][32 * Tile::PAD];  // two tiles in turn: one barrier per tile
+    __shared__ __attribute__((aligned(16))) T v_tiles[2][32 * Tile::PAD];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hb = lane >> 5;
     const int blocks = (P.R + kBackwardRows - 1) / kBackwardRows;
@@ -280,39 +280,63 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dq_mfma_kernel(B
 
     // every workgroup walks the keys anybody can see; what its own rows do not see is masked
     const int n_tiles = (P.Nc + P.Nb + 31) / 32;
+    // tile kt + 1 goes to LDS at the start of round kt (it was requested a round earlier), tile
+    // kt + 2 is requested then: one barrier per tile, a whole round to cover the round trip
     u32x4 k_raw = Tile::fetch(P.k, b, h, 0, P.R, tid), v_raw = Tile::fetch(P.v, b, h, 0, P.R, tid);
+    Tile::stash(k_tiles[0], tid, k_raw);
+    Tile::stash(v_tiles[0], tid, v_raw);
+    if (n_tiles > 1) {
+        k_raw = Tile::fetch(P.k, b, h, 32, P.R, tid);
+        v_raw = Tile::fetch(P.v, b, h, 32, P.R, tid);
+    }
     for (int kt = 0; kt < n_tiles; ++kt) {
-        __syncthreads();  // the previous tile has been read by everyone
-        Tile::stash(k_tile, tid, k_raw);
-        Tile::stash(v_tile, tid, v_raw);
-        __syncthreads();
+        __syncthreads();  // tile kt is complete; everyone has finished reading the other one
+        const T *k_tile = k_tiles[kt & 1], *v_tile = v_tiles[kt & 1];
         if (kt + 1 < n_tiles) {
-            k_raw = Tile::fetch(P.k, b, h, 32 * (kt + 1), P.R, tid);
-            v_raw = Tile::fetch(P.v, b, h, 32 * (kt + 1), P.R, tid);
+            Tile::stash(k_tiles[(kt + 1) & 1], tid, k_raw);
+            Tile::stash(v_tiles[(kt + 1) & 1], tid, v_raw);
+            if (kt + 2 < n_tiles) {
+                k_raw = Tile::fetch(P.k, b, h, 32 * (kt + 2), P.R, tid);
+                v_raw = Tile::fetch(P.v, b, h, 32 * (kt + 2), P.R, tid);
+            }
         }
-        f32x16 s, dp;
+        f32x16 s, dp;  // dp starts at -delta: the product leaves dP - delta
 #pragma unroll
-        for (int v = 0; v < 16; ++v) s[v] = dp[v] = 0.f;
+        for (int v = 0; v < 16; ++v) {
+            s[v] = 0.f;
+            dp[v] = -delta;
+        }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             s = Ops::mma(Tile::row_operand(k_tile, c, hb, ks), qf[ks], s);
             dp = Ops::mma(Tile::row_operand(v_tile, c, hb, ks), gf[ks], dp);
         }
         u32x4 dsb[2];
+        if (32 * kt + 32 <= P.Nc) {
+            // a tile of context keys: every row sees all of it (rows past the end are never stored)
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                float ds[2];
-#pragma unroll
-                for (int x = 0; x < 2; ++x) {
-                    const int v = 8 * t + 2 * e + x;
-                    const bool vis = 32 * kt + 8 * (v >> 2) + 4 * hb + (v & 3) < vis_end;
-                    const float p = fast_exp2(fmaf(s[v], c2, -lse2));
-                    ds[x] = vis ? p * (dp[v] - delta) : 0.f;
+                for (int e = 0; e < 4; ++e) {
+                    const int v = 8 * t + 2 * e;
+                    dsb[t][e] = pack2<T>(fast_exp2(fmaf(s[v], c2, -lse2)) * dp[v],
+                                         fast_exp2(fmaf(s[v + 1], c2, -lse2)) * dp[v + 1]);
                 }
-                dsb[t][e] = pack2<T>(ds[0], ds[1]);
-            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float ds[2];
+#pragma unroll
+                    for (int x = 0; x < 2; ++x) {
+                        const int v = 8 * t + 2 * e + x;
+                        const bool vis = 32 * kt + 8 * (v >> 2) + 4 * hb + (v & 3) < vis_end;
+                        ds[x] = vis ? fast_exp2(fmaf(s[v], c2, -lse2)) * dp[v] : 0.f;
+                    }
+                    dsb[t][e] = pack2<T>(ds[0], ds[1]);
+                }
+        }
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -340,11 +364,11 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
     typedef typename Ops::vec vec;
     typedef BackwardTile<T, DH> Tile;
     constexpr int KS = DH / 16, DB = DH / 32;
-    __shared__ __attribute__((aligned(16))) T q_tile[32 * Tile::PAD];
-    __shared__ __attribute__((aligned(16))) T g_tile[32 * Tile::PAD];
-    __shared__ __attribute__((aligned(16))) float lse2_s[32];
-    __shared__ __attribute__((aligned(16))) float delta_s[32];
-    __shared__ __attribute__((aligned(16))) int end_s[32];
+    __shared__ __attribute__((aligned(16))) T q_tiles[2][32 * Tile::PAD];  // two tiles in turn: one barrier per tile
+    __shared__ __attribute__((aligned(16))) T g_tiles[2][32 * Tile::PAD];
+    __shared__ __attribute__((aligned(16))) float lse2_t[2][32];
+    __shared__ __attribute__((aligned(16))) float delta_t[2][32];
+    __shared__ __attribute__((aligned(16))) int end_t[2][32];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hb = lane >> 5;
     const int blocks = (P.R + kBackwardRows - 1) / kBackwardRows;
@@ -386,42 +410,71 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
             st_end = backward_vis_end(P, i);
         }
     };
-    if (t_begin < t_end) fetch(t_begin);
+    auto stash = [&](int slot) {
+        Tile::stash(q_tiles[slot], tid, q_raw);
+        Tile::stash(g_tiles[slot], tid, g_raw);
+        if (tid < 32) {
+            lse2_t[slot][tid] = st_lse2;
+            delta_t[slot][tid] = st_delta;
+            end_t[slot][tid] = st_end;
+        }
+    };
+    // as in the dQ kernel: tile qt + 1 goes to LDS at the start of round qt, tile qt + 2 is requested then
+    if (t_begin < t_end) {
+        fetch(t_begin);
+        stash(0);
+        if (t_begin + 1 < t_end) fetch(t_begin + 1);
+    }
     for (int qt = t_begin; qt < t_end; ++qt) {
         __syncthreads();
-        Tile::stash(q_tile, tid, q_raw);
-        Tile::stash(g_tile, tid, g_raw);
-        if (tid < 32) {
-            lse2_s[tid] = st_lse2;
-            delta_s[tid] = st_delta;
-            end_s[tid] = st_end;
+        const int slot = (qt - t_begin) & 1;
+        const T *q_tile = q_tiles[slot], *g_tile = g_tiles[slot];
+        const float *lse2_s = lse2_t[slot], *delta_s = delta_t[slot];
+        const int *end_s = end_t[slot];
+        if (qt + 1 < t_end) {
+            stash(slot ^ 1);
+            if (qt + 2 < t_end) fetch(qt + 2);
         }
-        __syncthreads();
-        if (qt + 1 < t_end) fetch(qt + 1);
+        // rows of the accumulators are queries 8g + 4hb + r of the tile: their statistics come from
+        // LDS; dp starts at -delta of its row, so that the product leaves dP - delta
         f32x16 s, dp;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) s[v] = dp[v] = 0.f;
+        for (int g = 0; g < 4; ++g) {
+            const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&delta_s[8 * g + 4 * hb]);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                s[4 * g + r] = 0.f;
+                dp[4 * g + r] = -d4[r];
+            }
+        }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             s = Ops::mma(Tile::row_operand(q_tile, c, hb, ks), kf[ks], s);
             dp = Ops::mma(Tile::row_operand(g_tile, c, hb, ks), vf[ks], dp);
         }
-        // rows of the accumulator are queries 8g + 4hb + r of the tile: their statistics from LDS
         u32x4 pb[2], dsb[2];
+        // context keys under a full tile of rows: everything is visible (wave-uniform)
+        const bool all_visible = key0 + 32 * wave + 32 <= P.Nc && 32 * qt + 32 <= P.R;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const f32x4 l4 = *reinterpret_cast<const f32x4 *>(&lse2_s[8 * g + 4 * hb]);
-            const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&delta_s[8 * g + 4 * hb]);
-            const int4 e4 = *reinterpret_cast<const int4 *>(&end_s[8 * g + 4 * hb]);
-            const int ends[4] = {e4.x, e4.y, e4.z, e4.w};
             float p[4], ds[4];
+            if (all_visible) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int v = 4 * g + r;
-                const bool vis = kj < ends[r];
-                const float pr = fast_exp2(fmaf(s[v], c2, -l4[r]));
-                p[r] = vis ? pr : 0.f;
-                ds[r] = vis ? pr * (dp[v] - d4[r]) : 0.f;
+                for (int r = 0; r < 4; ++r) {
+                    p[r] = fast_exp2(fmaf(s[4 * g + r], c2, -l4[r]));
+                    ds[r] = p[r] * dp[4 * g + r];
+                }
+            } else {
+                const int4 e4 = *reinterpret_cast<const int4 *>(&end_s[8 * g + 4 * hb]);
+                const int ends[4] = {e4.x, e4.y, e4.z, e4.w};
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const bool vis = kj < ends[r];
+                    const float pr = fast_exp2(fmaf(s[4 * g + r], c2, -l4[r]));
+                    p[r] = vis ? pr : 0.f;
+                    ds[r] = vis ? pr * dp[4 * g + r] : 0.f;
+                }
             }
             const int t = g >> 1, e = 2 * (g & 1);
             pb[t][e] = pack2<T>(p[0], p[1]);

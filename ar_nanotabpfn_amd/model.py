@@ -23,7 +23,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
-from .attention import DenseMask, MultiheadAttention
+from .attention import DenseMask, MultiheadAttention, RowMask
 from .glue import add_layer_norm, bias_gelu, layer_fusable, layer_post, layer_post_pre, layer_pre, pack_weight
 
 __all__ = ["Embedder", "TwoStageTransformerLayer", "TwoStageTransformer", "MixtureGaussianHead", "ARTabPFN"]
@@ -207,12 +207,14 @@ class TwoStageTransformerLayer(nn.Module):
         return self.norm3(x_row + self.ff(x_row)), kv
 
     def forward(self, x: Tensor, mask_features, mask_rows) -> Tuple[Tensor, Tuple[Tensor, Tensor]]:
-        """``[B,R,C,D]`` under a dense mask (the bidirectional context pass) or the training row
-        mask.  While gradients are recorded the layer runs as differentiable modules."""
+        """``[B,R,C,D]`` under a dense mask (the bidirectional context pass, inference only) or the
+        training row mask.  Under the row mask, while gradients are recorded, the layer runs as
+        differentiable modules."""
         B, R, C, D = x.shape
         if C != 1:
             raise NotImplementedError("only the single-column layout (C = 1) is used by this model")
-        if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
+        if (isinstance(mask_rows, RowMask) and torch.is_grad_enabled()
+                and (x.requires_grad or any(p.requires_grad for p in self.parameters()))):
             out, kv = self._forward_recording(x.squeeze(2), mask_rows)
             return out.unsqueeze(2), kv
         x_row = self.feature_stage(x.squeeze(2))

@@ -27,6 +27,8 @@ Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
                                           configs[1], [3] and [4], timings on stderr)
        python bench.py --mix-ceiling     (instead: the instruction mix of one 32x32 score block from
                                           registers: what the SIMD's issue port allows)
+       python bench.py --training-attention  (instead: forward and backward of the training row
+                                          attention at the reference's training shapes)
 """
 
 from __future__ import annotations
@@ -326,6 +328,53 @@ def mix_ceiling(device):
     print(json.dumps({"mix_ceiling": rows}))
 
 
+def training_attention(device):
+    """Forward (with log-sum-exp) and backward of the row attention of one training step at the
+    shapes of the reference's training configuration (configs/train_tabular_online.yaml and the
+    defaults of train.py:44-64: 4 heads of 32, 32 buffer rows, 512 target rows, context 64 or
+    1024, batch 64 or 512), q/k/v as views of one projection output.  Algorithmic flops: 4 Dh per
+    visible (query, key) pair forward, 10 Dh backward (the kernels recompute S and dP in both
+    backward launches: 14 Dh executed)."""
+    import ar_nanotabpfn_amd.attention_kernels as ak
+    from ar_nanotabpfn_amd.attention import RowMask
+
+    H, D, Nb, Nt = 4, 32, 32, 512
+    rows = []
+
+    def timed(fn, n=20):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / n
+
+    for B, Nc in ((64, 64), (64, 1024), (512, 64), (512, 1024)):
+        R, A = Nc + Nb + Nt, Nt // (2 * Nb)
+        g = torch.Generator().manual_seed(0)
+        qkv = (torch.randn(B, R, 3, H, D, generator=g) * 0.7).to(device, torch.bfloat16)
+        q, k, v = (qkv[:, :, i].transpose(1, 2) for i in range(3))
+        dout = (torch.randn(B, R, H, D, generator=g) * 0.7).to(device, torch.bfloat16).transpose(1, 2)
+        pairs = int(RowMask(R, Nc, Nb, A).dense().sum()) * B * H
+        out, lse = ak._row_mask_forward(q, k, v, Nc, Nb, A, True, True)
+        us_f = timed(lambda: ak._row_mask_forward(q, k, v, Nc, Nb, A, True, True))
+        us_b = timed(lambda: ak.row_mask_attention_backward(q, k, v, out, dout, lse, Nc, Nb, A))
+        tensor_bytes = B * H * R * D * 2
+        rows.append(dict(B=B, Nc=Nc, Nb=Nb, Nt=Nt, visible_pairs=pairs, forward_us=round(us_f, 1), backward_us=round(us_b, 1),
+                         forward_tflops=round(4.0 * D * pairs / us_f * 1e-6, 1),
+                         backward_tflops=round(10.0 * D * pairs / us_b * 1e-6, 1),
+                         forward_gbs=round(4 * tensor_bytes / us_f * 1e-3, 1),
+                         backward_gbs=round(8 * tensor_bytes / us_b * 1e-3, 1)))
+        log(f"[training attention] B={B:3d} Nc={Nc:4d} R={R:4d}: forward {us_f:7.1f} us, backward {us_b:7.1f} us "
+            f"({rows[-1]['forward_tflops']} / {rows[-1]['backward_tflops']} TFLOP/s algorithmic, "
+            f"{rows[-1]['forward_gbs']} / {rows[-1]['backward_gbs']} GB/s of tensor bytes)")
+    print(json.dumps({"training_attention": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -342,6 +391,8 @@ def main():
                     help="only copy a 256 MiB buffer five times (reference kernel for scaling HBM counters)")
     ap.add_argument("--mix-ceiling", action="store_true",
                     help="only run the instruction mix of one score block from registers (issue-port ceiling of the kernel)")
+    ap.add_argument("--training-attention", action="store_true",
+                    help="only time forward and backward of the training row attention at the reference's training shapes")
     ap.add_argument("--kernel-shapes", action="store_true",
                     help="only time one decode layer-step at the attention shapes of configs[1], [3], [4]")
     args = ap.parse_args()
@@ -371,6 +422,9 @@ def main():
         return
     if args.mix_ceiling:
         mix_ceiling(torch.device("cuda:0"))
+        return
+    if args.training_attention:
+        training_attention(torch.device("cuda:0"))
         return
     device, dtype = torch.device("cuda:0"), torch.bfloat16
     model = build_model(device, dtype)

@@ -314,12 +314,16 @@ def test_training_step_under_bf16_autocast(device, monkeypatch):
     assert all(np.isfinite(losses)) and losses[-1] < losses[0] - 0.05, losses
 
 
-def test_dense_attention_refuses_to_record_gradients(device):
+def test_dense_attention_refuses_to_backpropagate(device):
+    """The dense (prefill) attention is inference-only: its forward works wherever it is called,
+    a gradient that reaches it raises instead of silently stopping."""
     from ar_nanotabpfn_amd.attention import MultiheadAttention, create_dense_mask
 
     attn = MultiheadAttention(64, 2).to(device=device, dtype=torch.bfloat16)
     x = torch.zeros(1, 8, 64, device=device, dtype=torch.bfloat16)
+    out, _ = attn(x, x, x, create_dense_mask(8, device=device))
     with pytest.raises(NotImplementedError):
-        attn(x, x, x, create_dense_mask(8, device=device))
+        out.float().sum().backward()
     with torch.no_grad():
-        attn(x, x, x, create_dense_mask(8, device=device))
+        out2, _ = attn(x, x, x, create_dense_mask(8, device=device))
+    assert torch.equal(out2, out.detach())
