@@ -190,6 +190,7 @@ __global__ __launch_bounds__(kPortableWaves * 64) void backward_dkv_portable_ker
 
 constexpr int kBackwardWaves = 4;                      // wavefronts per workgroup, 32 rows each
 constexpr int kBackwardRows = 32 * kBackwardWaves;     // query rows (dQ) / key rows (dK, dV) per workgroup
+static_assert(kBackwardWaves == 4, "the four LDS tiles of a workgroup double as one staging tile per wavefront");
 
 // A 32-row tile of a [.,.,rows,DH] tensor, row-major in LDS with a padded row (stride 32 or 96
 // bytes mod 128: what the transposing reads want), filled by the whole workgroup: 16-byte piece
@@ -234,8 +235,39 @@ __device__ __forceinline__ u32x4 backward_row_piece(const View &src, long b, lon
     return *reinterpret_cast<const u32x4 *>(view_row<T>(src, b, h, min(row, R - 1)) + 16 * ks + 8 * hb);
 }
 
+// A wavefront's transposed result (lane = row c of its 32 rows, accumulator registers = columns
+// 8g + 4hb + r of each 32-column block) to rows in global memory, through a wavefront-private LDS
+// tile, so that a row's DH elements leave as 16-byte pieces side by side instead of 8-byte pieces
+// of 32 different rows per store.  (LDS operations of one wavefront execute in order.)
 template <typename T, int DH>
-__global__ __launch_bounds__(kBackwardWaves * 64) void backward_dq_mfma_kernel(BackwardParams P) {
+__device__ __forceinline__ void backward_store_rows(T *tile, const f32x16 (&acc)[DH / 32], float mul, const View &dst,
+                                                    long b, long h, int row0, int R, int lane) {
+    typedef BackwardTile<T, DH> Tile;
+    const int c = lane & 31, hb = lane >> 5;
+#pragma unroll
+    for (int db = 0; db < DH / 32; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            u32x2 o;
+            o[0] = pack2<T>(acc[db][4 * g] * mul, acc[db][4 * g + 1] * mul);
+            o[1] = pack2<T>(acc[db][4 * g + 2] * mul, acc[db][4 * g + 3] * mul);
+            *reinterpret_cast<u32x2 *>(tile + c * Tile::PAD + 32 * db + 8 * g + 4 * hb) = o;
+        }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int pass = 0; pass < Tile::PIECES / 64; ++pass) {
+        const int idx = lane + 64 * pass, row = idx / Tile::CPR, piece = idx % Tile::CPR;
+        const u32x4 val = *reinterpret_cast<const u32x4 *>(tile + row * Tile::PAD + 8 * piece);
+        if (row0 + row < R) *reinterpret_cast<u32x4 *>(view_row<T>(dst, b, h, row0 + row) + 8 * piece) = val;
+    }
+    __builtin_amdgcn_wave_barrier();
+}
+
+// (head_dim 32 is held to 128 registers, four wavefronts per SIMD: measured 6 % faster than the
+// 130 the compiler takes unconstrained; the dK/dV kernel loses 12 % when held to the same)
+template <typename T, int DH>
+__global__ __launch_bounds__(kBackwardWaves * 64) __attribute__((amdgpu_waves_per_eu(DH == 32 ? 4 : 2)))
+void backward_dq_mfma_kernel(BackwardParams P) {
     typedef MfmaOps<T> Ops;
     typedef typename Ops::vec vec;
     typedef BackwardTile<T, DH> Tile;
@@ -344,18 +376,9 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dq_mfma_kernel(B
                 acc[db] = Ops::mma(Tile::col_operand(k_tile, lane, t, db), __builtin_bit_cast(vec, dsb[t]), acc[db]);
     }
 
-    if (qi < P.R) {
-        T *dqrow = view_row<T>(P.dq, b, h, qi);
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                u32x2 o;
-                o[0] = pack2<T>(acc[db][4 * g] * P.scale, acc[db][4 * g + 1] * P.scale);
-                o[1] = pack2<T>(acc[db][4 * g + 2] * P.scale, acc[db][4 * g + 3] * P.scale);
-                *reinterpret_cast<u32x2 *>(dqrow + 32 * db + 8 * g + 4 * hb) = o;
-            }
-    }
+    __syncthreads();  // the tiles are free: one per wavefront stages its rows
+    T *stage = wave < 2 ? k_tiles[wave] : v_tiles[wave - 2];
+    backward_store_rows<T, DH>(stage, acc, P.scale, P.dq, b, h, blk * kBackwardRows + 32 * wave, P.R, lane);
 }
 
 template <typename T, int DH>
@@ -379,6 +402,20 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
     const int kj = key0 + 32 * wave + c;        // this lane's key (column)
     const long stat0 = (b * P.H + h) * static_cast<long>(P.R);
 
+    if (key0 >= P.Nc + P.Nb) {
+        // target keys only: nobody sees them.  Zero rows, 16 bytes per lane, whole rows side by side.
+        constexpr int CPR = Tile::CPR;
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        for (int piece = tid; piece < kBackwardRows * CPR; piece += kBackwardWaves * 64) {
+            const int row = key0 + piece / CPR;
+            if (row < P.R) {
+                *reinterpret_cast<u32x4 *>(view_row<T>(P.dk, b, h, row) + 8 * (piece % CPR)) = zero;
+                *reinterpret_cast<u32x4 *>(view_row<T>(P.dv, b, h, row) + 8 * (piece % CPR)) = zero;
+            }
+        }
+        return;
+    }
+
     vec kf[KS], vf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -394,8 +431,8 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
         for (int v = 0; v < 16; ++v) acc_k[db][v] = acc_v[db][v] = 0.f;
 
     // Queries that can see a key of this workgroup: everybody while it holds a context key, the
-    // rows from the first buffer row on otherwise, nobody when it holds target keys only.
-    const int t_end = key0 < P.Nc + P.Nb ? (P.R + 31) / 32 : 0;
+    // rows from the first buffer row on otherwise.
+    const int t_end = (P.R + 31) / 32;
     const int t_begin = key0 < P.Nc ? 0 : P.Nc / 32;
     u32x4 q_raw = {0u, 0u, 0u, 0u}, g_raw = {0u, 0u, 0u, 0u};
     float st_lse2 = 0.f, st_delta = 0.f;
@@ -491,21 +528,10 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
             }
     }
 
-    if (kj < P.R) {
-        T *dkrow = view_row<T>(P.dk, b, h, kj), *dvrow = view_row<T>(P.dv, b, h, kj);
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                u32x2 ok, ov;
-                ok[0] = pack2<T>(acc_k[db][4 * g] * P.scale, acc_k[db][4 * g + 1] * P.scale);
-                ok[1] = pack2<T>(acc_k[db][4 * g + 2] * P.scale, acc_k[db][4 * g + 3] * P.scale);
-                ov[0] = pack2<T>(acc_v[db][4 * g], acc_v[db][4 * g + 1]);
-                ov[1] = pack2<T>(acc_v[db][4 * g + 2], acc_v[db][4 * g + 3]);
-                *reinterpret_cast<u32x2 *>(dkrow + 32 * db + 8 * g + 4 * hb) = ok;
-                *reinterpret_cast<u32x2 *>(dvrow + 32 * db + 8 * g + 4 * hb) = ov;
-            }
-    }
+    __syncthreads();  // the tiles are free: one per wavefront stages its rows
+    T *stage = wave < 2 ? q_tiles[wave] : g_tiles[wave - 2];
+    backward_store_rows<T, DH>(stage, acc_k, P.scale, P.dk, b, h, key0 + 32 * wave, P.R, lane);
+    backward_store_rows<T, DH>(stage, acc_v, 1.f, P.dv, b, h, key0 + 32 * wave, P.R, lane);
 }
 
 }  // namespace artab
