@@ -265,7 +265,17 @@ def test_training_step_gradients_match_torch_reference(device, monkeypatch):
         assert abs(float(model(xc, yc, xb, yb, xt, *masks, y_target=yt)) - loss_dev) <= 1e-5
 
 
-def test_training_step_under_bf16_autocast(device, monkeypatch):
+@pytest.mark.parametrize(
+    "cfg,B,Nc,Nb,Nt",
+    [
+        (dict(d_model=128, n_heads=4, n_layers=2, d_ff=128, num_features=5, buffer_size=16, num_components=4),
+         4, 200, 16, 96),
+        # the model and batch shape of the reference's configs/train_tabular_online.yaml (12 layers there)
+        (dict(d_model=128, n_heads=4, n_layers=4, d_ff=256, num_features=2, buffer_size=32, num_components=20),
+         8, 64, 32, 512),
+    ],
+)
+def test_training_step_under_bf16_autocast(device, monkeypatch, cfg, B, Nc, Nb, Nt):
     """The reference trains under bf16 autocast (train.py:289-292): q, k, v reach the row attention
     as bf16 and take the matrix-core kernels in both directions.  Parameter gradients against the
     plain PyTorch statement under the same autocast, and a few optimiser steps."""
@@ -273,10 +283,8 @@ def test_training_step_under_bf16_autocast(device, monkeypatch):
     from ar_nanotabpfn_amd.attention import create_dense_mask, create_row_mask
     from ar_nanotabpfn_amd.model import ARTabPFN
 
-    cfg = dict(d_model=128, n_heads=4, n_layers=2, d_ff=128, num_features=5, buffer_size=16, num_components=4)
     torch.manual_seed(0)
     model = ARTabPFN(**cfg).to(device)
-    B, Nc, Nb, Nt = 4, 200, 16, 96
     xc, yc, xb, yb, xt, yt = _training_problem(device, torch.float32, cfg, B, Nc, Nb, Nt)
     masks = (create_dense_mask(1, device=device), create_row_mask(Nc + Nb + Nt, Nc, Nb, device=device))
     calls = []
