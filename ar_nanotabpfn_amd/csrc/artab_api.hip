@@ -935,6 +935,13 @@ int artab_teacher_forcing_attention(const artab_view *q, const artab_view *k_ctx
     return launch_status(launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st), "teacher forcing (mfma)");
 }
 
+// More attending chunks than the target rows can fill change nothing; clamped so that
+// attending_chunks * Nb (the kernels' comparison) stays far from the integer range.
+static int clamp_attending_chunks(int attending_chunks, int R, int Nb) {
+    const int most = R / (Nb > 0 ? Nb : 1) + 1;
+    return attending_chunks < most ? attending_chunks : most;
+}
+
 int artab_row_mask_attention(const artab_view *q, const artab_view *k, const artab_view *v, const artab_view *out,
                              float *lse, int B, int H, int R, int Nc, int Nb, int attending_chunks, int Dh, float scale,
                              int dtype, int impl, void *stream) {
@@ -943,6 +950,7 @@ int artab_row_mask_attention(const artab_view *q, const artab_view *k, const art
         return fail(ARTAB_ERR_BAD_SHAPE, "row mask needs 1 <= Nc, 0 <= Nb, Nc + Nb <= R, attending_chunks >= 0 (got Nc=%d Nb=%d R=%d A=%d)",
                     Nc, Nb, R, attending_chunks);
     if (B == 0 || R == 0) return ARTAB_OK;
+    attending_chunks = clamp_attending_chunks(attending_chunks, R, Nb);
     ARTAB_TRY(check_view(q, "q", dtype, true));
     ARTAB_TRY(check_view(k, "k", dtype, true));
     ARTAB_TRY(check_view(v, "v", dtype, true));
@@ -1000,6 +1008,7 @@ int artab_row_mask_attention_backward(const artab_view *q, const artab_view *k, 
         aligned = aligned && vec_aligned(views[i], dtype, Dh);
     }
     if (!lse || !delta) return fail(ARTAB_ERR_NULL_POINTER, "lse and delta must be given");
+    attending_chunks = clamp_attending_chunks(attending_chunks, R, Nb);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool use_mfma = impl != ARTAB_IMPL_PORTABLE && (dtype == ARTAB_BF16 || dtype == ARTAB_F16) &&
                           (Dh == 32 || Dh == 64) && aligned;

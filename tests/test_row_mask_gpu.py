@@ -335,3 +335,20 @@ def test_dense_attention_refuses_to_backpropagate(device):
     with torch.no_grad():
         out2, _ = attn(x, x, x, create_dense_mask(8, device=device))
     assert torch.equal(out2, out.detach())
+
+
+def test_row_mask_attending_chunks_beyond_the_targets(device):
+    """More attending chunks than there are target rows (up to the largest int) mean "every chunk
+    attends": same output and gradients as the exact count."""
+    import ar_nanotabpfn_amd.attention_kernels as ak
+
+    B, H, D, Nc, Nb, T = 2, 2, 32, 40, 8, 64
+    R = Nc + Nb + T
+    q, k, v, dout = (randn((B, H, R, D), s, torch.bfloat16, 0.7).to(device) for s in (1, 2, 3, 4))
+    want, lse = ak._row_mask_forward(q, k, v, Nc, Nb, T // Nb, True, want_lse=True)
+    grads = ak.row_mask_attention_backward(q, k, v, want, dout, lse, Nc, Nb, T // Nb)
+    for chunks in (T // Nb + 5, 2 ** 31 - 1):
+        out, lse2 = ak._row_mask_forward(q, k, v, Nc, Nb, chunks, True, want_lse=True)
+        assert torch.equal(out, want) and torch.equal(lse2, lse)
+        for g, w in zip(ak.row_mask_attention_backward(q, k, v, out, dout, lse2, Nc, Nb, chunks), grads):
+            assert torch.equal(g, w)
