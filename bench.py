@@ -372,7 +372,70 @@ def training_attention(device):
         log(f"[training attention] B={B:3d} Nc={Nc:4d} R={R:4d}: forward {us_f:7.1f} us, backward {us_b:7.1f} us "
             f"({rows[-1]['forward_tflops']} / {rows[-1]['backward_tflops']} TFLOP/s algorithmic, "
             f"{rows[-1]['forward_gbs']} / {rows[-1]['backward_gbs']} GB/s of tensor bytes)")
-    print(json.dumps({"training_attention": rows}))
+    step = training_step(device)
+    print(json.dumps({"training_attention": rows, "training_step": step}))
+
+
+def training_step(device):
+    """One optimiser step of the reference's training configuration (configs/train_tabular_online.yaml:
+    12 layers, d_model 128, 4 heads, d_ff 256, 20 mixture components; batch 64 of 64 context + 32
+    buffer + 512 target rows; bf16 autocast, AdamW, gradient clipping at 1.0 as in train.py:289-310)
+    with the row attention on the device kernels in both directions, and the same step with the row
+    attention as PyTorch's scaled_dot_product_attention under the dense boolean mask."""
+    import torch.nn.functional as F
+
+    import ar_nanotabpfn_amd.attention_kernels as ak
+    from ar_nanotabpfn_amd.attention import RowMask, create_dense_mask, create_row_mask
+    from ar_nanotabpfn_amd.model import ARTabPFN
+
+    cfg = dict(d_model=128, n_heads=4, n_layers=12, d_ff=256, num_features=2, buffer_size=32, num_components=20)
+    B, Nc, Nb, Nt = 64, 64, 32, 512
+    torch.manual_seed(0)
+    model = ARTabPFN(**cfg).to(device)
+    opt = torch.optim.AdamW(model.parameters(), lr=1e-3, betas=(0.9, 0.95), weight_decay=0.0)
+    g = torch.Generator().manual_seed(1)
+    mk = lambda *s: torch.randn(*s, generator=g).to(device)  # noqa: E731
+    data = (mk(B, Nc, 2), mk(B, Nc), mk(B, Nb, 2), mk(B, Nb), mk(B, Nt, 2))
+    y_t = mk(B, Nt)
+    masks = (create_dense_mask(1, device=device), create_row_mask(Nc + Nb + Nt, Nc, Nb, device=device))
+
+    def sdpa_row_attention(q, k, v, context_len, buffer_len, attending_chunks, use_triton=True):
+        mask = RowMask(q.shape[2], context_len, buffer_len, attending_chunks).dense(q.device)
+        return F.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+
+    def one_step():
+        opt.zero_grad(set_to_none=True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            loss = model(*data, *masks, y_target=y_t)
+        loss.backward()
+        torch.nn.utils.clip_grad_norm_(model.parameters(), 1.0)
+        opt.step()
+        return loss
+
+    def timed(n=10):
+        for _ in range(3):
+            one_step()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            loss = one_step()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n, loss.item()
+
+    ms_dev, loss_dev = timed()
+    device_attention = ak.row_mask_attention
+    ak.row_mask_attention = sdpa_row_attention
+    try:
+        ms_ref, loss_ref = timed()
+    finally:
+        ak.row_mask_attention = device_attention
+    log(f"[training step] 12 layers, B={B}, rows {Nc}+{Nb}+{Nt}, bf16 autocast + AdamW: {ms_dev:.2f} ms per step with the "
+        f"device row attention, {ms_ref:.2f} ms with scaled_dot_product_attention under the dense mask")
+    return dict(config="train_tabular_online.yaml", B=B, Nc=Nc, Nb=Nb, Nt=Nt, ms_per_step=round(ms_dev, 3),
+                ms_per_step_sdpa_dense_mask=round(ms_ref, 3), loss_after=round(loss_dev, 4),
+                loss_after_sdpa=round(loss_ref, 4))
 
 
 def main():
