@@ -312,8 +312,8 @@ void backward_dq_mfma_kernel(BackwardParams P) {
 
     // every workgroup walks the keys anybody can see; what its own rows do not see is masked
     const int n_tiles = (P.Nc + P.Nb + 31) / 32;
-    // tile kt + 1 goes to LDS at the start of round kt (it was requested a round earlier), tile
-    // kt + 2 is requested then: one barrier per tile, a whole round to cover the round trip
+    // tile kt + 1 goes to LDS at the start of iteration kt (it was requested one iteration earlier), tile
+    // kt + 2 is requested then: one barrier per tile, a whole iteration to cover the memory round trip
     u32x4 k_raw = Tile::fetch(P.k, b, h, 0, P.R, tid), v_raw = Tile::fetch(P.v, b, h, 0, P.R, tid);
     Tile::stash(k_tiles[0], tid, k_raw);
     Tile::stash(v_tiles[0], tid, v_raw);
@@ -456,7 +456,7 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
             end_t[slot][tid] = st_end;
         }
     };
-    // as in the dQ kernel: tile qt + 1 goes to LDS at the start of round qt, tile qt + 2 is requested then
+    // as in the dQ kernel: tile qt + 1 goes to LDS at the start of iteration qt, tile qt + 2 is requested then
     if (t_begin < t_end) {
         fetch(t_begin);
         stash(0);
