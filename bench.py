@@ -29,6 +29,9 @@ Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
                                           registers: what the SIMD's issue port allows)
        python bench.py --training-attention  (instead: forward and backward of the training row
                                           attention at the reference's training shapes)
+       python bench.py --training-step   (instead: one optimiser step of the reference's training
+                                          configuration; launches from autograd's worker thread —
+                                          not for runs under rocprofv3 --pmc)
 """
 
 from __future__ import annotations
@@ -372,8 +375,7 @@ def training_attention(device):
         log(f"[training attention] B={B:3d} Nc={Nc:4d} R={R:4d}: forward {us_f:7.1f} us, backward {us_b:7.1f} us "
             f"({rows[-1]['forward_tflops']} / {rows[-1]['backward_tflops']} TFLOP/s algorithmic, "
             f"{rows[-1]['forward_gbs']} / {rows[-1]['backward_gbs']} GB/s of tensor bytes)")
-    step = training_step(device)
-    print(json.dumps({"training_attention": rows, "training_step": step}))
+    print(json.dumps({"training_attention": rows}))
 
 
 def training_step(device):
@@ -433,9 +435,9 @@ def training_step(device):
         ak.row_mask_attention = device_attention
     log(f"[training step] 12 layers, B={B}, rows {Nc}+{Nb}+{Nt}, bf16 autocast + AdamW: {ms_dev:.2f} ms per step with the "
         f"device row attention, {ms_ref:.2f} ms with scaled_dot_product_attention under the dense mask")
-    return dict(config="train_tabular_online.yaml", B=B, Nc=Nc, Nb=Nb, Nt=Nt, ms_per_step=round(ms_dev, 3),
-                ms_per_step_sdpa_dense_mask=round(ms_ref, 3), loss_after=round(loss_dev, 4),
-                loss_after_sdpa=round(loss_ref, 4))
+    print(json.dumps({"training_step": dict(
+        config="train_tabular_online.yaml", B=B, Nc=Nc, Nb=Nb, Nt=Nt, ms_per_step=round(ms_dev, 3),
+        ms_per_step_sdpa_dense_mask=round(ms_ref, 3), loss_after=round(loss_dev, 4), loss_after_sdpa=round(loss_ref, 4))}))
 
 
 def main():
@@ -456,6 +458,8 @@ def main():
                     help="only run the instruction mix of one score block from registers (issue-port ceiling of the kernel)")
     ap.add_argument("--training-attention", action="store_true",
                     help="only time forward and backward of the training row attention at the reference's training shapes")
+    ap.add_argument("--training-step", action="store_true",
+                    help="only time one optimiser step of the reference's training configuration")
     ap.add_argument("--kernel-shapes", action="store_true",
                     help="only time one decode layer-step at the attention shapes of configs[1], [3], [4]")
     args = ap.parse_args()
@@ -488,6 +492,9 @@ def main():
         return
     if args.training_attention:
         training_attention(torch.device("cuda:0"))
+        return
+    if args.training_step:
+        training_step(torch.device("cuda:0"))
         return
     device, dtype = torch.device("cuda:0"), torch.bfloat16
     model = build_model(device, dtype)
