@@ -192,15 +192,22 @@ constexpr int kBackwardWaves = 4;                      // wavefronts per workgro
 constexpr int kBackwardRows = 32 * kBackwardWaves;     // query rows (dQ) / key rows (dK, dV) per workgroup
 static_assert(kBackwardWaves == 4, "the four LDS tiles of a workgroup double as one staging tile per wavefront");
 
-// A 32-row tile of a [.,.,rows,DH] tensor, row-major in LDS with a padded row (stride 32 or 96
-// bytes mod 128: what the transposing reads want), filled by the whole workgroup: 16-byte piece
-// `tid` (row tid / CPR, piece tid % CPR); rows past the end re-read the last row (finite values
-// that the mask keeps out of every result).
+// A 32-row tile of a [.,.,rows,DH] tensor in LDS, filled by the whole workgroup (16-byte piece
+// `tid`: row tid / CPR, piece tid % CPR; rows past the end re-read the last row: finite values that
+// the mask keeps out of every result).  Layout: blocks of 16 columns, each block 32 rows of
+// 32 bytes side by side (1 KiB).  Both kinds of operand reads are then free of bank conflicts: a
+// row operand (lane = row c, half hb of the block) is 64 lanes x 16 bytes in one contiguous KiB,
+// and the 16 lanes that a transposing read combines (4 rows x 4 groups of 4 columns) cover 128
+// contiguous bytes.  (With padded whole rows, 96 bytes apart at head_dim 32, a third to a half of
+// the LDS cycles of these kernels were bank conflicts; removing them was worth 1 %: the LDS pipe
+// is not what the kernels wait for.)  The array is sized for the padded form, which the epilogue
+// still uses to stage results (backward_store_rows).
 template <typename T, int DH>
 struct BackwardTile {
     static constexpr int PAD = DH + 16;
     static constexpr int CPR = DH / 8;
     static constexpr int PIECES = 32 * CPR;  // <= 256 = threads of the workgroup
+    static constexpr int BLOCK = 32 * 16;    // elements of a 16-column block
     static __device__ __forceinline__ u32x4 fetch(const View &src, long b, long h, int row0, int R, int tid) {
         u32x4 raw = {0u, 0u, 0u, 0u};
         if (tid < PIECES)
@@ -208,21 +215,24 @@ struct BackwardTile {
         return raw;
     }
     static __device__ __forceinline__ void stash(T *tile, int tid, const u32x4 &raw) {
-        if (tid < PIECES) *reinterpret_cast<u32x4 *>(tile + (tid / CPR) * PAD + 8 * (tid % CPR)) = raw;
+        const int row = tid / CPR, piece = tid % CPR;
+        if (tid < PIECES) *reinterpret_cast<u32x4 *>(tile + (piece >> 1) * BLOCK + row * 16 + 8 * (piece & 1)) = raw;
     }
     // operand of a product contracted over head_dim, for the lane's row c: 8 elements at 16 ks + 8 hb
     static __device__ __forceinline__ typename MfmaOps<T>::vec row_operand(const T *tile, int c, int hb, int ks) {
         return __builtin_bit_cast(typename MfmaOps<T>::vec,
-                                  *reinterpret_cast<const u32x4 *>(tile + c * PAD + 16 * ks + 8 * hb));
+                                  *reinterpret_cast<const u32x4 *>(tile + ks * BLOCK + c * 16 + 8 * hb));
     }
     // operand of a product contracted over the tile's rows (step t: rows 16 t .. 16 t + 15 in the
-    // enumeration of an accumulator used as the other operand), for output dimension 32 db + c
+    // enumeration of an accumulator used as the other operand), for output dimension 32 db + c:
+    // the lane hands the transposing read four consecutive elements of row 4 hb + (lane % 16) / 4
+    // (+ 8 for the second read) at column 16 ((lane / 16) % 2) + 4 (lane % 4) of the 32-column block
     static __device__ __forceinline__ typename MfmaOps<T>::vec col_operand(const T *tile, int lane, int t, int db) {
         const int hb = lane >> 5;
-        const int rd = (4 * hb + ((lane & 15) >> 2)) * PAD + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-        const T *p = tile + (16 * t) * PAD + 32 * db + rd;
+        const int row = 16 * t + 4 * hb + ((lane & 15) >> 2);
+        const T *p = tile + (2 * db + ((lane >> 4) & 1)) * BLOCK + row * 16 + 4 * (lane & 3);
         s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(p));
-        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(p + 8 * PAD));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(p + 8 * 16));
         typedef short s16x8 __attribute__((ext_vector_type(8)));
         s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         return __builtin_bit_cast(typename MfmaOps<T>::vec, both);
