@@ -295,6 +295,7 @@ void backward_dq_mfma_kernel(BackwardParams P) {
 
     vec qf[KS], gf[KS];
     float part = 0.f;
+    const float c2 = P.scale * kLog2e;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         const u32x4 qr = backward_row_piece<T>(P.q, b, h, qi, P.R, ks, hb);
@@ -305,12 +306,17 @@ void backward_dq_mfma_kernel(BackwardParams P) {
             part = fmaf(unpack_lo<T>(gr[e]), unpack_lo<T>(orw[e]), part);
             part = fmaf(unpack_hi<T>(gr[e]), unpack_hi<T>(orw[e]), part);
         }
-        qf[ks] = __builtin_bit_cast(vec, qr);
+        // scale * log2(e) folded into the queries and rounded to the input type, as the forward
+        // does (the rounding model of the reference kernel, triton_kernels.py:120-121): the scores
+        // come out of the matrix pipe in base-2 units and P is the forward's P
+        u32x4 sc;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sc[e] = pack2<T>(unpack_lo<T>(qr[e]) * c2, unpack_hi<T>(qr[e]) * c2);
+        qf[ks] = __builtin_bit_cast(vec, sc);
         gf[ks] = __builtin_bit_cast(vec, gr);
     }
     const float delta = part + __shfl_xor(part, 32, 64);
     const float lse2 = P.lse[stat] * kLog2e;
-    const float c2 = P.scale * kLog2e;
     const int vis_end = backward_vis_end(P, qi);
     if (qi < P.R && hb == 0) P.delta[stat] = delta;
 
@@ -342,7 +348,8 @@ void backward_dq_mfma_kernel(BackwardParams P) {
                 v_raw = Tile::fetch(P.v, b, h, 32 * (kt + 2), P.R, tid);
             }
         }
-        f32x16 s, dp;  // dp starts at -delta: the product leaves dP - delta
+        f32x16 s, dp;  // dp starts at -delta: the product leaves dP - delta.  (Starting s at -lse2
+                       // as well costs 16 more registers than four wavefronts per SIMD leave: measured slower.)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             s[v] = 0.f;
@@ -361,8 +368,7 @@ void backward_dq_mfma_kernel(BackwardParams P) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int v = 8 * t + 2 * e;
-                    dsb[t][e] = pack2<T>(fast_exp2(fmaf(s[v], c2, -lse2)) * dp[v],
-                                         fast_exp2(fmaf(s[v + 1], c2, -lse2)) * dp[v + 1]);
+                    dsb[t][e] = pack2<T>(fast_exp2(s[v] - lse2) * dp[v], fast_exp2(s[v + 1] - lse2) * dp[v + 1]);
                 }
         } else {
 #pragma unroll
@@ -374,7 +380,7 @@ void backward_dq_mfma_kernel(BackwardParams P) {
                     for (int x = 0; x < 2; ++x) {
                         const int v = 8 * t + 2 * e + x;
                         const bool vis = 32 * kt + 8 * (v >> 2) + 4 * hb + (v & 3) < vis_end;
-                        ds[x] = vis ? fast_exp2(fmaf(s[v], c2, -lse2)) * dp[v] : 0.f;
+                        ds[x] = vis ? fast_exp2(s[v] - lse2) * dp[v] : 0.f;
                     }
                     dsb[t][e] = pack2<T>(ds[0], ds[1]);
                 }
@@ -427,12 +433,18 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
     }
 
     vec kf[KS], vf[KS];
+    const float c2 = P.scale * kLog2e;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-        kf[ks] = __builtin_bit_cast(vec, backward_row_piece<T>(P.k, b, h, kj, P.R, ks, hb));
+        // scale * log2(e) folded into the keys (this kernel's register operand) and rounded to the
+        // input type: scores in base-2 units straight from the matrix pipe
+        const u32x4 kr = backward_row_piece<T>(P.k, b, h, kj, P.R, ks, hb);
+        u32x4 sc;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sc[e] = pack2<T>(unpack_lo<T>(kr[e]) * c2, unpack_hi<T>(kr[e]) * c2);
+        kf[ks] = __builtin_bit_cast(vec, sc);
         vf[ks] = __builtin_bit_cast(vec, backward_row_piece<T>(P.v, b, h, kj, P.R, ks, hb));
     }
-    const float c2 = P.scale * kLog2e;
 
     f32x16 acc_k[DB], acc_v[DB];
 #pragma unroll
@@ -452,8 +464,8 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
         g_raw = Tile::fetch(P.dout, b, h, 32 * qt, P.R, tid);
         if (tid < 32) {
             const int i = 32 * qt + tid;
-            st_lse2 = P.lse[stat0 + min(i, P.R - 1)] * kLog2e;
-            st_delta = P.delta[stat0 + min(i, P.R - 1)];
+            st_lse2 = -P.lse[stat0 + min(i, P.R - 1)] * kLog2e;  // negated: the accumulators start from them
+            st_delta = -P.delta[stat0 + min(i, P.R - 1)];
             st_end = backward_vis_end(P, i);
         }
     };
@@ -482,16 +494,17 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
             stash(slot ^ 1);
             if (qt + 2 < t_end) fetch(qt + 2);
         }
-        // rows of the accumulators are queries 8g + 4hb + r of the tile: their statistics come from
-        // LDS; dp starts at -delta of its row, so that the product leaves dP - delta
+        // rows of the accumulators are queries 8g + 4hb + r of the tile: the accumulators start at
+        // -lse2 and -delta of their rows, read from LDS, so that the products leave log2 P and dP - delta
         f32x16 s, dp;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
+            const f32x4 l4 = *reinterpret_cast<const f32x4 *>(&lse2_s[8 * g + 4 * hb]);
             const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&delta_s[8 * g + 4 * hb]);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                s[4 * g + r] = 0.f;
-                dp[4 * g + r] = -d4[r];
+                s[4 * g + r] = l4[r];
+                dp[4 * g + r] = d4[r];
             }
         }
 #pragma unroll
@@ -504,12 +517,11 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
         const bool all_visible = key0 + 32 * wave + 32 <= P.Nc && 32 * qt + 32 <= P.R;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            const f32x4 l4 = *reinterpret_cast<const f32x4 *>(&lse2_s[8 * g + 4 * hb]);
             float p[4], ds[4];
             if (all_visible) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    p[r] = fast_exp2(fmaf(s[4 * g + r], c2, -l4[r]));
+                    p[r] = fast_exp2(s[4 * g + r]);
                     ds[r] = p[r] * dp[4 * g + r];
                 }
             } else {
@@ -518,7 +530,7 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const bool vis = kj < ends[r];
-                    const float pr = fast_exp2(fmaf(s[4 * g + r], c2, -l4[r]));
+                    const float pr = fast_exp2(s[4 * g + r]);
                     p[r] = vis ? pr : 0.f;
                     ds[r] = vis ? pr * dp[4 * g + r] : 0.f;
                 }
