@@ -285,7 +285,7 @@ void backward_dq_mfma_kernel(BackwardParams P) {
     __shared__ __attribute__((aligned(16))) T k_tiles[2][32 * Tile::PAD];  // two tiles in turn: one barrier per tile
     __shared__ __attribute__((aligned(16))) T v_tiles[2][32 * Tile::PAD];
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hb = lane >> 5;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, c = lane & 31, hb = lane >> 5;
     const int blocks = (P.R + kBackwardRows - 1) / kBackwardRows;
     const int blk = blockIdx.x % blocks;
     const int h = (blockIdx.x / blocks) % P.H;
@@ -409,7 +409,7 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
     __shared__ __attribute__((aligned(16))) float delta_t[2][32];
     __shared__ __attribute__((aligned(16))) int end_t[2][32];
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, hb = lane >> 5;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, c = lane & 31, hb = lane >> 5;
     const int blocks = (P.R + kBackwardRows - 1) / kBackwardRows;
     const int blk = blockIdx.x % blocks;
     const int h = (blockIdx.x / blocks) % P.H;
@@ -513,20 +513,30 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
             dp = Ops::mma(Tile::row_operand(g_tile, c, hb, ks), vf[ks], dp);
         }
         u32x4 pb[2], dsb[2];
-        // context keys under a full tile of rows: everything is visible (wave-uniform)
-        const bool all_visible = key0 + 32 * wave + 32 <= P.Nc && 32 * qt + 32 <= P.R;
+        // context keys under a full tile of rows: everything is visible.  One wavefront-uniform
+        // branch around the whole block (`wave` is a scalar: the compiler must not turn the two
+        // paths into lane masks and issue the exponentials of both).
+        if (key0 + 32 * wave + 32 <= P.Nc && 32 * qt + 32 <= P.R) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            float p[4], ds[4];
-            if (all_visible) {
+            for (int g = 0; g < 4; ++g) {
+                float p[4], ds[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     p[r] = fast_exp2(s[4 * g + r]);
                     ds[r] = p[r] * dp[4 * g + r];
                 }
-            } else {
+                const int t = g >> 1, e = 2 * (g & 1);
+                pb[t][e] = pack2<T>(p[0], p[1]);
+                pb[t][e + 1] = pack2<T>(p[2], p[3]);
+                dsb[t][e] = pack2<T>(ds[0], ds[1]);
+                dsb[t][e + 1] = pack2<T>(ds[2], ds[3]);
+            }
+        } else {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
                 const int4 e4 = *reinterpret_cast<const int4 *>(&end_s[8 * g + 4 * hb]);
                 const int ends[4] = {e4.x, e4.y, e4.z, e4.w};
+                float p[4], ds[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const bool vis = kj < ends[r];
@@ -534,12 +544,12 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
                     p[r] = vis ? pr : 0.f;
                     ds[r] = vis ? pr * dp[4 * g + r] : 0.f;
                 }
+                const int t = g >> 1, e = 2 * (g & 1);
+                pb[t][e] = pack2<T>(p[0], p[1]);
+                pb[t][e + 1] = pack2<T>(p[2], p[3]);
+                dsb[t][e] = pack2<T>(ds[0], ds[1]);
+                dsb[t][e + 1] = pack2<T>(ds[2], ds[3]);
             }
-            const int t = g >> 1, e = 2 * (g & 1);
-            pb[t][e] = pack2<T>(p[0], p[1]);
-            pb[t][e + 1] = pack2<T>(p[2], p[3]);
-            dsb[t][e] = pack2<T>(ds[0], ds[1]);
-            dsb[t][e + 1] = pack2<T>(ds[2], ds[3]);
         }
 #pragma unroll
         for (int db = 0; db < DB; ++db)
