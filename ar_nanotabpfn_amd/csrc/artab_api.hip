@@ -697,6 +697,11 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
         const long rows = fit > kStreamShortRows ? fit : kStreamShortRows;
         D.stream_short_rows = env_int("ARTAB_STREAM_SHORT", static_cast<int>(rows < 1 << 20 ? rows : 1 << 20));  // env: tuning hook
     }
+    if (side_stream && side_stream != stream) {  // the two passes share the compute units
+        F.beside_rows = n_buf_device;
+        F.beside_n = n_buf;
+        F.dense_below = env_int("ARTAB_DENSE_BELOW", 128);  // env: tuning hook
+    }
     D.buf_part_o = static_cast<char *>(workspace) + static_cast<size_t>(pl.n_split) * rows * Dh * 2;
     D.buf_part_lse = F.part_lse + static_cast<size_t>(pl.n_split) * rows;
     hipStream_t side = (side_stream && side_stream != stream) ? static_cast<hipStream_t>(side_stream) : st;

@@ -98,6 +98,15 @@ struct FlashParams {
     int mode;
     int rm_nc, rm_attend;  // row-mask mode: context rows in front of the Nb buffer rows, attending chunks
     int force_robust;  // 1: skip the fast path (testing the online-softmax path)
+    // A buffer pass runs beside this launch on the same compute units and streams `beside_rows`
+    // rows per pair (read from device memory, or `beside_n` when the pointer is null).  From
+    // `dense_below` rows on the context pass leaves the straight-line form of its tile loop alone
+    // (0: no limit): measured at B=1024, H=8, N_ctx=16384 the straight-line form is 3 % faster alone
+    // and worth 1.9 % of a decode step beside a short buffer pass; beside a long one the context
+    // pass waits for its tiles behind the streaming loads either way and the denser issue only
+    // takes slots from the buffer pass (256 steps: +0.3 % with the limit at 128 rows, 0 without).
+    const int *beside_rows;
+    int beside_n, dense_below;
     unsigned *started;  // optional counter that the first thread of the grid advances at once: "the
                         // launches ahead of this one on its queue are complete" for a watcher on
                         // another queue (queue_order.h); the kernel's own work does not depend on it
@@ -938,6 +947,8 @@ void flash_kernel(FlashParams P) {
         };
 
         __builtin_amdgcn_s_setprio(3);
+        // (read here, in front of the prologue's requests: where it is used the loop would wait for it)
+        const int beside_now = P.dense_below > 0 && P.beside_rows ? *P.beside_rows : P.beside_n;
         {
             // the first three tiles are requested together with the queries: full tiles by direct
             // loads into their stages, a ragged or buffer tile among the first two through registers
@@ -961,6 +972,64 @@ void flash_kernel(FlashParams P) {
         // with nothing but full context tiles the whole slice is steady state; otherwise the last
         // two full tiles have to request tiles of the other kind and take the general route
         const int n_steady = n_tiles == n_main ? n_main : n_main - 2;
+        // The bulk of a long slice: groups of four full tiles that each have three full tiles
+        // behind them.  Nothing about such a tile depends on its index — the wait is for a constant
+        // number of direct loads, the request three ahead is unconditional — so the group is
+        // straight-line code (the general steady tile below spends a dozen scalar branches on
+        // these decisions); the priority steps sit between groups, at multiples of four.
+        const int n_fast = n_main >= 12 ? ((n_steady < n_main - 3 ? n_steady : n_main - 3) & ~3) : 0;
+        bool dense = n_fast > 0;
+        if (dense && P.dense_below > 0)  // (a scalar: the choice must stay a wavefront-uniform branch)
+            dense = __builtin_amdgcn_readfirstlane(beside_now) < P.dense_below;
+        if (dense) {
+            const bool two = n_dma == 2;  // direct loads of this wavefront per tile: one or two
+            auto fast_tile = [&](auto stage_) {
+                // this tile's loads have landed, those of the next two tiles may be under way
+                if (two)
+                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(4));
+                else
+                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(2));
+                __syncthreads();
+                constexpr int into = (decltype(stage_)::value + 3) % 4;
+#pragma unroll
+                for (int r = 0; r < NR; ++r) {
+                    if (r == 0 || two) {
+                        const unsigned m0v = lds_base + into * STAGE_BYTES + (wave + NW * r) * 1024;
+                        unsigned m0_saved;
+                        asm volatile(
+                            "s_mov_b32 %0, m0\n\t"
+                            "s_mov_b32 m0, %1\n\t"
+                            "global_load_lds_dwordx4 %2, %3\n\t"
+                            "s_mov_b32 m0, %0"
+                            : "=&s"(m0_saved)
+                            : "s"(m0v), "v"(d_off[r]), "s"(d_src[r]));
+                    }
+                    d_src[r] += d_step[r];
+                }
+#pragma unroll
+                for (int sb = 0; sb < SB; ++sb) block(stage_, sb, BoolTag<false>{}, 0, true, 0);
+            };
+            // the priority falls with progress (see the general steady tile): steps between groups
+            const int q1 = (n_main / 4) & ~3, q2 = (n_main / 2) & ~3, q3 = (3 * n_main / 4) & ~3;
+#pragma nounroll
+            for (int part = 0; part < 4; ++part) {
+                int end = part == 0 ? q1 : part == 1 ? q2 : part == 2 ? q3 : n_fast;
+                end = end < n_fast ? end : n_fast;
+#pragma nounroll
+                for (; it < end; it += 4) {
+                    fast_tile(std::integral_constant<int, 0>{});
+                    fast_tile(std::integral_constant<int, 1>{});
+                    fast_tile(std::integral_constant<int, 2>{});
+                    fast_tile(std::integral_constant<int, 3>{});
+                }
+                if (part == 0 && it == q1)
+                    __builtin_amdgcn_s_setprio(2);
+                else if (part == 1 && it == q2)
+                    __builtin_amdgcn_s_setprio(1);
+                else if (part == 2 && it == q3)
+                    __builtin_amdgcn_s_setprio(0);
+            }
+        }
         while (it < n_steady) {  // stages as compile-time constants: every LDS offset is an immediate
             tile(it, std::integral_constant<int, 0>{}, BoolTag<true>{});
             if (++it >= n_steady) break;
