@@ -228,7 +228,7 @@ def log_density_bench(device, dtype, model, with_cpu):
 # Measured with rocprofv3 (median over the decode launches): 10337.7 KiB x 2.0 fetched,
 # 14336.0 KiB written (the partial outputs leave in 16-bit, their LSE in fp32; about 3 MB read and
 # 6 MB written are the registers the kernel's prologue parks in scratch memory).
-CONTEXT_PASS_HBM_BYTES = int(10337.7 * 1024 * 2.0 + 14336.0 * 1024)
+CONTEXT_PASS_HBM_BYTES = int(9339.5 * 1024 * 2.0 + 10240.0 * 1024)
 
 
 def kernel_shapes(device):
