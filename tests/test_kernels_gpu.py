@@ -360,6 +360,29 @@ def test_decode_attention_config3_full_size(device, n_buf):
     _full_size_decode(device, 1024, 8, 16384, n_buf, 256, seed=3 + n_buf)
 
 
+def test_context_pass_tile_loop_forms_agree_bit_for_bit(device, monkeypatch):
+    """Beside a buffer pass the context pass runs the bulk of its tile loop as straight-line code
+    while the committed buffer is short and tile by tile beyond (``ARTAB_DENSE_BELOW`` rows, read
+    with the length on the device): the same products in the same order, so the partial slots are
+    identical whichever form ran (configs[3] shape, 37 buffer rows, limit forced to either side)."""
+    ak = _ak()
+    B, H, Nc, D, Lq, n_buf, cap = 1024, 8, 16384, 32, 2, 37, 64
+    g = torch.Generator(device=device).manual_seed(21)
+    draw = lambda *shape: (torch.randn(*shape, generator=g, device=device) * 0.6).to(torch.bfloat16)  # noqa: E731
+    q, k_ctx, v_ctx = draw(B, H, Lq, D), draw(H, Nc, D), draw(H, Nc, D)
+    k_cache, v_cache, k_new, v_new = draw(B, H, cap, D), draw(B, H, cap, D), draw(B, H, 1, D), draw(B, H, 1, D)
+    nbuf = torch.tensor([n_buf], device=device, dtype=torch.int32)
+    side = torch.cuda.Stream(device=device)
+    outs = []
+    for limit in ("1", "100000"):
+        monkeypatch.setenv("ARTAB_DENSE_BELOW", limit)
+        parts = ak.decode_attention(q, k_ctx, v_ctx, k_cache.clone(), v_cache.clone(), cap - 1, k_new, v_new,
+                                    side_stream=side, leave_partials=True, n_buf_device=nbuf)
+        outs.append(parts.merged())
+        torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1])
+
+
 @pytest.mark.parametrize("n_buf", [1, 130, 255])
 def test_decode_attention_config4_full_size(device, n_buf):
     """BASELINE configs[4] layer-step: B=2048 trajectories, 16 heads, N_ctx=4096, buffer up to 256."""
