@@ -237,25 +237,28 @@ void flash_kernel(FlashParams P) {
         for (int j = 0; j < QB; ++j) {
             const T *qrow = view_row<T>(P.q, qb[j], h, qi[j] >= 0 ? qi[j] : 0) + 8 * hb;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                qraw[j][ks] = u32x4{0u, 0u, 0u, 0u};
-                if (qi[j] >= 0) qraw[j][ks] = *reinterpret_cast<const u32x4 *>(qrow + 16 * ks);
-            }
+            // unconditional: a column past the last row re-reads the group's first row (a valid
+            // address) and is zeroed when it is scaled.  A load under a lane mask, merged with
+            // zeros, made the compiler wait for the queries right here, a memory round trip in
+            // front of the first tile requests.
+            for (int ks = 0; ks < KS; ++ks) qraw[j][ks] = *reinterpret_cast<const u32x4 *>(qrow + 16 * ks);
         }
     };
     bool q_scaled = false;
     auto scale_q = [&](const u32x4(&qraw)[QB][KS]) {
         q_scaled = true;
 #pragma unroll
-        for (int j = 0; j < QB; ++j)
+        for (int j = 0; j < QB; ++j) {
+            const float qs = qi[j] >= 0 ? P.qscale : 0.f;  // columns past the last row carry zero queries
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 u32x4 sc;
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    sc[e] = pack2<T>(unpack_lo<T>(qraw[j][ks][e]) * P.qscale, unpack_hi<T>(qraw[j][ks][e]) * P.qscale);
+                    sc[e] = pack2<T>(unpack_lo<T>(qraw[j][ks][e]) * qs, unpack_hi<T>(qraw[j][ks][e]) * qs);
                 qreg[j][ks] = __builtin_bit_cast(vec, sc);
             }
+        }
     };
 
     // ---- prefill: this tile's own K/V rows go to the cache.
