@@ -46,11 +46,12 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodePa
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int c = lane & 31, hb = lane >> 5;
 
-    // what phase 2 needs from global memory is requested first: its round trips (the buffer rows
-    // come from HBM) run under phase 1
+    // what phase 2 needs from global memory is requested early, so that its round trips (the
+    // buffer rows come from HBM) run under phase 1 — but behind the queries and the first two
+    // context blocks: loads return in the order they were requested, and the first product must
+    // not wait for the buffer rows
     const long b2 = b0 + wave;
     BufferHead<T, DH, LQ> head2;
-    if (b2 < P.B) decode_buffer_request<T, DH, LQ>(P, b2, h, lane, head2);
 
     // ---- phase 1: context.  Column c = (trajectory c / LQ, query c % LQ); columns past the end
     // carry zero queries (their results are never read).
@@ -59,13 +60,18 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodePa
         const long b = b0 + c / LQ;
         const bool live = c < NCOL && b < P.B;
         const T *qrow = view_row<T>(P.q, live ? b : 0, h, live ? c % LQ : 0);
+        // Loaded without a lane mask (an idle column re-reads a valid row and is zeroed by its
+        // scale): a masked load merged with zeros made the compiler wait for the queries on the
+        // spot, and with them for the buffer rows of phase 2 requested just before.
+        const float qs = live ? P.qscale : 0.f;
+        u32x4 raw[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) raw[ks] = *reinterpret_cast<const u32x4 *>(qrow + 16 * ks + 8 * hb);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            u32x4 raw = {0u, 0u, 0u, 0u};
-            if (live) raw = *reinterpret_cast<const u32x4 *>(qrow + 16 * ks + 8 * hb);
             u32x4 sc;  // scale * log2(e) folded in and rounded to the input type (triton_kernels.py:120-121)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) sc[e] = pack2<T>(unpack_lo<T>(raw[e]) * P.qscale, unpack_hi<T>(raw[e]) * P.qscale);
+            for (int e = 0; e < 4; ++e) sc[e] = pack2<T>(unpack_lo<T>(raw[ks][e]) * qs, unpack_hi<T>(raw[ks][e]) * qs);
             qreg[ks] = __builtin_bit_cast(vec, sc);
         }
     }
@@ -182,6 +188,7 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodePa
         Raw r0, r1, r2;
         if (my_blocks > 0) fetch(wave, r0);
         if (my_blocks > 1) fetch(wave + NW, r1);
+        if (b2 < P.B) decode_buffer_request<T, DH, LQ>(P, b2, h, lane, head2);
         int i = 0;
         while (i < my_blocks) {
             if (i + 2 < my_blocks) fetch(wave + NW * (i + 2), r2);
