@@ -208,11 +208,12 @@ struct BackwardTile {
     static constexpr int CPR = DH / 8;
     static constexpr int PIECES = 32 * CPR;  // <= 256 = threads of the workgroup
     static constexpr int BLOCK = 32 * 16;    // elements of a 16-column block
+    // (every thread loads, without a lane mask: threads beyond the tile's pieces re-read one of
+    // them and never store it.  A masked load merged with zeros makes the compiler wait for the
+    // load where it is issued, and the prefetch of the next tile would hide nothing.)
     static __device__ __forceinline__ u32x4 fetch(const View &src, long b, long h, int row0, int R, int tid) {
-        u32x4 raw = {0u, 0u, 0u, 0u};
-        if (tid < PIECES)
-            raw = *reinterpret_cast<const u32x4 *>(view_row<T>(src, b, h, min(row0 + tid / CPR, R - 1)) + 8 * (tid % CPR));
-        return raw;
+        const int piece = tid % PIECES;
+        return *reinterpret_cast<const u32x4 *>(view_row<T>(src, b, h, min(row0 + piece / CPR, R - 1)) + 8 * (piece % CPR));
     }
     static __device__ __forceinline__ void stash(T *tile, int tid, const u32x4 &raw) {
         const int row = tid / CPR, piece = tid % CPR;
@@ -462,10 +463,12 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
     auto fetch = [&](int qt) {
         q_raw = Tile::fetch(P.q, b, h, 32 * qt, P.R, tid);
         g_raw = Tile::fetch(P.dout, b, h, 32 * qt, P.R, tid);
-        if (tid < 32) {
-            const int i = 32 * qt + tid;
-            st_lse2 = -P.lse[stat0 + min(i, P.R - 1)] * kLog2e;  // negated: the accumulators start from them
-            st_delta = -P.delta[stat0 + min(i, P.R - 1)];
+        {   // (all threads, as above; threads 32.. hold copies that are never stored)
+            const int i = 32 * qt + (tid & 31);
+            // (as loaded: any arithmetic on them here would wait for the loads, and with them for
+            // the tile requested just before; they are negated and scaled when they go to LDS)
+            st_lse2 = P.lse[stat0 + min(i, P.R - 1)];
+            st_delta = P.delta[stat0 + min(i, P.R - 1)];
             st_end = backward_vis_end(P, i);
         }
     };
@@ -473,8 +476,8 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
         Tile::stash(q_tiles[slot], tid, q_raw);
         Tile::stash(g_tiles[slot], tid, g_raw);
         if (tid < 32) {
-            lse2_t[slot][tid] = st_lse2;
-            delta_t[slot][tid] = st_delta;
+            lse2_t[slot][tid] = -st_lse2 * kLog2e;  // negated: the accumulators start from them
+            delta_t[slot][tid] = -st_delta;
             end_t[slot][tid] = st_end;
         }
     };
