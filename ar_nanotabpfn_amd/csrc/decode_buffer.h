@@ -89,7 +89,13 @@ struct BufferHead {
     bool slot_fits;
 };
 
-template <typename T, int DH, int LQ>
+// ALL_LANES: every lane group loads, without a lane mask — one past the last row re-reads the last
+// row, which the consumer masks by position.  Loads under a mask, merged with zeros, make the
+// compiler wait for them where they are issued, so a batch requested ahead hides nothing: the
+// streaming buffer kernel takes the unmasked form (2-7 % faster from 128 rows on).  The one-launch
+// kernel keeps the masked one: at a handful of rows the 31 idle lane groups' loads cost more than
+// the wait (11.4 against 11.9 us at one row).
+template <typename T, int DH, int LQ, bool ALL_LANES = false>
 __device__ __forceinline__ void decode_buffer_rows(const DecodeParams &P, long b, int h, int lane, int kv0, int n_buf,
                                                    int n_total, u32x4 (&kraw)[kDecodeUnroll],
                                                    u32x4 (&vraw)[kDecodeUnroll]) {
@@ -97,20 +103,30 @@ __device__ __forceinline__ void decode_buffer_rows(const DecodeParams &P, long b
     const int grp = lane / LPR, sub = lane % LPR;
 #pragma unroll
     for (int u = 0; u < kDecodeUnroll; ++u) {
-        const int kv = kv0 + u * RPW + grp;
-        kraw[u] = u32x4{0u, 0u, 0u, 0u};
-        vraw[u] = u32x4{0u, 0u, 0u, 0u};
-        if (kv < n_total) {
+        const int kv_raw = kv0 + u * RPW + grp;
+        if constexpr (ALL_LANES) {
+            const int kv = kv_raw < n_total ? kv_raw : (n_total > 0 ? n_total - 1 : 0);
             const bool is_new = P.has_new && kv == n_buf;
             const T *kr = is_new ? view_row<T>(P.knew, b, h, 0) : view_row<T>(P.kb, b, h, kv);
             const T *vr = is_new ? view_row<T>(P.vnew, b, h, 0) : view_row<T>(P.vb, b, h, kv);
             kraw[u] = *reinterpret_cast<const u32x4 *>(kr + 8 * sub);
             vraw[u] = *reinterpret_cast<const u32x4 *>(vr + 8 * sub);
+        } else {
+            const int kv = kv_raw;
+            kraw[u] = u32x4{0u, 0u, 0u, 0u};
+            vraw[u] = u32x4{0u, 0u, 0u, 0u};
+            if (kv < n_total) {
+                const bool is_new = P.has_new && kv == n_buf;
+                const T *kr = is_new ? view_row<T>(P.knew, b, h, 0) : view_row<T>(P.kb, b, h, kv);
+                const T *vr = is_new ? view_row<T>(P.vnew, b, h, 0) : view_row<T>(P.vb, b, h, kv);
+                kraw[u] = *reinterpret_cast<const u32x4 *>(kr + 8 * sub);
+                vraw[u] = *reinterpret_cast<const u32x4 *>(vr + 8 * sub);
+            }
         }
     }
 }
 
-template <typename T, int DH, int LQ>
+template <typename T, int DH, int LQ, bool ALL_LANES = false>
 __device__ __forceinline__ void decode_buffer_request(const DecodeParams &P, long b, int h, int lane,
                                                       BufferHead<T, DH, LQ> &hd) {
     const int sub = lane % (DH / 8);
@@ -118,13 +134,13 @@ __device__ __forceinline__ void decode_buffer_request(const DecodeParams &P, lon
     for (int i = 0; i < LQ; ++i) hd.qraw[i] = *reinterpret_cast<const u32x4 *>(view_row<T>(P.q, b, h, i) + 8 * sub);
     hd.n_buf = P.n_base + committed_rows(P, hd.slot_fits);
     hd.n_total = hd.n_buf + (P.has_new ? 1 : 0);
-    decode_buffer_rows<T, DH, LQ>(P, b, h, lane, 0, hd.n_buf, hd.n_total, hd.kraw, hd.vraw);
+    decode_buffer_rows<T, DH, LQ, ALL_LANES>(P, b, h, lane, 0, hd.n_buf, hd.n_total, hd.kraw, hd.vraw);
 }
 
 // The buffer pass of one (trajectory, head) pair by one wavefront: streams the committed buffer
 // rows, appends the new one, merges with the context partials `parts` and writes the final output.
 // `wave` (0 .. NWAVES-1) selects the wavefront's private LDS region.
-template <typename T, int DH, int LQ, int NWAVES, typename Parts>
+template <typename T, int DH, int LQ, int NWAVES, typename Parts, bool ALL_LANES = false>
 __device__ __forceinline__ void decode_buffer_pair(const DecodeParams &P, long b, int h, int wave, int lane,
                                                    const Parts &parts, const BufferHead<T, DH, LQ> &hd) {
     constexpr int LPR = DH / 8;    // lanes per key row
@@ -193,7 +209,7 @@ __device__ __forceinline__ void decode_buffer_pair(const DecodeParams &P, long b
             vraw[u] = vnext[u];
         }
         if (kv0 + RPW * kDecodeUnroll < n_total)
-            decode_buffer_rows<T, DH, LQ>(P, b, h, lane, kv0 + RPW * kDecodeUnroll, n_buf, n_total, knext, vnext);
+            decode_buffer_rows<T, DH, LQ, ALL_LANES>(P, b, h, lane, kv0 + RPW * kDecodeUnroll, n_buf, n_total, knext, vnext);
         float s[LQ][kDecodeUnroll];
 #pragma unroll
         for (int u = 0; u < kDecodeUnroll; ++u) {
@@ -319,8 +335,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(Decode
     const long b = pair / P.H;
     const int h = static_cast<int>(pair % P.H);
     BufferHead<T, DH, LQ> hd;
-    decode_buffer_request<T, DH, LQ>(P, b, h, lane, hd);
-    decode_buffer_pair<T, DH, LQ, kDecodeWaves>(P, b, h, wave, lane, parts, hd);
+    decode_buffer_request<T, DH, LQ, true>(P, b, h, lane, hd);
+    decode_buffer_pair<T, DH, LQ, kDecodeWaves, decltype(parts), true>(P, b, h, wave, lane, parts, hd);
 }
 
 }  // namespace artab
