@@ -571,8 +571,11 @@ def test_graph_sampling_ordered_by_counters_equals_event_ordered(device):
             if st.order is None:
                 pytest.skip("the two streams are served by one hardware queue here")
             assert pred.counter_ordering and st.order.failed() == 0
-            n_waits = 2 * (Nt - 1) * len(model.backbone.layers)  # per call of sample_sequence
-            assert st.order.state[0].item() == st.order.state[32].item() and st.order.state[0].item() % (n_waits // 2) == 0
+            # one signal per layer and step: two calls of sample_sequence, and the one replay of
+            # each recorded graph (one step, steps_per_graph steps) when they were recorded
+            n_steps = 2 * (Nt - 1) + 1 + pred.steps_per_graph
+            assert st.graph_many is not None
+            assert st.order.state[0].item() == st.order.state[32].item() == n_steps * len(model.backbone.layers)
         else:
             assert st.order is None
         results[ordered] = (y, [(l.k_buf_cache.clone(), l.v_buf_cache.clone()) for l in model.backbone.layers])
