@@ -48,6 +48,16 @@ __device__ __forceinline__ int committed_rows(const DecodeParams &P, bool &fits)
     return raw < 0 ? 0 : (raw > hi ? (hi > 0 ? hi : 0) : raw);
 }
 
+struct CommittedRows {
+    int n;
+    bool fits;
+};
+__device__ __forceinline__ CommittedRows read_committed_rows(const DecodeParams &P) {
+    CommittedRows c;
+    c.n = committed_rows(P, c.fits);
+    return c;
+}
+
 constexpr int kDecodeWaves = 4;
 constexpr int kDecodeUnroll = 4;
 constexpr int kSplitBatch = 8;  // context partials fetched per round of the merge
@@ -126,15 +136,23 @@ __device__ __forceinline__ void decode_buffer_rows(const DecodeParams &P, long b
     }
 }
 
+// (`rows`: the committed length as read_committed_rows() gave it — to a caller that read it
+// earlier, so that nothing here waits for it.)
 template <typename T, int DH, int LQ, bool ALL_LANES = false>
 __device__ __forceinline__ void decode_buffer_request(const DecodeParams &P, long b, int h, int lane,
-                                                      BufferHead<T, DH, LQ> &hd) {
+                                                      BufferHead<T, DH, LQ> &hd, const CommittedRows &rows) {
     const int sub = lane % (DH / 8);
 #pragma unroll
     for (int i = 0; i < LQ; ++i) hd.qraw[i] = *reinterpret_cast<const u32x4 *>(view_row<T>(P.q, b, h, i) + 8 * sub);
-    hd.n_buf = P.n_base + committed_rows(P, hd.slot_fits);
+    hd.n_buf = P.n_base + rows.n;
+    hd.slot_fits = rows.fits;
     hd.n_total = hd.n_buf + (P.has_new ? 1 : 0);
     decode_buffer_rows<T, DH, LQ, ALL_LANES>(P, b, h, lane, 0, hd.n_buf, hd.n_total, hd.kraw, hd.vraw);
+}
+template <typename T, int DH, int LQ, bool ALL_LANES = false>
+__device__ __forceinline__ void decode_buffer_request(const DecodeParams &P, long b, int h, int lane,
+                                                      BufferHead<T, DH, LQ> &hd) {
+    decode_buffer_request<T, DH, LQ, ALL_LANES>(P, b, h, lane, hd, read_committed_rows(P));
 }
 
 // The buffer pass of one (trajectory, head) pair by one wavefront: streams the committed buffer

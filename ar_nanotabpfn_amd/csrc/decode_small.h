@@ -47,11 +47,13 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodePa
     const int c = lane & 31, hb = lane >> 5;
 
     // what phase 2 needs from global memory is requested early, so that its round trips (the
-    // buffer rows come from HBM) run under phase 1 — but behind the queries and the first two
-    // context blocks: loads return in the order they were requested, and the first product must
-    // not wait for the buffer rows
+    // buffer rows come from HBM) run under phase 1 — but behind the first product: loads return
+    // in the order they were requested, and the first product must not wait for the buffer rows
     const long b2 = b0 + wave;
     BufferHead<T, DH, LQ> head2;
+    // (the committed length first of all: the form of phase 2's requests depends on it, and a
+    // value requested here has arrived when they are made)
+    const CommittedRows committed = read_committed_rows(P);
 
     // ---- phase 1: context.  Column c = (trajectory c / LQ, query c % LQ); columns past the end
     // carry zero queries (their results are never read).
@@ -183,22 +185,40 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodePa
         __builtin_amdgcn_wave_barrier();
     };
 
-    // blocks wave, wave + NW, ...: two requested ahead of the one being multiplied
+    // phase 2's requests: a handful of rows under a lane mask (the idle lane groups' loads would
+    // cost more than the wait that the masked form brings with it), from half a batch on every
+    // lane loads and nothing waits
+    constexpr int kBatch = kDecodeUnroll * 64 / (DH / 8);
+    const int n_total2 = P.n_base + committed.n + (P.has_new ? 1 : 0);
+
     {
+        // blocks wave, wave + NW, ...: two requested ahead of the one being multiplied.  Phase 2's
+        // requests follow the first product: loads return in the order of their requests, and the
+        // first product waits for everything requested before it.
         Raw r0, r1, r2;
         if (my_blocks > 0) fetch(wave, r0);
         if (my_blocks > 1) fetch(wave + NW, r1);
-        if (b2 < P.B) decode_buffer_request<T, DH, LQ>(P, b2, h, lane, head2);
         int i = 0;
+        if (my_blocks > 0) {
+            if (2 < my_blocks) fetch(wave + NW * 2, r2);
+            compute(wave, r0);
+            i = 1;
+        }
+        if (b2 < P.B) {
+            if (n_total2 > kBatch / 2)
+                decode_buffer_request<T, DH, LQ, true>(P, b2, h, lane, head2, committed);
+            else
+                decode_buffer_request<T, DH, LQ, false>(P, b2, h, lane, head2, committed);
+        }
         while (i < my_blocks) {
-            if (i + 2 < my_blocks) fetch(wave + NW * (i + 2), r2);
-            compute(wave + NW * i, r0);
-            if (++i >= my_blocks) break;
             if (i + 2 < my_blocks) fetch(wave + NW * (i + 2), r0);
             compute(wave + NW * i, r1);
             if (++i >= my_blocks) break;
             if (i + 2 < my_blocks) fetch(wave + NW * (i + 2), r1);
             compute(wave + NW * i, r2);
+            if (++i >= my_blocks) break;
+            if (i + 2 < my_blocks) fetch(wave + NW * (i + 2), r2);
+            compute(wave + NW * i, r0);
             ++i;
         }
     }
