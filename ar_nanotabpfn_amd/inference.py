@@ -77,6 +77,7 @@ class ARTabPFNPredictor:
         # one-step graph covers the remainder.  Measured at B=1024, N_ctx=16384: 1 step per graph
         # -1.7 %, 8 against 4 +0.2 %, 16 loses what the longer remainder of one-step replays costs.
         self.steps_per_graph = 8
+        self.single_steps_first = True  # order of the replays of a run: remainder steps, then the long graphs
         self.fuse_step_boundary = True  # last layer's tail, step tail and first layer's head as one launch
         self.min_chain_batch = 256   # groups smaller than this are not worth their fixed costs
         # Order the two streams of the recorded step through counters in device memory instead of
@@ -594,19 +595,21 @@ class ARTabPFNPredictor:
                 reset(st)
         k = self.steps_per_graph if gs.chains[0].graph_many is not None else 1
         n_many, n_single = (Nt - 1) // k if k > 1 else 0, (Nt - 1) % k if k > 1 else Nt - 1
+        # The one-step replays come first, so that the host queues the first long graph while
+        # they run (measured: nothing at 20 steps, +0.4 % at 256).
+        first_many = 0 if self.single_steps_first else n_many
+        order = [i < first_many or i >= first_many + n_single for i in range(n_many + n_single)]
         if len(gs.chains) == 1:
-            for _ in range(n_many):
-                gs.chains[0].graph_many.replay()
-            for _ in range(n_single):
-                gs.chains[0].graph.replay()
+            for many in order:
+                (gs.chains[0].graph_many if many else gs.chains[0].graph).replay()
         else:
             # every group replays its own step on its own stream; they meet again at the end
             for st in gs.chains:
                 st.stream.wait_stream(current)
-            for i in range(n_many + n_single):
+            for many in order:
                 for st in gs.chains:
                     with torch.cuda.stream(st.stream):
-                        (st.graph_many if i < n_many else st.graph).replay()
+                        (st.graph_many if many else st.graph).replay()
             for st in gs.chains:
                 current.wait_stream(st.stream)
         # the result is copied before the host waits for the failure flag of the counters, so that
