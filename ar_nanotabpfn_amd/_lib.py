@@ -3,6 +3,10 @@
 There is no CPU fallback: if the shared library has not been built the first use
 raises ``RuntimeError`` naming the build command, and tensors that are not on a
 HIP device are rejected.
+
+``libartab_bench.so`` (``include/artab_bench.h``) is a second link of the same object files with
+the benchmark aids added; ``benchmark_library()`` routes every call of this package through it for
+the duration of a ``with`` block.  Only ``bench.py`` does that.
 """
 
 from __future__ import annotations
@@ -15,8 +19,9 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libartab_attention.so")
+BENCH_LIB_PATH = os.path.join(_HERE, "libartab_bench.so")
 
-ABI_VERSION = 6  # ARTAB_VERSION of include/artab_attention.h
+ABI_VERSION = 7  # ARTAB_VERSION of include/artab_attention.h
 STATIC_SCRATCH_BYTES = 32 << 20  # ARTAB_STATIC_SCRATCH_BYTES
 ARTAB_BF16, ARTAB_F16, ARTAB_F32 = 0, 1, 2
 IMPL_AUTO, IMPL_PORTABLE, IMPL_MFMA = 0, 1, 2
@@ -78,9 +83,8 @@ SIGNATURES = {
     "artab_version": (_i, []),
     "artab_status_string": (ctypes.c_char_p, [_i]),
     "artab_last_error": (ctypes.c_char_p, []),
-    "artab_profile_begin": (_i, [_i]),
-    "artab_profile_end": (_i, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_i)]),
-    "artab_bench_instruction_mix": (_i, [_i, _i, _i, _i, _sz, _p, _p, _p]),
+    "artab_tuning_set": (_i, [ctypes.c_char_p, _i, _i]),
+    "artab_tuning_get": (_i, [ctypes.c_char_p, ctypes.POINTER(_i)]),
     "artab_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i]),
     "artab_context_attention": (_i, [_VP, _VP, _VP, _VP, _p, _i, _i, _i, _i, _i, _f, _i, _p, _sz, _i, _p]),
     "artab_decode_attention": (
@@ -138,33 +142,108 @@ SIGNATURES = {
     "artab_layer_post": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _f, _p, _p, _p, _p, _p, _p, _f, _p, _i64, _i, _i, _i, _p]),
 }
 
+# every symbol declared in include/artab_bench.h (exported by libartab_bench.so only)
+BENCH_SIGNATURES = {
+    "artab_profile_begin": (_i, [_i]),
+    "artab_profile_end": (_i, [ctypes.POINTER(_f), ctypes.POINTER(_i), _i]),
+    "artab_bench_instruction_mix": (_i, [_i, _i, _i, _i, _sz, _p, _p, _p]),
+}
+
+TUNING_KEYS = ("ARTAB_BM", "ARTAB_SPLIT", "ARTAB_SMALL", "ARTAB_STREAM", "ARTAB_STREAM_PER_CU", "ARTAB_STREAM_PRIO",
+               "ARTAB_STREAM_SHORT", "ARTAB_DENSE_BELOW", "ARTAB_ORDER_GATE_LAUNCH", "ARTAB_BN", "ARTAB_LEAN",
+               "ARTAB_LEAN_OCC", "ARTAB_NW", "ARTAB_TILE_ROWS")
+
 _lib: Optional[ctypes.CDLL] = None
+_product_lib: Optional[ctypes.CDLL] = None
+_bench_lib: Optional[ctypes.CDLL] = None
 
 
 def library_built() -> bool:
     return os.path.exists(LIB_PATH)
 
 
-def load() -> ctypes.CDLL:
-    """Load the shared library once; raise loudly when it is missing."""
-    global _lib
-    if _lib is not None:
-        return _lib
-    if not library_built():
+def _open(path: str, signatures) -> ctypes.CDLL:
+    if not os.path.exists(path):
         raise RuntimeError(
-            f"{LIB_PATH} is missing: the HIP extension has not been built. "
+            f"{path} is missing: the HIP extension has not been built. "
             "Build it with `python -m ar_nanotabpfn_amd.build_ext` (needs hipcc, targets gfx950). "
             "There is no CPU fallback for the attention path."
         )
-    lib = ctypes.CDLL(LIB_PATH)
-    for name, (restype, argtypes) in SIGNATURES.items():
+    lib = ctypes.CDLL(path)
+    for name, (restype, argtypes) in signatures.items():
         fn = getattr(lib, name)
         fn.restype = restype
         fn.argtypes = argtypes
     if lib.artab_version() != ABI_VERSION:
-        raise RuntimeError(f"{LIB_PATH}: ABI version {lib.artab_version()} != {ABI_VERSION}; rebuild the extension")
-    _lib = lib
+        raise RuntimeError(f"{path}: ABI version {lib.artab_version()} != {ABI_VERSION}; rebuild the extension")
     return lib
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library once; raise loudly when it is missing."""
+    global _lib, _product_lib
+    if _lib is not None:
+        return _lib
+    _product_lib = _open(LIB_PATH, SIGNATURES)
+    _lib = _product_lib
+    return _lib
+
+
+class benchmark_library:
+    """``with benchmark_library() as lib:`` — every call of this package goes through
+    ``libartab_bench.so`` inside the block (same kernels, plus the aids of include/artab_bench.h
+    on ``lib``), and through the product library again afterwards.  Overrides set with
+    ``tuning`` belong to the library they were set on."""
+
+    def __enter__(self) -> ctypes.CDLL:
+        global _lib, _bench_lib
+        load()
+        if _bench_lib is None:
+            _bench_lib = _open(BENCH_LIB_PATH, {**SIGNATURES, **BENCH_SIGNATURES})
+        _lib = _bench_lib
+        return _bench_lib
+
+    def __exit__(self, *exc):
+        global _lib
+        _lib = _product_lib
+        return False
+
+
+class tuning:
+    """``with tuning(ARTAB_SMALL=0, ARTAB_TILE_ROWS=16):`` sets route overrides of the loaded
+    library (``artab_tuning_set``) and restores the previous state on exit; ``None`` removes an
+    override.  ``tuning.set(...)`` / ``tuning.get(name)`` for callers that manage the lifetime
+    themselves (pytest fixtures)."""
+
+    def __init__(self, **overrides):
+        self.overrides = overrides
+        self.saved = {}
+
+    @staticmethod
+    def get(name: str) -> Optional[int]:
+        v = _i(0)
+        rc = load().artab_tuning_get(name.encode(), ctypes.byref(v))
+        if rc < 0:
+            check(rc)
+        return int(v.value) if rc == 1 else None
+
+    @staticmethod
+    def set(**overrides) -> None:
+        lib = load()
+        for name, value in overrides.items():
+            if value is None:
+                check(lib.artab_tuning_set(name.encode(), 0, 0))
+            else:
+                check(lib.artab_tuning_set(name.encode(), int(value), 1))
+
+    def __enter__(self):
+        self.saved = {k: tuning.get(k) for k in self.overrides}
+        tuning.set(**self.overrides)
+        return self
+
+    def __exit__(self, *exc):
+        tuning.set(**self.saved)
+        return False
 
 
 def dtype_code(dtype: torch.dtype) -> int:

@@ -514,7 +514,10 @@ class _RowMaskAttention(torch.autograd.Function):
         return out
 
     @staticmethod
+    @torch.autograd.function.once_differentiable
     def backward(ctx, dout):
+        # The device backward pass is not itself differentiable: asking for a second derivative
+        # raises instead of treating dq, dk, dv as constants.
         q, k, v, out, lse = ctx.saved_tensors
         context_len, buffer_len, attending_chunks, use_triton = ctx.mask
         dq, dk, dv = row_mask_attention_backward(q, k, v, out, dout, lse, context_len, buffer_len, attending_chunks,

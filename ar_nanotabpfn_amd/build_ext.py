@@ -1,10 +1,14 @@
-"""Build ``libartab_attention.so`` for gfx950 with hipcc (cross-compiles without a GPU).
+"""Build ``libartab_attention.so`` and ``libartab_bench.so`` for gfx950 with hipcc (cross-compiles
+without a GPU).
 
     python -m ar_nanotabpfn_amd.build_ext
 
 The device code is split over several translation units (the C ABI with the small kernels, the
 matrix-core attention kernel, the fused layer kernels per element type and kernel group) that are
-compiled side by side and linked into one shared library.
+compiled side by side.  The same objects are linked twice: with a launch observer that observes
+nothing into the drop-in library (exports: the ``artab_*`` functions of
+``include/artab_attention.h``), and with the benchmark hooks and the instruction-mix kernel into
+``libartab_bench.so`` (``include/artab_bench.h``), which only ``bench.py`` loads.
 """
 
 from __future__ import annotations
@@ -19,6 +23,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 OUT = os.path.join(HERE, "libartab_attention.so")
+OUT_BENCH = os.path.join(HERE, "libartab_bench.so")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -29,11 +34,19 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # MFMA accumulators live in VGPRs (no AGPR<->VGPR copies around every product)
     "-mllvm", "-amdgpu-mfma-vgpr-form",
+    # only the extern "C" entry points leave the library (see EXPORTS below)
+    "-fvisibility=hidden",
 ]
+
+# linker version script: the C ABI is every artab_* symbol, nothing else is exported
+EXPORTS = "{ global: artab_*; local: *; };\n"
 
 # (source, extra defines, object name)
 UNITS = [("artab_api.hip", [], "artab_api.o"), ("flash_launch.hip", [], "flash_launch.o"),
-         ("mix_bench.hip", [], "mix_bench.o"), ("backward_launch.hip", [], "backward_launch.o")]
+         ("backward_launch.hip", [], "backward_launch.o")]
+# objects that differ between the two libraries
+PRODUCT_ONLY = [("launch_observer_none.hip", [], "launch_observer_none.o")]
+BENCH_ONLY = [("bench_hooks.hip", [], "bench_hooks.o"), ("mix_bench.hip", [], "mix_bench.o")]
 for _bf16 in (1, 0):
     for _group in (0, 1, 2, 3):
         UNITS.append(("layer_launch.hip", [f"-DARTAB_LAYER_BF16={_bf16}", f"-DARTAB_LAYER_GROUP={_group}"],
@@ -59,18 +72,28 @@ def _run(cmd, verbose):
 
 
 def build(verbose: bool = True, jobs: int = 0) -> str:
-    """Compile every translation unit from source (every time it is called) and link the
-    library; returns the .so path."""
+    """Compile every translation unit from source (every time it is called) and link the two
+    libraries; returns the path of the drop-in library."""
     hipcc = find_hipcc()
     os.makedirs(OBJ_DIR, exist_ok=True)
-    jobs = jobs or min(len(UNITS), max(1, (os.cpu_count() or 2)), 8)
-    objs = [os.path.join(OBJ_DIR, o) for _, _, o in UNITS]
-    cmds = [[hipcc, *HIPCC_FLAGS, *defs, "-c", os.path.join(CSRC, src), "-o", obj]
-            for (src, defs, _), obj in zip(UNITS, objs)]
+    units = UNITS + PRODUCT_ONLY + BENCH_ONLY
+    jobs = jobs or min(len(units), max(1, (os.cpu_count() or 2)), 8)
+
+    def obj(u):
+        return os.path.join(OBJ_DIR, u[2])
+
+    cmds = [[hipcc, *HIPCC_FLAGS, *defs, "-c", os.path.join(CSRC, src), "-o", os.path.join(OBJ_DIR, o)]
+            for src, defs, o in units]
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(lambda c: _run(c, verbose), cmds))
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT + ".tmp", *objs], verbose)
-    os.replace(OUT + ".tmp", OUT)
+    exports = os.path.join(OBJ_DIR, "exports.map")
+    with open(exports, "w") as f:
+        f.write(EXPORTS)
+    for out, extra in ((OUT, PRODUCT_ONLY), (OUT_BENCH, BENCH_ONLY)):
+        objs = [obj(u) for u in UNITS + extra]
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", f"-Wl,--version-script={exports}",
+              "-o", out + ".tmp", *objs], verbose)
+        os.replace(out + ".tmp", out)
     return OUT
 
 

@@ -26,28 +26,39 @@ namespace artab {
 
 static thread_local char g_err[512] = "";
 
-// Optional timing of the MFMA context-pass launches (benchmark aid; off by default).
-// While enabled, each such launch is bracketed by a pair of HIP events on its stream.
-struct ProfileState {
-    bool enabled = false;
-    int capacity = 0, used = 0;
-    hipEvent_t *start = nullptr, *stop = nullptr;
+// Route and tile-size overrides: one slot per key, filled from the environment once (the static
+// initialiser below runs when the library is loaded) and afterwards only by artab_tuning_set().
+struct TuneSlot {
+    const char *name;
+    bool set;
+    int value;
 };
-static ProfileState g_prof;
-
-struct ProfileScope {
-    hipStream_t stream;
-    int slot;
-    explicit ProfileScope(hipStream_t st) : stream(st), slot(-1) {
-        if (g_prof.enabled && g_prof.used < g_prof.capacity) {
-            slot = g_prof.used++;
-            (void)hipEventRecord(g_prof.start[slot], stream);
+static TuneSlot g_tune[kTuneCount] = {
+    {"ARTAB_BM", false, 0},          {"ARTAB_SPLIT", false, 0},        {"ARTAB_SMALL", false, 0},
+    {"ARTAB_STREAM", false, 0},      {"ARTAB_STREAM_PER_CU", false, 0}, {"ARTAB_STREAM_PRIO", false, 0},
+    {"ARTAB_STREAM_SHORT", false, 0}, {"ARTAB_DENSE_BELOW", false, 0},  {"ARTAB_ORDER_GATE_LAUNCH", false, 0},
+    {"ARTAB_BN", false, 0},          {"ARTAB_LEAN", false, 0},         {"ARTAB_LEAN_OCC", false, 0},
+    {"ARTAB_NW", false, 0},          {"ARTAB_TILE_ROWS", false, 0},
+};
+static const bool g_tune_loaded = [] {
+    for (TuneSlot &t : g_tune) {
+        const char *v = getenv(t.name);
+        if (v && *v) {
+            t.set = true;
+            t.value = atoi(v);
         }
     }
-    ~ProfileScope() {
-        if (slot >= 0) (void)hipEventRecord(g_prof.stop[slot], stream);
-    }
-};
+    return true;
+}();
+
+int tune(Tune key, int fallback) { return g_tune[key].set ? g_tune[key].value : fallback; }
+
+static int tune_index(const char *name) {
+    if (!name) return -1;
+    for (int i = 0; i < kTuneCount; ++i)
+        if (strcmp(g_tune[i].name, name) == 0) return i;
+    return -1;
+}
 
 static int fail(int code, const char *fmt, ...) {
     va_list ap;
@@ -132,7 +143,7 @@ struct FlashPlan {
 // rows (no wavefronts of pure padding) or, for the unsplittable phases, when the
 // grid would not cover the chip.  Missing parallelism on long contexts comes from
 // slicing the context (each slice returns a normalised partial + log-sum-exp).
-// ARTAB_BM / ARTAB_SPLIT override the choice (tuning aid).
+// kTuneBM / kTuneSplit override the choice.
 static FlashPlan plan_flash(int B, int H, int Lq, int Nc, int Dh, bool stacked, bool allow_split) {
     FlashPlan pl;
     pl.n_groups = stacked ? 1 : B;
@@ -142,7 +153,7 @@ static FlashPlan plan_flash(int B, int H, int Lq, int Nc, int Dh, bool stacked, 
     while (bm > 64 && pl.G <= bm / 2) bm /= 2;
     if (!allow_split)
         while (bm > 64 && wgs(bm) < 512) bm /= 2;
-    const int bm_env = env_int("ARTAB_BM", 0);
+    const int bm_env = tune(kTuneBM, 0);
     if ((bm_env == 64 || bm_env == 128 || (bm_env == 256 && Dh != 128))) bm = bm_env;
     pl.BM = bm;
     pl.tiles_per_group = (pl.G + bm - 1) / bm;
@@ -158,7 +169,7 @@ static FlashPlan plan_flash(int B, int H, int Lq, int Nc, int Dh, bool stacked, 
         // (measured at 1024 stacked rows: 31 us with 16 slices, 30 us with 8) and cost the merge a
         // second round.
         if (n_split > 8 && base * 8 >= kTargetWorkgroups / 2) n_split = 8;
-        const int sp_env = env_int("ARTAB_SPLIT", 0);
+        const int sp_env = tune(kTuneSplit, 0);
         if (sp_env > 0) n_split = sp_env < max_split ? sp_env : max_split;
     }
     int per = (Nc + n_split - 1) / n_split;
@@ -176,9 +187,9 @@ static hipError_t launch_decode_lq(const DecodeParams &P, int Dh, hipStream_t st
     if (pairs == 0) return hipSuccess;
     dim3 grid(static_cast<unsigned>((pairs + kDecodeWaves - 1) / kDecodeWaves)), block(kDecodeWaves * 64);
     switch (Dh) {
-        case 32: hipLaunchKernelGGL((decode_buffer_kernel<T, 32, LQ>), grid, block, 0, stream, P); break;
-        case 64: hipLaunchKernelGGL((decode_buffer_kernel<T, 64, LQ>), grid, block, 0, stream, P); break;
-        default: hipLaunchKernelGGL((decode_buffer_kernel<T, 128, LQ>), grid, block, 0, stream, P); break;
+        case 32: launch_observed(kLaunchBuffer, decode_buffer_kernel<T, 32, LQ>, grid, block, 0, stream, P); break;
+        case 64: launch_observed(kLaunchBuffer, decode_buffer_kernel<T, 64, LQ>, grid, block, 0, stream, P); break;
+        default: launch_observed(kLaunchBuffer, decode_buffer_kernel<T, 128, LQ>, grid, block, 0, stream, P); break;
     }
     return hipGetLastError();
 }
@@ -194,7 +205,7 @@ static hipError_t launch_decode(const DecodeParams &P, int dtype, int Dh, int Lq
 // twice, and a context that a CU streams from L2 in a few microseconds (every workgroup reads its
 // head's whole context: 2.6 us for 1024 rows of 64 at the ~100 GB/s a CU draws from L2).
 static bool small_decode_applies(int B, int H, int Lq, int Nc, int Dh) {
-    if (env_int("ARTAB_SMALL", 1) == 0 || (Dh != 32 && Dh != 64) || Lq < 1 || Lq > 2) return false;
+    if (tune(kTuneSmall, 1) == 0 || (Dh != 32 && Dh != 64) || Lq < 1 || Lq > 2) return false;
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
@@ -209,14 +220,14 @@ static hipError_t launch_small_t(const DecodeParams &P, const View &kc, const Vi
     dim3 grid(static_cast<unsigned>((P.B + kSmallTraj - 1) / kSmallTraj) * P.H), block(kSmallWaves * 64);
     if (Dh == 32) {
         if (Lq == 1)
-            hipLaunchKernelGGL((decode_small_kernel<T, 32, 1>), grid, block, 0, stream, P, kc, vc, Nc);
+            launch_observed(kLaunchSmallDecode, decode_small_kernel<T, 32, 1>, grid, block, 0, stream, P, kc, vc, Nc);
         else
-            hipLaunchKernelGGL((decode_small_kernel<T, 32, 2>), grid, block, 0, stream, P, kc, vc, Nc);
+            launch_observed(kLaunchSmallDecode, decode_small_kernel<T, 32, 2>, grid, block, 0, stream, P, kc, vc, Nc);
     } else {
         if (Lq == 1)
-            hipLaunchKernelGGL((decode_small_kernel<T, 64, 1>), grid, block, 0, stream, P, kc, vc, Nc);
+            launch_observed(kLaunchSmallDecode, decode_small_kernel<T, 64, 1>, grid, block, 0, stream, P, kc, vc, Nc);
         else
-            hipLaunchKernelGGL((decode_small_kernel<T, 64, 2>), grid, block, 0, stream, P, kc, vc, Nc);
+            launch_observed(kLaunchSmallDecode, decode_small_kernel<T, 64, 2>, grid, block, 0, stream, P, kc, vc, Nc);
     }
     return hipGetLastError();
 }
@@ -234,19 +245,19 @@ static hipError_t launch_stream_t(const DecodeParams &P, int Lq, hipStream_t str
         cus = 256;
     const long tasks = (pairs + 3) / 4;  // of the 4-pair chunk shape; the 16-pair shape leaves the surplus idle
     long per_cu = 4;
-    if (const char *e = getenv("ARTAB_STREAM_PER_CU")) per_cu = atol(e) >= 1 && atol(e) <= 4 ? atol(e) : per_cu;  // tuning hook
+    if (const int v = tune(kTuneStreamPerCu, 0); v >= 1 && v <= 4) per_cu = v;
     dim3 grid(static_cast<unsigned>(tasks < per_cu * cus ? tasks : per_cu * cus)), block(64);
-    const int prio = env_int("ARTAB_STREAM_PRIO", 3);  // tuning aid
+    const int prio = tune(kTuneStreamPrio, 3);
     if (Lq == 1)
-        hipLaunchKernelGGL((decode_stream_kernel<T, 1>), grid, block, kStreamLdsBytes, stream, P);
+        launch_observed(kLaunchStreamBuffer, decode_stream_kernel<T, 1>, grid, block, kStreamLdsBytes, stream, P);
     else if (prio == 0)
-        hipLaunchKernelGGL((decode_stream_kernel<T, 2, 0>), grid, block, kStreamLdsBytes, stream, P);
+        launch_observed(kLaunchStreamBuffer, decode_stream_kernel<T, 2, 0>, grid, block, kStreamLdsBytes, stream, P);
     else if (prio == 1)
-        hipLaunchKernelGGL((decode_stream_kernel<T, 2, 1>), grid, block, kStreamLdsBytes, stream, P);
+        launch_observed(kLaunchStreamBuffer, decode_stream_kernel<T, 2, 1>, grid, block, kStreamLdsBytes, stream, P);
     else if (prio == 2)
-        hipLaunchKernelGGL((decode_stream_kernel<T, 2, 2>), grid, block, kStreamLdsBytes, stream, P);
+        launch_observed(kLaunchStreamBuffer, decode_stream_kernel<T, 2, 2>, grid, block, kStreamLdsBytes, stream, P);
     else
-        hipLaunchKernelGGL((decode_stream_kernel<T, 2>), grid, block, kStreamLdsBytes, stream, P);
+        launch_observed(kLaunchStreamBuffer, decode_stream_kernel<T, 2>, grid, block, kStreamLdsBytes, stream, P);
     return hipGetLastError();
 }
 
@@ -380,45 +391,19 @@ const char *artab_status_string(int status) {
 
 const char *artab_last_error(void) { return g_err; }
 
-int artab_profile_begin(int max_records) {
-    if (max_records <= 0) return fail(ARTAB_ERR_BAD_SHAPE, "max_records must be positive");
-    if (g_prof.capacity < max_records) {
-        for (int i = 0; i < g_prof.capacity; ++i) {
-            (void)hipEventDestroy(g_prof.start[i]);
-            (void)hipEventDestroy(g_prof.stop[i]);
-        }
-        delete[] g_prof.start;
-        delete[] g_prof.stop;
-        g_prof.start = new hipEvent_t[max_records];
-        g_prof.stop = new hipEvent_t[max_records];
-        g_prof.capacity = 0;
-        for (int i = 0; i < max_records; ++i) {
-            if (hipEventCreate(&g_prof.start[i]) != hipSuccess || hipEventCreate(&g_prof.stop[i]) != hipSuccess)
-                return fail(ARTAB_ERR_LAUNCH, "hipEventCreate failed");
-            g_prof.capacity = i + 1;
-        }
-    }
-    g_prof.used = 0;
-    g_prof.enabled = true;
+int artab_tuning_set(const char *name, int value, int enable) {
+    const int i = tune_index(name);
+    if (i < 0) return fail(ARTAB_ERR_UNSUPPORTED, "unknown tuning key %s", name ? name : "(null)");
+    g_tune[i].set = enable != 0;
+    g_tune[i].value = value;
     return ARTAB_OK;
 }
 
-int artab_profile_end(double *total_ms, int *records) {
-    g_prof.enabled = false;
-    double sum = 0.0;
-    int n = 0;
-    for (int i = 0; i < g_prof.used; ++i) {
-        if (hipEventSynchronize(g_prof.stop[i]) != hipSuccess) continue;
-        float ms = 0.f;
-        if (hipEventElapsedTime(&ms, g_prof.start[i], g_prof.stop[i]) == hipSuccess) {
-            sum += ms;
-            ++n;
-        }
-    }
-    if (total_ms) *total_ms = sum;
-    if (records) *records = n;
-    g_prof.used = 0;
-    return ARTAB_OK;
+int artab_tuning_get(const char *name, int *value) {
+    const int i = tune_index(name);
+    if (i < 0) return fail(ARTAB_ERR_UNSUPPORTED, "unknown tuning key %s", name ? name : "(null)");
+    if (value) *value = g_tune[i].value;
+    return g_tune[i].set ? 1 : 0;
 }
 
 size_t artab_workspace_bytes(int B, int H, int Lq, int Nc, int Dh, int dtype) {
@@ -487,7 +472,6 @@ int artab_context_attention(const artab_view *q, const artab_view *k_ctx, const 
         F.part_lse = split_lse_base(workspace, rows, Dh, pl.n_split);
     }
     {
-        ProfileScope prof(st);
         ARTAB_TRY(launch_status(launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st), "context attention (mfma)"));
     }
     if (pl.n_split > 1) {
@@ -576,7 +560,7 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
     const bool shared_ctx = (k_ctx->stride_b == 0 && v_ctx->stride_b == 0) || B == 1;
     bool use_mfma = impl != ARTAB_IMPL_PORTABLE && mfma_shape_ok(dtype, Dh) && aligned && shared_ctx;
     const long rows = static_cast<long>(B) * H * Lq;
-    if (use_mfma && !leave_partials && !order_state && env_int("ARTAB_STREAM", 0) == 0 &&
+    if (use_mfma && !leave_partials && !order_state && tune(kTuneStream, 0) == 0 &&
         small_decode_applies(B, H, Lq, Nc, Dh)) {
         DecodeParams D;
         memset(&D, 0, sizeof(D));
@@ -585,7 +569,6 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
         D.capacity = buf_capacity;
         D.qscale = scale * kLog2e;
         const View kc = dv(k_ctx), vc = dv(v_ctx);
-        ProfileScope prof(st);
         const hipError_t e = dtype == ARTAB_BF16 ? launch_small_t<bf16_t>(D, kc, vc, Nc, Dh, Lq, st)
                                                  : launch_small_t<f16_t>(D, kc, vc, Nc, Dh, Lq, st);
         return launch_status(e, "decode attention (one launch)");
@@ -599,7 +582,7 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
         // the streaming buffer pass exists for head_dim 32 (the shape whose context pass leaves room
         // for it on a SIMD); it is used when the caller offers a second stream to run it on
         stream_buf = need_buf && Dh == 32 &&
-                     ((side_stream && side_stream != stream) || env_int("ARTAB_STREAM", 0) != 0);
+                     ((side_stream && side_stream != stream) || tune(kTuneStream, 0) != 0);
         if (order_state && !(stream_buf && side_stream && side_stream != stream))
             return fail(ARTAB_ERR_UNSUPPORTED,
                         "counter-ordered decode needs the streaming buffer pass (head_dim 32, buffer rows) and a second stream");
@@ -677,10 +660,23 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
 
     if (!stream_buf) {
         {
-            ProfileScope prof(st);
             ARTAB_TRY(launch_status(launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st), "decode context pass"));
         }
         if (!need_ws) return ARTAB_OK;
+        if (!need_buf) {
+            // A split context and nothing else: no buffer row, no new row, and k_buf / v_buf may be
+            // NULL or hold no row at all.  The partials are merged by the elementwise kernel; the
+            // buffer kernel (which reads the cache) is not launched.
+            CombineParams C;
+            C.out = dv(out); C.part_o = F.part_o; C.part_lse = F.part_lse; C.lse = nullptr;
+            C.rows = rows; C.H = H; C.Lq = Lq; C.Dh = Dh; C.n_split = pl.n_split;
+            const unsigned cgrid = static_cast<unsigned>((rows * (Dh / 4) + 255) / 256);
+            if (dtype == ARTAB_BF16)
+                hipLaunchKernelGGL((combine_kernel<bf16_t>), dim3(cgrid), dim3(256), 0, st, C);
+            else
+                hipLaunchKernelGGL((combine_kernel<f16_t>), dim3(cgrid), dim3(256), 0, st, C);
+            return launch_status(hipGetLastError(), "decode combine (context only)");
+        }
         return launch_status(launch_decode(D, dtype, Dh, Lq, st), "decode buffer pass");
     }
 
@@ -695,12 +691,12 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
         const long per_row = static_cast<long>(B) * H * 2 * Dh * 2;  // K and V bytes of one buffer row of every pair
         const long fit = per_row > 0 ? kLastLevelCacheBytes / per_row : 0;
         const long rows = fit > kStreamShortRows ? fit : kStreamShortRows;
-        D.stream_short_rows = env_int("ARTAB_STREAM_SHORT", static_cast<int>(rows < 1 << 20 ? rows : 1 << 20));  // env: tuning hook
+        D.stream_short_rows = tune(kTuneStreamShort, static_cast<int>(rows < 1 << 20 ? rows : 1 << 20));
     }
     if (side_stream && side_stream != stream) {  // the two passes share the compute units
         F.beside_rows = n_buf_device;
         F.beside_n = n_buf;
-        F.dense_below = env_int("ARTAB_DENSE_BELOW", 128);  // env: tuning hook
+        F.dense_below = tune(kTuneDenseBelow, 128);
     }
     D.buf_part_o = static_cast<char *>(workspace) + static_cast<size_t>(pl.n_split) * rows * Dh * 2;
     D.buf_part_lse = F.part_lse + static_cast<size_t>(pl.n_split) * rows;
@@ -719,7 +715,6 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
         ARTAB_TRY(order_wait(order_state, ARTAB_ORDER_SIDE, order_timeout_us, side));
         hipError_t e_ctx, e_buf;
         {
-            ProfileScope prof(st);
             e_ctx = launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st);
         }
         e_buf = launch_stream(D, dtype, Lq, side);
@@ -746,7 +741,6 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
     }
     hipError_t e_ctx, e_buf, e_join = hipSuccess;
     {
-        ProfileScope prof(st);
         e_ctx = launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st);
     }
     e_buf = launch_stream(D, dtype, Lq, side);
@@ -936,7 +930,6 @@ int artab_teacher_forcing_attention(const artab_view *q, const artab_view *k_ctx
     F.n_split = 1; F.kv_per_split = pl.kv_per_split;
     F.qscale = scale * kLog2e;
     F.mode = kFlashTeacher;
-    ProfileScope prof(st);
     return launch_status(launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st), "teacher forcing (mfma)");
 }
 
@@ -991,7 +984,6 @@ int artab_row_mask_attention(const artab_view *q, const artab_view *k, const art
     F.n_split = 1; F.kv_per_split = pl.kv_per_split;
     F.qscale = scale * kLog2e;
     F.mode = kFlashRowMask;
-    ProfileScope prof(st);
     return launch_status(launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st), "row-mask attention (mfma)");
 }
 
@@ -1027,7 +1019,6 @@ int artab_row_mask_attention_backward(const artab_view *q, const artab_view *k, 
     P.B = B; P.H = H; P.R = R; P.Nc = Nc; P.Nb = Nb; P.attend = attending_chunks;
     P.Dh = Dh; P.scale = resolve_scale(scale, Dh); P.vec_ok = aligned ? 1 : 0;
     const int elem = dtype == ARTAB_BF16 ? kElemBf16 : dtype == ARTAB_F16 ? kElemF16 : kElemF32;
-    ProfileScope prof(st);
     return launch_status(launch_row_mask_backward(P, elem, use_mfma, st),
                          use_mfma ? "row-mask attention backward (mfma)" : "row-mask attention backward (portable)");
 }
@@ -1077,7 +1068,6 @@ int artab_prefill_attention(const artab_view *q, const artab_view *k, const arta
     F.n_split = 1; F.kv_per_split = pl.kv_per_split;
     F.qscale = scale * kLog2e;
     F.mode = kFlashPrefill;
-    ProfileScope prof(st);
     return launch_status(launch_flash_dtype(F, dtype == ARTAB_BF16, Dh, pl.BM, st), "prefill (mfma)");
 }
 
@@ -1268,7 +1258,7 @@ static int apply_partials_order(const artab_attention_partials *parts, FusedPost
         const int64_t grid =
             grid_of_launch >= 0 ? grid_of_launch : (rows + fused_tile_rows(rows) - 1) / fused_tile_rows(rows);
         const uint64_t us = parts->order_timeout_us ? parts->order_timeout_us : 2000000;
-        if (grid * 2 <= cus && env_int("ARTAB_ORDER_GATE_LAUNCH", 0) == 0) {
+        if (grid * 2 <= cus && tune(kTuneOrderGateLaunch, 0) == 0) {
             P.order_wait = parts->order_state;
             P.order_limit = us * 100ull;  // 100 MHz wall clock
         } else {

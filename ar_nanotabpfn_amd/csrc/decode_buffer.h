@@ -147,6 +147,16 @@ __device__ __forceinline__ void decode_buffer_request(const DecodeParams &P, lon
     hd.n_buf = P.n_base + rows.n;
     hd.slot_fits = rows.fits;
     hd.n_total = hd.n_buf + (P.has_new ? 1 : 0);
+    if (ALL_LANES && hd.n_total <= 0) {
+        // No row at all (an empty buffer and no new row: the call only merges context partials).
+        // The unmasked form would re-read "the last row" of a cache that may have none, or be NULL.
+#pragma unroll
+        for (int u = 0; u < kDecodeUnroll; ++u) {
+            hd.kraw[u] = u32x4{0u, 0u, 0u, 0u};
+            hd.vraw[u] = u32x4{0u, 0u, 0u, 0u};
+        }
+        return;
+    }
     decode_buffer_rows<T, DH, LQ, ALL_LANES>(P, b, h, lane, 0, hd.n_buf, hd.n_total, hd.kraw, hd.vraw);
 }
 template <typename T, int DH, int LQ, bool ALL_LANES = false>

@@ -6,8 +6,13 @@ namespace artab {
 
 constexpr int kFlashBN = 64;
 
-// Keys per LDS tile: 64, or 128 for head_dim 32 when ARTAB_BN=128 (tuning aid).
-static int flash_bn(int Dh) { return (Dh == 32 && env_int("ARTAB_BN", 64) == 128) ? 128 : 64; }
+// Keys per LDS tile: 64, or 128 for head_dim 32 when kTuneBN is 128.
+static int flash_bn(int Dh) { return (Dh == 32 && tune(kTuneBN, 64) == 128) ? 128 : 64; }
+
+template <typename Kernel>
+static void launch_one(Kernel kernel, unsigned grid, unsigned block, hipStream_t stream, const FlashParams &P) {
+    launch_observed(kLaunchFlash, kernel, dim3(grid), dim3(block), 0, stream, P);
+}
 
 template <typename T, int DH>
 static hipError_t launch_flash_bm(const FlashParams &P, int BM, hipStream_t stream) {
@@ -18,43 +23,43 @@ static hipError_t launch_flash_bm(const FlashParams &P, int BM, hipStream_t stre
     if constexpr (DH == 32) {
         if (flash_bn(DH) == 128) {
             if (BM == 256)
-                hipLaunchKernelGGL((flash_kernel<T, DH, 2, 4, 128>), dim3(grid), dim3(256), 0, stream, P);
+                launch_one(flash_kernel<T, DH, 2, 4, 128>, grid, 256, stream, P);
             else if (BM == 128)
-                hipLaunchKernelGGL((flash_kernel<T, DH, 1, 4, 128>), dim3(grid), dim3(256), 0, stream, P);
+                launch_one(flash_kernel<T, DH, 1, 4, 128>, grid, 256, stream, P);
             else
-                hipLaunchKernelGGL((flash_kernel<T, DH, 1, 2, 128>), dim3(grid), dim3(128), 0, stream, P);
+                launch_one(flash_kernel<T, DH, 1, 2, 128>, grid, 128, stream, P);
             return hipGetLastError();
         }
     }
     if constexpr (DH == 32) {
         // the lean pass: 256 query rows as eight wavefronts of one 32-row block each, four
-        // wavefronts per SIMD (ARTAB_LEAN=0 selects the software-pipelined form; tuning aid)
-        if (BM == 256 && env_int("ARTAB_LEAN", 1) != 0) {
+        // wavefronts per SIMD (kTuneLean = 0 selects the software-pipelined form)
+        if (BM == 256 && tune(kTuneLean, 1) != 0) {
             // 96 registers (five per SIMD by the register file) leave room for the streaming
-            // buffer pass beside four of these wavefronts; ARTAB_LEAN_OCC=4 takes 128 (tuning aid)
-            if (env_int("ARTAB_LEAN_OCC", 5) == 4)
-                hipLaunchKernelGGL((flash_kernel<T, DH, 1, 8, kFlashBN, true, 4>), dim3(grid), dim3(512), 0, stream, P);
+            // buffer pass beside four of these wavefronts; kTuneLeanOcc = 4 takes 128
+            if (tune(kTuneLeanOcc, 5) == 4)
+                launch_one(flash_kernel<T, DH, 1, 8, kFlashBN, true, 4>, grid, 512, stream, P);
             else if (P.mode == kFlashContext)  // the decode launch: nothing but the context pass compiled in
-                hipLaunchKernelGGL((flash_kernel<T, DH, 1, 8, kFlashBN, true, 5, true>), dim3(grid), dim3(512), 0, stream, P);
+                launch_one(flash_kernel<T, DH, 1, 8, kFlashBN, true, 5, true>, grid, 512, stream, P);
             else
-                hipLaunchKernelGGL((flash_kernel<T, DH, 1, 8, kFlashBN, true, 5>), dim3(grid), dim3(512), 0, stream, P);
+                launch_one(flash_kernel<T, DH, 1, 8, kFlashBN, true, 5>, grid, 512, stream, P);
             return hipGetLastError();
         }
     }
     if constexpr (DH <= 64) {
         if (BM == 256) {
-            hipLaunchKernelGGL((flash_kernel<T, DH, 2, 4, kFlashBN>), dim3(grid), dim3(256), 0, stream, P);
+            launch_one(flash_kernel<T, DH, 2, 4, kFlashBN>, grid, 256, stream, P);
             return hipGetLastError();
         }
-        if (BM == 128 && env_int("ARTAB_NW", 4) == 2) {  // two wavefronts of two query blocks each
-            hipLaunchKernelGGL((flash_kernel<T, DH, 2, 2, kFlashBN>), dim3(grid), dim3(128), 0, stream, P);
+        if (BM == 128 && tune(kTuneNW, 4) == 2) {  // two wavefronts of two query blocks each
+            launch_one(flash_kernel<T, DH, 2, 2, kFlashBN>, grid, 128, stream, P);
             return hipGetLastError();
         }
     }
     if (BM == 128) {
-        hipLaunchKernelGGL((flash_kernel<T, DH, 1, 4, kFlashBN>), dim3(grid), dim3(256), 0, stream, P);
+        launch_one(flash_kernel<T, DH, 1, 4, kFlashBN>, grid, 256, stream, P);
     } else {
-        hipLaunchKernelGGL((flash_kernel<T, DH, 1, 2, kFlashBN>), dim3(grid), dim3(128), 0, stream, P);
+        launch_one(flash_kernel<T, DH, 1, 2, kFlashBN>, grid, 128, stream, P);
     }
     return hipGetLastError();
 }

@@ -21,9 +21,9 @@ template <typename T, int TR>
 hipError_t launch_pre_r(const FusedPreParams &P, int D, hipStream_t st) {
     dim3 grid(static_cast<unsigned>((P.rows + TR - 1) / TR)), block(fused_waves(D) * 64);
     switch (D) {
-        case 128: hipLaunchKernelGGL((fused_pre_kernel<T, 128, TR>), grid, block, 0, st, P); break;
-        case 256: hipLaunchKernelGGL((fused_pre_kernel<T, 256, TR>), grid, block, 0, st, P); break;
-        default: hipLaunchKernelGGL((fused_pre_kernel<T, 512, TR>), grid, block, 0, st, P); break;
+        case 128: launch_observed(kLaunchLayer, fused_pre_kernel<T, 128, TR>, grid, block, 0, st, P); break;
+        case 256: launch_observed(kLaunchLayer, fused_pre_kernel<T, 256, TR>, grid, block, 0, st, P); break;
+        default: launch_observed(kLaunchLayer, fused_pre_kernel<T, 512, TR>, grid, block, 0, st, P); break;
     }
     return hipGetLastError();
 }
@@ -37,9 +37,9 @@ template <typename T, int D, int TR>
 hipError_t launch_post_d(const FusedPostParams &P, int F, hipStream_t st) {
     dim3 grid(static_cast<unsigned>((P.rows + TR - 1) / TR)), block(fused_waves(D) * 64);
     switch (F) {
-        case 128: hipLaunchKernelGGL((fused_post_kernel<T, D, 128, TR>), grid, block, 0, st, P); break;
-        case 256: hipLaunchKernelGGL((fused_post_kernel<T, D, 256, TR>), grid, block, 0, st, P); break;
-        default: hipLaunchKernelGGL((fused_post_kernel<T, D, 512, TR>), grid, block, 0, st, P); break;
+        case 128: launch_observed(kLaunchLayer, fused_post_kernel<T, D, 128, TR>, grid, block, 0, st, P); break;
+        case 256: launch_observed(kLaunchLayer, fused_post_kernel<T, D, 256, TR>, grid, block, 0, st, P); break;
+        default: launch_observed(kLaunchLayer, fused_post_kernel<T, D, 512, TR>, grid, block, 0, st, P); break;
     }
     return hipGetLastError();
 }
@@ -48,9 +48,9 @@ template <typename T, int D, int TR>
 hipError_t launch_post_pre_d(const FusedPostParams &P, const FusedPreParams &N, int F, hipStream_t st) {
     dim3 grid(static_cast<unsigned>((P.rows + TR - 1) / TR)), block(fused_waves(D) * 64);
     switch (F) {
-        case 128: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 128, TR>), grid, block, 0, st, P, N); break;
-        case 256: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 256, TR>), grid, block, 0, st, P, N); break;
-        default: hipLaunchKernelGGL((fused_post_pre_kernel<T, D, 512, TR>), grid, block, 0, st, P, N); break;
+        case 128: launch_observed(kLaunchLayer, fused_post_pre_kernel<T, D, 128, TR>, grid, block, 0, st, P, N); break;
+        case 256: launch_observed(kLaunchLayer, fused_post_pre_kernel<T, D, 256, TR>, grid, block, 0, st, P, N); break;
+        default: launch_observed(kLaunchLayer, fused_post_pre_kernel<T, D, 512, TR>, grid, block, 0, st, P, N); break;
     }
     return hipGetLastError();
 }
@@ -87,9 +87,9 @@ template <typename T, int D, int TR>
 hipError_t launch_sample_d(const SampleEmbedParams &P, int F, hipStream_t st) {
     dim3 grid(static_cast<unsigned>((P.B + TR - 1) / TR)), block(fused_waves(D) * 64);
     switch (F) {
-        case 128: hipLaunchKernelGGL((sample_embed_kernel<T, D, 128, TR>), grid, block, 0, st, P); break;
-        case 256: hipLaunchKernelGGL((sample_embed_kernel<T, D, 256, TR>), grid, block, 0, st, P); break;
-        default: hipLaunchKernelGGL((sample_embed_kernel<T, D, 512, TR>), grid, block, 0, st, P); break;
+        case 128: launch_observed(kLaunchLayer, sample_embed_kernel<T, D, 128, TR>, grid, block, 0, st, P); break;
+        case 256: launch_observed(kLaunchLayer, sample_embed_kernel<T, D, 256, TR>, grid, block, 0, st, P); break;
+        default: launch_observed(kLaunchLayer, sample_embed_kernel<T, D, 512, TR>, grid, block, 0, st, P); break;
     }
     return hipGetLastError();
 }
@@ -114,9 +114,9 @@ hipError_t launch_boundary_d(const FusedPostParams &P, const SampleEmbedParams &
     constexpr int TR = kFusedRowsSmall;
     dim3 grid(static_cast<unsigned>((S.B + TR / 2 - 1) / (TR / 2))), block(fused_waves(D) * 64);
     switch (F) {
-        case 128: hipLaunchKernelGGL((decode_step_boundary_kernel<T, D, 128, TR>), grid, block, 0, st, P, S, N); break;
-        case 256: hipLaunchKernelGGL((decode_step_boundary_kernel<T, D, 256, TR>), grid, block, 0, st, P, S, N); break;
-        default: hipLaunchKernelGGL((decode_step_boundary_kernel<T, D, 512, TR>), grid, block, 0, st, P, S, N); break;
+        case 128: launch_observed(kLaunchLayer, decode_step_boundary_kernel<T, D, 128, TR>, grid, block, 0, st, P, S, N); break;
+        case 256: launch_observed(kLaunchLayer, decode_step_boundary_kernel<T, D, 256, TR>, grid, block, 0, st, P, S, N); break;
+        default: launch_observed(kLaunchLayer, decode_step_boundary_kernel<T, D, 512, TR>, grid, block, 0, st, P, S, N); break;
     }
     return hipGetLastError();
 }

@@ -10,7 +10,7 @@
 // pipe draws, and with it lowers the clock the part sustains).
 #include <hip/hip_runtime.h>
 
-#include "../../include/artab_attention.h"
+#include "../../include/artab_bench.h"
 #include "common.h"
 
 namespace artab {

@@ -289,14 +289,13 @@ class DecodeStepBoundary:
 
     @staticmethod
     def supported(tail: "SampleEmbedStep", first_layer, last_layer, x: Tensor) -> bool:
-        import os
         F_ = last_layer.ff[0].out_features
         return (tail is not None and tail.advances and tail.args.F == F_ and first_layer.ff[0].out_features == F_
                 and first_layer.attn_rows.n_heads == last_layer.attn_rows.n_heads
                 and last_layer.fused_for(x) and first_layer.fused_for(x)
                 and tail.args.B <= DecodeStepBoundary.MAX_TRAJECTORIES
                 and tail.args.D <= DecodeStepBoundary.MAX_WIDTH
-                and os.environ.get("ARTAB_TILE_ROWS", "16") == "16")
+                and _lib.tuning.get("ARTAB_TILE_ROWS") in (None, 16))
 
     def __init__(self, tail: "SampleEmbedStep", first_layer, last_layer, y_next: Tensor, qkv_next: Tensor):
         B, D = tail.args.B, tail.args.D

@@ -61,6 +61,9 @@ class ARTabPFNPredictor:
         # Replay the decode step of sample_sequence from a recorded HIP graph (shared
         # layout on a HIP device only).  Set to False to launch every kernel from Python.
         self.use_hip_graph = True
+        # Instead of replaying the recorded graphs, issue the launches they hold one by one from the
+        # host: same kernels, streams, ordering and scratch memory (for instrumented runs).
+        self.launch_live = False
         self.fuse_step_tail = True   # head + draw + next embedding as one launch inside the graph
         # Run the HBM-bound buffer pass of a decode step on a second stream, next to the
         # compute-bound context pass (shared layout, HIP device).
@@ -539,7 +542,7 @@ class ARTabPFNPredictor:
                         self._first_step(st)
                     st.workspace_first = _lib.held_workspace(device)
             st.counters.zero_()
-            st.graph_first.replay()
+            self._run_recorded(st, "graph_first")
             y0 = emb1 = None
             if st.graph is None:  # the step graphs are still to be recorded: their warm-up starts from here
                 y0, emb1 = st.preds[:, 0:1].clone(), st.emb.clone()
@@ -601,7 +604,7 @@ class ARTabPFNPredictor:
         order = [i < first_many or i >= first_many + n_single for i in range(n_many + n_single)]
         if len(gs.chains) == 1:
             for many in order:
-                (gs.chains[0].graph_many if many else gs.chains[0].graph).replay()
+                self._run_recorded(gs.chains[0], "graph_many" if many else "graph")
         else:
             # every group replays its own step on its own stream; they meet again at the end
             for st in gs.chains:
@@ -609,7 +612,7 @@ class ARTabPFNPredictor:
             for many in order:
                 for st in gs.chains:
                     with torch.cuda.stream(st.stream):
-                        (st.graph_many if many else st.graph).replay()
+                        self._run_recorded(st, "graph_many" if many else "graph")
             for st in gs.chains:
                 current.wait_stream(st.stream)
         # the result is copied before the host waits for the failure flag of the counters, so that
@@ -636,28 +639,45 @@ class ARTabPFNPredictor:
             return False
         return all(layer.attn_rows.head_dim == 32 and layer.fused_for(x) for layer in self.backbone.layers)
 
+    def _issue_steps(self, st, n_steps: int) -> None:
+        """The launches of ``n_steps`` decode steps of one trajectory group, on the current stream
+        (and its side stream).  With counter ordering the side stream is forked once and rejoins
+        at the end; the per-layer dependencies between the two streams are the counters' waits."""
+        if st.order is None:
+            for _ in range(n_steps):
+                self._graph_step(st)
+            return
+        main = torch.cuda.current_stream()
+        side = self._side_stream(main.device, st.chain)
+        side.wait_stream(main)
+        st.order_active = st.order
+        try:
+            for _ in range(n_steps):
+                self._graph_step(st)
+        finally:
+            st.order_active = None
+            main.wait_stream(side)
+
     def _record_steps(self, st, n_steps: int) -> "torch.cuda.CUDAGraph":
-        """Record ``n_steps`` decode steps of one trajectory group into a HIP graph.  With counter
-        ordering the side stream joins the recording once and rejoins at the end; the per-layer
-        dependencies between the two streams are the counters' waits."""
+        """Record ``n_steps`` decode steps of one trajectory group into a HIP graph."""
         graph = torch.cuda.CUDAGraph()
         self.graph_recordings += 1
         with torch.cuda.graph(graph):
-            if st.order is None:
-                for _ in range(n_steps):
-                    self._graph_step(st)
-            else:
-                main = torch.cuda.current_stream()
-                side = self._side_stream(main.device, st.chain)
-                side.wait_stream(main)
-                st.order_active = st.order
-                try:
-                    for _ in range(n_steps):
-                        self._graph_step(st)
-                finally:
-                    st.order_active = None
-                    main.wait_stream(side)
+            self._issue_steps(st, n_steps)
         return graph
+
+    def _run_recorded(self, st, which: str) -> None:
+        """Replay one of the group's recorded graphs — or, with ``launch_live``, issue the very
+        launches it holds one by one from the host (same kernels, streams, ordering and scratch
+        memory; for instrumented runs, whose per-launch events cannot sit inside a graph)."""
+        if not self.launch_live:
+            getattr(st, which).replay()
+            return
+        with _lib.workspace_tag(1 + st.chain):
+            if which == "graph_first":
+                self._first_step(st)
+            else:
+                self._issue_steps(st, self.steps_per_graph if which == "graph_many" else 1)
 
     @staticmethod
     def _draw_step_variates(rand_u: Tensor, rand_n: Tensor) -> None:

@@ -13,30 +13,43 @@ reported separately.
 
 Prints one JSON line:
   metric/value   target-steps per second over the K timed steps (inputs resident in HBM)
+  full_run       the same for all 256 steps of the configuration, whatever K is, with the
+                 context pass's fraction of the bf16 matrix peak over those 256 steps
   roofline       the dominant kernel (MFMA context pass of the decode attention):
-                 algorithmic flops 4*B*H*Lq*N_ctx*Dh per launch over its average
-                 launch duration, measured with HIP events around every launch in a
-                 second, instrumented run of the same K steps; peak 2.5 PFLOP/s bf16
-  cpu_baseline   the numpy oracle (a port of the reference's arithmetic, float32) timed
-                 on this box's host cores on a bounded sample of the same workload
+                 algorithmic flops 4*B*H*Lq*N_ctx*Dh per launch over its average launch
+                 duration in steps 0..K-1.  Durations are the launches' own start and end time
+                 stamps (what a kernel trace reports), taken in a run that issues the launches
+                 of the recorded step live, through the benchmark build of the library; peak
+                 2.5 PFLOP/s bf16
+  cpu_baseline   the reference's CPU path (a PyTorch restatement of its op sequence,
+                 oracle/torch_cpu_path.py) timed on this box's host cores on a bounded
+                 sample of the same workload
   log_density    configs[2] (B=64 datasets, 512 context + 128 target rows): one
-                 teacher-forced evaluation on the GPU vs the same on the host CPU
+                 teacher-forced evaluation on the GPU vs the same on the host CPU, and what
+                 the result differs by from the exact value
+  config4        configs[4] (d_model 512, 16 heads, B=2048, N_ctx=4096): 4 outputs x 64 rows
+                 flattened into 256 scalar decode steps
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
-       python bench.py --kernel-shapes   (instead: one decode layer-step at the shapes of
-                                          configs[1], [3] and [4], timings on stderr)
-       python bench.py --mix-ceiling     (instead: the instruction mix of one 32x32 score block from
-                                          registers: what the SIMD's issue port allows)
-       python bench.py --training-attention  (instead: forward and backward of the training row
-                                          attention at the reference's training shapes)
-       python bench.py --training-step   (instead: one optimiser step of the reference's training
-                                          configuration; launches from autograd's worker thread —
-                                          not for runs under rocprofv3 --pmc)
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-config4]
+       python bench.py --config4            (instead: only the configs[4] leg)
+       python bench.py --kernel-shapes      (instead: one decode layer-step at the shapes of
+                                             configs[1], [3] and [4], timings on stderr)
+       python bench.py --reference-shapes   (instead: the shapes the reference's own benchmark
+                                             scripts print figures for: fp16, d_model 256, 8 heads,
+                                             8 layers, N_ctx 512, 32 targets, B in {1, 8, 64})
+       python bench.py --mix-ceiling        (instead: the instruction mix of one 32x32 score block
+                                             from registers: what the SIMD's issue port allows)
+       python bench.py --training-attention (instead: forward and backward of the training row
+                                             attention at the reference's training shapes)
+       python bench.py --training-step      (instead: one optimiser step of the reference's training
+                                             configuration; launches from autograd's worker thread —
+                                             not for runs under rocprofv3 --pmc)
 """
 
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import math
 import os
@@ -50,21 +63,26 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 
 CFG3 = dict(d_model=256, n_heads=8, n_layers=12, d_ff=256, num_features=10, buffer_size=256, num_components=5)
 B3, NC3, NT3 = 1024, 16384, 256
 B2, NC2, NT2 = 64, 512, 128
+CFG4 = dict(d_model=512, n_heads=16, n_layers=12, d_ff=256, num_features=21, buffer_size=256, num_components=5)
+B4, NC4, ROWS4, OUTS4 = 2048, 4096, 64, 4
+
+KIND_FLASH, KIND_STREAM_BUFFER, KIND_BUFFER, KIND_SMALL, KIND_LAYER = 0, 1, 2, 3, 4  # include/artab_bench.h
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def build_model(device, dtype):
+def build_model(device, dtype, cfg=CFG3):
     from ar_nanotabpfn_amd.model import ARTabPFN
 
     torch.manual_seed(0)
-    return ARTabPFN(**CFG3).eval().to(device=device, dtype=dtype)
+    return ARTabPFN(**cfg).eval().to(device=device, dtype=dtype)
 
 
 def gp_context(n, feats, seed, lengthscale=1.0, noise=0.05, n_rff=2048):
@@ -89,22 +107,86 @@ def decode_inputs(device, dtype):
     return x_context, y_context, x_target
 
 
-def run_decode(pred, x_context, y_context, x_target, steps, device, dtype):
-    """Prefill (untimed) + `steps` decode steps; returns (prefill_ms, decode_ms)."""
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
-    pred.init_kv_cache(B3, NT3, device, dtype)
+def config4_inputs(device, dtype):
+    """configs[4]: N_ctx=4096 context rows with x in R^20 and a 4-dim y from an independent random
+    tanh-MLP (20 -> 64 -> 64 -> 1) per output dimension; 64 target rows x 4 outputs.  The model is
+    scalar-y (ar_tabpfn/model/model.py:34, :310-312), so (row, output) pairs are flattened into
+    scalar rows: a row's features are its 20 x values and the output index as a 21st feature.
+    Context row i carries output i mod 4 and that output's y (N_ctx stays 4096, as the
+    configuration states); target step s is (row s // 4, output s mod 4): 256 sequential steps."""
+    g = torch.Generator().manual_seed(4)
+    F = 20
+    x_ctx = torch.randn(NC4, F, generator=g)
+    x_tgt = torch.randn(ROWS4, F, generator=g)
+    w1 = torch.randn(OUTS4, F, 64, generator=g) / F ** 0.5
+    w2 = torch.randn(OUTS4, 64, 64, generator=g) / 8.0
+    w3 = torch.randn(OUTS4, 64, 1, generator=g) / 8.0
+    y_all = (torch.tanh(torch.tanh(x_ctx @ w1) @ w2) @ w3).squeeze(-1).T  # [Nc, 4]
+    o_ctx = torch.arange(NC4) % OUTS4
+    y_ctx = y_all[torch.arange(NC4), o_ctx] + 0.1 * torch.randn(NC4, generator=g)
+    xc = torch.cat([x_ctx, o_ctx[:, None].float()], dim=1)
+    steps = torch.arange(ROWS4 * OUTS4)
+    xt = torch.cat([x_tgt[steps // OUTS4], (steps % OUTS4)[:, None].float()], dim=1)
+    x_context = xc.to(device, dtype).unsqueeze(0).expand(B4, -1, -1)
+    y_context = y_ctx.to(device, dtype).unsqueeze(0).expand(B4, -1)
+    x_target = xt.to(device, dtype).unsqueeze(0).expand(B4, -1, -1)
+    return x_context, y_context, x_target
+
+
+def prefill(pred, x_context, y_context, cap, device, dtype):
+    """Cache allocation + context prefill; returns the prefill's GPU time in ms."""
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    pred.init_kv_cache(x_context.shape[0], cap, device, dtype)
     torch.cuda.synchronize()
     ev[0].record()
     pred.prefill_context(x_context, y_context)
     ev[1].record()
     torch.cuda.synchronize()
+    return ev[0].elapsed_time(ev[1])
+
+
+def run_decode(pred, x_context, y_context, x_target, steps, device, dtype, cap=NT3):
+    """Prefill (untimed) + `steps` decode steps; returns (prefill_ms, decode_ms, host wall ms)."""
+    prefill_ms = prefill(pred, x_context, y_context, cap, device, dtype)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
     t0 = time.perf_counter()
-    ev[2].record()
+    ev[0].record()
     pred.decode_targets(x_target[:, :steps])
-    ev[3].record()
+    ev[1].record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
-    return ev[0].elapsed_time(ev[1]), ev[2].elapsed_time(ev[3]), wall_ms
+    return prefill_ms, ev[0].elapsed_time(ev[1]), wall_ms
+
+
+def observed_decode(pred, x_context, y_context, x_target, steps, device, dtype, cap=NT3):
+    """The decode run once more with the recorded step's launches issued live, one by one, through
+    the benchmark build of the library, every launch carrying events that receive its own start
+    and end time stamps.  Returns {kind: [ms per launch, in launch order]}; the prefill is outside
+    the observed region."""
+    from ar_nanotabpfn_amd import _lib
+
+    with _lib.benchmark_library() as bl:
+        pred.launch_live = True
+        try:
+            # a short run first: whatever this setting of the predictor still has to record is
+            # recorded here, unobserved (a launch that is being captured must not carry events)
+            run_decode(pred, x_context, y_context, x_target, min(steps, 12), device, dtype, cap)
+            prefill(pred, x_context, y_context, cap, device, dtype)
+            n_layers = len(pred.backbone.layers)
+            capacity = 5 * n_layers * (steps + 2) + 64
+            _lib.check(bl.artab_profile_begin(capacity))
+            pred.decode_targets(x_target[:, :steps])
+            ms = (ctypes.c_float * capacity)()
+            kinds = (ctypes.c_int * capacity)()
+            n = bl.artab_profile_end(ms, kinds, capacity)
+            if n < 0:
+                _lib.check(n)
+        finally:
+            pred.launch_live = False
+    out = {}
+    for i in range(min(n, capacity)):
+        out.setdefault(kinds[i], []).append(float(ms[i]))
+    return out
 
 
 def host_info():
@@ -129,16 +211,66 @@ def host_info():
             "blas_threads": blas}
 
 
-CPU_DECODE_B = 256            # trajectories of the CPU sample (a quarter of the batch; a step is linear in B)
+# ------------------------------------------------------------------------------------------------
+# host-CPU legs (the only users of oracle/ in this file, and only as the thing that is timed
+# beside the GPU, or as the exact value a GPU result is compared with)
+# ------------------------------------------------------------------------------------------------
+
+CPU_DECODE_B = 16             # trajectories of the CPU sample (a step is linear in B: 1/64 of the batch)
 CPU_DECODE_NBUF = (1, 128, 255)
 
 
-def cpu_decode_baseline(model, x_context, y_context, x_target, n_bufs=CPU_DECODE_NBUF, b_sample=CPU_DECODE_B):
-    """The numpy oracle (float32) on the host: one full 12-layer decode step of `b_sample`
-    trajectories at each buffer length in `n_bufs`, one warm-up and the median of three timed runs
-    each; the context K/V are random tensors of the right shape (the prefill is not part of the
-    timed GPU region either, and attention cost does not depend on values).  Returns seconds per
-    step of the FULL batch (the sample's median scaled by B / b_sample) averaged over `n_bufs`."""
+def cpu_decode_baseline(model, n_bufs=CPU_DECODE_NBUF, b_sample=CPU_DECODE_B):
+    """The reference's CPU path on the host: oracle/torch_cpu_path.py, a PyTorch restatement of
+    its op sequence (stride-0 expanded context K/V and materialised [B,H,Lq,Nc] scores,
+    triton_kernels.py:554-565; torch.cat of the buffer, inference.py:806-807; merge, :508-524;
+    head.sample), with torch.set_num_threads(os.cpu_count()).  One full 12-layer decode step
+    (autoregressive_decode with a buffer row, N_ctx=16384) of `b_sample` trajectories at each
+    buffer length in `n_bufs`: bf16 (the configuration's type) with 1 warm-up + median of 3, float32
+    for information at the middle length with 1 warm-up + 1.  The context K/V are random tensors
+    of the right shape (the prefill is outside the timed GPU region as well).  Returns, per dtype,
+    seconds per step of the FULL batch: the sample's time scaled by B / b_sample (every op of the
+    path is linear in the number of trajectories) and averaged over `n_bufs`."""
+    from oracle import torch_cpu_path as tp
+
+    torch.set_num_threads(os.cpu_count())
+    H, Dh, L = CFG3["n_heads"], CFG3["d_model"] // CFG3["n_heads"], CFG3["n_layers"]
+    res = {}
+    for dt, name, lens, reps in ((torch.bfloat16, "bf16", n_bufs, 3), (torch.float32, "f32", n_bufs[1:2], 1)):
+        tm = tp.TorchCpuModel(model.state_dict(), H, dt)
+        p = tp.TorchCpuPredictor(tm, "shared")
+        g = torch.Generator().manual_seed(0)
+        p.init_kv_cache(b_sample, NT3, context_len=NC3)
+        for i in range(L):
+            p.k_ctx[i].copy_(torch.randn(H, NC3, Dh, generator=g) * 0.5)
+            p.v_ctx[i].copy_(torch.randn(H, NC3, Dh, generator=g) * 0.5)
+            p.k_buf[i].copy_(torch.randn(b_sample, H, NT3, Dh, generator=g) * 0.5)
+            p.v_buf[i].copy_(torch.randn(b_sample, H, NT3, Dh, generator=g) * 0.5)
+        p.context_len = NC3
+        xt = torch.randn(b_sample, 2, CFG3["num_features"], generator=g).to(dt)
+        y_prev = torch.zeros(b_sample, 1, dtype=dt)
+        per_n = []
+        for n in lens:
+            times = []
+            for rep in range(reps + 1):  # the first run is the warm-up
+                p.buffer_len = n - 1
+                t0 = time.perf_counter()
+                with torch.no_grad():
+                    p.autoregressive_decode(xt[:, 1:2], xt[:, 0:1], y_prev, n % NT3)
+                if rep:
+                    times.append(time.perf_counter() - t0)
+            per_n.append(float(np.median(times)) * (B3 / b_sample))
+            log(f"[cpu] torch {name} decode step at n_buf={n}: median {np.median(times):.2f} s for {b_sample} "
+                f"trajectories -> {per_n[-1]:.1f} s for {B3} (extrapolated x{B3 // b_sample})")
+        res[name] = (float(np.mean(per_n)), per_n)
+    return res
+
+
+def cpu_decode_numpy(model, x_target, n_buf=128, b_sample=256):
+    """The numpy oracle in float32 (a port of the arithmetic, not of the op sequence: one einsum
+    per product, no expanded K/V): one decode step of `b_sample` trajectories at one buffer
+    length, 1 warm-up + 1 timed, scaled to the batch.  Kept next to the torch figure because it
+    is the faster CPU implementation of the two."""
     from oracle import model_oracle as mo
 
     sd = {k: v.detach().float().cpu().numpy() for k, v in model.state_dict().items()}
@@ -149,42 +281,108 @@ def cpu_decode_baseline(model, x_context, y_context, x_target, n_bufs=CPU_DECODE
     xt = x_target[:b_sample, :2].float().cpu().numpy()
     k_ctx = [rng.standard_normal((H, NC3, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
     v_ctx = [rng.standard_normal((H, NC3, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
-    per_n = []
-    for n in n_bufs:
-        k_buf = [rng.standard_normal((b_sample, H, n - 1, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
-        v_buf = [rng.standard_normal((b_sample, H, n - 1, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
-        emb = np.concatenate(
-            [om.embed_buffer(xt[:, 0:1], np.zeros((b_sample, 1), np.float32)) + om.ar_tokens[n % om.ar_tokens.shape[0]],
-             om.embed_target(xt[:, 1:2])], axis=1)
-        times = []
-        for rep in range(4):  # the first run is the warm-up
-            op.init_kv_cache(b_sample, NT3)
-            op.context_len, op.k_ctx, op.v_ctx = NC3, k_ctx, v_ctx
-            op.k_buf, op.v_buf, op.buffer_len = list(k_buf), list(v_buf), n - 1
-            t0 = time.perf_counter()
-            z = op.transformer_decode(emb, commit=1)
-            om.head_parameterize(z[:, -1:])
-            if rep:
-                times.append(time.perf_counter() - t0)
-        per_n.append(float(np.median(times)) * (B3 / b_sample))
-        log(f"[cpu] decode step at n_buf={n}: median {np.median(times):.2f} s for {b_sample} trajectories "
-            f"-> {per_n[-1]:.2f} s for {B3}")
-    return float(np.mean(per_n)), per_n
+    k_buf = [rng.standard_normal((b_sample, H, n_buf - 1, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
+    v_buf = [rng.standard_normal((b_sample, H, n_buf - 1, Dh), dtype=np.float32) * 0.5 for _ in range(L)]
+    emb = np.concatenate(
+        [om.embed_buffer(xt[:, 0:1], np.zeros((b_sample, 1), np.float32)) + om.ar_tokens[n_buf % om.ar_tokens.shape[0]],
+         om.embed_target(xt[:, 1:2])], axis=1)
+    t = 0.0
+    for rep in range(2):
+        op.init_kv_cache(b_sample, NT3)
+        op.context_len, op.k_ctx, op.v_ctx = NC3, k_ctx, v_ctx
+        op.k_buf, op.v_buf, op.buffer_len = list(k_buf), list(v_buf), n_buf - 1
+        t0 = time.perf_counter()
+        z = op.transformer_decode(emb, commit=1)
+        om.head_parameterize(z[:, -1:])
+        t = time.perf_counter() - t0
+    log(f"[cpu] numpy float32 decode step at n_buf={n_buf}: {t:.2f} s for {b_sample} trajectories")
+    return t * (B3 / b_sample)
 
 
-def log_density_bench(device, dtype, model, with_cpu):
-    from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
-
+def config2_data(device, dtype):
     g = torch.Generator().manual_seed(2)
     F = CFG3["num_features"]
     x = torch.randn(B2, NC2 + NT2, F, generator=g)
-    w1 = torch.randn(B2, F, 64, generator=g) / F**0.5
+    w1 = torch.randn(B2, F, 64, generator=g) / F ** 0.5
     w2 = torch.randn(B2, 64, 64, generator=g) / 8.0
     w3 = torch.randn(B2, 64, 1, generator=g) / 8.0
     y = (torch.tanh(torch.tanh(x @ w1) @ w2) @ w3).squeeze(-1) + 0.1 * torch.randn(B2, NC2 + NT2, generator=g)
     y = (y - y[:, :NC2].mean(1, keepdim=True)) / y[:, :NC2].std(1, keepdim=True)
     xd, yd = x.to(device, dtype), y.to(device, dtype)
-    args = (xd[:, :NC2], yd[:, :NC2], xd[:, NC2:], yd[:, NC2:])
+    return xd[:, :NC2], yd[:, :NC2], xd[:, NC2:], yd[:, NC2:]
+
+
+def log_density_accuracy(device, model, args, n_exact=16, n_f32=8):
+    """What the configs[2] log-density differs by from its exact value, nats per target.  Three
+    evaluations of the bf16 model on the first `n_exact` datasets: the product path (HIP attention,
+    fused layer kernels), the same model with float32 PyTorch attention and plain PyTorch layers
+    (oracle/torch_attention_f32.py), and the float64 numpy oracle on the same bf16 weights and
+    inputs (the exact value).  Then the same 12-layer model with float32 weights on `n_f32`
+    datasets through the device path against the float64 oracle: the case in which a tolerance of
+    1e-3 nats per target is well defined."""
+    import ar_nanotabpfn_amd.inference as inf
+    import ar_nanotabpfn_amd.model as model_mod
+    from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
+    from oracle import model_oracle as mo
+    from oracle import torch_attention_f32 as tref
+
+    def f64(t):
+        return t.detach().float().cpu().numpy().astype(np.float64)
+
+    def stats(a, b):
+        d = np.abs(a - b)
+        return {"mean": float(d.mean()), "p99": float(np.quantile(d, 0.99)), "max": float(d.max())}
+
+    sub = tuple(a[:n_exact] for a in args)
+    ll_hip = f64(ARTabPFNPredictor.from_trained_model(model, backend="flex_attention").evaluate_joint_density(*sub))
+
+    class Ref:  # the namespace the predictor calls, float32 attention inside
+        prefill_attention = staticmethod(tref.prefill_attention)
+        decode_attention = staticmethod(tref.decode_attention)
+        teacher_forcing_attention = staticmethod(tref.teacher_forcing_attention)
+        hybrid_teacher_forcing_attention = staticmethod(tref.hybrid_teacher_forcing_attention)
+
+    ak_saved, fus_saved = inf.ak, model_mod.layer_fusable
+    inf.ak, model_mod.layer_fusable = Ref, (lambda *a, **k: False)
+    try:
+        ll_f32attn = f64(ARTabPFNPredictor.from_trained_model(model, backend="flex_attention").evaluate_joint_density(*sub))
+    finally:
+        inf.ak, model_mod.layer_fusable = ak_saved, fus_saved
+    sd = {k: f64(v) for k, v in model.state_dict().items()}
+    om = mo.OracleModel(sd, CFG3["n_heads"])
+    ll_exact = mo.OraclePredictor(om, "per_dataset").evaluate_joint_density(*(f64(a) for a in sub))
+    res = {
+        "exact": "float64 numpy oracle on the same weights and inputs",
+        "bf16_model": {
+            "datasets": n_exact,
+            "hip_vs_exact": stats(ll_hip, ll_exact),
+            "f32attn_vs_exact": stats(ll_f32attn, ll_exact),
+            "hip_vs_f32attn": stats(ll_hip, ll_f32attn),
+        },
+    }
+    # the same architecture and data in float32 through the device path
+    model32 = build_model(device, torch.float32)
+    sub32 = tuple(a[:n_f32].float() for a in args)
+    ll32 = f64(ARTabPFNPredictor.from_trained_model(model32, backend="flex_attention").evaluate_joint_density(*sub32))
+    om32 = mo.OracleModel({k: f64(v) for k, v in model32.state_dict().items()}, CFG3["n_heads"])
+    ll32_exact = mo.OraclePredictor(om32, "per_dataset").evaluate_joint_density(*(f64(a) for a in sub32))
+    res["f32_model"] = {"datasets": n_f32, "hip_vs_exact": stats(ll32, ll32_exact)}
+    b = res["bf16_model"]
+    res["mean_abs_dlogp_hip_vs_f32attn"] = b["hip_vs_f32attn"]["mean"]
+    res["float32_attention_floor_mean_abs_dlogp"] = b["f32attn_vs_exact"]["mean"]
+    res["reading"] = (
+        "the 1e-3 nats/target tolerance is met by the float32 model through the device path (f32_model.hip_vs_exact); "
+        "a bf16 model cannot meet it with any attention kernel: with float32 attention the same bf16 model misses the "
+        "exact value by f32attn_vs_exact (8-bit rounding of every activation, twelve layers deep), and the HIP path "
+        "(hip_vs_exact) is no further from the exact value than that floor")
+    del model32
+    return res
+
+
+def log_density_bench(device, dtype, model, with_cpu):
+    from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
+
+    args = config2_data(device, dtype)
     pred = ARTabPFNPredictor.from_trained_model(model, backend="flex_attention")
     for _ in range(3):
         ll = pred.evaluate_joint_density(*args)
@@ -201,28 +399,167 @@ def log_density_bench(device, dtype, model, with_cpu):
     res = {"workload": "configs[2]: B=64 datasets x (512 context + 128 target rows), 12-layer d_model=256 bf16, "
                        "per-dataset contexts", "gpu_ms": round(gpu_ms, 3), "finite": bool(torch.isfinite(ll).all())}
     if with_cpu:
-        from oracle import model_oracle as mo
+        from oracle import torch_cpu_path as tp
 
-        # host leg: the numpy oracle in float32 on a bounded sample (the first 16 of the 64
-        # datasets; datasets are independent, so the evaluation is linear in their number), one
-        # warm-up and the median of three timed runs, scaled to the 64 datasets
-        sd = {k: v.detach().float().cpu().numpy() for k, v in model.state_dict().items()}
-        om = mo.OracleModel(sd, CFG3["n_heads"], compute=np.float32)
-        n_cpu = 16
-        a32 = [t[:n_cpu].float().cpu().numpy() for t in args]
-        times = []
-        for rep in range(4):
-            t0 = time.perf_counter()
-            ll_cpu = mo.OraclePredictor(om, "per_dataset").evaluate_joint_density(*a32)
-            if rep:
-                times.append(time.perf_counter() - t0)
-        cpu_s = float(np.median(times)) * (B2 / n_cpu)
-        d = np.abs(ll[:n_cpu].float().cpu().numpy() - ll_cpu)
-        res.update(cpu_s=round(cpu_s, 3), speedup=round(cpu_s * 1e3 / gpu_ms, 1),
-                   cpu_sample=f"numpy float32 oracle on {n_cpu} of the {B2} datasets, 1 warm-up + median of 3, x{B2 // n_cpu}",
-                   mean_abs_dlogp_vs_cpu_f32=float(d.mean()), max_abs_dlogp_vs_cpu_f32=float(d.max()))
-        log(f"[cpu] configs[2] log-density: {cpu_s:.2f} s for {B2} datasets (from {n_cpu})  (GPU {gpu_ms:.2f} ms)")
+        # host leg: the reference's per-dataset path restated in PyTorch (dense masked softmax over
+        # the full cache under the teacher-forcing mask, inference.py:422-471, :525-577), all 64
+        # datasets, torch.set_num_threads(os.cpu_count()); bf16 as the configuration specifies
+        # (1 warm-up + median of 3), float32 for information (1 warm-up + 1)
+        torch.set_num_threads(os.cpu_count())
+        cpu = {}
+        for dt, name, reps in ((torch.bfloat16, "bf16", 3), (torch.float32, "f32", 1)):
+            tm = tp.TorchCpuModel(model.state_dict(), CFG3["n_heads"], dt)
+            a_cpu = [t.to("cpu", dt) for t in args]
+            times = []
+            for rep in range(reps + 1):
+                t0 = time.perf_counter()
+                with torch.no_grad():
+                    ll_cpu = tp.TorchCpuPredictor(tm, "per_dataset").evaluate_joint_density(*a_cpu)
+                if rep:
+                    times.append(time.perf_counter() - t0)
+            cpu[name] = float(np.median(times))
+            log(f"[cpu] configs[2] log-density, torch {name}: {cpu[name]:.2f} s for {B2} datasets (GPU {gpu_ms:.2f} ms)")
+        res.update(cpu_s=round(cpu["bf16"], 3), cpu_s_f32=round(cpu["f32"], 3),
+                   speedup=round(cpu["bf16"] * 1e3 / gpu_ms, 1), speedup_vs_f32=round(cpu["f32"] * 1e3 / gpu_ms, 1),
+                   cpu_sample=f"oracle/torch_cpu_path.py (the reference's op sequence in PyTorch), all {B2} datasets, "
+                              f"{torch.get_num_threads()} threads; bf16: 1 warm-up + median of 3, float32: 1 warm-up + 1")
+        res["accuracy"] = log_density_accuracy(device, model, args)
     return res
+
+
+def config4_bench(device, observe=True):
+    """configs[4] end to end: the 12-layer d_model=512 / 16-head (head_dim 32) bf16 model, one shared
+    context of 4096 rows, B=2048 trajectories, 256 sequential scalar decode steps (config4_inputs
+    states the flattening).  Reports target-steps/s over the decode loop (prefill separately), the
+    context pass's fraction of the bf16 matrix peak, and the streaming buffer pass's HBM rate
+    (K and V rows of every trajectory and head, read once) against 8 TB/s."""
+    from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
+
+    dtype = torch.bfloat16
+    model = build_model(device, dtype, CFG4)
+    x_context, y_context, x_target = config4_inputs(device, dtype)
+    pred = ARTabPFNPredictor.from_trained_model(model, backend="triton_shared_context")
+    Nt = ROWS4 * OUTS4
+    torch.manual_seed(0)
+    run_decode(pred, x_context, y_context, x_target, 24, device, dtype, cap=Nt)
+    recorded = pred.graph_recordings
+    best = None
+    for _ in range(2):
+        r = run_decode(pred, x_context, y_context, x_target, Nt, device, dtype, cap=Nt)
+        best = r if best is None or r[1] < best[1] else best
+    if pred.graph_recordings != recorded:
+        sys.exit("bench.py: a HIP graph was recorded inside the timed region of the configs[4] leg")
+    prefill_ms, decode_ms, _ = best
+    H, Dh, L = CFG4["n_heads"], CFG4["d_model"] // CFG4["n_heads"], CFG4["n_layers"]
+    out = {
+        "workload": "configs[4] wide-head joint sampling: d_model=512, 16 heads (head_dim 32), 12 layers, bf16, shared context "
+                    "N_ctx=4096 (x in R^20 + output index as a 21st feature), B=2048 trajectories, 4 outputs x 64 target rows "
+                    "flattened into 256 sequential scalar decode steps (the reference model is scalar-y)",
+        "value": round(Nt / decode_ms * 1e3, 2), "unit": "target-steps/s", "steps": Nt,
+        "ms_per_step": round(decode_ms / Nt, 4), "prefill_ms": round(prefill_ms, 3),
+        "trajectory_steps_per_sec": round(Nt / decode_ms * 1e3 * B4, 1),
+    }
+    log(f"[config4] prefill {prefill_ms:.2f} ms; {Nt} decode steps in {decode_ms:.1f} ms = {out['value']} target-steps/s")
+    if observe:
+        obs = observed_decode(pred, x_context, y_context, x_target, Nt, device, dtype, cap=Nt)
+        ctx = obs.get(KIND_FLASH, [])
+        buf = obs.get(KIND_STREAM_BUFFER, [])
+        if len(ctx) == L * Nt and len(buf) == L * (Nt - 1):
+            ctx_ms = float(np.sum(ctx))
+            flops = 4.0 * B4 * H * NC4 * Dh * L * (1 + 2 * (Nt - 1))
+            # buffer pass of step t (t = 1 .. Nt-1) reads t-1 committed rows and the new one: t rows of K and V
+            row_bytes = 2.0 * B4 * H * Dh * 2
+            buf_by_step = np.asarray(buf).reshape(Nt - 1, L)
+            last = buf_by_step[-1].mean()
+            out.update({
+                "context_pass_avg_us": round(ctx_ms * 1e3 / len(ctx), 2),
+                "context_pass_frac": round(flops / (ctx_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                "buffer_pass_us_at_255_rows": round(float(last) * 1e3, 1),
+                "buffer_pass_gbs_at_255_rows": round(row_bytes * (Nt - 1) / (last * 1e-3) / 1e9, 1),
+                "buffer_pass_frac_of_hbm_peak_at_255_rows": round(row_bytes * (Nt - 1) / (last * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                "buffer_pass_gbs_whole_run": round(row_bytes * L * sum(range(1, Nt)) / (float(np.sum(buf)) * 1e-3) / 1e9, 1),
+                "layer_kernel_avg_us": round(float(np.mean(obs.get(KIND_LAYER, [0.0]))) * 1e3, 2),
+            })
+            log(f"[config4] context pass avg {out['context_pass_avg_us']} us ({out['context_pass_frac']} of peak); buffer pass "
+                f"at 255 rows {out['buffer_pass_us_at_255_rows']} us = {out['buffer_pass_gbs_at_255_rows']} GB/s")
+        else:
+            out["observed"] = f"unexpected launch counts: {len(ctx)} context passes, {len(buf)} buffer passes"
+    del pred, model
+    torch.cuda.empty_cache()
+    return out
+
+
+def reference_shapes(device):
+    """The shapes the reference's own benchmark scripts print figures for (it records none):
+    kernel K1 at (B, 8, 512, 64) fp16 with one query (ar_tabpfn/tests/test_triton_gpu.py:255-293,
+    :376-397) against the same product in plain PyTorch on the device (the script's own
+    comparison); predictor decode with fixed buffer values (:126-165, :399-479) and joint density
+    (tests/test_triton_joint_density.py:286-365) on a d_model=256 / 8-head / 8-layer fp16 model with
+    N_ctx=512, 32 targets, B in {1, 8, 64}, shared-context backend against the per-trajectory cache
+    backend.  Timed the way the scripts do: host wall clock around a synchronised call."""
+    import ar_nanotabpfn_amd.attention_kernels as ak
+    from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
+    from ar_nanotabpfn_amd.model import ARTabPFN
+
+    dt = torch.float16
+    rows = []
+
+    def wall(fn, iters, warm):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / iters * 1e3
+
+    def torch_context(q, k, v):  # pytorch_context_attention on the device (triton_kernels.py:549-567)
+        B = q.shape[0]
+        ke, ve = k.unsqueeze(0).expand(B, -1, -1, -1), v.unsqueeze(0).expand(B, -1, -1, -1)
+        s = torch.matmul(q, ke.transpose(-2, -1)) * q.shape[-1] ** -0.5
+        return torch.matmul(torch.softmax(s, dim=-1), ve), torch.logsumexp(s.float(), dim=-1)
+
+    for B, H, Nc, D in ((1, 8, 512, 64), (8, 8, 512, 64), (64, 8, 512, 64)):
+        torch.manual_seed(42)
+        q = torch.randn(B, H, 1, D, device=device, dtype=dt)
+        k, v = torch.randn(H, Nc, D, device=device, dtype=dt), torch.randn(H, Nc, D, device=device, dtype=dt)
+        ms = wall(lambda: ak.context_attention(q, k, v), 100, 10)
+        ms_t = wall(lambda: torch_context(q, k, v), 100, 10)
+        rows.append(dict(leg="kernel", B=B, H=H, Nc=Nc, Dh=D, ms=round(ms, 4), torch_ms=round(ms_t, 4)))
+        log(f"[reference shapes] kernel B={B:3d} H={H} N_ctx={Nc} D={D}: {ms:.3f} ms per call (host wall, 100 calls), "
+            f"plain PyTorch on the device {ms_t:.3f} ms")
+    Fe, Nc, Nt = 4, 512, 32
+    torch.manual_seed(0)
+    model = ARTabPFN(num_features=Fe, d_model=256, n_heads=8, n_layers=8, buffer_size=32, num_components=3).eval().to(device, dt)
+    for B in (1, 8, 64):
+        xc = torch.randn(1, Nc, Fe, device=device, dtype=dt).expand(B, -1, -1).contiguous()
+        yc = torch.randn(1, Nc, device=device, dtype=dt).expand(B, -1).contiguous()
+        xt, yt = torch.randn(B, Nt, Fe, device=device, dtype=dt), torch.randn(B, Nt, device=device, dtype=dt)
+        res = dict(B=B, Nc=Nc, Nt=Nt)
+        for backend, tag in (("triton_shared_context", "shared"), ("flex_attention", "per_trajectory")):
+            pred = ARTabPFNPredictor.from_trained_model(model, backend=backend)
+
+            def fixed_buffer_decode():
+                pred.init_kv_cache(B, Nt if tag == "shared" else Nc + Nt, device, dt)
+                pred.prefill_context(xc, yc)
+                outs = []
+                for t in range(Nt):
+                    tgt = pred.embedder.embed_target(xt[:, t:t + 1])
+                    if t == 0:
+                        emb, commit = tgt, 0
+                    else:
+                        buf = pred.embedder.embed_buffer(xt[:, t - 1:t], yt[:, t - 1:t]) + pred.ar_tokens[t % pred.ar_tokens.shape[0]]
+                        emb, commit = torch.cat([buf, tgt], dim=1), 1
+                    outs.append(pred.transformer_decode(emb, commit=commit)[:, -1:])
+                return torch.cat(outs, dim=1)
+
+            res[f"decode_{tag}_ms"] = round(wall(fixed_buffer_decode, 3, 1), 3)
+            res[f"sample_sequence_{tag}_ms"] = round(wall(lambda: pred.sample_sequence(xc, yc, xt), 3, 2), 3)
+            res[f"joint_density_{tag}_ms"] = round(wall(lambda: pred.evaluate_joint_density(xc, yc, xt, yt), 5, 2), 3)
+        rows.append(dict(leg="predictor", **res))
+        log(f"[reference shapes] predictor B={B:3d}: " + ", ".join(f"{k} {v}" for k, v in res.items() if k.endswith("_ms")))
+    print(json.dumps({"reference_shapes": rows}))
 
 
 # Measured with rocprofv3 (median over the decode launches): 10337.7 KiB x 2.0 fetched,
@@ -281,22 +618,25 @@ def kernel_shapes(device):
                 flops = 4.0 * B * H * Lq * (Nc + nn + (Lq - 1)) * Dh
                 byts = 2.0 * Dh * 2 * (H * Nc + B * H * (nn + (Lq - 1))) + 2.0 * 2 * B * H * Lq * Dh
                 out.append(dict(config=name, n_buf=nn, schedule=label, us=round(us, 1),
-                                tflops=round(flops / us / 1e6, 1), gbps=round(byts / us / 1e3, 1)))
+                                tflops=round(flops / us / 1e6, 1), gbps=round(byts / us / 1e3, 1),
+                                frac_of_hbm_peak=round(byts / us / 1e3 / HBM_PEAK_GBS, 4)))
                 log(f"[shape] {name} n_buf={nn:3d} {label:11s} {us:8.1f} us  {flops / us / 1e6:7.1f} TFLOP/s  "
-                    f"{byts / us / 1e3:7.1f} GB/s")
+                    f"{byts / us / 1e3:7.1f} GB/s ({byts / us / 1e3 / HBM_PEAK_GBS * 100:.1f} % of 8 TB/s)")
     print(json.dumps({"kernel_shapes": out}))
 
 
 def mix_ceiling(device):
     """The instruction mix of one 32x32 score block of the head_dim-32 kernel, issued from registers
-    with no memory traffic (``artab_bench_instruction_mix``): the rate the SIMD's issue port allows,
+    with no memory traffic (``artab_bench_instruction_mix`` of the benchmark library): the rate the SIMD's issue port allows,
     for the software-pipelined pass (row sum on v_dot2c) and the lean pass (row sum on the matrix
     pipe), on constant and on random operands, with two and four wavefronts per SIMD."""
-    import ctypes
-
     from ar_nanotabpfn_amd import _lib
 
-    lib = _lib.load()
+    with _lib.benchmark_library() as lib:
+        _mix_ceiling(device, lib, _lib)
+
+
+def _mix_ceiling(device, lib, _lib):
     iters = 20000
     names = {0: "pipelined pass: 4 mfma32 + 16 exp + 8 cvt + 8 dot2c", 1: "lean pass: 4 mfma32 + 2 mfma16 + 16 exp + 8 cvt",
              2: "matrix instructions of the lean pass alone", 3: "vector instructions of the lean pass alone"}
@@ -446,6 +786,8 @@ def main():
     ap.add_argument("--steps", type=int, default=NT3)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline legs")
+    ap.add_argument("--no-config4", action="store_true", help="skip the configs[4] leg of the default run")
+    ap.add_argument("--config4", action="store_true", help="only the configs[4] leg")
     ap.add_argument("--full-last-layer", action="store_true",
                     help="let the last layer of a decode step finish the buffer row too (its output is read by nobody)")
     ap.add_argument("--event-ordering", action="store_true",
@@ -462,6 +804,8 @@ def main():
                     help="only time one optimiser step of the reference's training configuration")
     ap.add_argument("--kernel-shapes", action="store_true",
                     help="only time one decode layer-step at the attention shapes of configs[1], [3], [4]")
+    ap.add_argument("--reference-shapes", action="store_true",
+                    help="only the shapes of the reference's own benchmark scripts (fp16, 8 layers, N_ctx 512, B in 1/8/64)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: trajectories are independent given the context, so more GPUs "
@@ -483,20 +827,18 @@ def main():
     from ar_nanotabpfn_amd import _lib
     from ar_nanotabpfn_amd.inference import ARTabPFNPredictor
 
-    lib = _lib.load()  # fails loudly when the extension is not built
-    if args.kernel_shapes:
-        kernel_shapes(torch.device("cuda:0"))
-        return
-    if args.mix_ceiling:
-        mix_ceiling(torch.device("cuda:0"))
-        return
-    if args.training_attention:
-        training_attention(torch.device("cuda:0"))
-        return
-    if args.training_step:
-        training_step(torch.device("cuda:0"))
-        return
+    _lib.load()  # fails loudly when the extension is not built
     device, dtype = torch.device("cuda:0"), torch.bfloat16
+    for flag, leg in ((args.kernel_shapes, kernel_shapes), (args.mix_ceiling, mix_ceiling),
+                      (args.training_attention, training_attention), (args.training_step, training_step),
+                      (args.reference_shapes, reference_shapes)):
+        if flag:
+            leg(device)
+            return
+    if args.config4:
+        print(json.dumps({"config4": config4_bench(device)}), flush=True)
+        return
+
     model = build_model(device, dtype)
     x_context, y_context, x_target = decode_inputs(device, dtype)
     pred = ARTabPFNPredictor.from_trained_model(model, backend="triton_shared_context")
@@ -520,41 +862,52 @@ def main():
     value = 1e3 / ms_per_step
     log(f"[gpu] prefill {prefill_ms:.2f} ms; {args.steps} decode steps in {decode_ms:.2f} ms "
         f"({ms_per_step:.3f} ms/step, host wall {wall_ms:.1f} ms)")
+    # the whole configuration (all 256 steps), whatever K is: same recorded graphs, replayed once more
+    if args.steps == NT3:
+        full_ms = decode_ms
+    else:
+        _, full_ms, _ = run_decode(pred, x_context, y_context, x_target, NT3, device, dtype)
+        if pred.graph_recordings != recorded:
+            sys.exit("bench.py: a HIP graph was recorded inside the 256-step run")
+    log(f"[gpu] all {NT3} decode steps in {full_ms:.2f} ms ({full_ms / NT3:.3f} ms/step)")
 
-    # instrumented re-run of the same steps: HIP events around every context-pass launch
-    import ctypes
-
-    # (launched kernel by kernel from Python: events cannot be recorded into a replayed graph)
-    pred.use_hip_graph = False
-    lib.artab_profile_begin(CFG3["n_layers"] * (args.steps + 1) + 64)
-    run_decode(pred, x_context, y_context, x_target, args.steps, device, dtype)
-    tot, cnt = ctypes.c_double(0.0), ctypes.c_int(0)
-    lib.artab_profile_end(ctypes.byref(tot), ctypes.byref(cnt))
-    # the same launches with the buffer pass after the context pass instead of beside it: the
-    # context-pass kernel with the chip to itself
-    pred.overlap_buffer_pass = False
-    lib.artab_profile_begin(CFG3["n_layers"] * (args.steps + 1) + 64)
-    run_decode(pred, x_context, y_context, x_target, args.steps, device, dtype)
-    tot_alone, cnt_alone = ctypes.c_double(0.0), ctypes.c_int(0)
-    lib.artab_profile_end(ctypes.byref(tot_alone), ctypes.byref(cnt_alone))
-    pred.overlap_buffer_pass = True
-    pred.use_hip_graph = True
-    # the first L launches are the prefill's dense passes, the first decode step has Lq=1
+    # Per-launch durations of the whole configuration: the launches of the recorded step issued
+    # live through the benchmark build of the library, each with its own start/end time stamps.
     H, Dh, L = CFG3["n_heads"], CFG3["d_model"] // CFG3["n_heads"], CFG3["n_layers"]
-    n_dec = cnt.value - L
-    # per-launch algorithmic flops: 4*B*H*Lq*Nc*Dh with Lq=1 for step 0 and 2 afterwards
-    flops_total = 4.0 * B3 * H * NC3 * Dh * L * (1 + 2 * (args.steps - 1))
-    # time of the decode launches = total - prefill launches; measure prefill launches separately
-    lib.artab_profile_begin(L + 8)
-    pred.init_kv_cache(B3, NT3, device, dtype)
-    pred.prefill_context(x_context, y_context)
-    ptot, pcnt = ctypes.c_double(0.0), ctypes.c_int(0)
-    lib.artab_profile_end(ctypes.byref(ptot), ctypes.byref(pcnt))
-    dec_kernel_ms = tot.value - ptot.value
-    alone_ms = tot_alone.value - ptot.value
-    avg_launch_us = dec_kernel_ms * 1e3 / max(n_dec, 1)
-    achieved = flops_total / (dec_kernel_ms * 1e-3) / 1e12 if dec_kernel_ms > 0 else 0.0
+    obs = observed_decode(pred, x_context, y_context, x_target, NT3, device, dtype)
+    ctx = np.asarray(obs.get(KIND_FLASH, []))
+    if len(ctx) != L * NT3:
+        sys.exit(f"bench.py: expected {L * NT3} context-pass launches in the observed run, saw {len(ctx)}")
+    ctx_by_step = ctx.reshape(NT3, L)  # ms; step 0 has one query per trajectory, the others two
+    buf_by_step = np.asarray(obs.get(KIND_STREAM_BUFFER, [])).reshape(NT3 - 1, L) if len(obs.get(KIND_STREAM_BUFFER, [])) == L * (NT3 - 1) else None
+    layer_ms = np.asarray(obs.get(KIND_LAYER, []))
+    # the same with the buffer pass after the context pass instead of beside it: the context-pass
+    # kernel with the chip to itself
+    pred.overlap_buffer_pass = False
+    alone = np.asarray(observed_decode(pred, x_context, y_context, x_target, NT3, device, dtype).get(KIND_FLASH, []))
+    pred.overlap_buffer_pass = True
+    flops_lq1 = 4.0 * B3 * H * NC3 * Dh
+
+    def frac_over(steps, by_step):
+        total_ms = float(by_step[:steps].sum())
+        flops = flops_lq1 * L * (1 + 2 * (steps - 1))
+        return flops / (total_ms * 1e-3) / 1e12, total_ms * 1e3 / (steps * L)
+
+    achieved, avg_launch_us = frac_over(args.steps, ctx_by_step)
+    achieved_full, avg_launch_us_full = frac_over(NT3, ctx_by_step)
+    alone_by_step = alone.reshape(NT3, L) if len(alone) == L * NT3 else None
+    achieved_alone, avg_alone_us = frac_over(NT3, alone_by_step) if alone_by_step is not None else (None, None)
+
+    # prefill launches (dense pass over the context), observed on their own
+    with _lib.benchmark_library() as bl:
+        pred.init_kv_cache(B3, NT3, device, dtype)
+        _lib.check(bl.artab_profile_begin(L + 8))
+        pred.prefill_context(x_context, y_context)
+        pms, pk = (ctypes.c_float * (L + 8))(), (ctypes.c_int * (L + 8))()
+        pn = bl.artab_profile_end(pms, pk, L + 8)
+    prefill_kernel_ms = sum(pms[i] for i in range(max(pn, 0)) if pk[i] == KIND_FLASH)
     prefill_flops = 4.0 * H * NC3 * NC3 * Dh * L
+
     roofline = {
         "kernel": "flash_kernel<bf16,32> context pass of artab_decode_attention",
         "bound": "mfma",
@@ -566,16 +919,32 @@ def main():
         # rocprofv3 --pmc runs of this script, the factors from the same counters on a 256 MiB copy
         # (--copy-calibration); algorithmic: K/V 16.8 MB + Q 1.0 MB read, 8.9 MB of partials written.
         "traffic": CONTEXT_PASS_HBM_BYTES,
-        "launches": n_dec,
+        "launches": int(args.steps * L),
         "avg_launch_us": round(avg_launch_us, 2),
+        "timing": "the launch's own start/end time stamps (hipExtLaunchKernelGGL events), launches of the recorded step "
+                  "issued live on the same two streams with the same ordering; steps 0..K-1",
         # In the timed schedule the buffer pass of the same layer runs beside this kernel and takes
-        # issue slots from it; these two are the kernel without that neighbour.
-        "avg_launch_us_alone": round(alone_ms * 1e3 / max(n_dec, 1), 2),
-        "frac_alone": round(flops_total / (alone_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4) if alone_ms > 0 else None,
-        "flops_per_launch_lq2": 4.0 * B3 * H * 2 * NC3 * Dh,
-        "prefill_tflops": round(prefill_flops / (ptot.value * 1e-3) / 1e12, 2) if ptot.value > 0 else None,
+        # issue slots from it; these two are the kernel without that neighbour (all 256 steps).
+        "avg_launch_us_alone": round(avg_alone_us, 2) if avg_alone_us else None,
+        "frac_alone": round(achieved_alone / MFMA_BF16_PEAK_TFLOPS, 4) if achieved_alone else None,
+        "flops_per_launch_lq2": 2 * flops_lq1,
+        "prefill_tflops": round(prefill_flops / (prefill_kernel_ms * 1e-3) / 1e12, 2) if prefill_kernel_ms > 0 else None,
     }
-    log(f"[gpu] context-pass kernel: {n_dec} launches, avg {avg_launch_us:.1f} us, {achieved:.1f} TFLOP/s")
+    log(f"[gpu] context-pass kernel: avg {avg_launch_us:.1f} us over steps 0..{args.steps - 1} ({achieved:.1f} TFLOP/s), "
+        f"{avg_launch_us_full:.1f} us over all {NT3} steps ({achieved_full:.1f} TFLOP/s), alone {avg_alone_us} us")
+    marks = [t for t in (1, 16, 64, 128, 192, 255) if t < NT3]
+    full_run = {
+        "steps": NT3,
+        "value": round(NT3 / full_ms * 1e3, 2),
+        "unit": "target-steps/s",
+        "ms_per_step": round(full_ms / NT3, 4),
+        "context_pass_avg_us": round(avg_launch_us_full, 2),
+        "context_pass_frac": round(achieved_full / MFMA_BF16_PEAK_TFLOPS, 4),
+        "context_pass_us_by_step": {str(t): round(float(ctx_by_step[t].mean()) * 1e3, 1) for t in marks},
+        "buffer_pass_us_by_step": ({str(t): round(float(buf_by_step[t - 1].mean()) * 1e3, 1) for t in marks}
+                                   if buf_by_step is not None else None),
+        "layer_kernel_avg_us": round(float(layer_ms.mean()) * 1e3, 2) if len(layer_ms) else None,
+    }
 
     out = {
         "metric": "ar_decode_target_steps_per_sec",
@@ -607,27 +976,49 @@ def main():
         if pred._graph_state is not None else None,
         "prefill_ms": round(prefill_ms, 3),
         "roofline": roofline,
+        "full_run": full_run,
     }
 
     if not args.no_cpu:
-        cpu_s, per_n = cpu_decode_baseline(model, x_context, y_context, x_target)
+        cpu = cpu_decode_baseline(model)
         host = host_info()
+        cpu_s, per_n = cpu["bf16"]
         out["cpu_baseline"] = {
-            "value": round(1.0 / cpu_s, 4),
+            "value": round(1.0 / cpu_s, 5),
             "unit": "target-steps/s",
-            "cores": host["blas_threads"] or host["torch_threads"],
+            "cores": host["torch_threads"],
             "kind": "port",
-            "dtype": "f32",
-            "sample": f"numpy float32 oracle (a port of the reference's arithmetic), one full 12-layer decode step "
-                      f"(N_ctx=16384) of {CPU_DECODE_B} of the {B3} trajectories at each of N_buf={list(CPU_DECODE_NBUF)}: "
-                      f"1 warm-up + median of 3, scaled x{B3 // CPU_DECODE_B} to the batch, mean over N_buf; "
-                      f"context K/V random (the prefill is outside the timed GPU region as well)",
-            "seconds_per_step_by_n_buf": [round(t, 3) for t in per_n],
+            "dtype": "bf16",
+            "sample": f"oracle/torch_cpu_path.py: the reference's op sequence in PyTorch (stride-0 expanded context K/V, "
+                      f"materialised [B,H,Lq,Nc] scores, torch.cat of the buffer, LSE merge, head.sample), one full 12-layer "
+                      f"decode step (N_ctx=16384) of {CPU_DECODE_B} of the {B3} trajectories at each of "
+                      f"N_buf={list(CPU_DECODE_NBUF)}: 1 warm-up + median of 3; EXTRAPOLATED x{B3 // CPU_DECODE_B} to the "
+                      f"batch (every op is linear in the number of trajectories), mean over N_buf; context K/V random (the "
+                      f"prefill is outside the timed GPU region as well)",
+            "seconds_per_step_by_n_buf": [round(t, 2) for t in per_n],
+            "float32_value": round(1.0 / cpu["f32"][0], 5),
+            "float32_seconds_per_step_at_n_buf_128": round(cpu["f32"][1][0], 2),
             "host": host,
+        }
+        np_s = cpu_decode_numpy(model, x_target)
+        out["cpu_baseline_numpy"] = {
+            "value": round(1.0 / np_s, 4), "unit": "target-steps/s", "kind": "port", "dtype": "f32",
+            "cores": host["blas_threads"] or host["torch_threads"],
+            "sample": "numpy float32 oracle (same arithmetic, one einsum per product instead of the reference's op "
+                      "sequence), one decode step of 256 of the 1024 trajectories at N_buf=128, 1 warm-up + 1 timed, "
+                      "EXTRAPOLATED x4 to the batch",
         }
     else:
         out["cpu_baseline"] = None
     out["log_density"] = log_density_bench(device, dtype, model, with_cpu=not args.no_cpu)
+    if not args.no_config4:
+        del pred
+        for layer in model.backbone.layers:  # the caches live on the layer modules (3.2 GB)
+            for name in ("k_ctx_cache", "v_ctx_cache", "k_buf_cache", "v_buf_cache", "k_cache", "v_cache"):
+                if hasattr(layer, name):
+                    delattr(layer, name)
+        torch.cuda.empty_cache()
+        out["config4"] = config4_bench(device)
     print(json.dumps(out), flush=True)
 
 

@@ -35,8 +35,12 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* the library is built with hidden visibility; what is declared here is what it exports */
+#if defined(__GNUC__) || defined(__clang__)
+#pragma GCC visibility push(default)
+#endif
 
-#define ARTAB_VERSION 6
+#define ARTAB_VERSION 7
 
 typedef enum artab_dtype {
     ARTAB_BF16 = 0,
@@ -75,33 +79,20 @@ const char *artab_status_string(int status);
 const char *artab_last_error(void);
 
 /*
- * Benchmark aid without a counterpart in the reference (which times whole calls with
- * perf_counter + synchronize, tests/test_triton_gpu.py:255-293).  Between
- * artab_profile_begin and artab_profile_end every launch of the MFMA attention kernel
- * (context pass of artab_context_attention / artab_decode_attention, teacher forcing,
- * prefill) is bracketed by a pair of HIP events on its stream; _end waits for them and
- * returns the summed kernel time and the number of launches.  These two calls create
- * events and synchronise, unlike every other entry point; not thread-safe.
+ * Route and tile-size overrides, for tests and tuning; no counterpart in the reference, and a
+ * drop-in caller never needs them.  Each key is also the name of an environment variable that is
+ * read ONCE, when the library is loaded; afterwards only artab_tuning_set changes a value, so the
+ * environment of the host process cannot change a kernel route between two calls.  Keys:
+ * ARTAB_BM, ARTAB_SPLIT, ARTAB_SMALL, ARTAB_STREAM, ARTAB_STREAM_PER_CU, ARTAB_STREAM_PRIO,
+ * ARTAB_STREAM_SHORT, ARTAB_DENSE_BELOW, ARTAB_ORDER_GATE_LAUNCH, ARTAB_BN, ARTAB_LEAN,
+ * ARTAB_LEAN_OCC, ARTAB_NW, ARTAB_TILE_ROWS (what each selects: csrc/launchers.h).
+ *   artab_tuning_set: enable != 0 sets the override to `value`, enable == 0 removes it (the
+ *                     library's own choice applies again).  Not thread-safe against running calls.
+ *   artab_tuning_get: returns 1 if an override is set (its value in *value), 0 if not.
+ * Both return ARTAB_ERR_UNSUPPORTED for an unknown key.
  */
-int artab_profile_begin(int max_records);
-int artab_profile_end(double *total_ms, int *records);
-
-/*
- * Benchmark aid without a counterpart in the reference: the instruction mix of one 32x32 score
- * block of the head_dim-32 attention kernel (ar_tabpfn/model/triton_kernels.py:131-162 is the
- * loop it stands for), issued from registers with no memory traffic, to measure what the SIMD's
- * issue port alone allows.  `workgroups` workgroups of four wavefronts run `iters` (even)
- * iterations; `lds_bytes` of dynamic LDS per workgroup fixes how many share a compute unit.
- *   variant 0: 4 MFMA 32x32x16 + 16 exp2 + 8 cvt_pk + 8 dot2c    (software-pipelined pass)
- *   variant 1: 4 MFMA 32x32x16 + 2 MFMA 16x16x32 + 16 exp2 + 8 cvt_pk   (lean pass)
- *   variant 2: the matrix instructions of variant 1 alone; 3: its vector instructions alone
- * random_data != 0 fills the operands with pseudo-random bf16 values instead of constants.
- *   out     float32 [workgroups * 256] (written, contents meaningless)
- *   stamps  uint64 [workgroups * 4][2] or NULL: per wavefront, shader cycles and 100 MHz ticks spent
- * The call only launches on `stream`; the caller times it.
- */
-int artab_bench_instruction_mix(int variant, int random_data, int workgroups, int iters, size_t lds_bytes,
-                                float *out, unsigned long long *stamps, void *stream);
+int artab_tuning_set(const char *name, int value, int enable);
+int artab_tuning_get(const char *name, int *value);
 
 /* Bytes of workspace the split-context paths need for the given problem
  * (artab_context_attention, artab_decode_attention).  0 means no workspace is
@@ -562,6 +553,9 @@ int artab_layer_post_pre_from_partials(const artab_attention_partials *partials,
                                        void *next_y, void *next_qkv,
                                        int64_t rows, int D, int F, int dtype, void *stream);
 
+#if defined(__GNUC__) || defined(__clang__)
+#pragma GCC visibility pop
+#endif
 #ifdef __cplusplus
 }
 #endif

@@ -1,10 +1,14 @@
-"""float32 PyTorch restatement of the attention entry points (TEST INFRASTRUCTURE).
+"""float32 PyTorch restatement of the attention entry points (TEST INFRASTRUCTURE ONLY — never
+imported by the shipped package).
 
 Same call signatures as ``ar_nanotabpfn_amd.attention_kernels``; every function
-up-casts to float32, evaluates one masked softmax over the concatenated key set and
-returns the input dtype.  It lets an end-to-end test run the same PyTorch-ROCm
-model twice on the same device, changing nothing but the attention implementation.
-It is itself checked against the numpy oracle in tests/test_predictor_gpu.py.
+up-casts to float32, evaluates one masked softmax over the concatenated key set
+(triton_kernels.py:204-240 is the reference's own statement of that equivalence) and
+returns the input dtype.  It lets an end-to-end test, and the log-density leg of
+bench.py, run the same PyTorch-ROCm model twice on the same device, changing nothing
+but the attention implementation: what is left between the two runs is the attention
+kernels' own error, and what both miss the float64 oracle by is the model's 16-bit
+rounding.  It is itself checked against the numpy oracle in tests/test_predictor_gpu.py.
 """
 
 import torch

@@ -19,3 +19,20 @@ def device():
     if not torch.cuda.is_available():
         pytest.skip("no HIP device")
     return torch.device("cuda:0")
+
+
+@pytest.fixture
+def tuning():
+    """``tuning(ARTAB_SMALL=0)``: route overrides of the loaded library (artab_tuning_set) for the
+    duration of one test; the state found before the test is restored afterwards."""
+    from ar_nanotabpfn_amd import _lib
+
+    saved = {}
+
+    def set_overrides(**overrides):
+        for key in overrides:
+            saved.setdefault(key, _lib.tuning.get(key))
+        _lib.tuning.set(**overrides)
+
+    yield set_overrides
+    _lib.tuning.set(**saved)

@@ -13,7 +13,7 @@ import pytest
 import torch
 
 from oracle import model_oracle as mo
-from tests import torch_attention_ref as tref
+from oracle import torch_attention_f32 as tref
 from tests.helpers import max_abs, to_np
 
 pytestmark = pytest.mark.gpu

@@ -20,17 +20,58 @@ def _lib():
     return _lib
 
 
+def _declared(header_name):
+    header = open(os.path.join(ROOT, "include", header_name)).read()
+    return set(re.findall(r"\b(artab_[a-z_]+)\s*\(", header)) - {"artab_view"}
+
+
+def _exported(path):
+    import subprocess
+
+    out = subprocess.run(["nm", "-D", "--defined-only", path], check=True, capture_output=True, text=True).stdout
+    return {line.split()[-1] for line in out.splitlines() if line.strip()}
+
+
 def test_library_exports_every_declared_symbol():
     L = _lib()
-    header = open(os.path.join(ROOT, "include", "artab_attention.h")).read()
-    declared = set(re.findall(r"\b(artab_[a-z_]+)\s*\(", header))
-    declared -= {"artab_view"}
+    declared = _declared("artab_attention.h")
     assert declared == set(L.SIGNATURES), (declared ^ set(L.SIGNATURES))
     lib = L.load()
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.artab_version() == L.ABI_VERSION == 6
+    assert lib.artab_version() == L.ABI_VERSION == 7
     assert lib.artab_status_string(0) == b"ok"
+
+
+def test_drop_in_library_exports_nothing_but_the_declared_abi():
+    """The drop-in library exports exactly the functions of include/artab_attention.h: no
+    benchmark aid, no C++ symbol.  The benchmark library adds those of include/artab_bench.h."""
+    L = _lib()
+    assert _exported(L.LIB_PATH) == _declared("artab_attention.h")
+    bench_only = _declared("artab_bench.h")
+    assert bench_only == set(L.BENCH_SIGNATURES)
+    assert _exported(L.BENCH_LIB_PATH) == _declared("artab_attention.h") | bench_only
+    for name in bench_only:
+        assert not hasattr(L.load(), name)
+
+
+def test_tuning_overrides_are_explicit_and_restorable(monkeypatch):
+    """Route overrides are set through the ABI; the environment is read when the library is
+    loaded and never again."""
+    L = _lib()
+    lib = L.load()
+    assert lib.artab_tuning_set(b"ARTAB_NO_SUCH_KEY", 1, 1) == L.ARTAB_ERR_UNSUPPORTED
+    for key in L.TUNING_KEYS:
+        assert L.tuning.get(key) is None or key in os.environ
+    monkeypatch.setenv("ARTAB_SMALL", "0")  # after the load: must not be seen
+    if "ARTAB_SMALL" not in os.environ or L.tuning.get("ARTAB_SMALL") is None:
+        assert L.tuning.get("ARTAB_SMALL") is None
+    with L.tuning(ARTAB_TILE_ROWS=32, ARTAB_DENSE_BELOW=0):
+        assert L.tuning.get("ARTAB_TILE_ROWS") == 32 and L.tuning.get("ARTAB_DENSE_BELOW") == 0
+        with L.tuning(ARTAB_TILE_ROWS=None):
+            assert L.tuning.get("ARTAB_TILE_ROWS") is None
+        assert L.tuning.get("ARTAB_TILE_ROWS") == 32
+    assert L.tuning.get("ARTAB_TILE_ROWS") is None and L.tuning.get("ARTAB_DENSE_BELOW") is None
 
 
 def test_workspace_query_is_host_only():

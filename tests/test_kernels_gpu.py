@@ -159,10 +159,10 @@ def _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, use_mfma,
 
 
 @pytest.fixture(params=[1, 0], ids=["one-launch", "general-route"])
-def small_route(request, monkeypatch):
+def small_route(request, tuning):
     """Small decode problems take a single-launch kernel (ARTAB_SMALL, on by default); with it
     switched off the same call goes through the context pass, the buffer pass and their merge."""
-    monkeypatch.setenv("ARTAB_SMALL", str(request.param))
+    tuning(ARTAB_SMALL=request.param)
     return request.param
 
 
@@ -216,12 +216,12 @@ def test_decode_attention_overlapped_matches_oracle(device, small_route, dtype, 
 
 
 @pytest.fixture(params=["0", "100000", "20", None], ids=["16-row-chunks", "4-row-chunks", "switch-at-20-rows", "by-length"])
-def stream_chunk_shape(request, monkeypatch):
+def stream_chunk_shape(request, tuning):
     """The streaming buffer pass reads 4 rows of 16 pairs or 16 rows of 4 pairs per request and
     picks by buffer length (ARTAB_STREAM_SHORT: the longest buffer that takes the first shape)."""
-    monkeypatch.setenv("ARTAB_SMALL", "0")
+    tuning(ARTAB_SMALL=0)
     if request.param is not None:
-        monkeypatch.setenv("ARTAB_STREAM_SHORT", request.param)
+        tuning(ARTAB_STREAM_SHORT=int(request.param))
     return request.param
 
 
@@ -360,7 +360,7 @@ def test_decode_attention_config3_full_size(device, n_buf):
     _full_size_decode(device, 1024, 8, 16384, n_buf, 256, seed=3 + n_buf)
 
 
-def test_context_pass_tile_loop_forms_agree_bit_for_bit(device, monkeypatch):
+def test_context_pass_tile_loop_forms_agree_bit_for_bit(device, tuning):
     """Beside a buffer pass the context pass runs the bulk of its tile loop as straight-line code
     while the committed buffer is short and tile by tile beyond (``ARTAB_DENSE_BELOW`` rows, read
     with the length on the device): the same products in the same order, so the partial slots are
@@ -375,7 +375,7 @@ def test_context_pass_tile_loop_forms_agree_bit_for_bit(device, monkeypatch):
     side = torch.cuda.Stream(device=device)
     outs = []
     for limit in ("1", "100000"):
-        monkeypatch.setenv("ARTAB_DENSE_BELOW", limit)
+        tuning(ARTAB_DENSE_BELOW=int(limit))
         parts = ak.decode_attention(q, k_ctx, v_ctx, k_cache.clone(), v_cache.clone(), cap - 1, k_new, v_new,
                                     side_stream=side, leave_partials=True, n_buf_device=nbuf)
         outs.append(parts.merged())
@@ -428,6 +428,23 @@ def test_decode_attention_config1_shape(device, small_route, n_buf):
 def test_decode_attention_long_context_split(device):
     """Many context slices + buffer pass + merge (the configs[3] schedule, smaller)."""
     _decode_case(device, torch.bfloat16, 128, 8, 2, 8192, 32, 100, 128, True, True, scale=0.6)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,Lq,Nc,D", [(64, 2, 8192, 32), (40, 1, 4200, 64), (300, 2, 2048, 32)])
+@pytest.mark.parametrize("cache", ["none", "zero-rows"])
+def test_decode_attention_split_context_without_any_buffer(device, dtype, B, Lq, Nc, D, cache):
+    """A shared context long enough to be cut into slices, no committed buffer row and no new
+    row, with no cache at all or one that holds zero rows: the call is context attention
+    (tests/test_triton_kernel.py:319-339 on the split route) and must not touch the cache."""
+    ak = _ak()
+    H = 8
+    q, k, v = _ctx_inputs(B, H, Lq, Nc, D, dtype, seed=11, scale=0.5)
+    kb = None if cache == "none" else torch.empty(B, H, 0, D, dtype=dtype, device=device)
+    out = ak.decode_attention(q.to(device), k.to(device), v.to(device), kb, kb, 0)
+    ref, _ = ao.context_attention(to_np(q), to_np(k), to_np(v))
+    assert out.shape == (B, H, Lq, D) and out.dtype == dtype
+    assert max_abs(to_np(out), ref) <= out_tol(dtype)
 
 
 def test_hybrid_attention_empty_buffer_is_context_only(device):
@@ -763,10 +780,10 @@ def _mk_norm(D, seed, dtype):
 
 
 @pytest.fixture(params=[16, 32])
-def tile_rows(request, monkeypatch):
+def tile_rows(request, tuning):
     """Both tile shapes of the layer kernels (token rows per workgroup): the library picks by row
     count, ARTAB_TILE_ROWS forces one."""
-    monkeypatch.setenv("ARTAB_TILE_ROWS", str(request.param))
+    tuning(ARTAB_TILE_ROWS=request.param)
     return request.param
 
 
@@ -1074,7 +1091,7 @@ def test_layer_post_pre_falls_back_when_not_covered(device):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,H,Lq,Nc,n_buf,cap", [(64, 4, 2, 4096, 9, 16), (33, 8, 2, 2048, 0, 8), (40, 8, 1, 4096, 5, 8)])
-def test_decode_partials_merged_in_layer_kernel(device, monkeypatch, tile_rows, dtype, B, H, Lq, Nc, n_buf, cap):
+def test_decode_partials_merged_in_layer_kernel(device, tuning, tile_rows, dtype, B, H, Lq, Nc, n_buf, cap):
     """decode_attention(leave_partials=True) + the layer kernels that merge the partials while
     loading, against the merged attention output fed to the same kernels: the merge is the same
     arithmetic rounded at the same point, so the results must agree bit for bit.  (Both legs on the
@@ -1082,7 +1099,7 @@ def test_decode_partials_merged_in_layer_kernel(device, monkeypatch, tile_rows, 
     from ar_nanotabpfn_amd import attention_kernels as ak
     from ar_nanotabpfn_amd import model as m
 
-    monkeypatch.setenv("ARTAB_SMALL", "0")
+    tuning(ARTAB_SMALL=0)
 
     D, Dh, F = 32 * H, 32, 256
     torch.manual_seed(2)
@@ -1125,7 +1142,7 @@ def test_decode_partials_merged_in_layer_kernel(device, monkeypatch, tile_rows, 
     (21, 512, 256, 16, 200, 2, 8, True),     # matrices deeper than the prefetch window
     (40, 128, 128, 4, 64, 0, 8, False),      # attention output given as a tensor (first target: context only)
 ])
-def test_decode_step_boundary_equals_its_three_launches(device, monkeypatch, dtype, B, D, F, H, Nc, n_buf, cap, partials):
+def test_decode_step_boundary_equals_its_three_launches(device, tuning, dtype, B, D, F, H, Nc, n_buf, cap, partials):
     """artab_decode_step_boundary against artab_layer_post(_from_partials) on the target rows,
     artab_decode_sample_embed and artab_layer_pre launched one after the other: predictions,
     embedding, the next step's feature stage and projections, and the loop counters, bit for bit."""
@@ -1133,7 +1150,7 @@ def test_decode_step_boundary_equals_its_three_launches(device, monkeypatch, dty
     from ar_nanotabpfn_amd import model as m
     from ar_nanotabpfn_amd.glue import DecodeStepBoundary, SampleEmbedStep
 
-    monkeypatch.setenv("ARTAB_SMALL", "0")
+    tuning(ARTAB_SMALL=0)
     Dh, Nt, K = D // H, 6, 5
     assert Dh == 32
     torch.manual_seed(4)
@@ -1259,12 +1276,12 @@ def test_queue_order_argument_checks(device):
 
 @pytest.mark.parametrize("absorb", [False, True])
 @pytest.mark.parametrize("B,H,Nc,cap", [(64, 8, 2048, 8), (600, 8, 1024, 12)])
-def test_decode_attention_ordered_by_counters_equals_event_ordered(device, monkeypatch, B, H, Nc, cap, absorb):
+def test_decode_attention_ordered_by_counters_equals_event_ordered(device, tuning, B, H, Nc, cap, absorb):
     """A run of decode steps whose two streams are ordered by device-side counters (one fork
     before the first call, one join after the last) against the same steps ordered by two events
     per call: same partials (bit for bit after the merge), same cache, no wait timed out."""
     ak = _ak()
-    monkeypatch.setenv("ARTAB_SMALL", "0")  # the event-ordered leg on the two-stream route as well
+    tuning(ARTAB_SMALL=0)  # the event-ordered leg on the two-stream route as well
     dtype, D = torch.bfloat16, 32
     q0, k_ctx, v_ctx = (t.to(device) for t in _ctx_inputs(B, H, 2, Nc, D, dtype, seed=1, scale=0.6))
     k_ref, v_ref = torch.zeros((B, H, cap, D), device=device, dtype=dtype), torch.zeros((B, H, cap, D), device=device, dtype=dtype)
@@ -1300,7 +1317,7 @@ def test_decode_attention_ordered_by_counters_equals_event_ordered(device, monke
 
 @pytest.mark.parametrize("gate_launch", [0, 1])
 @pytest.mark.parametrize("B,H,Nc,cap", [(64, 4, 4096, 8), (200, 8, 1024, 6)])
-def test_layer_kernels_wait_for_the_side_queue_themselves(device, monkeypatch, tile_rows, gate_launch, B, H, Nc, cap):
+def test_layer_kernels_wait_for_the_side_queue_themselves(device, tuning, tile_rows, gate_launch, B, H, Nc, cap):
     """Three layers of a decode step whose streams are ordered by counters, with the main
     stream's wait done by the layer kernels themselves (they wait for the buffer pass before
     they read the partials), repeated for several steps, against the event-ordered launches: bit
@@ -1309,7 +1326,7 @@ def test_layer_kernels_wait_for_the_side_queue_themselves(device, monkeypatch, t
     from ar_nanotabpfn_amd import attention_kernels as ak
     from ar_nanotabpfn_amd import model as m
 
-    monkeypatch.setenv("ARTAB_ORDER_GATE_LAUNCH", str(gate_launch))
+    tuning(ARTAB_ORDER_GATE_LAUNCH=gate_launch)
     dtype, Dh, F, n_layers = torch.bfloat16, 32, 128, 3
     D = H * Dh
     torch.manual_seed(3)
