@@ -146,6 +146,8 @@ SIGNATURES = {
 BENCH_SIGNATURES = {
     "artab_profile_begin": (_i, [_i]),
     "artab_profile_end": (_i, [ctypes.POINTER(_f), ctypes.POINTER(_i), _i]),
+    "artab_stamps_begin": (_i, [_i]),
+    "artab_stamps_end": (_i, [ctypes.POINTER(_f), _i]),
     "artab_bench_instruction_mix": (_i, [_i, _i, _i, _i, _sz, _p, _p, _p]),
 }
 

@@ -18,13 +18,28 @@ struct ObserverState {
 };
 static ObserverState g_obs;
 
-bool observe_launch(int kind, LaunchTiming *timing) {
-    if (!g_obs.enabled || g_obs.used >= g_obs.capacity) return false;
+// In-kernel time stamps of the matrix-core attention launches: device memory that the launches
+// (also recorded ones: a graph keeps the pointer) write into.  Never freed, so that a graph
+// recorded while stamps were on stays valid for the life of the process.
+struct StampState {
+    bool enabled = false;
+    unsigned long long *dev = nullptr;
+    int capacity = 0;
+};
+static StampState g_stamps;
+
+int observe_launch(int kind, LaunchTiming *timing) {
+    if (g_stamps.enabled && kind == kLaunchFlash) {
+        timing->stamps = g_stamps.dev;
+        timing->stamps_capacity = g_stamps.capacity;
+        return kObserveStamps;
+    }
+    if (!g_obs.enabled || g_obs.used >= g_obs.capacity) return 0;
     const int slot = g_obs.used++;
     g_obs.kind[slot] = kind;
     timing->start = g_obs.start[slot];
     timing->stop = g_obs.stop[slot];
-    return true;
+    return kObserveEvents;
 }
 
 }  // namespace artab
@@ -72,6 +87,45 @@ int artab_profile_end(float *each_ms, int *each_kind, int capacity) {
         ++n;
     }
     g_obs.used = 0;
+    return n;
+}
+
+int artab_stamps_begin(int capacity) {
+    if (capacity <= 0) return ARTAB_ERR_BAD_SHAPE;
+    if (hipDeviceSynchronize() != hipSuccess) return ARTAB_ERR_LAUNCH;
+    if (!g_stamps.dev) {
+        if (hipMalloc(reinterpret_cast<void **>(&g_stamps.dev), (4 + 2 * static_cast<size_t>(capacity)) * 8) != hipSuccess)
+            return ARTAB_ERR_WORKSPACE;
+        g_stamps.capacity = capacity;
+    } else if (capacity > g_stamps.capacity) {
+        return ARTAB_ERR_WORKSPACE;  // recorded launches hold the first array: it cannot grow
+    }
+    // header zero, every record (start = all ones, end = 0)
+    const size_t words = 4 + 2 * static_cast<size_t>(g_stamps.capacity);
+    unsigned long long *host = new unsigned long long[words];
+    for (size_t i = 0; i < words; ++i) host[i] = (i >= 4 && i % 2 == 0) ? ~0ull : 0ull;
+    const hipError_t e = hipMemcpy(g_stamps.dev, host, words * 8, hipMemcpyHostToDevice);
+    delete[] host;
+    if (e != hipSuccess) return ARTAB_ERR_LAUNCH;
+    g_stamps.enabled = true;
+    return ARTAB_OK;
+}
+
+int artab_stamps_end(float *each_us, int capacity) {
+    g_stamps.enabled = false;
+    if (!g_stamps.dev) return 0;
+    if (hipDeviceSynchronize() != hipSuccess) return ARTAB_ERR_LAUNCH;
+    const size_t words = 4 + 2 * static_cast<size_t>(g_stamps.capacity);
+    unsigned long long *host = new unsigned long long[words];
+    if (hipMemcpy(host, g_stamps.dev, words * 8, hipMemcpyDeviceToHost) != hipSuccess) {
+        delete[] host;
+        return ARTAB_ERR_LAUNCH;
+    }
+    const unsigned long long done = host[0];
+    const int n = static_cast<int>(done < static_cast<unsigned long long>(g_stamps.capacity) ? done : g_stamps.capacity);
+    for (int i = 0; i < n && i < capacity; ++i)
+        if (each_us) each_us[i] = static_cast<float>(host[4 + 2 * i + 1] - host[4 + 2 * i]) * 0.01f;  // 100 MHz ticks
+    delete[] host;
     return n;
 }
 

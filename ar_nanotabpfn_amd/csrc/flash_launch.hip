@@ -11,7 +11,18 @@ static int flash_bn(int Dh) { return (Dh == 32 && tune(kTuneBN, 64) == 128) ? 12
 
 template <typename Kernel>
 static void launch_one(Kernel kernel, unsigned grid, unsigned block, hipStream_t stream, const FlashParams &P) {
-    launch_observed(kLaunchFlash, kernel, dim3(grid), dim3(block), 0, stream, P);
+    LaunchTiming t;
+    const int how = observe_launch(kLaunchFlash, &t);
+    if (how == kObserveEvents) {
+        hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, stream, t.start, t.stop, 0, P);
+    } else if (how == kObserveStamps) {
+        FlashParams Q = P;
+        Q.stamps = t.stamps;
+        Q.stamps_capacity = t.stamps_capacity;
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, stream, Q);
+    } else {
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, stream, P);
+    }
 }
 
 template <typename T, int DH>

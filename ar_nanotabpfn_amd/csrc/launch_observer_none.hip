@@ -3,6 +3,6 @@
 
 namespace artab {
 
-bool observe_launch(int, LaunchTiming *) { return false; }
+int observe_launch(int, LaunchTiming *) { return 0; }
 
 }  // namespace artab

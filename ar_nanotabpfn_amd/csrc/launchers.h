@@ -58,15 +58,18 @@ enum LaunchKind : int {
     kLaunchLayer = 4,         // fused layer kernels (pre, post, boundary between two layers, step tail, step boundary)
 };
 struct LaunchTiming {
-    hipEvent_t start, stop;
+    hipEvent_t start, stop;          // kObserveEvents: the launch is made with these two events
+    unsigned long long *stamps;      // kObserveStamps: the kernel writes its own time stamps here
+    int stamps_capacity;             //   (kLaunchFlash only; legal inside a graph capture)
 };
-bool observe_launch(int kind, LaunchTiming *timing);
+enum : int { kObserveEvents = 1, kObserveStamps = 2 };
+int observe_launch(int kind, LaunchTiming *timing);  // 0 or one of the two
 
 template <typename Kernel, typename... Args>
 inline void launch_observed(int kind, Kernel kernel, dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream,
                             Args... args) {
     LaunchTiming t;
-    if (observe_launch(kind, &t))
+    if (observe_launch(kind, &t) == kObserveEvents)
         hipExtLaunchKernelGGL(kernel, grid, block, static_cast<uint32_t>(lds_bytes), stream, t.start, t.stop, 0, args...);
     else
         hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, args...);

@@ -110,7 +110,37 @@ struct FlashParams {
     unsigned *started;  // optional counter that the first thread of the grid advances at once: "the
                         // launches ahead of this one on its queue are complete" for a watcher on
                         // another queue (queue_order.h); the kernel's own work does not depend on it
+    // Benchmark builds only (null otherwise): time stamps of this launch from the 100 MHz wall
+    // clock.  stamps[0] counts finished launches and names this launch's record, stamps[1] is the
+    // ticket of the workgroups that have finished, records start at stamps[4]: (earliest start,
+    // latest end) over the workgroups of a launch.  Launches that share the array must not
+    // overlap in time (they are launches of one queue).
+    unsigned long long *stamps;
+    int stamps_capacity;
 };
+
+// A workgroup's entry into the record of its launch (first thread only).  Returns the record, or
+// null when stamps are off or the array is full.
+__device__ __forceinline__ unsigned long long *flash_stamp_begin(const FlashParams &P) {
+    if (!P.stamps) return nullptr;
+    const unsigned long long n =
+        __hip_atomic_load(&P.stamps[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (n >= static_cast<unsigned long long>(P.stamps_capacity)) return nullptr;
+    unsigned long long *rec = P.stamps + 4 + 2 * n;
+    __hip_atomic_fetch_min(&rec[0], wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return rec;
+}
+// A workgroup's exit (first thread only); the last one to leave closes the record.
+__device__ __forceinline__ void flash_stamp_end(const FlashParams &P, unsigned long long *rec) {
+    if (!P.stamps) return;
+    if (rec) __hip_atomic_fetch_max(&rec[1], wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned long long t =
+        __hip_atomic_fetch_add(&P.stamps[1], 1ull, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    if (t == gridDim.x - 1) {
+        __hip_atomic_store(&P.stamps[1], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_fetch_add(&P.stamps[0], 1ull, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
 
 // Probability mass (sum of 2^s over a row) the fast path accepts.
 constexpr float kFastMassMax = 1.2676506e30f;  // 2^100
@@ -165,8 +195,16 @@ void flash_kernel(FlashParams P) {
     // three stages; a stage is the K tile followed by the V tile, so that both have the same
     // stage stride and a stage index folds into the immediate offset of every LDS access
     constexpr int STAGE = BN * KPAD + BN * VPAD;
-    constexpr int NST = LEAN ? 4 : 3;  // stages: tiles are requested NST - 1 ahead at most
-    __shared__ __attribute__((aligned(16))) T kv_lds[NST * STAGE];
+#ifndef ARTAB_LEAN_STAGES
+#define ARTAB_LEAN_STAGES 4
+#endif
+    constexpr int NST = LEAN ? ARTAB_LEAN_STAGES : 3;  // stages: tiles are requested NST - 1 ahead at most
+    // The lean pass keeps its tiles unpadded, as 1 KiB chunks in the order the operand reads want
+    // them (see lean_pass): a stage is BN * DH elements of K and as many of V.  The robust pass,
+    // which may follow it in the same launch, needs two stages of the padded layout.
+    constexpr int LSTAGE = 2 * BN * DH;
+    constexpr int LDS_ELEMS = LEAN ? (NST * LSTAGE > 2 * STAGE ? NST * LSTAGE : 2 * STAGE) : NST * STAGE;
+    __shared__ __attribute__((aligned(1024))) T kv_lds[LDS_ELEMS];
     auto k_stage = [&](int st_) -> T * { return kv_lds + st_ * STAGE; };
     auto v_stage = [&](int st_) -> T * { return kv_lds + st_ * STAGE + BN * KPAD; };
     __shared__ int redo_flag;
@@ -177,6 +215,18 @@ void flash_kernel(FlashParams P) {
     if (LEAN && threadIdx.x == 0) redo_flag = 0;  // raised after the pass, at least one barrier later
     if (P.started && blockIdx.x == 0 && threadIdx.x == 0)
         __hip_atomic_fetch_add(P.started, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    // (kept by the first wavefront as a scalar: the record's address costs no vector register)
+    unsigned long long *stamp_rec = nullptr;
+    if (P.stamps && threadIdx.x < 64) {
+        unsigned long long r = 0;
+        if (threadIdx.x == 0) r = reinterpret_cast<unsigned long long>(flash_stamp_begin(P));
+        // (readfirstlane returns a signed int: both halves go through unsigned, or a low half with
+        // its top bit set would sign-extend over the high half)
+        const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(r >> 32)));
+        const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(r & 0xffffffffull)));
+        stamp_rec = reinterpret_cast<unsigned long long *>((static_cast<unsigned long long>(hi) << 32) |
+                                                           static_cast<unsigned long long>(lo));
+    }
 
     // ---- workgroup -> (kv-sharing group, q tile, context split); XCD-aware: the
     // hardware deals consecutive workgroup ids round-robin over the 8 XCDs, so all
@@ -186,7 +236,10 @@ void flash_kernel(FlashParams P) {
     const int xcd = blockIdx.x & 7;
     const int slot = blockIdx.x >> 3;
     const int kvg = (slot / W) * 8 + xcd;
-    if (kvg >= n_kvg) return;
+    if (kvg >= n_kvg) {
+        if (P.stamps && threadIdx.x == 0) flash_stamp_end(P, stamp_rec);
+        return;
+    }
     const int w_in = slot % W;
     const int split = w_in % P.n_split;
     const int tile = w_in / P.n_split;
@@ -714,7 +767,7 @@ void flash_kernel(FlashParams P) {
     //    row 1 (lanes 0..15, registers 0 and 1).  Two such products per block replace eight
     //    v_dot2c (which, issued between MFMAs, cost five times their nominal four cycles).
     //  * K and V tiles of a stage are one list of 16-byte pieces dealt over the whole workgroup.
-    // Four LDS stages, one barrier per tile, full tiles requested three ahead.
+    // NST LDS stages (four), one barrier per tile, full tiles requested NST - 1 ahead.
     auto lean_pass = [&]() {
         f32x4 lsum[QB][2];
 #pragma unroll
@@ -735,6 +788,29 @@ void flash_kernel(FlashParams P) {
         // the workgroup, NP rounds of NT pieces.  CHUNKS is a multiple of 64, so whether a piece
         // is K or V is uniform over a wavefront: sources are a scalar base plus a 32-bit lane
         // offset, and the base moves on by one tile with scalar arithmetic.
+        // ---- LDS layout of a lean stage.  No padding: every 1 KiB chunk is laid out so that the
+        // operand reads of a wavefront sweep whole bank rows.
+        //   K, chunk (sb, ks) [32 keys x 16 columns]: [hb][key][8 elements] — the A operand of S^T
+        //      for lane (c, hb) is the 16 bytes at hb*512 + c*16: 32 consecutive lanes read 512
+        //      consecutive bytes.
+        //   V, chunk (sb, cb) [32 keys x 16 columns]: [key][16 elements] — a transposing read takes
+        //      8 bytes per lane from rows 4*hb .. 4*hb+3 of one chunk: 16 consecutive lanes read 128
+        //      consecutive bytes.
+        // (With padded whole rows — 80-byte K rows, 96-byte V rows — a third of the LDS cycles of
+        // this pass were bank conflicts, and a stage was 11 KiB instead of 8.)
+        static_assert(DH % 16 == 0 && BN % 32 == 0, "chunks are 32 keys x 16 columns");
+        constexpr int CH = 512;                       // elements per chunk
+        constexpr int LK = BN * DH;                   // V region of a stage
+        auto k_off = [](int row, int col) {          // element offset of K[row][col] inside a stage
+            return ((row / 32) * KS + col / 16) * CH + ((col % 16) / 8) * 256 + (row % 32) * 8 + col % 8;
+        };
+        auto v_off = [](int row, int col) {
+            return LK + ((row / 32) * KS + col / 16) * CH + (row % 32) * 16 + col % 16;
+        };
+        const int lk_rd = hb * 256 + c * 8;                                               // + (sb*KS + ks) * CH
+        const int lv_rd = LK + (4 * hb + ((lane & 15) >> 2)) * 16 + ((lane >> 4) & 1) * CH + 4 * (lane & 3);
+        //                                              + (sb*KS + 2*db) * CH + (16*t + 8*u) * 16
+
         constexpr int NP = (2 * CHUNKS + NT - 1) / NT;
         static_assert(CHUNKS % 64 == 0, "K/V choice must be wavefront-uniform");
         bool p_on[NP], p_v[NP];
@@ -748,23 +824,22 @@ void flash_kernel(FlashParams P) {
             const int cidx = idx0 + lane - (p_v[x] ? CHUNKS : 0);
             p_row[x] = cidx / CPR;
             p_col[x] = (cidx % CPR) * 8;
-            p_dst[x] = p_v[x] ? BN * KPAD + p_row[x] * VPAD + p_col[x] : p_row[x] * KPAD + p_col[x];
+            p_dst[x] = p_v[x] ? v_off(p_row[x], p_col[x]) : k_off(p_row[x], p_col[x]);
         }
         u32x4 st_a[NP], st_b[NP];
 
         // Full context tiles (every row present, nothing masked): the steady state.
         const int n_main = (ctx_end - ctx_begin) / BN;
 
-        // In the steady state the tiles do not pass through registers at all: a stage is a whole
-        // number of KiB (K region and V region each), so it is filled by NI direct global->LDS
-        // loads of one KiB (lane l lands at base + 16 l), dealt over the wavefronts, each wholly
-        // inside K or inside V.  A lane whose 16 bytes fall into a row's padding re-reads the
-        // row's first piece (never used).  The loads are inline assembly: the compiler does not
-        // know of them and therefore does not drain them in front of every LDS read; they are
-        // waited for by hand (vmcnt) in front of the barrier that publishes their stage.
-        constexpr int STAGE_BYTES = STAGE * static_cast<int>(sizeof(T));
-        constexpr int NI = STAGE_BYTES / 1024, NKI = BN * KPAD * static_cast<int>(sizeof(T)) / 1024;
-        static_assert(STAGE_BYTES % 1024 == 0 && (BN * KPAD * sizeof(T)) % 1024 == 0, "stage must be whole KiB");
+        // In the steady state the tiles do not pass through registers at all: a stage is NI chunks
+        // of one KiB, each filled by one direct global->LDS load (lane l lands at base + 16 l; the
+        // lane's source address is whatever piece of the tile belongs there), dealt over the
+        // wavefronts.  The loads are inline assembly: the compiler does not know of them and
+        // therefore does not drain them in front of every LDS read; they are waited for by hand
+        // (vmcnt) in front of the barrier that publishes their stage.
+        constexpr int STAGE_BYTES = LSTAGE * static_cast<int>(sizeof(T));
+        constexpr int NI = STAGE_BYTES / 1024, NKI = NI / 2;
+        static_assert(STAGE_BYTES % 2048 == 0, "a stage is whole chunks of K and as many of V");
         constexpr int NR = (NI + NW - 1) / NW;
         static_assert(!LEAN || NR <= 2, "at most two direct loads per wavefront and tile");
         const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(kv_lds));
@@ -774,15 +849,15 @@ void flash_kernel(FlashParams P) {
         int n_dma = 0;  // direct loads this wavefront issues per tile
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
-            const int i = wave + NW * r;  // scalar
+            const int i = wave + NW * r;  // scalar: chunk of the stage
             const bool is_v = i >= NKI;
             const View &src = is_v ? P.vc : P.kc;
-            const int byte = (i - (is_v ? NKI : 0)) * 1024 + lane * 16;
-            const int row_bytes = (is_v ? VPAD : KPAD) * static_cast<int>(sizeof(T));
-            const int row = byte / row_bytes;
-            int piece = (byte % row_bytes) / 16;
-            piece = piece < CPR ? piece : 0;
-            d_off[r] = static_cast<unsigned>(row * src.sn * static_cast<long>(sizeof(T)) + piece * 16);
+            const int ch = i - (is_v ? NKI : 0);           // (sb, 16-column step) of the chunk
+            const int sbk = ch / KS, cs = ch % KS;
+            // lane l holds 16 bytes: K chunk [hb = l/32][key l%32], V chunk [key l/2][half l%2]
+            const int row = 32 * sbk + (is_v ? lane / 2 : lane % 32);
+            const int col = 16 * cs + 8 * (is_v ? lane % 2 : lane / 32);
+            d_off[r] = static_cast<unsigned>((row * src.sn + col) * static_cast<long>(sizeof(T)));
             d_step[r] = static_cast<long>(BN) * src.sn * static_cast<long>(sizeof(T));
             d_src[r] = reinterpret_cast<const char *>(view_row<T>(src, kvb, h, ctx_begin));
             if (i < NI) ++n_dma;
@@ -838,26 +913,26 @@ void flash_kernel(FlashParams P) {
         auto stash_tile = [&](auto stage_, const u32x4(&st)[NP]) {
 #pragma unroll
             for (int x = 0; x < NP; ++x)
-                if (p_on[x]) *reinterpret_cast<u32x4 *>(kv_lds + stage_ * STAGE + p_dst[x]) = st[x];
+                if (p_on[x]) *reinterpret_cast<u32x4 *>(kv_lds + stage_ * LSTAGE + p_dst[x]) = st[x];
         };
 
         // One 32-key block of the tile in `stage_` against this wavefront's queries.
         auto block = [&](auto stage_, int sb, auto mask_tag, int blk0, bool is_ctx, int seg_end) {
             constexpr bool MASK = decltype(mask_tag)::value;
-            const T *kt = kv_lds + stage_ * STAGE + k_rd;
-            const T *vt = kv_lds + stage_ * STAGE + BN * KPAD + v_rd;
+            const T *kt = kv_lds + stage_ * LSTAGE + lk_rd;
+            const T *vt = kv_lds + stage_ * LSTAGE + lv_rd;
             vec ak[KS];
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) ak[ks] = *reinterpret_cast<const vec *>(kt + 32 * sb * KPAD + 16 * ks);
+            for (int ks = 0; ks < KS; ++ks) ak[ks] = *reinterpret_cast<const vec *>(kt + (sb * KS + ks) * CH);
             vec av[DB][2];
 #pragma unroll
             for (int db = 0; db < DB; ++db)
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    const T *vp_ = vt + (32 * sb + 16 * t) * VPAD + 32 * db;
+                    const T *vp_ = vt + (sb * KS + 2 * db) * CH + 16 * t * 16;
                     s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(vp_));
                     s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) s16x4 *)(vp_ + 8 * VPAD));
+                        (__attribute__((address_space(3))) s16x4 *)(vp_ + 8 * 16));
                     typedef short s16x8 __attribute__((ext_vector_type(8)));
                     s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                     av[db][t] = __builtin_bit_cast(vec, both);
@@ -893,12 +968,12 @@ void flash_kernel(FlashParams P) {
             }
         };
 
-        // Tile `it` out of stage it % 4: barrier, request a later tile into a stage that is free,
-        // compute.  STEADY: a full, unmasked context tile; it requests the full tile three ahead (if
+        // Tile `it` out of stage it % NST: barrier, request a later tile into a stage that is free,
+        // compute.  STEADY: a full, unmasked context tile; it requests the full tile NST - 1 ahead (if
         // there is one) by direct global->LDS loads, into the stage that tile it - 1 has just left.
         // Otherwise: any tile; it requests the tile two ahead through registers and stores it after
         // the compute, unless that tile is a full one (then a direct load is or was under way).
-        // So full tiles 2 .. n_main - 1 arrive by direct loads (tile 2 from the prologue), all
+        // So full tiles 2 .. n_main - 1 arrive by direct loads (tiles 2 .. NST - 2 from the prologue), all
         // others through registers, and the tile in front of the first non-full one is never STEADY.
         auto tile = [&](int it, auto stage_, auto steady_tag) {
             constexpr bool STEADY = decltype(steady_tag)::value;
@@ -916,14 +991,19 @@ void flash_kernel(FlashParams P) {
                 // this tile's direct loads must have landed; those of the next two full tiles may
                 // still be on their way
                 const int behind = n_main - 1 - it;
-                switch ((behind >= 2 ? 2 : behind) * n_dma) {
+                switch ((behind >= NST - 2 ? NST - 2 : behind) * n_dma) {
                     case 0: __builtin_amdgcn_s_waitcnt(vmcnt_imm(0)); break;
                     case 1: __builtin_amdgcn_s_waitcnt(vmcnt_imm(1)); break;
                     case 2: __builtin_amdgcn_s_waitcnt(vmcnt_imm(2)); break;
-                    default: __builtin_amdgcn_s_waitcnt(vmcnt_imm(4)); break;
+                    case 3: __builtin_amdgcn_s_waitcnt(vmcnt_imm(3)); break;
+                    case 4: __builtin_amdgcn_s_waitcnt(vmcnt_imm(4)); break;
+                    case 5: __builtin_amdgcn_s_waitcnt(vmcnt_imm(5)); break;
+                    case 6: __builtin_amdgcn_s_waitcnt(vmcnt_imm(6)); break;
+                    default: __builtin_amdgcn_s_waitcnt(vmcnt_imm(8)); break;
                 }
+                static_assert(NST <= 6, "the wait counts above cover up to four tiles in flight, two loads each");
                 __syncthreads();
-                if (behind >= 3) dma_tile((stage_ + 3) % 4);
+                if (behind >= NST - 1) dma_tile((stage_ + NST - 1) % NST);
 #pragma unroll
                 for (int sb = 0; sb < SB; ++sb) block(stage_, sb, BoolTag<false>{}, 0, true, 0);
             } else {
@@ -945,7 +1025,7 @@ void flash_kernel(FlashParams P) {
                     else
                         block(stage_, sb, BoolTag<false>{}, blk0, is_ctx, seg_end);
                 }
-                if (fetch) stash_tile((stage_ + 2) % 4, st_a);
+                if (fetch) stash_tile((stage_ + 2) % NST, st_a);
             }
         };
 
@@ -965,7 +1045,9 @@ void flash_kernel(FlashParams P) {
                 dma_tile(std::integral_constant<int, 1>{});
             else if (n_tiles > 1)
                 gfetch(1, st_b);
-            if (n_main > 2) dma_tile(std::integral_constant<int, 2>{});
+#pragma unroll
+            for (int t = 2; t < NST - 1; ++t)
+                if (n_main > t) dma_tile(t);
             scale_q(qraw);
             if (n_main <= 0 && n_tiles > 0) stash_tile(std::integral_constant<int, 0>{}, st_a);
             if (n_main <= 1 && n_tiles > 1) stash_tile(std::integral_constant<int, 1>{}, st_b);
@@ -975,25 +1057,26 @@ void flash_kernel(FlashParams P) {
         // with nothing but full context tiles the whole slice is steady state; otherwise the last
         // two full tiles have to request tiles of the other kind and take the general route
         const int n_steady = n_tiles == n_main ? n_main : n_main - 2;
-        // The bulk of a long slice: groups of four full tiles that each have three full tiles
+        // The bulk of a long slice: groups of NST full tiles that each have NST - 1 full tiles
         // behind them.  Nothing about such a tile depends on its index — the wait is for a constant
-        // number of direct loads, the request three ahead is unconditional — so the group is
+        // number of direct loads, the request NST - 1 ahead is unconditional — so the group is
         // straight-line code (the general steady tile below spends a dozen scalar branches on
-        // these decisions); the priority steps sit between groups, at multiples of four.
-        const int n_fast = n_main >= 12 ? ((n_steady < n_main - 3 ? n_steady : n_main - 3) & ~3) : 0;
+        // these decisions); the priority steps sit between groups, at multiples of NST.
+        const int n_ahead = n_steady < n_main - (NST - 1) ? n_steady : n_main - (NST - 1);
+        const int n_fast = n_main >= 12 && n_ahead > 0 ? n_ahead / NST * NST : 0;
         bool dense = n_fast > 0;
         if (dense && P.dense_below > 0)  // (a scalar: the choice must stay a wavefront-uniform branch)
             dense = __builtin_amdgcn_readfirstlane(beside_now) < P.dense_below;
         if (dense) {
             const bool two = n_dma == 2;  // direct loads of this wavefront per tile: one or two
             auto fast_tile = [&](auto stage_) {
-                // this tile's loads have landed, those of the next two tiles may be under way
+                // this tile's loads have landed, those of the next NST - 2 tiles may be under way
                 if (two)
-                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(4));
+                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(2 * (NST - 2)));
                 else
-                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(2));
+                    __builtin_amdgcn_s_waitcnt(vmcnt_imm(NST - 2));
                 __syncthreads();
-                constexpr int into = (decltype(stage_)::value + 3) % 4;
+                constexpr int into = (decltype(stage_)::value + NST - 1) % NST;
 #pragma unroll
                 for (int r = 0; r < NR; ++r) {
                     if (r == 0 || two) {
@@ -1013,17 +1096,19 @@ void flash_kernel(FlashParams P) {
                 for (int sb = 0; sb < SB; ++sb) block(stage_, sb, BoolTag<false>{}, 0, true, 0);
             };
             // the priority falls with progress (see the general steady tile): steps between groups
-            const int q1 = (n_main / 4) & ~3, q2 = (n_main / 2) & ~3, q3 = (3 * n_main / 4) & ~3;
+            const int q1 = (n_main / 4) / NST * NST, q2 = (n_main / 2) / NST * NST, q3 = (3 * n_main / 4) / NST * NST;
 #pragma nounroll
             for (int part = 0; part < 4; ++part) {
                 int end = part == 0 ? q1 : part == 1 ? q2 : part == 2 ? q3 : n_fast;
                 end = end < n_fast ? end : n_fast;
 #pragma nounroll
-                for (; it < end; it += 4) {
+                for (; it < end; it += NST) {
                     fast_tile(std::integral_constant<int, 0>{});
                     fast_tile(std::integral_constant<int, 1>{});
                     fast_tile(std::integral_constant<int, 2>{});
                     fast_tile(std::integral_constant<int, 3>{});
+                    if constexpr (NST > 4) fast_tile(std::integral_constant<int, 4>{});
+                    if constexpr (NST > 5) fast_tile(std::integral_constant<int, 5>{});
                 }
                 if (part == 0 && it == q1)
                     __builtin_amdgcn_s_setprio(2);
@@ -1041,11 +1126,19 @@ void flash_kernel(FlashParams P) {
             tile(it, std::integral_constant<int, 2>{}, BoolTag<true>{});
             if (++it >= n_steady) break;
             tile(it, std::integral_constant<int, 3>{}, BoolTag<true>{});
+            if constexpr (NST > 4) {
+                if (++it >= n_steady) break;
+                tile(it, std::integral_constant<int, 4>{}, BoolTag<true>{});
+            }
+            if constexpr (NST > 5) {
+                if (++it >= n_steady) break;
+                tile(it, std::integral_constant<int, 5>{}, BoolTag<true>{});
+            }
             ++it;
         }
-        for (int stage = it % 4; it < n_tiles; ++it) {
+        for (int stage = it % NST; it < n_tiles; ++it) {
             tile(it, stage, BoolTag<false>{});
-            stage = stage == 3 ? 0 : stage + 1;
+            stage = stage == NST - 1 ? 0 : stage + 1;
         }
         // row sums: query c of this lane's block sits in lane c % 16, register c / 16; the total
         // already covers both halves, so only the hb = 0 lane carries it into the epilogue
@@ -1119,6 +1212,10 @@ void flash_kernel(FlashParams P) {
                 }
             if (P.lse && hb == 0) P.lse[orow_idx] = lse;
         }
+    }
+    if (P.stamps) {
+        __syncthreads();  // every wavefront of the workgroup has issued its stores
+        if (threadIdx.x == 0) flash_stamp_end(P, stamp_rec);
     }
 }
 

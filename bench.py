@@ -189,6 +189,40 @@ def observed_decode(pred, x_context, y_context, x_target, steps, device, dtype, 
     return out
 
 
+STAMP_CAPACITY = 12 * (NT3 + 8) + 64  # launches the stamp array of the benchmark library holds
+
+
+def stamped_decode(pred, x_context, y_context, x_target, steps, device, dtype, cap=NT3):
+    """The decode run as it is timed — replayed from recorded HIP graphs — with every launch of
+    the matrix-core attention kernel writing its own time stamps (benchmark build of the library:
+    earliest workgroup start to latest workgroup end on the 100 MHz wall clock).  The graphs are
+    recorded afresh under that build, replayed once unmeasured, then measured.  Returns
+    (decode_ms, [context-pass durations in us, launch order: `layers` per step])."""
+    from ar_nanotabpfn_amd import _lib
+
+    L = len(pred.backbone.layers)
+    with _lib.benchmark_library() as bl:
+        _lib.check(bl.artab_stamps_begin(STAMP_CAPACITY))
+        pred._graph_state = None  # record afresh: the recorded launches carry the stamp array
+        try:
+            run_decode(pred, x_context, y_context, x_target, min(steps, 12), device, dtype, cap)
+            recorded = pred.graph_recordings
+            _lib.check(bl.artab_stamps_begin(STAMP_CAPACITY))  # clears the records
+            _, decode_ms, _ = run_decode(pred, x_context, y_context, x_target, steps, device, dtype, cap)
+            buf = (ctypes.c_float * STAMP_CAPACITY)()
+            n = bl.artab_stamps_end(buf, STAMP_CAPACITY)
+            if n < 0:
+                _lib.check(n)
+            if pred.graph_recordings != recorded:
+                sys.exit("bench.py: a HIP graph was recorded inside the stamped run")
+        finally:
+            pred._graph_state = None  # later runs record with the drop-in library again
+    us = [float(buf[i]) for i in range(n)]
+    if n != L * (steps + 1):
+        sys.exit(f"bench.py: expected {L * (steps + 1)} stamped launches (prefill + {steps} steps), saw {n}")
+    return decode_ms, us[L:]  # the first L launches are the prefill's dense passes
+
+
 def host_info():
     """Cores, thread counts and CPU model of the host the CPU legs run on."""
     model = "unknown"
@@ -461,29 +495,30 @@ def config4_bench(device, observe=True):
     }
     log(f"[config4] prefill {prefill_ms:.2f} ms; {Nt} decode steps in {decode_ms:.1f} ms = {out['value']} target-steps/s")
     if observe:
+        _, ctx_us = stamped_decode(pred, x_context, y_context, x_target, Nt, device, dtype, cap=Nt)
         obs = observed_decode(pred, x_context, y_context, x_target, Nt, device, dtype, cap=Nt)
-        ctx = obs.get(KIND_FLASH, [])
         buf = obs.get(KIND_STREAM_BUFFER, [])
-        if len(ctx) == L * Nt and len(buf) == L * (Nt - 1):
-            ctx_ms = float(np.sum(ctx))
-            flops = 4.0 * B4 * H * NC4 * Dh * L * (1 + 2 * (Nt - 1))
+        ctx_ms = float(np.sum(ctx_us)) * 1e-3
+        flops = 4.0 * B4 * H * NC4 * Dh * L * (1 + 2 * (Nt - 1))
+        out.update({
+            "context_pass_avg_us": round(ctx_ms * 1e3 / len(ctx_us), 2),
+            "context_pass_frac": round(flops / (ctx_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+        })
+        if len(buf) == L * (Nt - 1):
             # buffer pass of step t (t = 1 .. Nt-1) reads t-1 committed rows and the new one: t rows of K and V
             row_bytes = 2.0 * B4 * H * Dh * 2
             buf_by_step = np.asarray(buf).reshape(Nt - 1, L)
             last = buf_by_step[-1].mean()
             out.update({
-                "context_pass_avg_us": round(ctx_ms * 1e3 / len(ctx), 2),
-                "context_pass_frac": round(flops / (ctx_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                 "buffer_pass_us_at_255_rows": round(float(last) * 1e3, 1),
                 "buffer_pass_gbs_at_255_rows": round(row_bytes * (Nt - 1) / (last * 1e-3) / 1e9, 1),
                 "buffer_pass_frac_of_hbm_peak_at_255_rows": round(row_bytes * (Nt - 1) / (last * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                 "buffer_pass_gbs_whole_run": round(row_bytes * L * sum(range(1, Nt)) / (float(np.sum(buf)) * 1e-3) / 1e9, 1),
                 "layer_kernel_avg_us": round(float(np.mean(obs.get(KIND_LAYER, [0.0]))) * 1e3, 2),
+                "buffer_and_layer_timing": "per-launch events in a run that issues the recorded step's launches live",
             })
-            log(f"[config4] context pass avg {out['context_pass_avg_us']} us ({out['context_pass_frac']} of peak); buffer pass "
-                f"at 255 rows {out['buffer_pass_us_at_255_rows']} us = {out['buffer_pass_gbs_at_255_rows']} GB/s")
-        else:
-            out["observed"] = f"unexpected launch counts: {len(ctx)} context passes, {len(buf)} buffer passes"
+        log(f"[config4] context pass avg {out['context_pass_avg_us']} us ({out['context_pass_frac']} of peak); buffer pass "
+            f"at 255 rows {out.get('buffer_pass_us_at_255_rows')} us = {out.get('buffer_pass_gbs_at_255_rows')} GB/s")
     del pred, model
     torch.cuda.empty_cache()
     return out
@@ -860,6 +895,9 @@ def main():
         sys.exit("bench.py: a HIP graph was recorded inside the timed region")
     ms_per_step = decode_ms / args.steps
     value = 1e3 / ms_per_step
+    chain0 = pred._graph_state.chains[0] if pred._graph_state is not None else None
+    step_boundary_fused = bool(chain0 is not None and getattr(chain0, "boundary", None) is not None)
+    stream_ordering = None if chain0 is None else ("counters" if getattr(chain0, "order", None) is not None else "events")
     log(f"[gpu] prefill {prefill_ms:.2f} ms; {args.steps} decode steps in {decode_ms:.2f} ms "
         f"({ms_per_step:.3f} ms/step, host wall {wall_ms:.1f} ms)")
     # the whole configuration (all 256 steps), whatever K is: same recorded graphs, replayed once more
@@ -871,21 +909,24 @@ def main():
             sys.exit("bench.py: a HIP graph was recorded inside the 256-step run")
     log(f"[gpu] all {NT3} decode steps in {full_ms:.2f} ms ({full_ms / NT3:.3f} ms/step)")
 
-    # Per-launch durations of the whole configuration: the launches of the recorded step issued
-    # live through the benchmark build of the library, each with its own start/end time stamps.
+    # Context-pass durations of the whole configuration, in the schedule that is timed: the recorded
+    # graphs replayed with the kernel writing its own time stamps (benchmark build of the library).
     H, Dh, L = CFG3["n_heads"], CFG3["d_model"] // CFG3["n_heads"], CFG3["n_layers"]
-    obs = observed_decode(pred, x_context, y_context, x_target, NT3, device, dtype)
-    ctx = np.asarray(obs.get(KIND_FLASH, []))
-    if len(ctx) != L * NT3:
-        sys.exit(f"bench.py: expected {L * NT3} context-pass launches in the observed run, saw {len(ctx)}")
-    ctx_by_step = ctx.reshape(NT3, L)  # ms; step 0 has one query per trajectory, the others two
-    buf_by_step = np.asarray(obs.get(KIND_STREAM_BUFFER, [])).reshape(NT3 - 1, L) if len(obs.get(KIND_STREAM_BUFFER, [])) == L * (NT3 - 1) else None
-    layer_ms = np.asarray(obs.get(KIND_LAYER, []))
+    stamped_ms, ctx_us = stamped_decode(pred, x_context, y_context, x_target, NT3, device, dtype)
+    ctx_by_step = np.asarray(ctx_us).reshape(NT3, L) * 1e-3  # ms; step 0 has one query per trajectory, the others two
+    log(f"[gpu] stamped run: {NT3} decode steps in {stamped_ms:.2f} ms (unstamped: {full_ms:.2f} ms)")
     # the same with the buffer pass after the context pass instead of beside it: the context-pass
     # kernel with the chip to itself
     pred.overlap_buffer_pass = False
-    alone = np.asarray(observed_decode(pred, x_context, y_context, x_target, NT3, device, dtype).get(KIND_FLASH, []))
+    _, alone_us = stamped_decode(pred, x_context, y_context, x_target, NT3, device, dtype)
     pred.overlap_buffer_pass = True
+    alone = np.asarray(alone_us) * 1e-3
+    # The other kernels of a step (buffer pass, layer kernels): the launches of the recorded step
+    # issued live through the benchmark build, each with events that receive its own start and end
+    # time stamps (about 2 us longer per launch than a kernel trace shows).
+    obs = observed_decode(pred, x_context, y_context, x_target, NT3, device, dtype)
+    buf_by_step = np.asarray(obs.get(KIND_STREAM_BUFFER, [])).reshape(NT3 - 1, L) if len(obs.get(KIND_STREAM_BUFFER, [])) == L * (NT3 - 1) else None
+    layer_ms = np.asarray(obs.get(KIND_LAYER, []))
     flops_lq1 = 4.0 * B3 * H * NC3 * Dh
 
     def frac_over(steps, by_step):
@@ -901,11 +942,12 @@ def main():
     # prefill launches (dense pass over the context), observed on their own
     with _lib.benchmark_library() as bl:
         pred.init_kv_cache(B3, NT3, device, dtype)
-        _lib.check(bl.artab_profile_begin(L + 8))
+        pcap = 8 * L + 8
+        _lib.check(bl.artab_profile_begin(pcap))
         pred.prefill_context(x_context, y_context)
-        pms, pk = (ctypes.c_float * (L + 8))(), (ctypes.c_int * (L + 8))()
-        pn = bl.artab_profile_end(pms, pk, L + 8)
-    prefill_kernel_ms = sum(pms[i] for i in range(max(pn, 0)) if pk[i] == KIND_FLASH)
+        pms, pk = (ctypes.c_float * pcap)(), (ctypes.c_int * pcap)()
+        pn = bl.artab_profile_end(pms, pk, pcap)
+    prefill_kernel_ms = sum(pms[i] for i in range(min(max(pn, 0), pcap)) if pk[i] == KIND_FLASH)
     prefill_flops = 4.0 * H * NC3 * NC3 * Dh * L
 
     roofline = {
@@ -921,8 +963,8 @@ def main():
         "traffic": CONTEXT_PASS_HBM_BYTES,
         "launches": int(args.steps * L),
         "avg_launch_us": round(avg_launch_us, 2),
-        "timing": "the launch's own start/end time stamps (hipExtLaunchKernelGGL events), launches of the recorded step "
-                  "issued live on the same two streams with the same ordering; steps 0..K-1",
+        "timing": "time stamps the kernel takes itself (earliest workgroup start to latest workgroup end, 100 MHz wall "
+                  "clock) in the recorded graphs as they are replayed for `value`; steps 0..K-1 of a 256-step run",
         # In the timed schedule the buffer pass of the same layer runs beside this kernel and takes
         # issue slots from it; these two are the kernel without that neighbour (all 256 steps).
         "avg_launch_us_alone": round(avg_alone_us, 2) if avg_alone_us else None,
@@ -970,13 +1012,12 @@ def main():
         # that layer is read by nobody; --full-last-layer computes it as the reference does: -0.7 %)
         "target_only_last_layer": bool(pred.target_only_last_layer),
         # last layer's tail + head/draw/embedding + first layer's head of the next step as one launch
-        "step_boundary_fused": bool(pred._graph_state is not None
-                                    and getattr(pred._graph_state.chains[0], "boundary", None) is not None),
-        "stream_ordering": ("counters" if getattr(pred._graph_state.chains[0], "order", None) is not None else "events")
-        if pred._graph_state is not None else None,
+        "step_boundary_fused": step_boundary_fused,
+        "stream_ordering": stream_ordering,
         "prefill_ms": round(prefill_ms, 3),
         "roofline": roofline,
         "full_run": full_run,
+        "stamped_run_ms_per_step": round(stamped_ms / NT3, 4),
     }
 
     if not args.no_cpu:
