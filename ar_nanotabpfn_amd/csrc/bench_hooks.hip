@@ -100,10 +100,10 @@ int artab_stamps_begin(int capacity) {
     } else if (capacity > g_stamps.capacity) {
         return ARTAB_ERR_WORKSPACE;  // recorded launches hold the first array: it cannot grow
     }
-    // header zero, every record (start = all ones, end = 0)
+    // counters and records zero, the slot that collects the earliest start all ones
     const size_t words = 4 + 2 * static_cast<size_t>(g_stamps.capacity);
     unsigned long long *host = new unsigned long long[words];
-    for (size_t i = 0; i < words; ++i) host[i] = (i >= 4 && i % 2 == 0) ? ~0ull : 0ull;
+    for (size_t i = 0; i < words; ++i) host[i] = i == 2 ? ~0ull : 0ull;  // [2]: earliest start so far
     const hipError_t e = hipMemcpy(g_stamps.dev, host, words * 8, hipMemcpyHostToDevice);
     delete[] host;
     if (e != hipSuccess) return ARTAB_ERR_LAUNCH;

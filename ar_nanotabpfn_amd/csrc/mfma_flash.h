@@ -112,34 +112,43 @@ struct FlashParams {
                         // another queue (queue_order.h); the kernel's own work does not depend on it
     // Benchmark builds only (null otherwise): time stamps of this launch from the 100 MHz wall
     // clock.  stamps[0] counts finished launches and names this launch's record, stamps[1] is the
-    // ticket of the workgroups that have finished, records start at stamps[4]: (earliest start,
-    // latest end) over the workgroups of a launch.  Launches that share the array must not
-    // overlap in time (they are launches of one queue).
+    // ticket of the workgroups that have finished, stamps[2] collects the earliest start of the
+    // launch under way, records start at stamps[4]: (earliest start, end of the last workgroup).
+    // Launches that share the array must not overlap in time (they are launches of one queue).
     unsigned long long *stamps;
     int stamps_capacity;
 };
 
-// A workgroup's entry into the record of its launch (first thread only).  Returns the record, or
-// null when stamps are off or the array is full.
-__device__ __forceinline__ unsigned long long *flash_stamp_begin(const FlashParams &P) {
-    if (!P.stamps) return nullptr;
-    const unsigned long long n =
-        __hip_atomic_load(&P.stamps[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (n >= static_cast<unsigned long long>(P.stamps_capacity)) return nullptr;
-    unsigned long long *rec = P.stamps + 4 + 2 * n;
-    __hip_atomic_fetch_min(&rec[0], wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return rec;
+// Reading the wall clock is a request to one unit of the chip: a launch in which every wavefront
+// reads it is several microseconds longer (measured: 4608 reads, +13 us on a 43 us launch).  So
+// few do: the first wavefront of the first kStampStarters workgroups at the start (the earliest of
+// them is the launch's start; workgroups are started in order), and the workgroup that takes the
+// last ticket at the end (it is the last to finish by definition).
+constexpr unsigned kStampStarters = 16;
+
+__device__ __forceinline__ void flash_stamp_start(const FlashParams &P) {  // first thread of a workgroup
+    if (P.stamps && blockIdx.x < kStampStarters)
+        __hip_atomic_fetch_min(&P.stamps[2], wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// A workgroup's exit (first thread only); the last one to leave closes the record.
-__device__ __forceinline__ void flash_stamp_end(const FlashParams &P, unsigned long long *rec) {
-    if (!P.stamps) return;
-    if (rec) __hip_atomic_fetch_max(&rec[1], wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+// First thread of a workgroup that is done.  Relaxed throughout: every access to the array is an
+// atomic at agent scope (they execute in the L2 / memory side, in order per address), and the next
+// reader is the next launch of the queue or the host after a synchronisation; an acquire/release
+// here would write back and invalidate the L2 once per workgroup.
+__device__ __forceinline__ void flash_stamp_end(const FlashParams &P) {
     const unsigned long long t =
-        __hip_atomic_fetch_add(&P.stamps[1], 1ull, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    if (t == gridDim.x - 1) {
-        __hip_atomic_store(&P.stamps[1], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_fetch_add(&P.stamps[0], 1ull, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_fetch_add(&P.stamps[1], 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (t != gridDim.x - 1) return;
+    const unsigned long long t1 = wall_clock64();
+    const unsigned long long n = __hip_atomic_load(&P.stamps[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned long long t0 =
+        __hip_atomic_exchange(&P.stamps[2], ~0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (n < static_cast<unsigned long long>(P.stamps_capacity)) {
+        __hip_atomic_store(&P.stamps[4 + 2 * n], t0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&P.stamps[5 + 2 * n], t1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    __hip_atomic_store(&P.stamps[1], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&P.stamps[0], n + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Probability mass (sum of 2^s over a row) the fast path accepts.
@@ -215,18 +224,7 @@ void flash_kernel(FlashParams P) {
     if (LEAN && threadIdx.x == 0) redo_flag = 0;  // raised after the pass, at least one barrier later
     if (P.started && blockIdx.x == 0 && threadIdx.x == 0)
         __hip_atomic_fetch_add(P.started, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-    // (kept by the first wavefront as a scalar: the record's address costs no vector register)
-    unsigned long long *stamp_rec = nullptr;
-    if (P.stamps && threadIdx.x < 64) {
-        unsigned long long r = 0;
-        if (threadIdx.x == 0) r = reinterpret_cast<unsigned long long>(flash_stamp_begin(P));
-        // (readfirstlane returns a signed int: both halves go through unsigned, or a low half with
-        // its top bit set would sign-extend over the high half)
-        const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(r >> 32)));
-        const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(r & 0xffffffffull)));
-        stamp_rec = reinterpret_cast<unsigned long long *>((static_cast<unsigned long long>(hi) << 32) |
-                                                           static_cast<unsigned long long>(lo));
-    }
+    if (threadIdx.x == 0) flash_stamp_start(P);
 
     // ---- workgroup -> (kv-sharing group, q tile, context split); XCD-aware: the
     // hardware deals consecutive workgroup ids round-robin over the 8 XCDs, so all
@@ -237,7 +235,7 @@ void flash_kernel(FlashParams P) {
     const int slot = blockIdx.x >> 3;
     const int kvg = (slot / W) * 8 + xcd;
     if (kvg >= n_kvg) {
-        if (P.stamps && threadIdx.x == 0) flash_stamp_end(P, stamp_rec);
+        if (P.stamps && threadIdx.x == 0) flash_stamp_end(P);
         return;
     }
     const int w_in = slot % W;
@@ -1215,7 +1213,7 @@ void flash_kernel(FlashParams P) {
     }
     if (P.stamps) {
         __syncthreads();  // every wavefront of the workgroup has issued its stores
-        if (threadIdx.x == 0) flash_stamp_end(P, stamp_rec);
+        if (threadIdx.x == 0) flash_stamp_end(P);
     }
 }
 

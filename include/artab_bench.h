@@ -41,14 +41,14 @@ int artab_profile_end(float *each_ms, int *each_kind, int capacity);
 
 /*
  * Time stamps taken by the matrix-core attention kernel itself (100 MHz wall clock: the earliest
- * start and the latest end over the workgroups of a launch), for launches that cannot carry
- * events: the ones inside a recorded HIP graph.  Between artab_stamps_begin and artab_stamps_end
+ * start over the first workgroups of a launch, the end of its last workgroup), for launches that
+ * cannot carry events: the ones inside a recorded HIP graph.  Between artab_stamps_begin and artab_stamps_end
  * every such launch this library makes -- or records -- points at one array in device memory that
  * the library allocates on the first call (hipMalloc; `capacity` launches; later calls may ask for
  * at most that many) and never frees, so a graph recorded in between stays valid.  _begin waits
  * for the device and clears the array; _end waits for the device, writes the durations of the
  * launches that completed since _begin, in order, in microseconds, and returns their number.
- * A stamped launch is a few atomic operations per workgroup longer than an unstamped one; what a
+ * A stamped launch is one atomic operation per workgroup longer than an unstamped one; what a
  * kernel trace reports for the same launch is longer by the dispatch's start-up and its final
  * cache write-back, which a kernel cannot see.  Launches that share the array must be launches
  * of one queue (the context passes of a decode run are).
