@@ -438,7 +438,13 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         // scale * log2(e) folded into the keys (this kernel's register operand) and rounded to the
-        // input type: scores in base-2 units straight from the matrix pipe
+        // input type: scores in base-2 units straight from the matrix pipe.  The forward and the dQ
+        // kernel round q * scale * log2(e) instead, so the P recomputed here is not bit for bit the
+        // forward's: the two roundings differ by up to 2^-9 of a score, i.e. P by |s| * 2^-9
+        // relative (about 1 % at |s| = 10 in base-2 units).  That is inside the 16-bit tolerance
+        // the gradients are held to (2e-2 of the gradient's scale, against the float64 oracle);
+        // folding the factor into the Q tile instead would put it into the A operand of
+        // dK^T += Q^T dS as well and cost a multiply per staged element.
         const u32x4 kr = backward_row_piece<T>(P.k, b, h, kj, P.R, ks, hb);
         u32x4 sc;
 #pragma unroll
