@@ -442,7 +442,7 @@ __global__ __launch_bounds__(kBackwardWaves * 64) void backward_dkv_mfma_kernel(
         // kernel round q * scale * log2(e) instead, so the P recomputed here is not bit for bit the
         // forward's: the two roundings differ by up to 2^-9 of a score, i.e. P by |s| * 2^-9
         // relative (about 1 % at |s| = 10 in base-2 units).  That is inside the 16-bit tolerance
-        // the gradients are held to (2e-2 of the gradient's scale, against the float64 oracle);
+        // the gradients are held to (2e-2 of the gradient's scale, against a float64 evaluation);
         // folding the factor into the Q tile instead would put it into the A operand of
         // dK^T += Q^T dS as well and cost a multiply per staged element.
         const u32x4 kr = backward_row_piece<T>(P.k, b, h, kj, P.R, ks, hb);

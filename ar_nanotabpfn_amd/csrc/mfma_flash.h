@@ -447,10 +447,14 @@ void flash_kernel(FlashParams P) {
     auto fetch = [&](int it) { fetch_into(it, kst, vst); };
     auto stash = [&](int buf) { stash_from(buf, kst, vst); };
 
-    // ---- per-lane LDS read offsets (elements).
-    const int k_rd = c * KPAD + 8 * hb;                                       // + 32*sb*KPAD + 16*ks
-    const int v_rd = (4 * hb + ((lane & 15) >> 2)) * VPAD + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-    //                                            + (32*sb + 16*t + 8*u)*VPAD + 32*db
+    // ---- per-lane LDS read offsets (elements) of the padded layout (robust and pipelined pass).
+    // Worked out inside those passes, from a lane index the compiler cannot trace: computed here
+    // they would stay live across the lean pass, which has no register to spare for them.
+    auto k_rd_of = [&]() { const int l = opaque(lane); return (l & 31) * KPAD + 8 * (l >> 5); };  // + 32*sb*KPAD + 16*ks
+    auto v_rd_of = [&]() {
+        const int l = opaque(lane);
+        return (4 * (l >> 5) + ((l & 15) >> 2)) * VPAD + 16 * ((l >> 4) & 1) + 4 * (l & 3);
+    };  //                                        + (32*sb + 16*t + 8*u)*VPAD + 32*db
 
     float m_run[QB], l_run[QB];
     f32x16 o_acc[QB][DB];
@@ -459,6 +463,7 @@ void flash_kernel(FlashParams P) {
     // with a running maximum; otherwise p = 2^s is accumulated as is.
     auto run_pass = [&](auto robust_tag) {
         constexpr bool ROBUST = decltype(robust_tag)::value;
+        const int k_rd = k_rd_of(), v_rd = v_rd_of();
 #pragma unroll
         for (int j = 0; j < QB; ++j) {
             m_run[j] = ROBUST ? -INFINITY : 0.f;
@@ -595,6 +600,7 @@ void flash_kernel(FlashParams P) {
     // stages with one barrier per tile: tile it+2 is stored while tile it is
     // computed and block 0 of tile it+1 is already being multiplied.
     auto fast_pass = [&]() {
+        const int k_rd = k_rd_of(), v_rd = v_rd_of();
 #pragma unroll
         for (int j = 0; j < QB; ++j) {
             m_run[j] = 0.f;
@@ -811,20 +817,25 @@ void flash_kernel(FlashParams P) {
 
         constexpr int NP = (2 * CHUNKS + NT - 1) / NT;
         static_assert(CHUNKS % 64 == 0, "K/V choice must be wavefront-uniform");
-        bool p_on[NP], p_v[NP];
-        int p_row[NP], p_col[NP];
-        int p_dst[NP];       // element offset inside a stage
-#pragma unroll
-        for (int x = 0; x < NP; ++x) {
+        // Where piece x of this thread sits: worked out where a (rare) register-staged tile needs it,
+        // from a lane index the compiler cannot trace — computed up front these values would sit in
+        // registers through the steady loop, and at 96 registers that means scratch memory written
+        // in the prologue of every launch.
+        struct Piece {
+            bool on, v;
+            int row, col, dst;  // row and column in the tile; element offset inside a stage
+        };
+        auto piece = [&](int x) {
+            Piece pc;
             const int idx0 = wave * 64 + x * NT;  // scalar: first piece of this wavefront in round x
-            p_on[x] = idx0 < 2 * CHUNKS;
-            p_v[x] = idx0 >= CHUNKS;
-            const int cidx = idx0 + lane - (p_v[x] ? CHUNKS : 0);
-            p_row[x] = cidx / CPR;
-            p_col[x] = (cidx % CPR) * 8;
-            p_dst[x] = p_v[x] ? v_off(p_row[x], p_col[x]) : k_off(p_row[x], p_col[x]);
-        }
-        u32x4 st_a[NP], st_b[NP];
+            pc.on = idx0 < 2 * CHUNKS;
+            pc.v = idx0 >= CHUNKS;
+            const int cidx = idx0 + opaque(lane) - (pc.v ? CHUNKS : 0);
+            pc.row = cidx / CPR;
+            pc.col = (cidx % CPR) * 8;
+            pc.dst = pc.v ? v_off(pc.row, pc.col) : k_off(pc.row, pc.col);
+            return pc;
+        };
 
         // Full context tiles (every row present, nothing masked): the steady state.
         const int n_main = (ctx_end - ctx_begin) / BN;
@@ -893,8 +904,9 @@ void flash_kernel(FlashParams P) {
             rows_left = (is_ctx ? ctx_end : P.Nb) - kv0;
 #pragma unroll
             for (int x = 0; x < NP; ++x) {
-                const View &src = p_v[x] ? vs_ : ks_;
-                g_src[x] = view_row<T>(src, bb, h, kv0) + p_row[x] * src.sn + p_col[x];
+                const Piece pc = piece(x);
+                const View &src = pc.v ? vs_ : ks_;
+                g_src[x] = view_row<T>(src, bb, h, kv0) + pc.row * src.sn + pc.col;
                 g_step[x] = static_cast<long>(BN) * src.sn;
             }
         };
@@ -903,7 +915,8 @@ void flash_kernel(FlashParams P) {
 #pragma unroll
             for (int x = 0; x < NP; ++x) {
                 st[x] = u32x4{0u, 0u, 0u, 0u};
-                if (p_on[x] && (rows_left >= BN || p_row[x] < rows_left)) st[x] = *reinterpret_cast<const u32x4 *>(g_src[x]);
+                const Piece pc = piece(x);
+                if (pc.on && (rows_left >= BN || pc.row < rows_left)) st[x] = *reinterpret_cast<const u32x4 *>(g_src[x]);
                 g_src[x] += g_step[x];
             }
             rows_left -= BN;
@@ -911,7 +924,10 @@ void flash_kernel(FlashParams P) {
         auto stash_tile = [&](auto stage_, const u32x4(&st)[NP]) {
 #pragma unroll
             for (int x = 0; x < NP; ++x)
-                if (p_on[x]) *reinterpret_cast<u32x4 *>(kv_lds + stage_ * LSTAGE + p_dst[x]) = st[x];
+            {
+                const Piece pc = piece(x);
+                if (pc.on) *reinterpret_cast<u32x4 *>(kv_lds + stage_ * LSTAGE + pc.dst) = st[x];
+            }
         };
 
         // One 32-key block of the tile in `stage_` against this wavefront's queries.
@@ -1008,6 +1024,7 @@ void flash_kernel(FlashParams P) {
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // direct loads of the steady state
                 __syncthreads();
                 const bool fetch = it + 2 < n_tiles && it + 2 >= n_main;
+                u32x4 st_a[NP];  // (local: a staging register that lived across the steady loop would be parked in scratch)
                 if (fetch) gfetch(it + 2, st_a);
                 const bool is_ctx = it < ctx_tiles;
                 const int kv0 = is_ctx ? ctx_begin + it * BN : (it - ctx_tiles) * BN;
@@ -1031,24 +1048,31 @@ void flash_kernel(FlashParams P) {
         // (read here, in front of the prologue's requests: where it is used the loop would wait for it)
         const int beside_now = P.dense_below > 0 && P.beside_rows ? *P.beside_rows : P.beside_n;
         {
-            // the first three tiles are requested together with the queries: full tiles by direct
-            // loads into their stages, a ragged or buffer tile among the first two through registers
+            // the first NST - 1 tiles are requested together with the queries, full tiles by direct
+            // loads into their stages.  A ragged or buffer tile among the first two goes through
+            // registers and is stored at once (small problems only: nothing there is worth keeping
+            // staging registers alive across the query scaling, which at 96 registers would park
+            // them in scratch memory on every launch, the common one included).
             u32x4 qraw[QB][KS];
             request_q(qraw);
-            if (n_main > 0)
+            if (n_main > 0) {
                 dma_tile(std::integral_constant<int, 0>{});
-            else if (n_tiles > 0)
-                gfetch(0, st_a);
-            if (n_main > 1)
+            } else if (n_tiles > 0) {
+                u32x4 st[NP];
+                gfetch(0, st);
+                stash_tile(std::integral_constant<int, 0>{}, st);
+            }
+            if (n_main > 1) {
                 dma_tile(std::integral_constant<int, 1>{});
-            else if (n_tiles > 1)
-                gfetch(1, st_b);
+            } else if (n_tiles > 1) {
+                u32x4 st[NP];
+                gfetch(1, st);
+                stash_tile(std::integral_constant<int, 1>{}, st);
+            }
 #pragma unroll
             for (int t = 2; t < NST - 1; ++t)
                 if (n_main > t) dma_tile(t);
             scale_q(qraw);
-            if (n_main <= 0 && n_tiles > 0) stash_tile(std::integral_constant<int, 0>{}, st_a);
-            if (n_main <= 1 && n_tiles > 1) stash_tile(std::integral_constant<int, 1>{}, st_b);
         }
 
         int it = 0;

@@ -30,7 +30,7 @@ Prints one JSON line:
   config4        configs[4] (d_model 512, 16 heads, B=2048, N_ctx=4096): 4 outputs x 64 rows
                  flattened into 256 scalar decode steps
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-config4]
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-config4] [--timed-only]
        python bench.py --config4            (instead: only the configs[4] leg)
        python bench.py --kernel-shapes      (instead: one decode layer-step at the shapes of
                                              configs[1], [3] and [4], timings on stderr)
@@ -461,7 +461,7 @@ def log_density_bench(device, dtype, model, with_cpu):
     return res
 
 
-def config4_bench(device, observe=True):
+def config4_bench(device, observe=True, event_ordering=False):
     """configs[4] end to end: the 12-layer d_model=512 / 16-head (head_dim 32) bf16 model, one shared
     context of 4096 rows, B=2048 trajectories, 256 sequential scalar decode steps (config4_inputs
     states the flattening).  Reports target-steps/s over the decode loop (prefill separately), the
@@ -473,6 +473,8 @@ def config4_bench(device, observe=True):
     model = build_model(device, dtype, CFG4)
     x_context, y_context, x_target = config4_inputs(device, dtype)
     pred = ARTabPFNPredictor.from_trained_model(model, backend="triton_shared_context")
+    if event_ordering:
+        pred.counter_ordering = False
     Nt = ROWS4 * OUTS4
     torch.manual_seed(0)
     run_decode(pred, x_context, y_context, x_target, 24, device, dtype, cap=Nt)
@@ -823,6 +825,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline legs")
     ap.add_argument("--no-config4", action="store_true", help="skip the configs[4] leg of the default run")
     ap.add_argument("--config4", action="store_true", help="only the configs[4] leg")
+    ap.add_argument("--timed-only", action="store_true",
+                    help="warm-up and the K timed steps only (for runs under a profiler: no instrumented re-runs, "
+                         "no CPU legs, no other configurations); with --config4: that leg without its instrumented runs")
     ap.add_argument("--full-last-layer", action="store_true",
                     help="let the last layer of a decode step finish the buffer row too (its output is read by nobody)")
     ap.add_argument("--event-ordering", action="store_true",
@@ -871,7 +876,8 @@ def main():
             leg(device)
             return
     if args.config4:
-        print(json.dumps({"config4": config4_bench(device)}), flush=True)
+        print(json.dumps({"config4": config4_bench(device, observe=not args.timed_only,
+                                                   event_ordering=args.event_ordering)}), flush=True)
         return
 
     model = build_model(device, dtype)
@@ -900,6 +906,11 @@ def main():
     stream_ordering = None if chain0 is None else ("counters" if getattr(chain0, "order", None) is not None else "events")
     log(f"[gpu] prefill {prefill_ms:.2f} ms; {args.steps} decode steps in {decode_ms:.2f} ms "
         f"({ms_per_step:.3f} ms/step, host wall {wall_ms:.1f} ms)")
+    if args.timed_only:
+        print(json.dumps({"metric": "ar_decode_target_steps_per_sec", "value": round(value, 2), "unit": "target-steps/s",
+                          "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+                          "stream_ordering": stream_ordering, "timed_only": True}), flush=True)
+        return
     # the whole configuration (all 256 steps), whatever K is: same recorded graphs, replayed once more
     if args.steps == NT3:
         full_ms = decode_ms
@@ -1059,7 +1070,7 @@ def main():
                 if hasattr(layer, name):
                     delattr(layer, name)
         torch.cuda.empty_cache()
-        out["config4"] = config4_bench(device)
+        out["config4"] = config4_bench(device, event_ordering=args.event_ordering)
     print(json.dumps(out), flush=True)
 
 
