@@ -134,6 +134,24 @@ __device__ __forceinline__ void load_row64_to_lds(const void *global_src, unsign
     __builtin_amdgcn_global_load_lds(global_src, lds_dst + 3024, 16, 48, 0);
 }
 
+// Kernel arguments are read with scalar loads through a cache that a launch finds cold, and the
+// compiler places each load where its field is first used: a prologue that steers by a dozen
+// fields of a 400-byte argument block pays one miss (200-300 ns) per 64-byte line, one after the
+// other.  Called first thing in a kernel, this touches every line of the first `BYTES` bytes of
+// the argument segment with one batch of loads and one wait; the loads that follow hit the cache.
+template <int BYTES>
+__device__ __forceinline__ void warm_kernel_arguments() {
+    typedef const unsigned __attribute__((address_space(4))) *ConstPtr;
+    ConstPtr ka = (ConstPtr)__builtin_amdgcn_kernarg_segment_ptr();
+    constexpr int LINES = (BYTES + 63) / 64;
+    static_assert(LINES >= 1 && LINES <= 16, "argument blocks of up to 1 KiB");
+    unsigned w[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) w[i] = ka[16 * (i < LINES ? i : LINES - 1)];
+    asm volatile("" ::"s"(w[0]), "s"(w[1]), "s"(w[2]), "s"(w[3]), "s"(w[4]), "s"(w[5]), "s"(w[6]), "s"(w[7]), "s"(w[8]),
+                 "s"(w[9]), "s"(w[10]), "s"(w[11]), "s"(w[12]), "s"(w[13]), "s"(w[14]), "s"(w[15]));
+}
+
 // A value again, as one the compiler cannot trace (typically the lane index): what rarely
 // executed code derives from it (rows, base addresses) is then computed where it is used instead
 // of being kept in registers across a hot loop that does not need it.

@@ -9,28 +9,39 @@ constexpr int kFlashBN = 64;
 // Keys per LDS tile: 64, or 128 for head_dim 32 when kTuneBN is 128.
 static int flash_bn(int Dh) { return (Dh == 32 && tune(kTuneBN, 64) == 128) ? 128 : 64; }
 
+// Grid of a launch: x = 8 * slices (the XCD in the low three bits), y = query tiles of a group,
+// z = blocks of eight (group, head) pairs.  grid.z is limited to 65535: beyond that (more than
+// half a million pairs) the blocks are spread over several launches.
+constexpr int kMaxGridZ = 65535;
+
 template <typename Kernel>
-static void launch_one(Kernel kernel, unsigned grid, unsigned block, hipStream_t stream, const FlashParams &P) {
-    LaunchTiming t;
-    const int how = observe_launch(kLaunchFlash, &t);
-    if (how == kObserveEvents) {
-        hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, stream, t.start, t.stop, 0, P);
-    } else if (how == kObserveStamps) {
-        FlashParams Q = P;
-        Q.stamps = t.stamps;
-        Q.stamps_capacity = t.stamps_capacity;
-        hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, stream, Q);
-    } else {
-        hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, stream, P);
+static void launch_one(Kernel kernel, dim3 grid, unsigned block, hipStream_t stream, const FlashParams &P0) {
+    const int z_total = static_cast<int>(grid.z);
+    for (int z0 = 0; z0 < z_total; z0 += kMaxGridZ) {
+        FlashParams P = P0;
+        P.kvg_block0 = z0;
+        grid.z = static_cast<unsigned>(z_total - z0 < kMaxGridZ ? z_total - z0 : kMaxGridZ);
+        LaunchTiming t;
+        const int how = observe_launch(kLaunchFlash, &t);
+        if (how == kObserveEvents) {
+            hipExtLaunchKernelGGL(kernel, grid, dim3(block), 0, stream, t.start, t.stop, 0, P);
+        } else if (how == kObserveStamps) {
+            P.stamps = t.stamps;
+            P.stamps_capacity = t.stamps_capacity;
+            hipLaunchKernelGGL(kernel, grid, dim3(block), 0, stream, P);
+        } else {
+            hipLaunchKernelGGL(kernel, grid, dim3(block), 0, stream, P);
+        }
     }
 }
 
 template <typename T, int DH>
 static hipError_t launch_flash_bm(const FlashParams &P, int BM, hipStream_t stream) {
-    const int W = P.tiles_per_group * P.n_split;
-    const int n_kvg = P.H * P.n_groups;
-    const unsigned grid = static_cast<unsigned>(((n_kvg + 7) / 8) * W * 8);
-    if (grid == 0) return hipSuccess;
+    const long n_kvg = static_cast<long>(P.H) * P.n_groups;
+    if (n_kvg == 0 || P.tiles_per_group <= 0 || P.n_split <= 0) return hipSuccess;
+    if (P.tiles_per_group > 65535) return hipErrorInvalidConfiguration;  // 16 million query rows per group
+    const dim3 grid(static_cast<unsigned>(8 * P.n_split), static_cast<unsigned>(P.tiles_per_group),
+                    static_cast<unsigned>((n_kvg + 7) / 8));
     if constexpr (DH == 32) {
         if (flash_bn(DH) == 128) {
             if (BM == 256)
@@ -90,3 +101,9 @@ hipError_t launch_flash_dtype(const FlashParams &P, bool is_bf16, int Dh, int BM
 
 
 }  // namespace artab
+
+#ifdef ARTAB_PHASES
+extern "C" __attribute__((visibility("default"))) int artab_phase_read(unsigned long long *host, int n) {
+    return hipMemcpyFromSymbol(host, HIP_SYMBOL(artab::g_phase), sizeof(unsigned long long) * n);
+}
+#endif

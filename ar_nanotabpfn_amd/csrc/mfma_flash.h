@@ -117,6 +117,7 @@ struct FlashParams {
     // Launches that share the array must not overlap in time (they are launches of one queue).
     unsigned long long *stamps;
     int stamps_capacity;
+    int kvg_block0;  // first block of eight (group, head) pairs of this launch (grid.z counts from here)
 };
 
 // Reading the wall clock is a request to one unit of the chip: a launch in which every wavefront
@@ -127,7 +128,7 @@ struct FlashParams {
 constexpr unsigned kStampStarters = 16;
 
 __device__ __forceinline__ void flash_stamp_start(const FlashParams &P) {  // first thread of a workgroup
-    if (P.stamps && blockIdx.x < kStampStarters)
+    if (P.stamps && blockIdx.x < kStampStarters && blockIdx.y == 0 && blockIdx.z == 0)
         __hip_atomic_fetch_min(&P.stamps[2], wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -138,7 +139,7 @@ __device__ __forceinline__ void flash_stamp_start(const FlashParams &P) {  // fi
 __device__ __forceinline__ void flash_stamp_end(const FlashParams &P) {
     const unsigned long long t =
         __hip_atomic_fetch_add(&P.stamps[1], 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (t != gridDim.x - 1) return;
+    if (t != static_cast<unsigned long long>(gridDim.x) * gridDim.y * gridDim.z - 1) return;
     const unsigned long long t1 = wall_clock64();
     const unsigned long long n = __hip_atomic_load(&P.stamps[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const unsigned long long t0 =
@@ -151,6 +152,16 @@ __device__ __forceinline__ void flash_stamp_end(const FlashParams &P) {
     __hip_atomic_store(&P.stamps[0], n + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+#ifdef ARTAB_PHASES
+__device__ unsigned long long g_phase[1024 * 16];
+#define PHASE_WG (blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z))
+#define PHASE(i) do { if (threadIdx.x == 0) g_phase[PHASE_WG * 16 + (i)] = __builtin_amdgcn_s_memtime(); } while (0)
+#define PHASEW(i) do { if (threadIdx.x == 448) g_phase[PHASE_WG * 16 + (i)] = __builtin_amdgcn_s_memtime(); } while (0)
+#else
+#define PHASE_WG 0u
+#define PHASE(i)
+#define PHASEW(i)
+#endif
 // Probability mass (sum of 2^s over a row) the fast path accepts.
 constexpr float kFastMassMax = 1.2676506e30f;  // 2^100
 constexpr float kFastMassMin = 7.8886091e-31f; // 2^-100
@@ -187,6 +198,7 @@ struct BoolTag {
 template <typename T, int DH, int QB, int NW, int BN, bool LEAN = false, int OCC = 1, bool PLAIN = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
 void flash_kernel(FlashParams P) {
+    warm_kernel_arguments<sizeof(FlashParams)>();
     typedef MfmaOps<T> Ops;
     typedef typename Ops::vec vec;
     constexpr int KS = DH / 16;
@@ -222,28 +234,39 @@ void flash_kernel(FlashParams P) {
     // (release: whatever this queue's earlier launches wrote is visible to the watcher that sees
     // the new count)
     if (LEAN && threadIdx.x == 0) redo_flag = 0;  // raised after the pass, at least one barrier later
-    if (P.started && blockIdx.x == 0 && threadIdx.x == 0)
+    if (P.started && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
         __hip_atomic_fetch_add(P.started, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
     if (threadIdx.x == 0) flash_stamp_start(P);
+    PHASE(0);
+#ifdef ARTAB_PHASES
+    if (threadIdx.x == 0 && PHASE_WG < 8) g_phase[PHASE_WG * 16 + 6] = wall_clock64();
+#endif
 
-    // ---- workgroup -> (kv-sharing group, q tile, context split); XCD-aware: the
-    // hardware deals consecutive workgroup ids round-robin over the 8 XCDs, so all
-    // workgroups that stream the same K/V are given ids congruent modulo 8.
-    const int W = P.tiles_per_group * P.n_split;
+    // ---- workgroup -> (kv-sharing group, q tile, context split).  The grid is three-dimensional
+    // so that none of this takes an integer division (three of them were 0.4 us of every launch):
+    // x = xcd + 8 * split, y = q tile, z = block of eight (group, head) pairs.  XCD-aware: the
+    // hardware deals workgroups round-robin over the 8 XCDs in the order x, y, z, and grid.x is a
+    // multiple of 8, so all workgroups that stream the same K/V (same pair, any tile and split)
+    // run on the XCD `x mod 8` and share its L2.
     const int n_kvg = P.H * P.n_groups;
     const int xcd = blockIdx.x & 7;
-    const int slot = blockIdx.x >> 3;
-    const int kvg = (slot / W) * 8 + xcd;
+    const int split = __builtin_amdgcn_readfirstlane(blockIdx.x >> 3);
+    const int tile = __builtin_amdgcn_readfirstlane(blockIdx.y);
+    const int kvg = __builtin_amdgcn_readfirstlane((P.kvg_block0 + static_cast<int>(blockIdx.z)) * 8 + xcd);
     if (kvg >= n_kvg) {
         if (P.stamps && threadIdx.x == 0) flash_stamp_end(P);
         return;
     }
-    const int w_in = slot % W;
-    const int split = w_in % P.n_split;
-    const int tile = w_in / P.n_split;
-    const int h = kvg % P.H;
-    const int g = kvg / P.H;
+    int h_ = kvg, g_ = 0;
+    if (P.n_groups != 1) {  // (a branch, not a select: the shared-context launches skip the division)
+        h_ = kvg % P.H;
+        g_ = kvg / P.H;
+    }
+    // scalars by construction; said explicitly because base addresses built from them are scalar
+    // operands of the direct-to-LDS loads
+    const int h = __builtin_amdgcn_readfirstlane(h_), g = __builtin_amdgcn_readfirstlane(g_);
     const long kvb = P.n_groups == 1 ? 0 : g;  // batch entry whose K/V this group reads
+    PHASE(8);
 
     const int tid = threadIdx.x;
     // wavefront index as a scalar: everything derived from it (the wavefront's rows, its
@@ -258,7 +281,6 @@ void flash_kernel(FlashParams P) {
     // been requested too, so that the kernel's first memory round trips overlap.
     vec qreg[QB][KS];
     int qi[QB];  // query index i within its batch entry, or -1
-    long qb[QB];
     // Batch entry b and index i of the query in column `col` (0..31) of block j of this wavefront;
     // false beyond the last row.  The epilogue asks again (with a column the compiler cannot
     // trace back to the lane index) instead of keeping addresses alive across the key loop.
@@ -278,15 +300,22 @@ void flash_kernel(FlashParams P) {
 #pragma unroll
     for (int j = 0; j < QB; ++j) {
         int i;
-        const bool valid = query_of(j, c, qb[j], i);
+        long b;
+        const bool valid = query_of(j, c, b, i);
         qi[j] = valid ? i : -1;
     }
-    // Raw query fragments of this lane (addresses recomputed from qb/qi: nothing extra stays live
-    // across the key loop), and their scaled, rounded form in qreg.
-    auto request_q = [&](u32x4(&qraw)[QB][KS]) {
+    PHASE(9);
+    // Raw query fragments of this lane, and their scaled, rounded form in qreg.  `ln` is the lane
+    // index: a pass that may run after the key loop (the robust one) hands it over as a value the
+    // compiler cannot trace, so that rows and addresses are worked out afresh there instead of
+    // staying live (parked in scratch memory at this register budget) across the loop.
+    auto request_q = [&](u32x4(&qraw)[QB][KS], int ln) {
 #pragma unroll
         for (int j = 0; j < QB; ++j) {
-            const T *qrow = view_row<T>(P.q, qb[j], h, qi[j] >= 0 ? qi[j] : 0) + 8 * hb;
+            long b;
+            int i;
+            const bool valid = query_of(j, ln & 31, b, i);
+            const T *qrow = view_row<T>(P.q, b, h, valid ? i : 0) + 8 * (ln >> 5);
 #pragma unroll
             // unconditional: a column past the last row re-reads the group's first row (a valid
             // address) and is zeroed when it is scaled.  A load under a lane mask, merged with
@@ -296,11 +325,12 @@ void flash_kernel(FlashParams P) {
         }
     };
     bool q_scaled = false;
-    auto scale_q = [&](const u32x4(&qraw)[QB][KS]) {
+    auto scale_q = [&](const u32x4(&qraw)[QB][KS], int ln) {
         q_scaled = true;
 #pragma unroll
         for (int j = 0; j < QB; ++j) {
-            const float qs = qi[j] >= 0 ? P.qscale : 0.f;  // columns past the last row carry zero queries
+            // columns past the last row carry zero queries
+            const float qs = row0_w + 32 * j + (ln & 31) < P.G ? P.qscale : 0.f;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 u32x4 sc;
@@ -370,6 +400,7 @@ void flash_kernel(FlashParams P) {
         buf_tiles = (wg_max + BN - 1) / BN;
     }
     const int n_tiles = ctx_tiles + buf_tiles;
+    PHASE(10);
 
     // ---- staging: global -> registers -> LDS.  Each thread owns NCH 16-byte chunks
     // (row st_row, column st_col) of the K tile and the same of V; their global
@@ -476,8 +507,9 @@ void flash_kernel(FlashParams P) {
 
         if (!q_scaled) {  // else the fast pass has left qreg ready
             u32x4 qraw[QB][KS];
-            request_q(qraw);
-            scale_q(qraw);
+            const int ln = opaque(lane);
+            request_q(qraw, ln);
+            scale_q(qraw, ln);
         }
         if (n_tiles > 0) {
             fetch(0);
@@ -613,10 +645,10 @@ void flash_kernel(FlashParams P) {
         // the first two tiles and the queries are requested together: one memory round trip
         // before the loop instead of three
         u32x4 kst1[NCH], vst1[NCH], qraw[QB][KS];
-        request_q(qraw);
+        request_q(qraw, lane);
         if (n_tiles > 0) fetch(0);
         if (n_tiles > 1) fetch_into(1, kst1, vst1);
-        scale_q(qraw);
+        scale_q(qraw, lane);
         if (n_tiles > 0) stash(0);
         if (n_tiles > 1) stash_from(1, kst1, vst1);
         __syncthreads();
@@ -773,6 +805,7 @@ void flash_kernel(FlashParams P) {
     //  * K and V tiles of a stage are one list of 16-byte pieces dealt over the whole workgroup.
     // NST LDS stages (four), one barrier per tile, full tiles requested NST - 1 ahead.
     auto lean_pass = [&]() {
+        PHASE(11);
         f32x4 lsum[QB][2];
 #pragma unroll
         for (int j = 0; j < QB; ++j) {
@@ -1044,6 +1077,7 @@ void flash_kernel(FlashParams P) {
             }
         };
 
+        PHASE(12);
         __builtin_amdgcn_s_setprio(3);
         // (read here, in front of the prologue's requests: where it is used the loop would wait for it)
         const int beside_now = P.dense_below > 0 && P.beside_rows ? *P.beside_rows : P.beside_n;
@@ -1054,26 +1088,40 @@ void flash_kernel(FlashParams P) {
             // staging registers alive across the query scaling, which at 96 registers would park
             // them in scratch memory on every launch, the common one included).
             u32x4 qraw[QB][KS];
-            request_q(qraw);
-            if (n_main > 0) {
+            if (PHASE_WG >= 8) PHASE(6);
+            request_q(qraw, lane);
+            if (n_main >= NST - 1) {
+                // The common case on a path of its own: where it shares basic blocks with the
+                // register-staged tiles below, the compiler has to assume one of their loads
+                // pending when the paths meet and drains the memory counter — the queries
+                // included — in front of the first direct load: a whole round trip.
                 dma_tile(std::integral_constant<int, 0>{});
-            } else if (n_tiles > 0) {
-                u32x4 st[NP];
-                gfetch(0, st);
-                stash_tile(std::integral_constant<int, 0>{}, st);
-            }
-            if (n_main > 1) {
                 dma_tile(std::integral_constant<int, 1>{});
-            } else if (n_tiles > 1) {
-                u32x4 st[NP];
-                gfetch(1, st);
-                stash_tile(std::integral_constant<int, 1>{}, st);
-            }
 #pragma unroll
-            for (int t = 2; t < NST - 1; ++t)
-                if (n_main > t) dma_tile(t);
-            scale_q(qraw);
+                for (int t = 2; t < NST - 1; ++t) dma_tile(t);
+            } else {
+                if (n_main > 0) {
+                    dma_tile(std::integral_constant<int, 0>{});
+                } else if (n_tiles > 0) {
+                    u32x4 st[NP];
+                    gfetch(0, st);
+                    stash_tile(std::integral_constant<int, 0>{}, st);
+                }
+                if (n_main > 1) {
+                    dma_tile(std::integral_constant<int, 1>{});
+                } else if (n_tiles > 1) {
+                    u32x4 st[NP];
+                    gfetch(1, st);
+                    stash_tile(std::integral_constant<int, 1>{}, st);
+                }
+#pragma unroll
+                for (int t = 2; t < NST - 1; ++t)
+                    if (n_main > t) dma_tile(t);
+            }
+            if (PHASE_WG >= 8) PHASE(7);
+            scale_q(qraw, lane);
         }
+        PHASE(1);
 
         int it = 0;
         // with nothing but full context tiles the whole slice is steady state; otherwise the last
@@ -1126,6 +1174,7 @@ void flash_kernel(FlashParams P) {
 #pragma nounroll
                 for (; it < end; it += NST) {
                     fast_tile(std::integral_constant<int, 0>{});
+                    if (it == 0) PHASE(2);
                     fast_tile(std::integral_constant<int, 1>{});
                     fast_tile(std::integral_constant<int, 2>{});
                     fast_tile(std::integral_constant<int, 3>{});
@@ -1162,6 +1211,8 @@ void flash_kernel(FlashParams P) {
             tile(it, stage, BoolTag<false>{});
             stage = stage == NST - 1 ? 0 : stage + 1;
         }
+        PHASE(3);
+        PHASEW(5);
         // row sums: query c of this lane's block sits in lane c % 16, register c / 16; the total
         // already covers both halves, so only the hb = 0 lane carries it into the epilogue
 #pragma unroll
@@ -1201,6 +1252,9 @@ void flash_kernel(FlashParams P) {
 
     // ---- epilogue: normalise, write output (final or split partial) and log-sum-exp.
     const long total_rows = static_cast<long>(P.B) * P.H * P.Lq;
+    // (the half of the wavefront again, from a lane index the compiler cannot trace: kept from the
+    // prologue it would be parked in scratch memory across the key loop)
+    const int hb_e = opaque(lane) >> 5;
 #pragma unroll
     for (int j = 0; j < QB; ++j) {
         float l_tot = l_run[j] + __shfl_xor(l_run[j], 32, 64);
@@ -1219,9 +1273,9 @@ void flash_kernel(FlashParams P) {
                 for (int gq = 0; gq < 4; ++gq) {
                     u32x2 val = {pack2<T>(o_acc[j][db][4 * gq] * inv, o_acc[j][db][4 * gq + 1] * inv),
                                  pack2<T>(o_acc[j][db][4 * gq + 2] * inv, o_acc[j][db][4 * gq + 3] * inv)};
-                    *reinterpret_cast<u32x2 *>(po + 32 * db + 8 * gq + 4 * hb) = val;
+                    *reinterpret_cast<u32x2 *>(po + 32 * db + 8 * gq + 4 * hb_e) = val;
                 }
-            if (hb == 0) P.part_lse[static_cast<long>(split) * total_rows + orow_idx] = lse;
+            if (hb_e == 0) P.part_lse[static_cast<long>(split) * total_rows + orow_idx] = lse;
         } else {
             T *orow = view_row<T>(P.out, ob, h, oi);
 #pragma unroll
@@ -1230,11 +1284,15 @@ void flash_kernel(FlashParams P) {
                 for (int gq = 0; gq < 4; ++gq) {
                     u32x2 val = {pack2<T>(o_acc[j][db][4 * gq] * inv, o_acc[j][db][4 * gq + 1] * inv),
                                  pack2<T>(o_acc[j][db][4 * gq + 2] * inv, o_acc[j][db][4 * gq + 3] * inv)};
-                    *reinterpret_cast<u32x2 *>(orow + 32 * db + 8 * gq + 4 * hb) = val;
+                    *reinterpret_cast<u32x2 *>(orow + 32 * db + 8 * gq + 4 * hb_e) = val;
                 }
-            if (P.lse && hb == 0) P.lse[orow_idx] = lse;
+            if (P.lse && hb_e == 0) P.lse[orow_idx] = lse;
         }
     }
+    PHASE(4);
+#ifdef ARTAB_PHASES
+    if (threadIdx.x == 0 && PHASE_WG < 8) g_phase[PHASE_WG * 16 + 7] = wall_clock64();
+#endif
     if (P.stamps) {
         __syncthreads();  // every wavefront of the workgroup has issued its stores
         if (threadIdx.x == 0) flash_stamp_end(P);
