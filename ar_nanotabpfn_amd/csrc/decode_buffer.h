@@ -355,6 +355,7 @@ __device__ __forceinline__ void decode_buffer_pair(const DecodeParams &P, long b
 
 template <typename T, int DH, int LQ>
 __global__ __launch_bounds__(kDecodeWaves * 64) void decode_buffer_kernel(DecodeParams P) {
+    warm_kernel_arguments<sizeof(DecodeParams)>();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const long pair = static_cast<long>(blockIdx.x) * kDecodeWaves + wave;  // b*H + h
     if (pair >= static_cast<long>(P.B) * P.H) return;

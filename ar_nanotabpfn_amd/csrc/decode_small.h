@@ -29,6 +29,7 @@ constexpr int kSmallTraj = 8;  // trajectories per workgroup: one per wavefront 
 
 template <typename T, int DH, int LQ>
 __global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodeParams P, View kc, View vc, int Nc) {
+    warm_kernel_arguments<sizeof(DecodeParams) + 2 * sizeof(View) + sizeof(int)>();
     typedef MfmaOps<T> Ops;
     typedef typename Ops::vec vec;
     constexpr int KS = DH / 16, DB = DH / 32, NW = kSmallWaves, NCOL = kSmallTraj * LQ;

@@ -461,6 +461,7 @@ __device__ __forceinline__ void decode_stream_body(const DecodeParams &P, unsign
 // pins the shape.  Dynamic LDS: kStreamLdsBytes.
 template <typename T, int LQ, int PRIO = 3, int KEYS = 0>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void decode_stream_kernel(DecodeParams P) {
+    warm_kernel_arguments<sizeof(DecodeParams)>();
     extern __shared__ __attribute__((aligned(16))) unsigned char stream_lds[];
     bool slot_fits;
     const int n_buf = committed_rows(P, slot_fits);

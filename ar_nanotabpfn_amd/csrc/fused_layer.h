@@ -710,6 +710,7 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
 
 template <typename T, int D, int TR>
 __global__ __launch_bounds__(fused_waves(D) * 64) void fused_pre_kernel(FusedPreParams P) {
+    warm_kernel_arguments<sizeof(FusedPreParams)>();
     constexpr int NW = fused_waves(D), LD = D + 8;
     __shared__ __attribute__((aligned(16))) T a0[TR * LD];
     __shared__ __attribute__((aligned(16))) T a1[TR * LD];
@@ -877,6 +878,7 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
 
 template <typename T, int D, int F, int TR>
 __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_kernel(FusedPostParams P) {
+    warm_kernel_arguments<sizeof(FusedPostParams)>();
     constexpr int NW = fused_waves(D), LDD = D + 8, LDF = F + 8, LDM = LDD > LDF ? LDD : LDF;
     __shared__ __attribute__((aligned(16))) T a0[TR * LDM];
     __shared__ __attribute__((aligned(16))) T a1[TR * LDD];
@@ -893,6 +895,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_kernel(FusedPo
 // never leaves LDS, and one launch (with its fixed cost) disappears per layer boundary.
 template <typename T, int D, int F, int TR>
 __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_pre_kernel(FusedPostParams P, FusedPreParams N) {
+    warm_kernel_arguments<sizeof(FusedPostParams) + sizeof(FusedPreParams)>();
     constexpr int NW = fused_waves(D), LDD = D + 8, LDF = F + 8, LDM = LDD > LDF ? LDD : LDF;
     __shared__ __attribute__((aligned(16))) T a0[TR * LDM];
     __shared__ __attribute__((aligned(16))) T a1[TR * LDD];
@@ -1231,6 +1234,7 @@ __device__ __forceinline__ void advance_loop_counters(const SampleEmbedParams &P
 
 template <typename T, int D, int F, int TR>
 __global__ __launch_bounds__(fused_waves(D) * 64) void sample_embed_kernel(SampleEmbedParams P) {
+    warm_kernel_arguments<sizeof(SampleEmbedParams)>();
     constexpr int NW = fused_waves(D);
     constexpr int LDD = D + 8, LDF = F + 8;
     __shared__ __attribute__((aligned(16))) T a0[TR * LDD];  // z = norm(x_last)
@@ -1262,6 +1266,7 @@ template <typename T, int D, int F, int TR>
 __global__ __launch_bounds__(fused_waves(D) * 64) void decode_step_boundary_kernel(FusedPostParams P,
                                                                                     SampleEmbedParams S,
                                                                                     FusedPreParams N) {
+    warm_kernel_arguments<sizeof(FusedPostParams) + sizeof(SampleEmbedParams) + sizeof(FusedPreParams)>();
     constexpr int TJ = TR / 2;
     constexpr int NW = fused_waves(D), LDD = D + 8, LDF = F + 8, LDM = LDD > LDF ? LDD : LDF;
     __shared__ __attribute__((aligned(16))) T a0[TR * LDM];
