@@ -101,9 +101,3 @@ hipError_t launch_flash_dtype(const FlashParams &P, bool is_bf16, int Dh, int BM
 
 
 }  // namespace artab
-
-#ifdef ARTAB_PHASES
-extern "C" __attribute__((visibility("default"))) int artab_phase_read(unsigned long long *host, int n) {
-    return hipMemcpyFromSymbol(host, HIP_SYMBOL(artab::g_phase), sizeof(unsigned long long) * n);
-}
-#endif

@@ -152,16 +152,6 @@ __device__ __forceinline__ void flash_stamp_end(const FlashParams &P) {
     __hip_atomic_store(&P.stamps[0], n + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-#ifdef ARTAB_PHASES
-__device__ unsigned long long g_phase[1024 * 16];
-#define PHASE_WG (blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z))
-#define PHASE(i) do { if (threadIdx.x == 0) g_phase[PHASE_WG * 16 + (i)] = __builtin_amdgcn_s_memtime(); } while (0)
-#define PHASEW(i) do { if (threadIdx.x == 448) g_phase[PHASE_WG * 16 + (i)] = __builtin_amdgcn_s_memtime(); } while (0)
-#else
-#define PHASE_WG 0u
-#define PHASE(i)
-#define PHASEW(i)
-#endif
 // Probability mass (sum of 2^s over a row) the fast path accepts.
 constexpr float kFastMassMax = 1.2676506e30f;  // 2^100
 constexpr float kFastMassMin = 7.8886091e-31f; // 2^-100
@@ -237,10 +227,6 @@ void flash_kernel(FlashParams P) {
     if (P.started && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
         __hip_atomic_fetch_add(P.started, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
     if (threadIdx.x == 0) flash_stamp_start(P);
-    PHASE(0);
-#ifdef ARTAB_PHASES
-    if (threadIdx.x == 0 && PHASE_WG < 8) g_phase[PHASE_WG * 16 + 6] = wall_clock64();
-#endif
 
     // ---- workgroup -> (kv-sharing group, q tile, context split).  The grid is three-dimensional
     // so that none of this takes an integer division (three of them were 0.4 us of every launch):
@@ -266,7 +252,6 @@ void flash_kernel(FlashParams P) {
     // operands of the direct-to-LDS loads
     const int h = __builtin_amdgcn_readfirstlane(h_), g = __builtin_amdgcn_readfirstlane(g_);
     const long kvb = P.n_groups == 1 ? 0 : g;  // batch entry whose K/V this group reads
-    PHASE(8);
 
     const int tid = threadIdx.x;
     // wavefront index as a scalar: everything derived from it (the wavefront's rows, its
@@ -304,7 +289,6 @@ void flash_kernel(FlashParams P) {
         const bool valid = query_of(j, c, b, i);
         qi[j] = valid ? i : -1;
     }
-    PHASE(9);
     // Raw query fragments of this lane, and their scaled, rounded form in qreg.  `ln` is the lane
     // index: a pass that may run after the key loop (the robust one) hands it over as a value the
     // compiler cannot trace, so that rows and addresses are worked out afresh there instead of
@@ -400,7 +384,6 @@ void flash_kernel(FlashParams P) {
         buf_tiles = (wg_max + BN - 1) / BN;
     }
     const int n_tiles = ctx_tiles + buf_tiles;
-    PHASE(10);
 
     // ---- staging: global -> registers -> LDS.  Each thread owns NCH 16-byte chunks
     // (row st_row, column st_col) of the K tile and the same of V; their global
@@ -805,7 +788,6 @@ void flash_kernel(FlashParams P) {
     //  * K and V tiles of a stage are one list of 16-byte pieces dealt over the whole workgroup.
     // NST LDS stages (four), one barrier per tile, full tiles requested NST - 1 ahead.
     auto lean_pass = [&]() {
-        PHASE(11);
         f32x4 lsum[QB][2];
 #pragma unroll
         for (int j = 0; j < QB; ++j) {
@@ -1077,7 +1059,6 @@ void flash_kernel(FlashParams P) {
             }
         };
 
-        PHASE(12);
         __builtin_amdgcn_s_setprio(3);
         // (read here, in front of the prologue's requests: where it is used the loop would wait for it)
         const int beside_now = P.dense_below > 0 && P.beside_rows ? *P.beside_rows : P.beside_n;
@@ -1088,7 +1069,6 @@ void flash_kernel(FlashParams P) {
             // staging registers alive across the query scaling, which at 96 registers would park
             // them in scratch memory on every launch, the common one included).
             u32x4 qraw[QB][KS];
-            if (PHASE_WG >= 8) PHASE(6);
             request_q(qraw, lane);
             if (n_main >= NST - 1) {
                 // The common case on a path of its own: where it shares basic blocks with the
@@ -1118,10 +1098,8 @@ void flash_kernel(FlashParams P) {
                 for (int t = 2; t < NST - 1; ++t)
                     if (n_main > t) dma_tile(t);
             }
-            if (PHASE_WG >= 8) PHASE(7);
             scale_q(qraw, lane);
         }
-        PHASE(1);
 
         int it = 0;
         // with nothing but full context tiles the whole slice is steady state; otherwise the last
@@ -1174,7 +1152,6 @@ void flash_kernel(FlashParams P) {
 #pragma nounroll
                 for (; it < end; it += NST) {
                     fast_tile(std::integral_constant<int, 0>{});
-                    if (it == 0) PHASE(2);
                     fast_tile(std::integral_constant<int, 1>{});
                     fast_tile(std::integral_constant<int, 2>{});
                     fast_tile(std::integral_constant<int, 3>{});
@@ -1211,8 +1188,6 @@ void flash_kernel(FlashParams P) {
             tile(it, stage, BoolTag<false>{});
             stage = stage == NST - 1 ? 0 : stage + 1;
         }
-        PHASE(3);
-        PHASEW(5);
         // row sums: query c of this lane's block sits in lane c % 16, register c / 16; the total
         // already covers both halves, so only the hb = 0 lane carries it into the epilogue
 #pragma unroll
@@ -1289,10 +1264,6 @@ void flash_kernel(FlashParams P) {
             if (P.lse && hb_e == 0) P.lse[orow_idx] = lse;
         }
     }
-    PHASE(4);
-#ifdef ARTAB_PHASES
-    if (threadIdx.x == 0 && PHASE_WG < 8) g_phase[PHASE_WG * 16 + 7] = wall_clock64();
-#endif
     if (P.stamps) {
         __syncthreads();  // every wavefront of the workgroup has issued its stores
         if (threadIdx.x == 0) flash_stamp_end(P);
