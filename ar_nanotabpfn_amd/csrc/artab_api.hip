@@ -36,7 +36,8 @@ struct TuneSlot {
 static TuneSlot g_tune[kTuneCount] = {
     {"ARTAB_BM", false, 0},          {"ARTAB_SPLIT", false, 0},        {"ARTAB_SMALL", false, 0},
     {"ARTAB_STREAM", false, 0},      {"ARTAB_STREAM_PER_CU", false, 0}, {"ARTAB_STREAM_PRIO", false, 0},
-    {"ARTAB_STREAM_SHORT", false, 0}, {"ARTAB_DENSE_BELOW", false, 0},  {"ARTAB_ORDER_GATE_LAUNCH", false, 0},
+    {"ARTAB_STREAM_SHORT", false, 0}, {"ARTAB_STREAM_CALM", false, 0},  {"ARTAB_DENSE_BELOW", false, 0},
+    {"ARTAB_ORDER_GATE_LAUNCH", false, 0},
     {"ARTAB_BN", false, 0},          {"ARTAB_LEAN", false, 0},         {"ARTAB_LEAN_OCC", false, 0},
     {"ARTAB_NW", false, 0},          {"ARTAB_TILE_ROWS", false, 0},
 };
@@ -692,6 +693,17 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
         const long fit = per_row > 0 ? kLastLevelCacheBytes / per_row : 0;
         const long rows = fit > kStreamShortRows ? fit : kStreamShortRows;
         D.stream_short_rows = tune(kTuneStreamShort, static_cast<int>(rows < 1 << 20 ? rows : 1 << 20));
+        // Wave priority of the streaming pass: raised only once the pass is long enough to be what the
+        // layer waits for.  A short buffer pass ends long before the context pass beside it, and at
+        // the raised priority it only takes issue slots from that one (measured at B=1024, H=8:
+        // base priority +1.0 % target-steps/s over steps 0..63, -3 % over steps 64..95; the buffers
+        // hold 64 MiB at the switch).  Only while one round of tasks covers all pairs (16 pairs per
+        // task, two wavefronts per compute unit beside the context pass): with more rounds than
+        // that the pass is nearly as long as its neighbour from the first row on (B=2048, H=16:
+        // -0.3 % with a switch at 16 rows, so none there).
+        const long one_round = 16L * 2 * 256;
+        const long calm = per_row > 0 && static_cast<long>(B) * H <= one_round ? (64L << 20) / per_row : 0;
+        D.stream_calm_rows = tune(kTuneStreamCalm, static_cast<int>(calm < 1 << 20 ? calm : 1 << 20));
     }
     if (side_stream && side_stream != stream) {  // the two passes share the compute units
         F.beside_rows = n_buf_device;

@@ -27,6 +27,7 @@ struct DecodeParams {
     int n_buf;    // committed buffer rows
     const int *n_buf_dev;  // when set, the committed length is read from here at run time
     int stream_short_rows;  // streaming variant: buffers longer than this are read 16 rows x 4 pairs at a time
+    int stream_calm_rows;   // streaming variant: buffers up to this length are streamed at the base wave priority
     int n_base;   // rows of kb/vb that precede the counted ones (a per-trajectory context stored in
                   // front of the buffer rows); 0 for a shared context
     int has_new;  // 1: row n_buf comes from knew/vnew, is attended and appended

@@ -466,8 +466,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4))) void de
     bool slot_fits;
     const int n_buf = committed_rows(P, slot_fits);
     // This wavefront shares its SIMD with older, compute-bound ones; without a raised priority it
-    // is only issued in their gaps.  It issues little: the priority costs them little.
-    __builtin_amdgcn_s_setprio(PRIO);
+    // is only issued in their gaps.  It issues little: the priority costs them little — but not
+    // nothing, so a buffer short enough to be done long before its neighbours stays at the base priority.
+    if (n_buf + (P.has_new ? 1 : 0) > P.stream_calm_rows) __builtin_amdgcn_s_setprio(PRIO);
     if (KEYS == 4 || (KEYS == 0 && n_buf + (P.has_new ? 1 : 0) <= P.stream_short_rows))
         decode_stream_body<T, LQ, 4>(P, stream_lds, n_buf, slot_fits);
     else

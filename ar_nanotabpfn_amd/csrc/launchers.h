@@ -25,6 +25,7 @@ enum Tune : int {
     kTuneStreamPerCu,     // ARTAB_STREAM_PER_CU: workgroups of the streaming buffer pass per compute unit (1..4)
     kTuneStreamPrio,      // ARTAB_STREAM_PRIO: wave priority of the streaming buffer pass (0..3)
     kTuneStreamShort,     // ARTAB_STREAM_SHORT: buffer rows above which the streaming pass reads 16-row chunks
+    kTuneStreamCalm,      // ARTAB_STREAM_CALM: buffer rows up to which the streaming pass keeps the base wave priority
     kTuneDenseBelow,      // ARTAB_DENSE_BELOW: buffer rows below which the context pass runs its straight-line tile groups
     kTuneOrderGateLaunch, // ARTAB_ORDER_GATE_LAUNCH: 1 makes the layer kernel's wait for the side queue a launch of its own
     kTuneBN,              // ARTAB_BN: keys per LDS tile at head_dim 32 (64/128)
