@@ -152,7 +152,7 @@ BENCH_SIGNATURES = {
 }
 
 TUNING_KEYS = ("ARTAB_BM", "ARTAB_SPLIT", "ARTAB_SMALL", "ARTAB_STREAM", "ARTAB_STREAM_PER_CU", "ARTAB_STREAM_PRIO",
-               "ARTAB_STREAM_SHORT", "ARTAB_STREAM_CALM", "ARTAB_DENSE_BELOW", "ARTAB_ORDER_GATE_LAUNCH", "ARTAB_BN", "ARTAB_LEAN",
+               "ARTAB_STREAM_SHORT", "ARTAB_STREAM_CALM", "ARTAB_DENSE_BELOW", "ARTAB_CTX_YIELD", "ARTAB_ORDER_GATE_LAUNCH", "ARTAB_BN", "ARTAB_LEAN",
                "ARTAB_LEAN_OCC", "ARTAB_NW", "ARTAB_TILE_ROWS")
 
 _lib: Optional[ctypes.CDLL] = None

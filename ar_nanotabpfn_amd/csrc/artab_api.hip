@@ -37,7 +37,7 @@ static TuneSlot g_tune[kTuneCount] = {
     {"ARTAB_BM", false, 0},          {"ARTAB_SPLIT", false, 0},        {"ARTAB_SMALL", false, 0},
     {"ARTAB_STREAM", false, 0},      {"ARTAB_STREAM_PER_CU", false, 0}, {"ARTAB_STREAM_PRIO", false, 0},
     {"ARTAB_STREAM_SHORT", false, 0}, {"ARTAB_STREAM_CALM", false, 0},  {"ARTAB_DENSE_BELOW", false, 0},
-    {"ARTAB_ORDER_GATE_LAUNCH", false, 0},
+    {"ARTAB_CTX_YIELD", false, 0},    {"ARTAB_ORDER_GATE_LAUNCH", false, 0},
     {"ARTAB_BN", false, 0},          {"ARTAB_LEAN", false, 0},         {"ARTAB_LEAN_OCC", false, 0},
     {"ARTAB_NW", false, 0},          {"ARTAB_TILE_ROWS", false, 0},
 };
@@ -709,6 +709,16 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
         F.beside_rows = n_buf_device;
         F.beside_n = n_buf;
         F.dense_below = tune(kTuneDenseBelow, 128);
+        // From the buffer length at which the buffer pass is about to become the longer kernel of
+        // the two, the context pass runs one priority step lower: it is no longer what the layer
+        // waits for.  Estimated from the work: buffer bytes at 5 TB/s against context flops at
+        // 900 TFLOP/s, switch at 0.8 of the context pass's time (146 rows at B=1024, H=8,
+        // N_ctx=16384; 36 at B=2048, H=16, N_ctx=4096).  Measured: +0.9 % target-steps/s over 256
+        // steps at the first shape (switch anywhere in 128..192), +1.0 % at the second.
+        const double ctx_flops = 4.0 * B * H * Lq * static_cast<double>(Nc) * Dh;
+        const double per_row = static_cast<double>(B) * H * 2 * Dh * 2;
+        const double yield_rows = per_row > 0 ? ctx_flops * 4.4e-3 / per_row : 0;
+        F.yield_from = tune(kTuneCtxYield, static_cast<int>(yield_rows < 1 ? 1 : (yield_rows < 1 << 20 ? yield_rows : 1 << 20)));
     }
     D.buf_part_o = static_cast<char *>(workspace) + static_cast<size_t>(pl.n_split) * rows * Dh * 2;
     D.buf_part_lse = F.part_lse + static_cast<size_t>(pl.n_split) * rows;

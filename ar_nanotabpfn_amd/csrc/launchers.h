@@ -27,6 +27,7 @@ enum Tune : int {
     kTuneStreamShort,     // ARTAB_STREAM_SHORT: buffer rows above which the streaming pass reads 16-row chunks
     kTuneStreamCalm,      // ARTAB_STREAM_CALM: buffer rows up to which the streaming pass keeps the base wave priority
     kTuneDenseBelow,      // ARTAB_DENSE_BELOW: buffer rows below which the context pass runs its straight-line tile groups
+    kTuneCtxYield,        // ARTAB_CTX_YIELD: buffer rows from which the context pass lowers its wave priority (0: never)
     kTuneOrderGateLaunch, // ARTAB_ORDER_GATE_LAUNCH: 1 makes the layer kernel's wait for the side queue a launch of its own
     kTuneBN,              // ARTAB_BN: keys per LDS tile at head_dim 32 (64/128)
     kTuneLean,            // ARTAB_LEAN: 0 selects the software-pipelined pass at head_dim 32

@@ -107,6 +107,7 @@ struct FlashParams {
     // takes slots from the buffer pass (256 steps: +0.3 % with the limit at 128 rows, 0 without).
     const int *beside_rows;
     int beside_n, dense_below;
+    int yield_from;  // rows of the neighbouring buffer pass from which this pass lowers its wave priority (0: never)
     unsigned *started;  // optional counter that the first thread of the grid advances at once: "the
                         // launches ahead of this one on its queue are complete" for a watcher on
                         // another queue (queue_order.h); the kernel's own work does not depend on it
@@ -854,6 +855,7 @@ void flash_kernel(FlashParams P) {
 
         // Full context tiles (every row present, nothing masked): the steady state.
         const int n_main = (ctx_end - ctx_begin) / BN;
+        bool yield_ = false;  // set once the neighbour's length is known (below)
 
         // In the steady state the tiles do not pass through registers at all: a stage is NI chunks
         // of one KiB, each filled by one direct global->LDS load (lane l lands at base + 16 l; the
@@ -1011,12 +1013,13 @@ void flash_kernel(FlashParams P) {
                 // first: left alone, one workgroup runs ahead and the other finishes the slice with
                 // the SIMDs half empty.  The priority falls with progress, so whoever is behind is
                 // served first (measured: the slower workgroup of a pair ends 2.5 us earlier).
-                if (it == n_main / 4)
-                    __builtin_amdgcn_s_setprio(2);
-                else if (it == n_main / 2)
-                    __builtin_amdgcn_s_setprio(1);
-                else if (it == 3 * n_main / 4)
+                if (it == n_main / 4) {
+                    if (yield_) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(2);
+                } else if (it == n_main / 2) {
+                    if (yield_) __builtin_amdgcn_s_setprio(0); else __builtin_amdgcn_s_setprio(1);
+                } else if (it == 3 * n_main / 4) {
                     __builtin_amdgcn_s_setprio(0);
+                }
                 // this tile's direct loads must have landed; those of the next two full tiles may
                 // still be on their way
                 const int behind = n_main - 1 - it;
@@ -1061,7 +1064,7 @@ void flash_kernel(FlashParams P) {
 
         __builtin_amdgcn_s_setprio(3);
         // (read here, in front of the prologue's requests: where it is used the loop would wait for it)
-        const int beside_now = P.dense_below > 0 && P.beside_rows ? *P.beside_rows : P.beside_n;
+        const int beside_now = (P.dense_below > 0 || P.yield_from > 0) && P.beside_rows ? *P.beside_rows : P.beside_n;
         {
             // the first NST - 1 tiles are requested together with the queries, full tiles by direct
             // loads into their stages.  A ragged or buffer tile among the first two goes through
@@ -1115,6 +1118,10 @@ void flash_kernel(FlashParams P) {
         bool dense = n_fast > 0;
         if (dense && P.dense_below > 0)  // (a scalar: the choice must stay a wavefront-uniform branch)
             dense = __builtin_amdgcn_readfirstlane(beside_now) < P.dense_below;
+        // Beside a buffer pass that is the longer kernel of the two, this pass gives way: one
+        // priority step lower throughout, so the neighbour's few instructions never queue behind it.
+        yield_ = P.yield_from > 0 && __builtin_amdgcn_readfirstlane(beside_now) >= P.yield_from;
+        if (yield_) __builtin_amdgcn_s_setprio(2);
         if (dense) {
             const bool two = n_dma == 2;  // direct loads of this wavefront per tile: one or two
             auto fast_tile = [&](auto stage_) {
