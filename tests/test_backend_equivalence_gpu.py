@@ -237,7 +237,7 @@ def to_np_f64(a):
 
 def test_config3_full_size_sampling_counter_ordered_equals_event_ordered(device):
     """configs[3] at its full shape (B=1024, N_ctx=16384, 12 layers, bf16): eleven sampled targets
-    from the recorded step (graphs of four steps, then a remainder), once with the two queues
+    from the recorded step (a graph of eight steps and one-step graphs for the remainder), once with the two queues
     ordered through the counters in device memory and once through events.  Same variates in:
     predictions and every buffer K/V row must be bit-identical — a partial read before the buffer
     pass had released it, or a stale line of the workspace that every layer reuses, would differ."""
