@@ -98,6 +98,25 @@ def test_context_attention_per_dataset_context(device, dtype):
     assert max_abs(to_np(lse), ref_lse) <= lse_tol(dtype)
 
 
+def test_context_attention_more_head_groups_than_one_grid_holds(device):
+    """Per-dataset contexts with more than 65535 x 8 (dataset, head) pairs: the matrix-core kernel's
+    grid counts blocks of eight pairs in its z dimension, so the call is spread over two launches.
+    The first and the last datasets against the oracle, everything against the portable kernel."""
+    ak = _ak()
+    B, H, Lq, Nc, D = 66000, 8, 1, 32, 32
+    g = torch.Generator(device=device).manual_seed(5)
+    mk = lambda *shape: (torch.randn(*shape, generator=g, device=device) * 0.6).to(torch.bfloat16)
+    q, k, v = mk(B, H, Lq, D), mk(B, H, Nc, D), mk(B, H, Nc, D)
+    out, lse = ak.context_attention(q, k, v)
+    out_p, lse_p = ak.context_attention(q, k, v, use_triton=False)
+    assert float((out.float() - out_p.float()).abs().max()) <= 2e-2
+    assert float((lse - lse_p).abs().max()) <= 2.5e-3
+    for sl in (slice(0, 3), slice(B - 3, B)):
+        ref_out, ref_lse = ao.context_attention(to_np(q[sl]), to_np(k[sl]), to_np(v[sl]))
+        assert max_abs(to_np(out[sl]), ref_out) <= 2e-2
+        assert max_abs(to_np(lse[sl]), ref_lse) <= 2.5e-3
+
+
 def test_context_attention_split_context_large(device):
     """Long context, few query rows: the split-context schedule with the LSE combine."""
     ak = _ak()
