@@ -272,6 +272,31 @@ def test_decode_attention_stream_chunk_shapes(device, stream_chunk_shape, dtype,
     _decode_case(device, dtype, B, H, Lq, Nc, D, n_buf, cap, with_new, True, scale=0.6, overlapped=True)
 
 
+@pytest.mark.parametrize("n_buf", [5, 150])
+def test_decode_attention_wave_priorities_do_not_change_results(device, tuning, n_buf):
+    """The two passes of an overlapped call choose their wave priorities from the buffer length
+    (ARTAB_STREAM_CALM: the buffer pass stays at the base priority up to that many rows;
+    ARTAB_CTX_YIELD: the context pass runs a step lower from that many rows on).  Priorities decide
+    who is issued first, never what is computed: every setting must give the same bits."""
+    ak = _ak()
+    tuning(ARTAB_SMALL=0)
+    dtype, B, H, Nc, D, cap = torch.bfloat16, 96, 8, 4096, 32, 160
+    q, k_ctx, v_ctx = (t.to(device) for t in _ctx_inputs(B, H, 2, Nc, D, dtype, seed=11, scale=0.6))
+    kb, vb = randn((B, H, cap, D), 12, dtype, 0.6).to(device), randn((B, H, cap, D), 13, dtype, 0.6).to(device)
+    kn, vn = randn((B, H, 1, D), 14, dtype, 0.6).to(device), randn((B, H, 1, D), 15, dtype, 0.6).to(device)
+    side = torch.cuda.Stream(device=device)
+    outs = []
+    for calm, give_way in ((None, None), (0, 0), (1000, 1), (0, 1), (1000, 0)):
+        tuning(ARTAB_STREAM_CALM=calm, ARTAB_CTX_YIELD=give_way)
+        outs.append(ak.decode_attention(q, k_ctx, v_ctx, kb.clone(), vb.clone(), n_buf, kn, vn, side_stream=side))
+        torch.cuda.synchronize()
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+    ref, _, _ = ao.decode_step_attention(to_np(q), to_np(k_ctx), to_np(v_ctx), to_np(kb[:, :, :n_buf]),
+                                         to_np(vb[:, :, :n_buf]), to_np(kn), to_np(vn))
+    assert max_abs(to_np(outs[0]), ref) <= 2e-2
+
+
 def test_decode_attention_overlapped_device_length_in_graph(device):
     """The overlapped call recorded into a graph (fork/join inside the capture) with the buffer
     length in device memory: every replay appends one row and must equal the eager plain call."""
