@@ -234,8 +234,11 @@ static hipError_t launch_small_t(const DecodeParams &P, const View &kc, const Vi
 }
 
 // The streaming buffer pass: one wavefront per workgroup.  Two of them fit on a CU beside the context
-// pass; the grid holds up to four per CU, so that with more tasks than that (B*H above 8192) the
-// rest moves in as the context pass leaves (measured at B*H = 32768, 255 rows: 276 -> 257 us).
+// pass, four or five once it has left (LDS).  The grid holds one workgroup per task up to 32 per CU:
+// which wavefront takes which task is then the dispatcher's decision, made when a slot frees up,
+// not a static deal that leaves the late starters with a full share (measured at B*H = 32768, 256
+// steps: 500 target-steps/s with 4 per CU, 506 with 6, 508 with 16, 512 with 32; at B*H = 8192,
+// where 8 per CU already is one per task, no difference).
 template <typename T>
 static hipError_t launch_stream_t(const DecodeParams &P, int Lq, hipStream_t stream) {
     const long pairs = static_cast<long>(P.B) * P.H;
@@ -245,8 +248,8 @@ static hipError_t launch_stream_t(const DecodeParams &P, int Lq, hipStream_t str
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
         cus = 256;
     const long tasks = (pairs + 3) / 4;  // of the 4-pair chunk shape; the 16-pair shape leaves the surplus idle
-    long per_cu = 4;
-    if (const int v = tune(kTuneStreamPerCu, 0); v >= 1 && v <= 4) per_cu = v;
+    long per_cu = 32;
+    if (const int v = tune(kTuneStreamPerCu, 0); v >= 1 && v <= 32) per_cu = v;
     dim3 grid(static_cast<unsigned>(tasks < per_cu * cus ? tasks : per_cu * cus)), block(64);
     const int prio = tune(kTuneStreamPrio, 3);
     if (Lq == 1)

@@ -22,7 +22,7 @@ enum Tune : int {
     kTuneSplit,           // ARTAB_SPLIT: number of context slices
     kTuneSmall,           // ARTAB_SMALL: 0 keeps small decode calls off the one-launch kernel
     kTuneStream,          // ARTAB_STREAM: 1 takes the streaming buffer pass without a second stream
-    kTuneStreamPerCu,     // ARTAB_STREAM_PER_CU: workgroups of the streaming buffer pass per compute unit (1..4)
+    kTuneStreamPerCu,     // ARTAB_STREAM_PER_CU: workgroups of the streaming buffer pass per compute unit (1..32)
     kTuneStreamPrio,      // ARTAB_STREAM_PRIO: wave priority of the streaming buffer pass (0..3)
     kTuneStreamShort,     // ARTAB_STREAM_SHORT: buffer rows above which the streaming pass reads 16-row chunks
     kTuneStreamCalm,      // ARTAB_STREAM_CALM: buffer rows up to which the streaming pass keeps the base wave priority
