@@ -25,6 +25,7 @@
 
 namespace artab {
 
+
 constexpr int kFusedRows = 32;       // token rows per workgroup ...
 constexpr int kFusedRowsSmall = 16;  // ... or, when that leaves most of the chip idle, 16: a decode step has
                                      // 2048 rows = 64 workgroups of 32, and everything a workgroup does
@@ -333,9 +334,10 @@ constexpr int kMergeBatch = 9;  // partials fetched per round (8 context slices 
 // and before the merge arithmetic — the place to begin() the next weight stream —, `per_slot(u)`,
 // u = 0 .. kMergeBatch-1, between the slots of the merge arithmetic of the last item: the place for
 // that stream's request_share(u, kMergeBatch), so that its requests queue while the merge computes.
-template <typename T, int D, int NT, int TR, typename Hook, typename SlotHook>
+template <typename T, int D, int NT, int TR, typename WaitHook, typename Hook, typename SlotHook>
 __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const FusedPostParams &P, long row0,
-                                                       int valid, int tid, Hook on_arrival, SlotHook per_slot) {
+                                                       int valid, int tid, WaitHook before_last_slot, Hook on_arrival,
+                                                       SlotHook per_slot) {
     const int dh = D / P.H;          // head dim, a multiple of 8
     const PartialIndex where(P.Lq, P.H, dh);
     const unsigned tok0 = static_cast<unsigned>(row0);  // the launcher keeps rows below 2^31
@@ -346,12 +348,19 @@ __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const
     if (P.n_slots <= kMergeBatch) {
         // Common case: every slot of two items is requested before anything is used, so the
         // thread pays one memory round trip per pair of items (rows beyond `valid` read the
-        // last valid row and are zeroed afterwards: no divergent loads).
+        // last valid row and are zeroed afterwards: no divergent loads).  The last slot is the one
+        // another queue may still be writing (the buffer pass's partial): `before_last_slot()` —
+        // the caller's wait for that queue — runs between the requests for the slots in front of
+        // it and the request for it, so the wait's own round trip travels with the former.
         constexpr int G = ITEMS % 2 == 0 ? 2 : 1;
+        constexpr int NC = kMergeBatch - 1;  // slots in front of the last one, at most
+        const int n_front = P.n_slots - 1;
 #pragma unroll
         for (int it0 = 0; it0 < ITEMS; it0 += G) {
             float lv[G][kMergeBatch];
             u32x4 ov[G][kMergeBatch];
+            const T *po_[G];
+            const float *pl_[G];
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 const int idx = tid + (it0 + g) * NT;
@@ -359,14 +368,20 @@ __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const
                 unsigned prow;
                 int d0;
                 where.locate(tok0 + (r < valid ? r : valid - 1), ch, prow, d0);
-                const T *po = static_cast<const T *>(P.part_o) + static_cast<long>(prow) * dh + d0;
-                const float *pl = P.part_lse + prow;
+                po_[g] = static_cast<const T *>(P.part_o) + static_cast<long>(prow) * dh + d0;
+                pl_[g] = P.part_lse + prow;
 #pragma unroll
-                for (int u = 0; u < kMergeBatch; ++u) {
-                    const int sl = u < P.n_slots ? u : P.n_slots - 1;
-                    lv[g][u] = pl[sl * P.part_rows];
-                    ov[g][u] = *reinterpret_cast<const u32x4 *>(po + sl * o_step);
+                for (int u = 0; u < NC; ++u) {
+                    const int sl = u < n_front ? u : (n_front > 0 ? n_front - 1 : 0);  // repeats are never used
+                    lv[g][u] = pl_[g][sl * P.part_rows];
+                    ov[g][u] = *reinterpret_cast<const u32x4 *>(po_[g] + sl * o_step);
                 }
+            }
+            if (it0 == 0) before_last_slot();
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                lv[g][NC] = pl_[g][n_front * P.part_rows];
+                ov[g][NC] = *reinterpret_cast<const u32x4 *>(po_[g] + n_front * o_step);
             }
             if (it0 + G >= ITEMS) {  // the last round of loads
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
@@ -377,13 +392,13 @@ __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const
             for (int g = 0; g < G; ++g) {
                 const int idx = tid + (it0 + g) * NT;
                 const int r = idx / CPR, ch = idx % CPR;
-                float mx = -INFINITY;
+                float mx = lv[g][NC];
 #pragma unroll
-                for (int u = 0; u < kMergeBatch; ++u) mx = fmaxf(mx, lv[g][u]);  // repeats of the last slot change nothing
+                for (int u = 0; u < NC; ++u) mx = fmaxf(mx, lv[g][u]);  // repeats of a slot change nothing
                 float wsum = 0.f, acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int u = 0; u < kMergeBatch; ++u) {
-                    if (u < P.n_slots) {
+                for (int u = 0; u < kMergeBatch; ++u) {  // slots in their order; the last one last
+                    if (u < n_front || u == NC) {
                         const float w = merge_weight(lv[g][u], mx);
                         wsum += w;
 #pragma unroll
@@ -408,6 +423,7 @@ __device__ __forceinline__ void stage_merged_attention(T *dst, int lds_ld, const
         }
         return;
     }
+    before_last_slot();
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     on_arrival();
 #pragma unroll
@@ -772,12 +788,18 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
     // the first weights travel while the partials are waited for, fetched and merged
     if (kWhole) w_o.start(static_cast<const T *>(P.w_o), nbd, lane, tile);
     if (P.part_o) {
-        if (P.order_wait) {  // the buffer pass's partial comes from the other queue
-            if (tid == 0) order_wait_device(P.order_wait, 0, P.order_limit);
-            __syncthreads();
-        }
+        // (The order of these requests was measured both other ways round — the partials in front
+        // of the weights, the wait in front of everything: the compute unit's address unit is what
+        // the prologue queues for, 16 clocks per 16-byte-per-lane request of a wavefront, and either
+        // change makes the first product wait longer for its weights than it gains on the merge.)
         stage_merged_attention<T, D, NT, TR>(
             a0, LDD, P, row0, valid, tid,
+            [&]() {
+                if (P.order_wait) {  // the buffer pass's partial (the last slot) comes from the other queue
+                    if (tid == 0) order_wait_device(P.order_wait, 0, P.order_limit);
+                    __syncthreads();
+                }
+            },
             [&]() { if (kWhole && ff_active) w_1.begin(static_cast<const T *>(P.w_1), nbf, lane, tile); },
             [&](int u) { if (kWhole && ff_active) w_1.request_share(u, kMergeBatch); });
         if (!kWhole) {

@@ -54,14 +54,19 @@ __device__ __forceinline__ void order_wait_device(unsigned *state, int side, uns
     const unsigned own = order_load(state + (side ? kOrderSide : kOrderMain));
     unsigned seen = order_load(other);  // both requests travel together: one round trip when nothing is pending
     const unsigned target = side ? own + 1u : own;
-    const unsigned long long t0 = wall_clock64();
-    while (static_cast<int>(seen - target) < 0) {
-        if (order_load(failed) != 0u || wall_clock64() - t0 > limit_ticks) {
-            atomicAdd(failed, 1u);
-            break;
-        }
-        __builtin_amdgcn_s_sleep(8);
-        seen = order_load(other);
+    if (static_cast<int>(seen - target) < 0) {
+        // (the wall clock is read only when there is something to wait for: it is one unit of the
+        // chip, and 128 workgroups asking it on their critical path is time the common case —
+        // nothing pending — does not have to spend)
+        const unsigned long long t0 = wall_clock64();
+        do {
+            if (order_load(failed) != 0u || wall_clock64() - t0 > limit_ticks) {
+                atomicAdd(failed, 1u);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(8);
+            seen = order_load(other);
+        } while (static_cast<int>(seen - target) < 0);
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 }
