@@ -199,8 +199,21 @@ struct WeightStream {
             wf[p][b] = *reinterpret_cast<const vec *>(wl[b] + ((p + rot) & (KS - 1)) * TL::kStepStride);
     }
 
-    // The requests that fall to step `ks` of a product of `n_steps` steps when this stream's PF
-    // requests are spread evenly over it.
+    // A product offers the caller kPoints places for the requests of a later stream: one behind
+    // each of its KS contraction steps (0 .. KS-1) and, in four groups (tail_points), KS more in
+    // its epilogue, where the address unit would otherwise idle while the wavefronts exchange row
+    // statistics.
+    static constexpr int kTail = KS;  // (three times as many, i.e. a quarter of the requests at the steps: no difference)
+    static constexpr int kPoints = KS + kTail;
+    template <typename StepHook>
+    static __device__ __forceinline__ void tail_points(int group, StepHook &steps) {
+#pragma unroll
+        for (int i = 0; i < kTail; ++i)
+            if (i * 4 / kTail == group) steps(KS + i);
+    }
+
+    // The requests that fall to point `ks` of `n_steps` when this stream's PF requests are spread
+    // evenly over them.
     __device__ __forceinline__ void request_share(int ks, int n_steps) {
 #pragma unroll
         for (int p = 0; p < PF; ++p)
@@ -223,17 +236,18 @@ struct WeightStream {
 
     // `before` runs ahead of the product — the place to begin() a later stream —, `per_step(ks)`
     // behind the MFMAs of every contraction step — the place for that stream's
-    // request_share(ks, KS); the fragment registers of step ks are free by then, so the later
-    // stream may be this very object (the matrix two ahead goes where the current one was).  For a
-    // stream deeper than its prefetch window both run up front, which is start() of the later
-    // stream ahead of this product.
+    // request_share(ks, kPoints); the fragment registers of step ks are free by then, so the later
+    // stream may be this very object (the matrix two ahead goes where the current one was).  The
+    // caller passes the same hook to tail_points() at four places of the product's epilogue for the
+    // points KS .. kPoints-1.  For a stream deeper than its prefetch window all points run up
+    // front, which is start() of the later stream ahead of this product.
     template <typename Hook = NoHook, typename StepHook = NoHook>
     __device__ __forceinline__ void run(acc_t (&acc)[NB], const T *a_lds, int ld, int c, int hb,
                                         Hook on_arrival = Hook{}, StepHook per_step = StepHook{}) {
         on_arrival();
         if (!kWhole) {
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) per_step(ks);
+            for (int ks = 0; ks < kPoints; ++ks) per_step(ks);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
@@ -528,10 +542,12 @@ enum VecSlot : int { kVecG1 = 0, kVecB1, kVecG2, kVecB2, kVecBias1, kVecG3, kVec
 // red_a / red_b ([NW*32] each) by the pairwise update of Chan et al., which is as robust as the
 // two-pass form.  Callers separate two calls by a barrier (the one that publishes the normalised
 // tile does).
-template <typename T, int NB, int NW, int TR>
+template <typename T, int NB, int NW, int TR, typename Hook = NoHook>
 __device__ __forceinline__ void row_mean_rstd(const float (&v)[NB][Tile<T, TR>::kVals], float *red_a, float *red_b,
-                                              int wave, int c, int hb, int N, float eps, float &mean, float &rstd) {
+                                              int wave, int c, int hb, int N, float eps, float &mean, float &rstd,
+                                              Hook at = Hook{}) {
     typedef Tile<T, TR> TL;
+    at(0);
     constexpr float kLocal = NB * TL::kBlock;
     float s = 0.f;
 #pragma unroll
@@ -553,7 +569,9 @@ __device__ __forceinline__ void row_mean_rstd(const float (&v)[NB][Tile<T, TR>::
         red_a[wave * TR + c] = lmean;
         red_b[wave * TR + c] = q;
     }
+    at(1);
     __syncthreads();
+    at(2);
     float lm[NW], tot = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
@@ -596,15 +614,15 @@ __device__ __forceinline__ void unstage_tile(T *dst, long ld, const T *src, int 
 
 // LayerNorm over the tile rows of v (statistics across all wavefronts), result written as T
 // into the LDS tile `dst` at this lane's (row c, accumulator columns).
-template <typename T, int NB, int NW, int TR>
+template <typename T, int NB, int NW, int TR, typename Hook = NoHook>
 __device__ __forceinline__ void layer_norm_to_lds(const float (&v)[NB][Tile<T, TR>::kVals],
                                                   const float (&gam)[NB][Tile<T, TR>::kVals],
                                                   const float (&bet)[NB][Tile<T, TR>::kVals], const int (&nblk)[NB],
                                                   T *dst, int ld, float *red_a, float *red_b, int wave, int c, int hb,
-                                                  int N, float eps) {
+                                                  int N, float eps, Hook at = Hook{}) {
     typedef Tile<T, TR> TL;
     float mean, rstd;
-    row_mean_rstd<T, NB, NW, TR>(v, red_a, red_b, wave, c, hb, N, eps, mean, rstd);
+    row_mean_rstd<T, NB, NW, TR>(v, red_a, red_b, wave, c, hb, N, eps, mean, rstd, at);
 #pragma unroll
     for (int b = 0; b < NB; ++b)
 #pragma unroll
@@ -614,6 +632,7 @@ __device__ __forceinline__ void layer_norm_to_lds(const float (&v)[NB][Tile<T, T
             for (int e = 0; e < 4; ++e) o[e] = (v[b][4 * g + e] - mean) * rstd * gam[b][4 * g + e] + bet[b][4 * g + e];
             store4f<T>(dst + c * ld + TL::col(nblk[b], g, hb), o[0], o[1], o[2], o[3]);
         }
+    at(3);
 }
 
 // Body of the pre kernel on one TR-row tile.  a0: x tile (row stride D + 8), staged here from
@@ -672,8 +691,9 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
     {
         typename TL::acc_t acc[NB];
         // whole-matrix streams: the k weights go where W_fo's fragments were, step by step
+        auto k_steps = [&](int ks) { if (kWhole) w_a.request_share(ks, WeightStream<T, D, NB, TR>::kPoints); };
         w_a.run(acc, a0, LD, c, hb, [&]() { if (kWhole) w_a.begin(static_cast<const T *>(P.w_qkv), nb_k, lane, tile); },
-                [&](int ks) { if (kWhole) w_a.request_share(ks, WeightStream<T, D, NB, TR>::KS); });
+                k_steps);
         float v[NB][VB];
 #pragma unroll
         for (int b = 0; b < NB; ++b)
@@ -684,7 +704,9 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[b][4 * g + e] = acc[b][4 * g + e] + r[e];
             }
-        layer_norm_to_lds<T, NB, NW, TR>(v, gam, bet, nblk, a1, LD, red_a, red_b, wave, c, hb, D, P.eps);
+        layer_norm_to_lds<T, NB, NW, TR>(v, gam, bet, nblk, a1, LD, red_a, red_b, wave, c, hb, D, P.eps, [&](int e) {
+            if (kWhole) WeightStream<T, D, NB, TR>::tail_points(e, k_steps);
+        });
     }
     __syncthreads();  // y complete in a1; a0 no longer read
     unstage_tile<T, D, NT, TR>(static_cast<T *>(P.y) + row0 * D, D, a1, LD, valid, tid);
@@ -697,6 +719,13 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
         typename TL::acc_t acc[NB];
         // whole-matrix streams: the v weights follow the q weights through w_b during the q pass (k
         // is on its way already); deeper ones: the next pass's weights ahead of this pass
+        auto steps = [&](int ks) {
+            if (kWhole) {
+                if (part == 0) w_b.request_share(ks, WeightStream<T, D, NB, TR>::kPoints);
+            } else if (part < 2) {
+                nxt.request_share(ks, WeightStream<T, D, NB, TR>::kPoints);
+            }
+        };
         cur.run(acc, a1, LD, c, hb,
                 [&]() {
                     if (kWhole) {
@@ -705,21 +734,19 @@ __device__ __forceinline__ void fused_pre_body(const FusedPreParams &P, T *a0, T
                         nxt.begin(static_cast<const T *>(P.w_qkv), part == 0 ? nb_k : nb_v, lane, tile);
                     }
                 },
-                [&](int ks) {
-                    if (kWhole) {
-                        if (part == 0) w_b.request_share(ks, WeightStream<T, D, NB, TR>::KS);
-                    } else if (part < 2) {
-                        nxt.request_share(ks, WeightStream<T, D, NB, TR>::KS);
-                    }
-                });
+                steps);
+        if (kWhole) WeightStream<T, D, NB, TR>::tail_points(0, steps);
         if (part) __syncthreads();  // the previous pass has been copied out of a0
+        if (kWhole) WeightStream<T, D, NB, TR>::tail_points(1, steps);
 #pragma unroll
         for (int b = 0; b < NB; ++b)
 #pragma unroll
             for (int g = 0; g < GB; ++g)
                 store4f<T>(a0 + c * LD + TL::col(nblk[b], g, hb), acc[b][4 * g], acc[b][4 * g + 1],
                            acc[b][4 * g + 2], acc[b][4 * g + 3]);
+        if (kWhole) WeightStream<T, D, NB, TR>::tail_points(2, steps);
         __syncthreads();
+        if (kWhole) WeightStream<T, D, NB, TR>::tail_points(3, steps);
         unstage_tile<T, D, NT, TR>(static_cast<T *>(P.qkv) + row0 * (3 * D) + part * D, 3 * D, a0, LD, valid, tid);
     }
 }
@@ -743,9 +770,10 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_pre_kernel(FusedPre
 // WRITE_OUT the tile is stored to P.out; otherwise it is left in a0, synchronised, for the
 // caller (the next layer's pre body).
 // The caller's requests for what follows this body ride on its last two products:
-// `mid_begin()` / `mid_steps(ks)` around the feed-forward product's contraction steps,
-// `last_begin()` / `last_steps(ks)` around the last product's (see WeightStream::run).  The fused
-// layer boundary requests the next layer's first two matrices there.
+// `mid_begin()` / `mid_steps(ks)` around the feed-forward product's contraction steps and in its
+// epilogue, `last_begin()` / `last_steps(ks)` around the last product's (ks = 0 .. kPoints-1 of
+// the product's stream, see WeightStream::run).  The fused layer boundary requests the next
+// layer's first two matrices there.
 template <typename T, int D, int F, int TR, bool WRITE_OUT, typename MidBegin, typename MidSteps, typename LastBegin,
           typename LastSteps>
 __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0, T *a1, float *red_a, float *red_b,
@@ -820,17 +848,18 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
         load_cols<T, NBD, TR>(vecs + kVecG2 * vec_ld, nbd, hb, gam);
         load_cols<T, NBD, TR>(vecs + kVecB2 * vec_ld, nbd, hb, bet);
         typename TL::acc_t acc[NBD];
+        auto w2_steps = [&](int ks) { if (kWhole) w_2.request_share(ks, WeightStream<T, D, NBD, TR>::kPoints); };
         {   // W_o arrived with the prologue; W_1 is on its way and must not be waited for here
             WeightStream<T, D, NBD, TR> &w = w_o;
 #pragma unroll
             for (int b = 0; b < NBD; ++b)
 #pragma unroll
                 for (int q = 0; q < TL::kVals; ++q) acc[b][q] = 0.f;
-            // W_2 goes where W_o's fragments were, step by step: two matrices (W_1, W_2) are then
-            // on their way while this product's epilogue runs, and the memory pipeline never idles
+            // W_2 goes where W_o's fragments were, half of it step by step and half from the
+            // epilogue: two matrices (W_1, W_2) are on their way while the row statistics are
+            // exchanged, and the address unit has requests to accept while the wavefronts wait
             if (kWhole) w_2.begin(static_cast<const T *>(P.w_2), nbd, lane, tile);
-            w.multiply(acc, a0, LDD, c, hb,
-                       [&](int ks) { if (kWhole) w_2.request_share(ks, WeightStream<T, D, NBD, TR>::KS); });
+            w.multiply(acc, a0, LDD, c, hb, w2_steps);
         }
         if (!kWhole) w_2.start(static_cast<const T *>(P.w_2), nbd, lane, tile);
         float v[NBD][VB];
@@ -843,7 +872,9 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[b][4 * g + e] = acc[b][4 * g + e] + r[e];
             }
-        layer_norm_to_lds<T, NBD, NW, TR>(v, gam, bet, nbd, a1, LDD, red_a, red_b, wave, c, hb, D, P.eps2);
+        layer_norm_to_lds<T, NBD, NW, TR>(v, gam, bet, nbd, a1, LDD, red_a, red_b, wave, c, hb, D, P.eps2, [&](int e) {
+            if (kWhole) WeightStream<T, D, NBD, TR>::tail_points(e, w2_steps);
+        });
     }
     __syncthreads();  // x1 complete in a1; every wavefront is done reading a0
 
@@ -853,8 +884,9 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
         load_cols<T, NBF, TR>(vecs + kVecBias1 * vec_ld, nbf, hb, bias);
         typename TL::acc_t acc[NBF];
         w_1.run(acc, a1, LDD, c, hb, mid_begin, mid_steps);
+        if (kWhole) WeightStream<T, D, NBF, TR>::tail_points(0, mid_steps);
 #pragma unroll
-        for (int b = 0; b < NBF; ++b)
+        for (int b = 0; b < NBF; ++b) {
 #pragma unroll
             for (int g = 0; g < GB; ++g) {
                 float o[4];
@@ -865,10 +897,17 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
                 }
                 store4f<T>(a0 + c * LDF + TL::col(nbf[b], g, hb), o[0], o[1], o[2], o[3]);
             }
+            // the rest of the caller's requests between the blocks of the activation
+            if (kWhole) {
+                if (NBF == 1 || b == 0) WeightStream<T, D, NBF, TR>::tail_points(1, mid_steps);
+                if (NBF == 1 || b == NBF / 2) WeightStream<T, D, NBF, TR>::tail_points(2, mid_steps);
+                if (b == NBF - 1) WeightStream<T, D, NBF, TR>::tail_points(3, mid_steps);
+            }
+        }
     } else {  // a wavefront that sits the feed-forward product out still makes the caller's requests
         mid_begin();
 #pragma unroll
-        for (int ks = 0; ks < WeightStream<T, D, NBF, TR>::KS; ++ks) mid_steps(ks);
+        for (int ks = 0; ks < WeightStream<T, D, NBF, TR>::kPoints; ++ks) mid_steps(ks);
     }
     float gam[NBD][VB], bet[NBD][VB], bias[NBD][VB];
     load_cols<T, NBD, TR>(vecs + kVecG3 * vec_ld, nbd, hb, gam);
@@ -892,7 +931,9 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
             }
         // every wavefront must be done with its last read of a0 (the product above) before the
         // result is written into it: the barrier inside the statistics orders exactly that
-        layer_norm_to_lds<T, NBD, NW, TR>(v, gam, bet, nbd, a0, LDD, red_a, red_b, wave, c, hb, D, P.eps3);
+        layer_norm_to_lds<T, NBD, NW, TR>(v, gam, bet, nbd, a0, LDD, red_a, red_b, wave, c, hb, D, P.eps3, [&](int e) {
+            if (kWhole) WeightStream<T, F, NBD, TR>::tail_points(e, last_steps);
+        });
     }
     __syncthreads();
     if (WRITE_OUT) unstage_tile<T, D, NT, TR>(static_cast<T *>(P.out) + row0 * D, D, a0, LDD, valid, tid);
@@ -943,7 +984,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_pre_kernel(Fus
     fused_post_body<T, D, F, TR, false>(
         P, a0, a1, red_a, red_b, row0, valid,
         [&]() { if (kWhole) next_fo.begin(w_fo, nblk, lane); },
-        [&](int ks) { if (kWhole) next_fo.request_share(ks, WeightStream<T, D, NBF, TR>::KS); },
+        [&](int ks) { if (kWhole) next_fo.request_share(ks, WeightStream<T, D, NBF, TR>::kPoints); },
         [&]() {
             if (kWhole)
                 next_q.begin(w_q, nblk, lane);
@@ -952,9 +993,9 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_pre_kernel(Fus
         },
         [&](int ks) {
             if (kWhole)
-                next_q.request_share(ks, WeightStream<T, F, NB, TR>::KS);
+                next_q.request_share(ks, WeightStream<T, F, NB, TR>::kPoints);
             else
-                next_fo.request_share(ks, WeightStream<T, F, NB, TR>::KS);
+                next_fo.request_share(ks, WeightStream<T, F, NB, TR>::kPoints);
         },
         vecs, VW);
     fused_pre_body<T, D, TR, true, kWhole>(N, a0, a1, red_a, red_b, row0, valid, next_fo, next_q, vecs, VW);
@@ -1348,7 +1389,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void decode_step_boundary_kern
     fused_post_body<T, D, F, TR, false>(
         P, a0, a1, red_a, red_b, row0, valid,
         [&]() { if (kWhole && head_active) w_h1.begin(w_h1p, nbf, lane, tile_t); },
-        [&](int ks) { if (kWhole && head_active) w_h1.request_share(ks, WeightStream<T, D, NBF, TR>::KS); },
+        [&](int ks) { if (kWhole && head_active) w_h1.request_share(ks, WeightStream<T, D, NBF, TR>::kPoints); },
         NoHook{}, NoHook{}, vecs, VW, tile_t);
     SampleEmbedParams S2 = S;  // the same tail, its small operands read from their LDS copies
     S2.norm_g = h_g; S2.norm_b = h_b; S2.w_x = h_wx; S2.b_x = h_bx; S2.w_y = h_wy; S2.b_y = h_by;
