@@ -153,7 +153,7 @@ BENCH_SIGNATURES = {
 
 TUNING_KEYS = ("ARTAB_BM", "ARTAB_SPLIT", "ARTAB_SMALL", "ARTAB_STREAM", "ARTAB_STREAM_PER_CU", "ARTAB_STREAM_PRIO",
                "ARTAB_STREAM_SHORT", "ARTAB_STREAM_CALM", "ARTAB_DENSE_BELOW", "ARTAB_CTX_YIELD", "ARTAB_ORDER_GATE_LAUNCH", "ARTAB_BN", "ARTAB_LEAN",
-               "ARTAB_LEAN_OCC", "ARTAB_NW", "ARTAB_TILE_ROWS")
+               "ARTAB_LEAN_OCC", "ARTAB_NW", "ARTAB_TILE_ROWS", "ARTAB_LAYER_FETCHERS")
 
 _lib: Optional[ctypes.CDLL] = None
 _product_lib: Optional[ctypes.CDLL] = None

@@ -39,7 +39,7 @@ static TuneSlot g_tune[kTuneCount] = {
     {"ARTAB_STREAM_SHORT", false, 0}, {"ARTAB_STREAM_CALM", false, 0},  {"ARTAB_DENSE_BELOW", false, 0},
     {"ARTAB_CTX_YIELD", false, 0},    {"ARTAB_ORDER_GATE_LAUNCH", false, 0},
     {"ARTAB_BN", false, 0},          {"ARTAB_LEAN", false, 0},         {"ARTAB_LEAN_OCC", false, 0},
-    {"ARTAB_NW", false, 0},          {"ARTAB_TILE_ROWS", false, 0},
+    {"ARTAB_NW", false, 0},          {"ARTAB_TILE_ROWS", false, 0},    {"ARTAB_LAYER_FETCHERS", false, 0},
 };
 static const bool g_tune_loaded = [] {
     for (TuneSlot &t : g_tune) {

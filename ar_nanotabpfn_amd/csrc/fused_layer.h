@@ -954,6 +954,39 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_kernel(FusedPo
                                        vecs, VW);
 }
 
+// Body of a fetcher workgroup: reads its share of the matrices w[0 .. N-1] (kib[i] KiB each) once
+// into `junk` (1 KiB of LDS that nobody reads), which brings their lines into the L2 of the XCD it
+// runs on.  Share `part` of `n_parts`, dealt in pieces of 1 KiB over the wavefronts.
+//
+// Between the decode step's layer kernels the context pass streams its keys and values through the
+// L2s, so a layer kernel finds its weights in the memory-side cache at best.  Its weight streams
+// request a matrix one product ahead, which hides that latency only in part: at 2048 rows a
+// product with its epilogue takes 1.5 us, 1.3 us with the lines in L2 and 1.0 us with them in the
+// compute unit's own cache.  A launch that leaves compute units idle therefore carries extra
+// workgroups, behind those that own rows, which do nothing but fetch; each XCD gets its own (ids
+// are dealt round-robin over the 8 XCDs).  Fetching from the workgroups that own rows instead,
+// ahead of their own requests, gains half as much: the prologue's requests are then accepted
+// 0.8 us later, whether the extra loads touch one word per line or read whole lines.
+template <int N, int NT>
+__device__ __forceinline__ void fetch_weights_to_l2(const void *const (&w)[N], const int (&kib)[N], void *junk,
+                                                    int part, int n_parts) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    int total = 0;
+#pragma unroll
+    for (int i = 0; i < N; ++i) total += kib[i];
+    for (int g = part * (NT / 64) + wave; g < total; g += n_parts * (NT / 64)) {
+        const char *p = static_cast<const char *>(w[0]);
+        int l = g;
+#pragma unroll
+        for (int i = 1; i < N; ++i) {
+            if (l < kib[i - 1]) break;
+            l -= kib[i - 1];
+            p = static_cast<const char *>(w[i]);
+        }
+        load_to_lds_16(p + (static_cast<long>(l) << 10) + 16 * lane, junk);
+    }
+}
+
 // The post part of layer L and the pre part of layer L+1 on the same rows: the layer output
 // never leaves LDS, and one launch (with its fixed cost) disappears per layer boundary.
 template <typename T, int D, int F, int TR>
@@ -964,6 +997,19 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_pre_kernel(Fus
     __shared__ __attribute__((aligned(16))) T a1[TR * LDD];
     __shared__ float red_a[NW * TR], red_b[NW * TR];
     const long row0 = static_cast<long>(blockIdx.x) * TR;
+    if (row0 >= P.rows) {
+        // a fetcher (see fetch_weights_to_l2): workgroup `part` of the `n_parts` fetchers of its XCD
+        const int n_tiles = static_cast<int>((P.rows + TR - 1) / TR), xcd = blockIdx.x & 7;
+        const int first = n_tiles + ((xcd - n_tiles) & 7);  // this XCD's first fetcher
+        const int part = (static_cast<int>(blockIdx.x) - first) >> 3;
+        const int n_parts = (static_cast<int>(gridDim.x) - first + 7) >> 3;
+        constexpr int KD = sizeof(T) * D * D / 1024, KF = sizeof(T) * D * F / 1024;  // KiB per matrix
+        const char *w_q = static_cast<const char *>(N.w_qkv);
+        const void *const w[7] = {P.w_o, P.w_1, P.w_2, N.w_fo, w_q, w_q + sizeof(T) * D * D, w_q + 2 * sizeof(T) * D * D};
+        const int kib[7] = {KD, KF, KF, KD, KD, KD, KD};
+        fetch_weights_to_l2<7, NW * 64>(w, kib, a0, part, n_parts);
+        return;
+    }
     const int valid = static_cast<int>(min(static_cast<long>(TR), P.rows - row0));
     constexpr int NB = fused_blocks<T, TR>(D, NW);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;

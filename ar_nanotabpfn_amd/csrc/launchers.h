@@ -34,6 +34,7 @@ enum Tune : int {
     kTuneLeanOcc,         // ARTAB_LEAN_OCC: 4 gives the lean pass 128 registers
     kTuneNW,              // ARTAB_NW: 2 = two wavefronts of two query blocks for 128-row tiles
     kTuneTileRows,        // ARTAB_TILE_ROWS: token rows per workgroup of the layer kernels (16/32)
+    kTuneLayerFetchers,   // ARTAB_LAYER_FETCHERS: weight-fetching workgroups per XCD of a layer-boundary launch (0..32)
     kTuneCount
 };
 // The override of `key` if one is set, else `fallback` (artab_api.hip).

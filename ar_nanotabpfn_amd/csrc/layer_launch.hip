@@ -44,9 +44,22 @@ hipError_t launch_post_d(const FusedPostParams &P, int F, hipStream_t st) {
     return hipGetLastError();
 }
 
+// Fetcher workgroups (fetch_weights_to_l2) of a layer-boundary launch of `tiles` row tiles: 8 per
+// XCD (16 and 32 measured the same or worse) while the tiles leave a quarter of the compute units
+// idle, none beyond.
+int layer_fetchers(long tiles) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        cus = 256;
+    const int per_xcd = tune(kTuneLayerFetchers, 4 * tiles <= 3L * cus ? 8 : 0);
+    return 8 * (per_xcd < 0 ? 0 : (per_xcd > 32 ? 32 : per_xcd));
+}
+
 template <typename T, int D, int TR>
 hipError_t launch_post_pre_d(const FusedPostParams &P, const FusedPreParams &N, int F, hipStream_t st) {
-    dim3 grid(static_cast<unsigned>((P.rows + TR - 1) / TR)), block(fused_waves(D) * 64);
+    const long tiles = (P.rows + TR - 1) / TR;
+    dim3 grid(static_cast<unsigned>(tiles + layer_fetchers(tiles))), block(fused_waves(D) * 64);
     switch (F) {
         case 128: launch_observed(kLaunchLayer, fused_post_pre_kernel<T, D, 128, TR>, grid, block, 0, st, P, N); break;
         case 256: launch_observed(kLaunchLayer, fused_post_pre_kernel<T, D, 256, TR>, grid, block, 0, st, P, N); break;

@@ -85,7 +85,8 @@ const char *artab_last_error(void);
  * environment of the host process cannot change a kernel route between two calls.  Keys:
  * ARTAB_BM, ARTAB_SPLIT, ARTAB_SMALL, ARTAB_STREAM, ARTAB_STREAM_PER_CU, ARTAB_STREAM_PRIO,
  * ARTAB_STREAM_SHORT, ARTAB_STREAM_CALM, ARTAB_DENSE_BELOW, ARTAB_CTX_YIELD, ARTAB_ORDER_GATE_LAUNCH,
- * ARTAB_BN, ARTAB_LEAN, ARTAB_LEAN_OCC, ARTAB_NW, ARTAB_TILE_ROWS (what each selects: csrc/launchers.h).
+ * ARTAB_BN, ARTAB_LEAN, ARTAB_LEAN_OCC, ARTAB_NW, ARTAB_TILE_ROWS, ARTAB_LAYER_FETCHERS (what each
+ * selects: csrc/launchers.h).
  *   artab_tuning_set: enable != 0 sets the override to `value`, enable == 0 removes it (the
  *                     library's own choice applies again).  Not thread-safe against running calls.
  *   artab_tuning_get: returns 1 if an override is set (its value in *value), 0 if not.

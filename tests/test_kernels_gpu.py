@@ -1117,6 +1117,27 @@ def test_layer_post_pre_equals_post_then_pre(device, tile_rows, dtype, rows, D, 
         assert a.shape == b.shape and torch.equal(a, b)
 
 
+@pytest.mark.parametrize("fetchers", [0, 3, 32])
+@pytest.mark.parametrize("rows", [16 * 13 + 5, 16 * 8])
+def test_layer_post_pre_with_weight_fetching_workgroups(device, tuning, fetchers, rows):
+    """A layer-boundary launch may carry workgroups that only fetch weights into the L2 (per XCD,
+    behind the workgroups that own rows): whatever their number, and whether or not the row tiles
+    end on a multiple of the 8 XCDs, the results are those of the two separate launches."""
+    from ar_nanotabpfn_amd import model as m
+
+    D, F, H, dtype = 256, 256, 8, torch.bfloat16
+    torch.manual_seed(1)
+    la = m.TwoStageTransformerLayer(D, H, F).to(device=device, dtype=dtype)
+    lb = m.TwoStageTransformerLayer(D, H, F).to(device=device, dtype=dtype)
+    y = randn((rows, 1, D), 2, dtype, 1.0).to(device)
+    attn = randn((rows, 1, H, D // H), 3, dtype).to(device).transpose(1, 2)
+    ref = lb.pre_attention(la.finish(y, attn))
+    tuning(ARTAB_LAYER_FETCHERS=fetchers, ARTAB_TILE_ROWS=16)
+    got = la.finish_then_pre(y, attn, lb)
+    for a, b in zip(ref, got):
+        assert a.shape == b.shape and torch.equal(a, b)
+
+
 def test_layer_post_pre_falls_back_when_not_covered(device):
     """float32 layers (or widths outside the fused kernels) compose the same result from the
     separate pieces."""
