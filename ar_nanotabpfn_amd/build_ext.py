@@ -34,6 +34,10 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # MFMA accumulators live in VGPRs (no AGPR<->VGPR copies around every product)
     "-mllvm", "-amdgpu-mfma-vgpr-form",
+    # leading scalar kernel arguments (up to 8 of them) arrive in SGPRs, placed there by the command
+    # processor, instead of being loaded from the argument segment by the kernel's first
+    # instructions; kernels whose first argument is a struct are unaffected
+    "-mllvm", "-amdgpu-kernarg-preload-count=8",
     # only the extern "C" entry points leave the library (see EXPORTS below)
     "-fvisibility=hidden",
 ]

@@ -152,6 +152,33 @@ __device__ __forceinline__ void warm_kernel_arguments() {
                  "s"(w[9]), "s"(w[10]), "s"(w[11]), "s"(w[12]), "s"(w[13]), "s"(w[14]), "s"(w[15]));
 }
 
+// The same in two halves, for a kernel whose first memory requests need nothing but arguments that
+// arrive in registers (the leading scalar arguments of a kernel are preloaded into SGPRs by the
+// command processor when the unit is compiled with -amdgpu-kernarg-preload-count): request()
+// starts the loads, the kernel issues those first requests, await() is the one wait.
+template <int BYTES>
+struct KernelArgumentLines {
+    unsigned w[16];
+    // (Inline assembly: as ordinary loads the compiler moves them down to await(), behind the
+    // requests they are meant to travel beside.  The compiler does not know that the registers of
+    // w are written late: EVERY path of the kernel must pass await() before it ends or branches
+    // far, or a register it has reused in the meantime is overwritten when the load lands.)
+    __device__ __forceinline__ void request() {
+        typedef const unsigned __attribute__((address_space(4))) *ConstPtr;
+        ConstPtr ka = (ConstPtr)__builtin_amdgcn_kernarg_segment_ptr();
+        constexpr int LINES = (BYTES + 63) / 64;
+        static_assert(LINES >= 1 && LINES <= 16, "argument blocks of up to 1 KiB");
+#pragma unroll
+        for (int i = 0; i < LINES; ++i) asm volatile("s_load_dword %0, %1, %2" : "=s"(w[i]) : "s"(ka), "n"(64 * i));
+    }
+    __device__ __forceinline__ void await() const {
+        constexpr int LINES = (BYTES + 63) / 64;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < LINES; ++i) asm volatile("" ::"s"(w[i]));
+    }
+};
+
 // A value again, as one the compiler cannot trace (typically the lane index): what rarely
 // executed code derives from it (rows, base addresses) is then computed where it is used instead
 // of being kept in registers across a hot loop that does not need it.

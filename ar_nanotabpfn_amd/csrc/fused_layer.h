@@ -773,13 +773,15 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_pre_kernel(FusedPre
 // `mid_begin()` / `mid_steps(ks)` around the feed-forward product's contraction steps and in its
 // epilogue, `last_begin()` / `last_steps(ks)` around the last product's (ks = 0 .. kPoints-1 of
 // the product's stream, see WeightStream::run).  The fused layer boundary requests the next
-// layer's first two matrices there.
+// layer's first two matrices there.  `after_first_requests()` runs behind the requests for W_o,
+// which need nothing of P but w_o: a kernel that receives that pointer in a register waits for
+// the rest of its arguments there.
 template <typename T, int D, int F, int TR, bool WRITE_OUT, typename MidBegin, typename MidSteps, typename LastBegin,
-          typename LastSteps>
+          typename LastSteps, typename First = NoHook>
 __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0, T *a1, float *red_a, float *red_b,
                                                 long row0, int valid, MidBegin mid_begin, MidSteps mid_steps,
                                                 LastBegin last_begin, LastSteps last_steps, T *vecs, int vec_ld,
-                                                int tile = -1) {
+                                                int tile = -1, First after_first_requests = First{}) {
     typedef Tile<T, TR> TL;
     constexpr int NW = fused_waves(D), NT = NW * 64;
     constexpr int LDD = D + 8, LDF = F + 8;
@@ -800,7 +802,13 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
     WeightStream<T, D, NBD, TR> w_o;
     WeightStream<T, D, NBF, TR> w_1;
     WeightStream<T, F, NBD, TR> w_2;
-    // prologue: everything this tile needs from memory is requested before anything is waited for
+    // whole-matrix streams follow the request-on-arrival rule of WeightStream
+    constexpr bool kWhole = WeightStream<T, D, NBD, TR>::kWhole && WeightStream<T, D, NBF, TR>::kWhole &&
+                            WeightStream<T, F, NBD, TR>::kWhole;
+    // prologue: everything this tile needs from memory is requested before anything is waited for;
+    // the first weights travel while the partials are waited for, fetched and merged
+    if (kWhole) w_o.start(static_cast<const T *>(P.w_o), nbd, lane, tile);
+    after_first_requests();
     dma_tile<T, D, NT, TR>(a1, LDD, static_cast<const T *>(P.y) + row0 * P.ldy, P.ldy, valid, tid);
     if (!P.part_o)
         dma_tile<T, D, NT, TR>(a0, LDD, static_cast<const T *>(P.attn) + row0 * P.lda, P.lda, valid, tid);
@@ -810,11 +818,6 @@ __device__ __forceinline__ void fused_post_body(const FusedPostParams &P, T *a0,
     dma_vector<T, D, NT>(vecs + kVecG3 * vec_ld, P.g3, tid, 3);
     dma_vector<T, D, NT>(vecs + kVecB3 * vec_ld, P.b3, tid, 4);
     dma_vector<T, D, NT>(vecs + kVecBias2 * vec_ld, P.bias_2, tid, 5);
-    // whole-matrix streams follow the request-on-arrival rule of WeightStream
-    constexpr bool kWhole = WeightStream<T, D, NBD, TR>::kWhole && WeightStream<T, D, NBF, TR>::kWhole &&
-                            WeightStream<T, F, NBD, TR>::kWhole;
-    // the first weights travel while the partials are waited for, fetched and merged
-    if (kWhole) w_o.start(static_cast<const T *>(P.w_o), nbd, lane, tile);
     if (P.part_o) {
         // (The order of these requests was measured both other ways round — the partials in front
         // of the weights, the wait in front of everything: the compute unit's address unit is what
@@ -990,8 +993,15 @@ __device__ __forceinline__ void fetch_weights_to_l2(const void *const (&w)[N], c
 // The post part of layer L and the pre part of layer L+1 on the same rows: the layer output
 // never leaves LDS, and one launch (with its fixed cost) disappears per layer boundary.
 template <typename T, int D, int F, int TR>
-__global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_pre_kernel(FusedPostParams P, FusedPreParams N) {
-    warm_kernel_arguments<sizeof(FusedPostParams) + sizeof(FusedPreParams)>();
+__global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_pre_kernel(const void *w_o, long rows,
+                                                                              FusedPostParams P0, FusedPreParams N) {
+    // w_o and rows (= P0.w_o, P0.rows) arrive in registers: the requests for the first matrix go
+    // out while the rest of the arguments is on its way from memory
+    KernelArgumentLines<16 + sizeof(FusedPostParams) + sizeof(FusedPreParams)> arguments;
+    arguments.request();
+    FusedPostParams P = P0;
+    P.w_o = w_o;
+    P.rows = rows;
     constexpr int NW = fused_waves(D), LDD = D + 8, LDF = F + 8, LDM = LDD > LDF ? LDD : LDF;
     __shared__ __attribute__((aligned(16))) T a0[TR * LDM];
     __shared__ __attribute__((aligned(16))) T a1[TR * LDD];
@@ -999,6 +1009,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_pre_kernel(Fus
     const long row0 = static_cast<long>(blockIdx.x) * TR;
     if (row0 >= P.rows) {
         // a fetcher (see fetch_weights_to_l2): workgroup `part` of the `n_parts` fetchers of its XCD
+        arguments.await();
         const int n_tiles = static_cast<int>((P.rows + TR - 1) / TR), xcd = blockIdx.x & 7;
         const int first = n_tiles + ((xcd - n_tiles) & 7);  // this XCD's first fetcher
         const int part = (static_cast<int>(blockIdx.x) - first) >> 3;
@@ -1019,7 +1030,6 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_pre_kernel(Fus
     WeightStream<T, D, NB, TR> next_fo, next_q;
     constexpr int VW = D > F ? D : F;
     __shared__ __attribute__((aligned(16))) T vecs[kVecSlots * VW];
-    stage_pre_vectors<T, D, NW * 64>(N, vecs, VW, threadIdx.x);  // visible after the first barrier below
     // Whole-matrix streams: the next layer's W_fo is requested during the feed-forward product and
     // its q weights during the last product.  Deeper ones: W_fo ahead of the last product, the q
     // weights by the pre body (the order that measured best for them).
@@ -1043,7 +1053,11 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_pre_kernel(Fus
             else
                 next_fo.request_share(ks, WeightStream<T, F, NB, TR>::kPoints);
         },
-        vecs, VW);
+        vecs, VW, -1,
+        [&]() {
+            arguments.await();
+            stage_pre_vectors<T, D, NW * 64>(N, vecs, VW, threadIdx.x);  // visible after the body's first barrier
+        });
     fused_pre_body<T, D, TR, true, kWhole>(N, a0, a1, red_a, red_b, row0, valid, next_fo, next_q, vecs, VW);
 }
 

@@ -61,9 +61,9 @@ hipError_t launch_post_pre_d(const FusedPostParams &P, const FusedPreParams &N, 
     const long tiles = (P.rows + TR - 1) / TR;
     dim3 grid(static_cast<unsigned>(tiles + layer_fetchers(tiles))), block(fused_waves(D) * 64);
     switch (F) {
-        case 128: launch_observed(kLaunchLayer, fused_post_pre_kernel<T, D, 128, TR>, grid, block, 0, st, P, N); break;
-        case 256: launch_observed(kLaunchLayer, fused_post_pre_kernel<T, D, 256, TR>, grid, block, 0, st, P, N); break;
-        default: launch_observed(kLaunchLayer, fused_post_pre_kernel<T, D, 512, TR>, grid, block, 0, st, P, N); break;
+        case 128: launch_observed(kLaunchLayer, fused_post_pre_kernel<T, D, 128, TR>, grid, block, 0, st, P.w_o, P.rows, P, N); break;
+        case 256: launch_observed(kLaunchLayer, fused_post_pre_kernel<T, D, 256, TR>, grid, block, 0, st, P.w_o, P.rows, P, N); break;
+        default: launch_observed(kLaunchLayer, fused_post_pre_kernel<T, D, 512, TR>, grid, block, 0, st, P.w_o, P.rows, P, N); break;
     }
     return hipGetLastError();
 }
