@@ -14,23 +14,46 @@ static int flash_bn(int Dh) { return (Dh == 32 && tune(kTuneBN, 64) == 128) ? 12
 // half a million pairs) the blocks are spread over several launches.
 constexpr int kMaxGridZ = 65535;
 
+// The leading kernel arguments of a launch (FlashEarly): filled for a context-mode launch over one
+// shared context whose K and V have the same head and row strides, all within 31 bits.
+static FlashEarly flash_early(const FlashParams &P) {
+    FlashEarly e = {nullptr, nullptr, 0, 0, 0, 0, 0, 0};
+    constexpr long kIntMax = 0x7fffffffL;
+    if (P.mode == kFlashContext && P.n_groups == 1 && P.kc.sh == P.vc.sh && P.kc.sn == P.vc.sn && P.kc.sn > 0 &&
+        P.kc.sn <= kIntMax && P.kc.sh >= 0 && P.kc.sh <= kIntMax) {
+        e.k = P.kc.p;
+        e.v = P.vc.p;
+        e.sh = static_cast<int>(P.kc.sh);
+        e.sn = static_cast<int>(P.kc.sn);
+        e.kv_per_split = P.kv_per_split;
+        e.nc = P.Nc;
+        e.n_kvg = P.H;
+    }
+    return e;
+}
+
 template <typename Kernel>
 static void launch_one(Kernel kernel, dim3 grid, unsigned block, hipStream_t stream, const FlashParams &P0) {
     const int z_total = static_cast<int>(grid.z);
+    FlashEarly e = flash_early(P0);
     for (int z0 = 0; z0 < z_total; z0 += kMaxGridZ) {
         FlashParams P = P0;
         P.kvg_block0 = z0;
+        e.block0 = z0;
         grid.z = static_cast<unsigned>(z_total - z0 < kMaxGridZ ? z_total - z0 : kMaxGridZ);
         LaunchTiming t;
         const int how = observe_launch(kLaunchFlash, &t);
         if (how == kObserveEvents) {
-            hipExtLaunchKernelGGL(kernel, grid, dim3(block), 0, stream, t.start, t.stop, 0, P);
+            hipExtLaunchKernelGGL(kernel, grid, dim3(block), 0, stream, t.start, t.stop, 0, e.k, e.v, e.sh, e.sn,
+                                  e.kv_per_split, e.nc, e.n_kvg, e.block0, P);
         } else if (how == kObserveStamps) {
             P.stamps = t.stamps;
             P.stamps_capacity = t.stamps_capacity;
-            hipLaunchKernelGGL(kernel, grid, dim3(block), 0, stream, P);
+            hipLaunchKernelGGL(kernel, grid, dim3(block), 0, stream, e.k, e.v, e.sh, e.sn, e.kv_per_split, e.nc, e.n_kvg,
+                               e.block0, P);
         } else {
-            hipLaunchKernelGGL(kernel, grid, dim3(block), 0, stream, P);
+            hipLaunchKernelGGL(kernel, grid, dim3(block), 0, stream, e.k, e.v, e.sh, e.sn, e.kv_per_split, e.nc, e.n_kvg,
+                               e.block0, P);
         }
     }
 }

@@ -80,6 +80,19 @@ struct MfmaOps<f16_t> {
 
 enum FlashMode : int { kFlashContext = 0, kFlashTeacher = 1, kFlashPrefill = 2, kFlashRowMask = 3 };
 
+// The leading, scalar arguments of the kernel, which the command processor places in registers
+// before the first instruction runs (the unit is compiled with -amdgpu-kernarg-preload-count=8):
+// what a plain context launch over one shared context needs to request its first K/V tiles.
+// sn == 0: no early requests (several context groups, K and V laid out differently, strides beyond
+// 32 bits, any other mode); the kernel then works from FlashParams alone.
+struct FlashEarly {
+    const char *k, *v;   // kc.p, vc.p
+    int sh, sn;          // head and row stride of both, in elements
+    int kv_per_split, nc;
+    int n_kvg;           // H (one group)
+    int block0;          // = FlashParams::kvg_block0
+};
+
 struct FlashParams {
     View q, kc, vc, kb, vb, out;
     View kcache, vcache;
@@ -188,8 +201,11 @@ struct BoolTag {
 // wavefront whatever the mode).
 template <typename T, int DH, int QB, int NW, int BN, bool LEAN = false, int OCC = 1, bool PLAIN = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
-void flash_kernel(FlashParams P) {
-    warm_kernel_arguments<sizeof(FlashParams)>();
+void flash_kernel(const char *early_k, const char *early_v, int early_sh, int early_sn, int early_kvps, int early_nc,
+                  int early_nkvg, int early_block0, FlashParams P) {
+    // The leading arguments arrive in registers (FlashEarly); the struct is on its way from memory.
+    KernelArgumentLines<sizeof(FlashEarly) + sizeof(FlashParams)> arguments;
+    arguments.request();
     typedef MfmaOps<T> Ops;
     typedef typename Ops::vec vec;
     constexpr int KS = DH / 16;
@@ -224,6 +240,88 @@ void flash_kernel(FlashParams P) {
 
     // (release: whatever this queue's earlier launches wrote is visible to the watcher that sees
     // the new count)
+    const int tid = threadIdx.x;
+    // wavefront index as a scalar: everything derived from it (the wavefront's rows, its
+    // teacher-forcing key limits) then steers scalar branches instead of exec-mask ones
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+
+    // ---- direct loads of the lean pass.  In its steady state the tiles do not pass through
+    // registers at all: a stage is NI chunks of one KiB, each filled by one direct global->LDS
+    // load (lane l lands at base + 16 l; the lane's source address is whatever piece of the tile
+    // belongs there), dealt over the wavefronts.  The loads are inline assembly: the compiler does
+    // not know of them and therefore does not drain them in front of every LDS read; they are
+    // waited for by hand (vmcnt) in front of the barrier that publishes their stage.
+    constexpr int STAGE_BYTES = LSTAGE * static_cast<int>(sizeof(T));
+    constexpr int NI = STAGE_BYTES / 1024, NKI = NI / 2;
+    static_assert(STAGE_BYTES % 2048 == 0, "a stage is whole chunks of K and as many of V");
+    constexpr int NR = (NI + NW - 1) / NW;
+    static_assert(!LEAN || NR <= 2, "at most two direct loads per wavefront and tile");
+    const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(kv_lds));
+    unsigned d_off[NR];    // this lane's byte offset inside a tile
+    const char *d_src[NR]; // the next tile to request (scalar)
+    long d_step[NR];       // bytes from one tile to the next
+    int n_dma = 0;         // direct loads this wavefront issues per tile
+#pragma unroll
+    for (int r = 0; r < NR; ++r)
+        if (wave + NW * r < NI) ++n_dma;
+    // chunk i of a stage (K chunks, then V chunks) of a source with row stride sn
+    auto direct_load_lane = [&](int i, long sn, unsigned &off, long &step) {
+        const bool is_v = i >= NKI;
+        const int ch = i - (is_v ? NKI : 0);  // (sb, 16-column step) of the chunk
+        const int sbk = ch / KS, cs = ch % KS;
+        // lane l holds 16 bytes: K chunk [hb = l/32][key l%32], V chunk [key l/2][half l%2]
+        const int row = 32 * sbk + (is_v ? lane / 2 : lane % 32);
+        const int col = 16 * cs + 8 * (is_v ? lane % 2 : lane / 32);
+        off = static_cast<unsigned>((row * sn + col) * static_cast<long>(sizeof(T)));
+        step = static_cast<long>(BN) * sn * static_cast<long>(sizeof(T));
+    };
+    auto dma_tile = [&](auto stage_) {
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int i = wave + NW * r;
+            if (i < NI) {
+                const unsigned m0v = lds_base + stage_ * STAGE_BYTES + i * 1024;
+                unsigned m0_saved;  // M0 (the LDS base of a direct load) is left as it was found
+                asm volatile(
+                    "s_mov_b32 %0, m0\n\t"
+                    "s_mov_b32 m0, %1\n\t"
+                    "global_load_lds_dwordx4 %2, %3\n\t"
+                    "s_mov_b32 m0, %0"
+                    : "=&s"(m0_saved)
+                    : "s"(m0v), "v"(d_off[r]), "s"(d_src[r]));
+            }
+            d_src[r] += d_step[r];
+        }
+    };
+    // The plain context launch requests its first NST - 1 tiles right here, from the arguments that
+    // arrived in registers: the tiles travel while the argument struct is fetched and the rest of
+    // the prologue (a chain of scalar loads and branches, about a microsecond) runs.
+    bool early_tiles = false;
+    if constexpr (LEAN && PLAIN) {
+        if (early_sn > 0) {
+            const int kvg_e =
+                __builtin_amdgcn_readfirstlane((early_block0 + static_cast<int>(blockIdx.z)) * 8 + (blockIdx.x & 7));
+            const int begin_e = __builtin_amdgcn_readfirstlane(blockIdx.x >> 3) * early_kvps;
+            const int end_e = min(early_nc, begin_e + early_kvps);
+            if (kvg_e < early_nkvg && (end_e - begin_e) / BN >= NST - 1) {
+                early_tiles = true;
+#pragma unroll
+                for (int r = 0; r < NR; ++r) {
+                    const int i = wave + NW * r;
+                    direct_load_lane(i, early_sn, d_off[r], d_step[r]);
+                    d_src[r] = (i >= NKI ? early_v : early_k) +
+                               (static_cast<long>(kvg_e) * early_sh + static_cast<long>(begin_e) * early_sn) *
+                                   static_cast<long>(sizeof(T));
+                }
+                dma_tile(std::integral_constant<int, 0>{});
+                dma_tile(std::integral_constant<int, 1>{});
+#pragma unroll
+                for (int t = 2; t < NST - 1; ++t) dma_tile(t);
+            }
+        }
+    }
+    arguments.await();
+
     if (LEAN && threadIdx.x == 0) redo_flag = 0;  // raised after the pass, at least one barrier later
     if (P.started && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
         __hip_atomic_fetch_add(P.started, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
@@ -254,10 +352,6 @@ void flash_kernel(FlashParams P) {
     const int h = __builtin_amdgcn_readfirstlane(h_), g = __builtin_amdgcn_readfirstlane(g_);
     const long kvb = P.n_groups == 1 ? 0 : g;  // batch entry whose K/V this group reads
 
-    const int tid = threadIdx.x;
-    // wavefront index as a scalar: everything derived from it (the wavefront's rows, its
-    // teacher-forcing key limits) then steers scalar branches instead of exec-mask ones
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int c = lane & 31, hb = lane >> 5;
     const int row0_wg = tile * BM;
     const int row0_w = row0_wg + wave * ROWS_W;
@@ -857,55 +951,18 @@ void flash_kernel(FlashParams P) {
         const int n_main = (ctx_end - ctx_begin) / BN;
         bool yield_ = false;  // set once the neighbour's length is known (below)
 
-        // In the steady state the tiles do not pass through registers at all: a stage is NI chunks
-        // of one KiB, each filled by one direct global->LDS load (lane l lands at base + 16 l; the
-        // lane's source address is whatever piece of the tile belongs there), dealt over the
-        // wavefronts.  The loads are inline assembly: the compiler does not know of them and
-        // therefore does not drain them in front of every LDS read; they are waited for by hand
-        // (vmcnt) in front of the barrier that publishes their stage.
-        constexpr int STAGE_BYTES = LSTAGE * static_cast<int>(sizeof(T));
-        constexpr int NI = STAGE_BYTES / 1024, NKI = NI / 2;
-        static_assert(STAGE_BYTES % 2048 == 0, "a stage is whole chunks of K and as many of V");
-        constexpr int NR = (NI + NW - 1) / NW;
-        static_assert(!LEAN || NR <= 2, "at most two direct loads per wavefront and tile");
-        const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(kv_lds));
-        unsigned d_off[NR];
-        const char *d_src[NR];
-        long d_step[NR];
-        int n_dma = 0;  // direct loads this wavefront issues per tile
-#pragma unroll
-        for (int r = 0; r < NR; ++r) {
-            const int i = wave + NW * r;  // scalar: chunk of the stage
-            const bool is_v = i >= NKI;
-            const View &src = is_v ? P.vc : P.kc;
-            const int ch = i - (is_v ? NKI : 0);           // (sb, 16-column step) of the chunk
-            const int sbk = ch / KS, cs = ch % KS;
-            // lane l holds 16 bytes: K chunk [hb = l/32][key l%32], V chunk [key l/2][half l%2]
-            const int row = 32 * sbk + (is_v ? lane / 2 : lane % 32);
-            const int col = 16 * cs + 8 * (is_v ? lane % 2 : lane / 32);
-            d_off[r] = static_cast<unsigned>((row * src.sn + col) * static_cast<long>(sizeof(T)));
-            d_step[r] = static_cast<long>(BN) * src.sn * static_cast<long>(sizeof(T));
-            d_src[r] = reinterpret_cast<const char *>(view_row<T>(src, kvb, h, ctx_begin));
-            if (i < NI) ++n_dma;
-        }
-        auto dma_tile = [&](auto stage_) {
+        // (the direct-load machinery — d_off, d_src, d_step, dma_tile — sits at kernel scope: the
+        // plain context launch starts it from its leading arguments before this pass is reached)
+        if (!early_tiles) {
 #pragma unroll
             for (int r = 0; r < NR; ++r) {
-                const int i = wave + NW * r;
-                if (i < NI) {
-                    const unsigned m0v = lds_base + stage_ * STAGE_BYTES + i * 1024;
-                    unsigned m0_saved;  // M0 (the LDS base of a direct load) is left as it was found
-                    asm volatile(
-                        "s_mov_b32 %0, m0\n\t"
-                        "s_mov_b32 m0, %1\n\t"
-                        "global_load_lds_dwordx4 %2, %3\n\t"
-                        "s_mov_b32 m0, %0"
-                        : "=&s"(m0_saved)
-                        : "s"(m0v), "v"(d_off[r]), "s"(d_src[r]));
-                }
-                d_src[r] += d_step[r];
+                const int i = wave + NW * r;  // scalar: chunk of the stage
+                const bool is_v = i >= NKI;
+                const View &src = is_v ? P.vc : P.kc;
+                direct_load_lane(i, src.sn, d_off[r], d_step[r]);
+                d_src[r] = reinterpret_cast<const char *>(view_row<T>(src, kvb, h, ctx_begin));
             }
-        };
+        }
 
         // Every other tile (the partial last context tile, buffer tiles of teacher forcing) goes
         // the general way: per-lane pointers, row guards, zero fill.
@@ -1078,10 +1135,12 @@ void flash_kernel(FlashParams P) {
                 // register-staged tiles below, the compiler has to assume one of their loads
                 // pending when the paths meet and drains the memory counter — the queries
                 // included — in front of the first direct load: a whole round trip.
-                dma_tile(std::integral_constant<int, 0>{});
-                dma_tile(std::integral_constant<int, 1>{});
+                if (!early_tiles) {
+                    dma_tile(std::integral_constant<int, 0>{});
+                    dma_tile(std::integral_constant<int, 1>{});
 #pragma unroll
-                for (int t = 2; t < NST - 1; ++t) dma_tile(t);
+                    for (int t = 2; t < NST - 1; ++t) dma_tile(t);
+                }
             } else {
                 if (n_main > 0) {
                     dma_tile(std::integral_constant<int, 0>{});
