@@ -49,6 +49,7 @@ static void launch_one(Kernel kernel, dim3 grid, unsigned block, hipStream_t str
         } else if (how == kObserveStamps) {
             P.stamps = t.stamps;
             P.stamps_capacity = t.stamps_capacity;
+            e.block0 |= kFlashStampedBit;
             hipLaunchKernelGGL(kernel, grid, dim3(block), 0, stream, e.k, e.v, e.sh, e.sn, e.kv_per_split, e.nc, e.n_kvg,
                                e.block0, P);
         } else {

@@ -90,8 +90,9 @@ struct FlashEarly {
     int sh, sn;          // head and row stride of both, in elements
     int kv_per_split, nc;
     int n_kvg;           // H (one group)
-    int block0;          // = FlashParams::kvg_block0
+    int block0;          // = FlashParams::kvg_block0; bit 30 (kFlashStampedBit) set: FlashParams::stamps is set
 };
+constexpr int kFlashStampedBit = 1 << 30;
 
 struct FlashParams {
     View q, kc, vc, kb, vb, out;
@@ -141,9 +142,12 @@ struct FlashParams {
 // last ticket at the end (it is the last to finish by definition).
 constexpr unsigned kStampStarters = 16;
 
-__device__ __forceinline__ void flash_stamp_start(const FlashParams &P) {  // first thread of a workgroup
+// `t_entry`: the clock as the workgroup read it with its first instructions (a stamped launch says
+// so in its leading arguments, see FlashEarly::block0), or 0.
+__device__ __forceinline__ void flash_stamp_start(const FlashParams &P, unsigned long long t_entry) {  // first thread of a workgroup
     if (P.stamps && blockIdx.x < kStampStarters && blockIdx.y == 0 && blockIdx.z == 0)
-        __hip_atomic_fetch_min(&P.stamps[2], wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_fetch_min(&P.stamps[2], t_entry ? t_entry : wall_clock64(), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // First thread of a workgroup that is done.  Relaxed throughout: every access to the array is an
@@ -297,10 +301,14 @@ void flash_kernel(const char *early_k, const char *early_v, int early_sh, int ea
     // arrived in registers: the tiles travel while the argument struct is fetched and the rest of
     // the prologue (a chain of scalar loads and branches, about a microsecond) runs.
     bool early_tiles = false;
+    unsigned long long t_entry = 0;  // a stamped launch starts its clock here, not behind the arguments' arrival
+    if ((early_block0 & kFlashStampedBit) && blockIdx.x < kStampStarters && blockIdx.y == 0 && blockIdx.z == 0 &&
+        wave == 0)
+        t_entry = wall_clock64();
     if constexpr (LEAN && PLAIN) {
         if (early_sn > 0) {
-            const int kvg_e =
-                __builtin_amdgcn_readfirstlane((early_block0 + static_cast<int>(blockIdx.z)) * 8 + (blockIdx.x & 7));
+            const int kvg_e = __builtin_amdgcn_readfirstlane(
+                ((early_block0 & ~kFlashStampedBit) + static_cast<int>(blockIdx.z)) * 8 + (blockIdx.x & 7));
             const int begin_e = __builtin_amdgcn_readfirstlane(blockIdx.x >> 3) * early_kvps;
             const int end_e = min(early_nc, begin_e + early_kvps);
             if (kvg_e < early_nkvg && (end_e - begin_e) / BN >= NST - 1) {
@@ -325,7 +333,7 @@ void flash_kernel(const char *early_k, const char *early_v, int early_sh, int ea
     if (LEAN && threadIdx.x == 0) redo_flag = 0;  // raised after the pass, at least one barrier later
     if (P.started && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
         __hip_atomic_fetch_add(P.started, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-    if (threadIdx.x == 0) flash_stamp_start(P);
+    if (threadIdx.x == 0) flash_stamp_start(P, t_entry);
 
     // ---- workgroup -> (kv-sharing group, q tile, context split).  The grid is three-dimensional
     // so that none of this takes an integer division (three of them were 0.4 us of every launch):
