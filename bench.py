@@ -599,10 +599,10 @@ def reference_shapes(device):
     print(json.dumps({"reference_shapes": rows}))
 
 
-# Measured with rocprofv3 (median over the decode launches): 9338.5 KiB x 2.0 fetched,
+# Measured with rocprofv3 (median over the decode launches): 9344.0 KiB x 2.0 fetched,
 # 10240.0 KiB written (the partial outputs leave in 16-bit, their LSE in fp32 as 8-byte pieces that
 # cost a 32-byte sector each: 1.5 MiB more than the values; no scratch memory).
-CONTEXT_PASS_HBM_BYTES = int(9338.5 * 1024 * 2.0 + 10240.0 * 1024)
+CONTEXT_PASS_HBM_BYTES = int(9344.0 * 1024 * 2.0 + 10240.0 * 1024)
 
 
 def kernel_shapes(device):
