@@ -219,16 +219,24 @@ template <typename T>
 static hipError_t launch_small_t(const DecodeParams &P, const View &kc, const View &vc, int Nc, int Dh, int Lq,
                                  hipStream_t stream) {
     dim3 grid(static_cast<unsigned>((P.B + kSmallTraj - 1) / kSmallTraj) * P.H), block(kSmallWaves * 64);
+    // the context as leading scalar arguments (the caller has checked that the strides fit)
+    const char *kp = kc.p, *vp = vc.p;
+    const int ksh = static_cast<int>(kc.sh), ksn = static_cast<int>(kc.sn), vsh = static_cast<int>(vc.sh),
+              vsn = static_cast<int>(vc.sn);
     if (Dh == 32) {
         if (Lq == 1)
-            launch_observed(kLaunchSmallDecode, decode_small_kernel<T, 32, 1>, grid, block, 0, stream, P, kc, vc, Nc);
+            launch_observed(kLaunchSmallDecode, decode_small_kernel<T, 32, 1>, grid, block, 0, stream, kp, vp, ksh, ksn, vsh,
+                            vsn, P.H, Nc, P);
         else
-            launch_observed(kLaunchSmallDecode, decode_small_kernel<T, 32, 2>, grid, block, 0, stream, P, kc, vc, Nc);
+            launch_observed(kLaunchSmallDecode, decode_small_kernel<T, 32, 2>, grid, block, 0, stream, kp, vp, ksh, ksn, vsh,
+                            vsn, P.H, Nc, P);
     } else {
         if (Lq == 1)
-            launch_observed(kLaunchSmallDecode, decode_small_kernel<T, 64, 1>, grid, block, 0, stream, P, kc, vc, Nc);
+            launch_observed(kLaunchSmallDecode, decode_small_kernel<T, 64, 1>, grid, block, 0, stream, kp, vp, ksh, ksn, vsh,
+                            vsn, P.H, Nc, P);
         else
-            launch_observed(kLaunchSmallDecode, decode_small_kernel<T, 64, 2>, grid, block, 0, stream, P, kc, vc, Nc);
+            launch_observed(kLaunchSmallDecode, decode_small_kernel<T, 64, 2>, grid, block, 0, stream, kp, vp, ksh, ksn, vsh,
+                            vsn, P.H, Nc, P);
     }
     return hipGetLastError();
 }
@@ -564,7 +572,11 @@ static int decode_impl(const artab_view *q, const artab_view *k_ctx, const artab
     const bool shared_ctx = (k_ctx->stride_b == 0 && v_ctx->stride_b == 0) || B == 1;
     bool use_mfma = impl != ARTAB_IMPL_PORTABLE && mfma_shape_ok(dtype, Dh) && aligned && shared_ctx;
     const long rows = static_cast<long>(B) * H * Lq;
-    if (use_mfma && !leave_partials && !order_state && tune(kTuneStream, 0) == 0 &&
+    // (the one-launch kernel takes the context's strides as 32-bit arguments)
+    const auto fits_int = [](int64_t v) { return v >= 0 && v <= 0x7fffffffLL; };
+    const bool ctx_strides_small = fits_int(k_ctx->stride_h) && fits_int(k_ctx->stride_n) &&
+                                   fits_int(v_ctx->stride_h) && fits_int(v_ctx->stride_n);
+    if (use_mfma && !leave_partials && !order_state && tune(kTuneStream, 0) == 0 && ctx_strides_small &&
         small_decode_applies(B, H, Lq, Nc, Dh)) {
         DecodeParams D;
         memset(&D, 0, sizeof(D));

@@ -27,9 +27,16 @@ namespace artab {
 constexpr int kSmallWaves = 8;
 constexpr int kSmallTraj = 8;  // trajectories per workgroup: one per wavefront in phase 2
 
+// The context arrives as the kernel's leading scalar arguments (base pointers; head and row
+// strides in elements, within 31 bits: the launcher checks; head count; length), which the
+// command processor preloads into SGPRs: the first two key blocks of every wavefront are
+// requested before the argument struct, a cold miss of 750 cycles, has been fetched.
 template <typename T, int DH, int LQ>
-__global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodeParams P, View kc, View vc, int Nc) {
-    warm_kernel_arguments<sizeof(DecodeParams) + 2 * sizeof(View) + sizeof(int)>();
+__global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(const char *kc_p, const char *vc_p, int kc_sh,
+                                                                        int kc_sn, int vc_sh, int vc_sn, int n_heads,
+                                                                        int Nc, DecodeParams P) {
+    KernelArgumentLines<40 + sizeof(DecodeParams)> arguments;
+    arguments.request();
     typedef MfmaOps<T> Ops;
     typedef typename Ops::vec vec;
     constexpr int KS = DH / 16, DB = DH / 32, NW = kSmallWaves, NCOL = kSmallTraj * LQ;
@@ -42,10 +49,58 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodePa
     __shared__ float part_lse2[NW][NCOL];
     __shared__ __attribute__((aligned(16))) float part_o[NW][NCOL][DH];
 
-    const int h = blockIdx.x % P.H;
-    const long b0 = static_cast<long>(blockIdx.x / P.H) * kSmallTraj;
+    const int h = blockIdx.x % n_heads;
+    const long b0 = static_cast<long>(blockIdx.x / n_heads) * kSmallTraj;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int c = lane & 31, hb = lane >> 5;
+    const T *const kc_h = reinterpret_cast<const T *>(kc_p) + static_cast<long>(h) * kc_sh;  // this head's context
+    const T *const vc_h = reinterpret_cast<const T *>(vc_p) + static_cast<long>(h) * vc_sh;
+
+    const int n_blocks = (Nc + 31) / 32;
+    const int my_blocks = wave < n_blocks ? (n_blocks - wave + NW - 1) / NW : 0;
+    // operands of a block as they come from global memory: K in MFMA order (row c, 8 elements at
+    // 16 ks + 8 hb), V as 16-byte pieces of a row-major tile (piece lane + 64 x)
+    struct Raw {
+        u32x4 k[KS];
+        u32x4 v[VP];
+    };
+    // Row pointers of the block to be requested next (blocks wave, wave + NW, ... in order): full
+    // blocks advance them by NW * 32 rows; the context's ragged last block computes clamped rows the
+    // long way (rows past the end re-read the last one: their scores are masked and their
+    // probabilities are zero, only finite values are needed).
+    const long k_step = static_cast<long>(NW) * 32 * kc_sn, v_step = static_cast<long>(NW) * 32 * vc_sn;
+    const T *k_ptr = kc_h + static_cast<long>(min(32 * wave + c, Nc - 1)) * kc_sn + 8 * hb;
+    const T *v_ptr[VP];
+#pragma unroll
+    for (int x = 0; x < VP; ++x)
+        v_ptr[x] = vc_h + static_cast<long>(min(32 * wave + (lane + 64 * x) / CPR, Nc - 1)) * vc_sn + 8 * ((lane + 64 * x) % CPR);
+    auto fetch = [&](int blk, Raw &r) {
+        if (32 * blk + 32 <= Nc) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) r.k[ks] = *reinterpret_cast<const u32x4 *>(k_ptr + 16 * ks);
+#pragma unroll
+            for (int x = 0; x < VP; ++x) r.v[x] = *reinterpret_cast<const u32x4 *>(v_ptr[x]);
+        } else {
+            const T *kr = kc_h + static_cast<long>(min(32 * blk + c, Nc - 1)) * kc_sn + 8 * hb;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) r.k[ks] = *reinterpret_cast<const u32x4 *>(kr + 16 * ks);
+#pragma unroll
+            for (int x = 0; x < VP; ++x) {
+                const int idx = lane + 64 * x;
+                r.v[x] = *reinterpret_cast<const u32x4 *>(vc_h + static_cast<long>(min(32 * blk + idx / CPR, Nc - 1)) * vc_sn +
+                                                          8 * (idx % CPR));
+            }
+        }
+        k_ptr += k_step;
+#pragma unroll
+        for (int x = 0; x < VP; ++x) v_ptr[x] += v_step;
+    };
+    // blocks wave, wave + NW, ...: two requested ahead of the one being multiplied; the first two
+    // right here, from the arguments that arrived in registers
+    Raw r0, r1, r2;
+    if (my_blocks > 0) fetch(wave, r0);
+    if (my_blocks > 1) fetch(wave + NW, r1);
+    arguments.await();
 
     // what phase 2 needs from global memory is requested early, so that its round trips (the
     // buffer rows come from HBM) run under phase 1 — but behind the first product: loads return
@@ -78,46 +133,6 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodePa
             qreg[ks] = __builtin_bit_cast(vec, sc);
         }
     }
-
-    const int n_blocks = (Nc + 31) / 32;
-    const int my_blocks = wave < n_blocks ? (n_blocks - wave + NW - 1) / NW : 0;
-    // operands of a block as they come from global memory: K in MFMA order (row c, 8 elements at
-    // 16 ks + 8 hb), V as 16-byte pieces of a row-major tile (piece lane + 64 x)
-    struct Raw {
-        u32x4 k[KS];
-        u32x4 v[VP];
-    };
-    // Row pointers of the block to be requested next (blocks wave, wave + NW, ... in order): full
-    // blocks advance them by NW * 32 rows; the context's ragged last block computes clamped rows the
-    // long way (rows past the end re-read the last one: their scores are masked and their
-    // probabilities are zero, only finite values are needed).
-    const long k_step = static_cast<long>(NW) * 32 * kc.sn, v_step = static_cast<long>(NW) * 32 * vc.sn;
-    const T *k_ptr = view_row<T>(kc, 0, h, min(32 * wave + c, Nc - 1)) + 8 * hb;
-    const T *v_ptr[VP];
-#pragma unroll
-    for (int x = 0; x < VP; ++x)
-        v_ptr[x] = view_row<T>(vc, 0, h, min(32 * wave + (lane + 64 * x) / CPR, Nc - 1)) + 8 * ((lane + 64 * x) % CPR);
-    auto fetch = [&](int blk, Raw &r) {
-        if (32 * blk + 32 <= Nc) {
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) r.k[ks] = *reinterpret_cast<const u32x4 *>(k_ptr + 16 * ks);
-#pragma unroll
-            for (int x = 0; x < VP; ++x) r.v[x] = *reinterpret_cast<const u32x4 *>(v_ptr[x]);
-        } else {
-            const T *kr = view_row<T>(kc, 0, h, min(32 * blk + c, Nc - 1)) + 8 * hb;
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) r.k[ks] = *reinterpret_cast<const u32x4 *>(kr + 16 * ks);
-#pragma unroll
-            for (int x = 0; x < VP; ++x) {
-                const int idx = lane + 64 * x;
-                r.v[x] = *reinterpret_cast<const u32x4 *>(view_row<T>(vc, 0, h, min(32 * blk + idx / CPR, Nc - 1)) +
-                                                          8 * (idx % CPR));
-            }
-        }
-        k_ptr += k_step;
-#pragma unroll
-        for (int x = 0; x < VP; ++x) v_ptr[x] += v_step;
-    };
 
     f32x16 o_acc[DB];
 #pragma unroll
@@ -193,12 +208,8 @@ __global__ __launch_bounds__(kSmallWaves * 64) void decode_small_kernel(DecodePa
     const int n_total2 = P.n_base + committed.n + (P.has_new ? 1 : 0);
 
     {
-        // blocks wave, wave + NW, ...: two requested ahead of the one being multiplied.  Phase 2's
-        // requests follow the first product: loads return in the order of their requests, and the
-        // first product waits for everything requested before it.
-        Raw r0, r1, r2;
-        if (my_blocks > 0) fetch(wave, r0);
-        if (my_blocks > 1) fetch(wave + NW, r1);
+        // Phase 2's requests follow the first product: loads return in the order of their
+        // requests, and the first product waits for everything requested before it.
         int i = 0;
         if (my_blocks > 0) {
             if (2 < my_blocks) fetch(wave + NW * 2, r2);
