@@ -1019,6 +1019,7 @@ __global__ __launch_bounds__(fused_waves(D) * 64) void fused_post_pre_kernel(con
         const void *const w[7] = {P.w_o, P.w_1, P.w_2, N.w_fo, w_q, w_q + sizeof(T) * D * D, w_q + 2 * sizeof(T) * D * D};
         const int kib[7] = {KD, KF, KF, KD, KD, KD, KD};
         fetch_weights_to_l2<7, NW * 64>(w, kib, a0, part, n_parts);
+        wait_all_loads();  // the LDS they land in is this workgroup's until it ends
         return;
     }
     const int valid = static_cast<int>(min(static_cast<long>(TR), P.rows - row0));
