@@ -117,6 +117,26 @@ def test_context_attention_more_head_groups_than_one_grid_holds(device):
         assert max_abs(to_np(lse[sl]), ref_lse) <= 2.5e-3
 
 
+def test_context_attention_first_tiles_from_leading_arguments(device):
+    """The plain context launch over one shared context requests its first K/V tiles from leading
+    scalar kernel arguments when K and V have the same strides, and from the argument struct like
+    every other launch when they have not: the same numbers either way, and the oracle's."""
+    ak = _ak()
+    B, H, Lq, Nc, D = 512, 8, 2, 2048, 32
+    q, k, v = _ctx_inputs(B, H, Lq, Nc, D, torch.bfloat16, scale=0.6)  # k, v: [H, Nc, D], shared
+    qd, kd, vd = q.to(device), k.to(device), v.to(device)
+    out_a, lse_a = ak.context_attention(qd, kd, vd)
+    wide = torch.zeros(H, Nc, 2 * D, device=device, dtype=torch.bfloat16)
+    wide[..., :D] = kd
+    k_strided = wide[..., :D]  # rows twice as far apart as V's
+    assert k_strided.stride(1) != vd.stride(1)
+    out_b, lse_b = ak.context_attention(qd, k_strided, vd)
+    assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b)
+    ref_out, ref_lse = ao.context_attention(to_np(q[:4]), to_np(k), to_np(v))
+    assert max_abs(to_np(out_a[:4]), ref_out) <= 2e-2
+    assert max_abs(to_np(lse_a[:4]), ref_lse) <= 1e-3
+
+
 def test_context_attention_split_context_large(device):
     """Long context, few query rows: the split-context schedule with the LSE combine."""
     ak = _ak()
