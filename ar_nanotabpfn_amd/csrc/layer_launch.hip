@@ -48,10 +48,15 @@ hipError_t launch_post_d(const FusedPostParams &P, int F, hipStream_t st) {
 // XCD (16 and 32 measured the same or worse) while the tiles leave a quarter of the compute units
 // idle, none beyond.
 int layer_fetchers(long tiles) {
+    static int cus_of[16] = {0};  // per device, asked once (a launch of the eager paths should not pay for it)
     int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-        cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) dev = -1;
+    if (dev >= 0) cus = cus_of[dev];
+    if (cus <= 0) {
+        if (dev < 0 || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        if (dev >= 0) cus_of[dev] = cus;
+    }
     const int per_xcd = tune(kTuneLayerFetchers, 4 * tiles <= 3L * cus ? 8 : 0);
     return 8 * (per_xcd < 0 ? 0 : (per_xcd > 32 ? 32 : per_xcd));
 }
